@@ -1,0 +1,155 @@
+/*
+ * tpk.h - C ABI of libtpk_hip.so: the spatial-search kernels of torch-points-kernels for
+ * AMD MI355X (gfx950).
+ *
+ * Every entry point takes plain device pointers and sizes, launches on the HIP stream
+ * passed as `stream` (a hipStream_t cast to void*; NULL = the null stream), never
+ * allocates, never synchronises the host and keeps no state between calls.  The caller
+ * owns all memory.  All arrays are dense row-major ("contiguous").  Outputs need not be
+ * initialised: every element of every output array is written by the call.
+ *
+ * Return value: TPK_OK (0); a negative TPK_ERR_* for a rejected argument (nothing was
+ * launched); or a positive hipError_t reported by the launch.  tpk_status_string() turns
+ * any of them into text.
+ *
+ * Each declaration names the interface of the reference (torch-points3d/
+ * torch-points-kernels, paths relative to its checkout) that it stands in for: the
+ * `*_kernel_wrapper` launchers its pybind host functions call.
+ */
+#ifndef TPK_H
+#define TPK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TPK_OK 0
+#define TPK_ERR_INVALID_ARG (-1) /* negative size, NULL pointer with non-empty data, ... */
+#define TPK_ERR_UNSUPPORTED (-2) /* valid request outside what the kernels cover */
+#define TPK_ERR_WORKSPACE (-3)   /* workspace missing or too small */
+
+/* Library version, major*10000 + minor*100 + patch. */
+int tpk_version(void);
+
+/* Text for a status returned by any entry point (static storage). */
+const char* tpk_status_string(int status);
+
+/* ---------------------------------------------------------------------------------------
+ * Furthest point sampling.
+ * Replaces furthest_point_sampling_kernel_wrapper(b, n, m, dataset, temp, idxs)
+ * (cuda/src/sampling_gpu.cu:146-201, declared cuda/src/sampling.cpp:5-6).
+ *   xyz  (b, n, 3) float32          idx_out (b, npoint) int32
+ * Starts at point 0; squared distances; points with x*x+y*y+z*z <= 1e-3 are never
+ * updated nor selected; ties resolve as the reference's block reduction does.
+ * `workspace` replaces the reference's `temp` tensor: it is needed only when n exceeds
+ * what one workgroup keeps in registers; tpk_fps_workspace_bytes() says how many bytes
+ * (0 = none needed, NULL may be passed).
+ * ------------------------------------------------------------------------------------- */
+size_t tpk_fps_workspace_bytes(int b, int n);
+int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* workspace,
+                size_t workspace_bytes, int32_t* idx_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Ball query, dense layout.
+ * Replaces query_ball_point_kernel_dense_wrapper(b, n, m, radius, nsample, new_xyz, xyz,
+ * idx, dist_out) (cuda/src/ball_query_gpu.cu:97-106, declared cuda/src/ball_query.cpp:5-7).
+ *   new_xyz (b, m, 3) query centres   xyz (b, n, 3) support
+ *   idx (b, m, nsample) int64         dist (b, m, nsample) float32 (squared)
+ * First `nsample` support points in index order with d2 < radius*radius; unused idx slots
+ * repeat the first hit (0 when there is none), unused dist slots are -1.
+ * ------------------------------------------------------------------------------------- */
+int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int nsample,
+                             const float* new_xyz, const float* xyz, int64_t* idx, float* dist,
+                             void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Ball query, packed variable-length layout.
+ * Replaces query_ball_point_kernel_partial_wrapper(batch_size, size_x, size_y, radius,
+ * nsample, x, y, batch_x, batch_y, idx_out, dist_out) (cuda/src/ball_query_gpu.cu:108-118,
+ * declared cuda/src/ball_query.cpp:9-13) together with the offset construction in front of
+ * it (cuda/src/ball_query.cpp:64-73): this entry takes the SORTED per-point cloud ids
+ * themselves and finds each cloud's range on the device, so no device-to-host copy and no
+ * cloud count are needed.
+ *   x (size_x, 3) support   y (size_y, 3) queries   batch_x (size_x) / batch_y (size_y) int64
+ *   idx (size_y, nsample) int64 (indices into x)    dist (size_y, nsample) float32
+ * First `nsample` points of the query's own cloud in index order with d2 <= radius*radius;
+ * unused slots are -1 in both outputs.
+ * ------------------------------------------------------------------------------------- */
+int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int nsample,
+                               const float* x, const float* y, const int64_t* batch_x,
+                               const int64_t* batch_y, int64_t* idx, float* dist, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Three nearest neighbours.
+ * Replaces three_nn_kernel_wrapper(b, n, m, unknown, known, dist2, idx)
+ * (cuda/src/interpolate_gpu.cu:67-76, declared cuda/src/interpolate.cpp:5-6).
+ *   unknown (b, n, 3)   known (b, m, 3)
+ *   dist2 (b, n, 3) float32 squared distances, ascending   idx (b, n, 3) int32
+ * Equal distances keep the lower index first; with m < 3 the missing entries are
+ * (+inf, 0).
+ * ------------------------------------------------------------------------------------- */
+int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* known,
+                     float* dist2, int32_t* idx, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Three-point interpolation, forward and backward.
+ * Replace three_interpolate_kernel_wrapper(b, c, m, n, points, idx, weight, out) and
+ * three_interpolate_grad_kernel_wrapper(b, c, n, m, grad_out, idx, weight, grad_points)
+ * (cuda/src/interpolate_gpu.cu:109-118 and :154-164, declared cuda/src/interpolate.cpp:7-10).
+ *   points (b, c, m)   idx (b, n, 3) int32 in [0, m)   weight (b, n, 3)
+ *   out (b, c, n) = sum_t points[b, c, idx[b, n, t]] * weight[b, n, t]
+ *   grad_points (b, c, m) += grad_out (b, c, n) scattered back (fully written, no pre-zero)
+ * ------------------------------------------------------------------------------------- */
+int tpk_three_interpolate_f32(int b, int c, int m, int n, const float* points,
+                              const int32_t* idx, const float* weight, float* out, void* stream);
+int tpk_three_interpolate_grad_f32(int b, int c, int n, int m, const float* grad_out,
+                                   const int32_t* idx, const float* weight, float* grad_points,
+                                   void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Grouping (gather of feature columns), forward and backward.
+ * The reference has no native code for this: it is `features.gather(2, idx repeated over
+ * channels)` plus autograd (torch_points_kernels/torchpoints.py:129-146).  These two entry
+ * points compute the same without materialising the repeated index.
+ *   features (b, c, n)   idx (b, npoint, nsample) int64 in [0, n)
+ *   out (b, c, npoint, nsample) = features[b, c, idx[b, p, s]]
+ *   grad_features (b, c, n) = scatter-add of grad_out (fully written, no pre-zero)
+ * ------------------------------------------------------------------------------------- */
+int tpk_group_f32(int b, int c, int n, int npoint, int nsample, const float* features,
+                  const int64_t* idx, float* out, void* stream);
+int tpk_group_grad_f32(int b, int c, int n, int npoint, int nsample, const float* grad_out,
+                       const int64_t* idx, float* grad_features, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Chamfer distance, forward (both directions) and backward.
+ * Replace chamfer_dist_kernel_wrapper(xyz1, xyz2) and chamfer_dist_grad_kernel_wrapper(
+ * xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2) (cuda/src/chamfer_dist_gpu.cu:157-184 and
+ * :215-245, declared cuda/include/chamfer_dist.h:4-15), which take tensors; here they take
+ * the raw arrays.
+ *   xyz1 (b, n, 3)  xyz2 (b, m, 3)
+ *   dist1 (b, n) squared distance of each xyz1 point to its nearest xyz2 point, idx1 (b, n)
+ *   int32 its index (lowest index on ties); dist2 (b, m), idx2 (b, m) the other direction.
+ *   grad_xyz1 (b, n, 3), grad_xyz2 (b, m, 3): fully written, no pre-zero needed.
+ * n == 0 or m == 0 yields zeros, as the reference's zero-initialised outputs do.
+ * ------------------------------------------------------------------------------------- */
+int tpk_chamfer_fwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2, float* dist1,
+                        float* dist2, int32_t* idx1, int32_t* idx2, void* stream);
+int tpk_chamfer_fwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
+                        double* dist1, double* dist2, int32_t* idx1, int32_t* idx2,
+                        void* stream);
+int tpk_chamfer_bwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2,
+                        const int32_t* idx1, const int32_t* idx2, const float* grad_dist1,
+                        const float* grad_dist2, float* grad_xyz1, float* grad_xyz2,
+                        void* stream);
+int tpk_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
+                        const int32_t* idx1, const int32_t* idx2, const double* grad_dist1,
+                        const double* grad_dist2, double* grad_xyz1, double* grad_xyz2,
+                        void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPK_H */

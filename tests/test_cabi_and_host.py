@@ -1,0 +1,113 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library exports what include/tpk.h
+declares, the Python layer mirrors the reference's error behaviour, and nothing falls back
+to a CPU implementation."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tpk.h")
+LIB = os.path.join(ROOT, "torch-points-kernels_amd", "torch_points_kernels", "libtpk_hip.so")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tpk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_symbols()
+    for want in (
+        "tpk_fps_f32", "tpk_fps_workspace_bytes", "tpk_ball_query_dense_f32", "tpk_ball_query_partial_f32",
+        "tpk_three_nn_f32", "tpk_three_interpolate_f32", "tpk_three_interpolate_grad_f32", "tpk_group_f32",
+        "tpk_group_grad_f32", "tpk_chamfer_fwd_f32", "tpk_chamfer_fwd_f64", "tpk_chamfer_bwd_f32",
+        "tpk_chamfer_bwd_f64", "tpk_status_string", "tpk_version",
+    ):
+        assert want in names
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(LIB), "libtpk_hip.so is not built (run torch-points-kernels_amd/build.py)"
+    lib = ctypes.CDLL(LIB)
+    for name in _declared_symbols():
+        assert hasattr(lib, name), name
+    lib.tpk_status_string.restype = ctypes.c_char_p
+    assert lib.tpk_status_string(0) == b"ok"
+    assert b"invalid" in lib.tpk_status_string(-1)
+    assert lib.tpk_version() >= 100
+    lib.tpk_fps_workspace_bytes.restype = ctypes.c_size_t
+    assert lib.tpk_fps_workspace_bytes(4, 16384) == 0
+    assert lib.tpk_fps_workspace_bytes(4, 50000) == 4 * 50000 * 4
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    lib = ctypes.CDLL(LIB)
+    null = ctypes.c_void_p(0)
+    # negative sizes / missing pointers are rejected before anything is launched
+    assert lib.tpk_three_nn_f32(-1, 4, 4, null, null, null, null, null) == -1
+    assert lib.tpk_three_nn_f32(1, 4, 4, null, null, null, null, null) == -1
+    assert lib.tpk_ball_query_dense_f32(1, 4, 4, ctypes.c_float(0.1), -3, null, null, null, null, null) == -1
+    assert lib.tpk_fps_f32(1, 4, 2, null, null, ctypes.c_size_t(0), null, null) == -1
+    # empty problems succeed trivially
+    assert lib.tpk_three_nn_f32(0, 4, 4, null, null, null, null, null) == 0
+    assert lib.tpk_group_f32(0, 1, 1, 1, 1, null, null, null, null) == 0
+
+
+def test_python_api_errors_match_the_reference(tpk):
+    x = torch.zeros(2, 10, 3)
+    # reference torchpoints.py:32-33
+    with pytest.raises(ValueError):
+        tpk.furthest_point_sample(x, 11)
+    # reference torchpoints.py:57-58
+    with pytest.raises(ValueError):
+        tpk.three_nn(torch.zeros(1, 2, 3), x[:1])
+    # reference torchpoints.py:201-218
+    with pytest.raises(Exception, match="mode should be defined"):
+        tpk.ball_query(0.1, 4, x, x, mode=None)
+    with pytest.raises(Exception, match="should be provided"):
+        tpk.ball_query(0.1, 4, x[0], x[0], mode="partial_dense")
+    with pytest.raises(Exception, match="should not be provided"):
+        tpk.ball_query(0.1, 4, x, x, mode="dense", batch_x=torch.zeros(10).long())
+    with pytest.raises(Exception, match="unrecognized mode"):
+        tpk.ball_query(0.1, 4, x, x, mode="sparse")
+    with pytest.raises(AssertionError):
+        tpk.ball_query(0.1, 4, x[0], x[0], mode="DENSE")
+    with pytest.raises(AssertionError):
+        tpk.ball_query(0.1, 4, x[0], x[0], mode="PARTIAL_DENSE", batch_x=torch.zeros(3).long(),
+                       batch_y=torch.zeros(10).long())
+    # reference chamfer_dist.py:43-44 and :10-11
+    from torch_points_kernels.chamfer_dist import ChamferFunction, chamfer_dist
+
+    with pytest.raises(ValueError):
+        chamfer_dist(torch.zeros(4, 3), torch.zeros(1, 4, 3))
+    with pytest.raises(NotImplementedError):
+        ChamferFunction.apply(x, x)
+
+
+def test_cpu_tensors_raise_instead_of_falling_back(tpk):
+    x = torch.rand(1, 16, 3)
+    with pytest.raises(NotImplementedError):
+        tpk.ball_query(0.5, 4, x, x)
+    with pytest.raises(NotImplementedError):
+        tpk.furthest_point_sample(x, 4)
+    with pytest.raises(NotImplementedError):
+        tpk.three_nn(x, x)
+    with pytest.raises(NotImplementedError):
+        tpk.three_interpolate(torch.rand(1, 2, 16), torch.zeros(1, 16, 3, dtype=torch.int32), torch.rand(1, 16, 3))
+    with pytest.raises(NotImplementedError):
+        tpk.grouping_operation(torch.rand(1, 2, 16), torch.zeros(1, 4, 2, dtype=torch.long))
+
+
+def test_product_package_does_not_reference_the_oracle():
+    pkg = os.path.join(ROOT, "torch-points-kernels_amd")
+    for dirpath, _, files in os.walk(pkg):
+        if os.sep + "build" in dirpath:
+            continue
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)

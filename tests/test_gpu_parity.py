@@ -1,0 +1,516 @@
+"""Parity of the HIP path with the oracle, on the GPU, through the package's public API
+(Python layer -> points_cuda extension -> C ABI -> kernels).
+
+Bar: integer outputs (neighbour / sample / argmin indices, hit counts) bit-exact; ball-query,
+three_nn and chamfer distances bit-exact too (same unfused fp32 arithmetic); interpolated
+features bit-exact forward; gradients (atomic accumulation, unordered) within
+rtol 1e-5 / atol 1e-6 of the oracle's in-order sums.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    print("\n[gpu-case] %s" % request.node.nodeid, file=sys.stderr, flush=True)
+    yield
+    torch.cuda.synchronize()
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+# ------------------------------------------------------------------ known answers on the GPU
+
+
+def test_kat_ball_query_dense(tpk, dev):
+    # reference test/test_ballquerry.py:18-23
+    a = torch.tensor([[[0, 0, 0], [1, 0, 0], [2, 0, 0]], [[0, 0, 0], [1, 0, 0], [2, 0, 0]]]).float().to(dev)
+    b = torch.tensor([[[0, 0, 0]], [[3, 0, 0]]]).float().to(dev)
+    idx, dist = tpk.ball_query(1.01, 2, a, b)
+    assert idx.dtype == torch.int64 and dist.dtype == torch.float32
+    np.testing.assert_array_equal(_np(idx), [[[0, 1]], [[2, 2]]])
+    np.testing.assert_array_equal(_np(dist), np.array([[[0, 1]], [[1, -1]]], np.float32))
+    with pytest.raises(NotImplementedError):
+        tpk.ball_query(1.01, 2, a, b, sort=True)  # reference torchpoints.py:152-153
+
+
+def test_kat_ball_query_partial(tpk, dev):
+    # reference test/test_ballquerry.py:63-78
+    x = torch.tensor([[10, 0, 0], [0.1, 0, 0], [0.2, 0, 0], [0.1, 0, 0]]).float().to(dev)
+    y = torch.tensor([[0, 0, 0]]).float().to(dev)
+    bx = torch.tensor([0, 0, 0, 1]).long().to(dev)
+    by = torch.tensor([0]).long().to(dev)
+    idx, dist2 = tpk.ball_query(0.2, 4, x, y, mode="PARTIAL_DENSE", batch_x=bx, batch_y=by)
+    np.testing.assert_array_equal(_np(idx), [[1, 2, -1, -1]])
+    np.testing.assert_array_almost_equal(_np(dist2), np.array([[0.01, 0.04, -1, -1]], np.float32))
+
+
+def test_kat_fps(tpk, dev):
+    # reference test/test_fps.py:13-16
+    pts = torch.tensor([[[0, 0, 0], [1, 0, 0], [2, 0, 0]], [[-1, 1, 0], [0, 0, 10], [0, 0, 2]]]).float().to(dev)
+    out = tpk.furthest_point_sample(pts, 2)
+    assert out.dtype == torch.int32
+    np.testing.assert_array_equal(_np(out), [[0, 2], [0, 1]])
+
+
+def test_kat_three_nn(tpk, dev):
+    # reference test/test_knn.py:14-20 (values; the GPU op returns euclidean distances)
+    support = torch.tensor([[[0, 0, 0], [1, 0, 0], [2, 0, 0]]]).float().to(dev)
+    query = torch.tensor([[[0, 0, 0]] * 3]).float().to(dev)
+    dist, idx = tpk.three_nn(query, support)
+    assert idx.dtype == torch.int32
+    np.testing.assert_array_equal(_np(idx)[0, 0], [0, 1, 2])
+    np.testing.assert_array_equal(_np(dist)[0, 0], [0.0, 1.0, 2.0])
+
+
+def test_kat_grouping(tpk, dev):
+    # reference test/test_grouping.py:13-41
+    features = torch.tensor(
+        [[[0, 10, 0], [1, 11, 0], [2, 12, 0]], [[100, 110, 120], [101, 111, 121], [102, 112, 122]]]
+    ).float()
+    idx = torch.tensor([[[1, 0], [0, 0]], [[0, 1], [1, 2]]]).long()
+    expected = np.array(
+        [
+            [[[10, 0], [0, 0]], [[11, 1], [1, 1]], [[12, 2], [2, 2]]],
+            [[[100, 110], [110, 120]], [[101, 111], [111, 121]], [[102, 112], [112, 122]]],
+        ]
+    )
+    np.testing.assert_array_equal(_np(tpk.grouping_operation(features.to(dev), idx.to(dev))), expected)
+
+
+def test_kat_chamfer(tpk, dev):
+    # reference test/test_chamfer_dist.py:28-39
+    from torch_points_kernels.chamfer_dist import chamfer_dist
+
+    xyz1 = torch.tensor([[[0, 0, 0], [1, 1, 1], [2, 0, 1]]]).float().to(dev)
+    xyz2 = torch.tensor([[[1, 0, 0], [1, 2, 1]]]).float().to(dev)
+    assert abs(chamfer_dist(xyz1, xyz2).item() - 2.333333) < 1e-5
+    assert abs(chamfer_dist(xyz1, xyz2, True).item() - 3.0) < 1e-5
+
+
+# ------------------------------------------------------------------ ball query
+
+
+@pytest.mark.parametrize(
+    "B,N,M,r,ns",
+    [
+        (2, 100, 37, 0.3, 8),       # less than one tile, ragged query block
+        (3, 2049, 65, 0.15, 16),    # one point past a tile boundary
+        (2, 5000, 200, 0.08, 32),   # several tiles, some balls empty
+        (1, 3000, 40, 0.6, 64),     # most balls overflow nsample (early exit)
+        (2, 300, 10, 5.0, 500),     # nsample larger than the cloud
+        (1, 64, 5, 0.2, 1),
+    ],
+)
+def test_ball_query_dense_parity(tpk, oracle, dev, B, N, M, r, ns):
+    g = torch.Generator().manual_seed(100 + N + M)
+    xyz = torch.rand(B, N, 3, generator=g)
+    new_xyz = torch.rand(B, M, 3, generator=g)
+    idx, dist = tpk.ball_query(r, ns, xyz.to(dev), new_xyz.to(dev), mode="dense")
+    want_idx, want_dist = oracle.ball_query_dense(r, ns, xyz.numpy(), new_xyz.numpy())
+    np.testing.assert_array_equal(_np(idx), want_idx)
+    np.testing.assert_array_equal(_np(dist), want_dist)
+
+
+def test_ball_query_dense_boundary_and_empty(tpk, oracle, dev):
+    # points exactly on the sphere are excluded (strict <); empty support gives zeros / -1
+    xyz = torch.tensor([[[0, 0, 0], [0.5, 0, 0], [0.25, 0, 0], [5, 5, 5]]]).float()
+    q = torch.tensor([[[1.0, 0, 0], [100, 0, 0], [0, 0, 0]]]).float()
+    idx, dist = tpk.ball_query(0.5, 3, xyz.to(dev), q.to(dev))
+    wi, wd = oracle.ball_query_dense(0.5, 3, xyz.numpy(), q.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), wd)
+    idx, dist = tpk.ball_query(0.5, 3, torch.zeros(2, 0, 3).to(dev), torch.zeros(2, 4, 3).to(dev))
+    assert (idx == 0).all() and (dist == -1).all()
+
+
+def _packed_case(seed, sizes, qfrac, jitter):
+    g = torch.Generator().manual_seed(seed)
+    xs, ys, bx, by = [], [], [], []
+    for c, n in enumerate(sizes):
+        cloud = torch.rand(n, 3, generator=g)
+        nq = max(0, int(n * qfrac))
+        q = cloud[torch.sort(torch.randperm(n, generator=g)[:nq]).values] + jitter
+        xs.append(cloud)
+        ys.append(q)
+        bx.append(torch.full((n,), c, dtype=torch.long))
+        by.append(torch.full((nq,), c, dtype=torch.long))
+    return torch.cat(xs), torch.cat(ys), torch.cat(bx), torch.cat(by)
+
+
+@pytest.mark.parametrize(
+    "sizes,qfrac,r,ns",
+    [
+        ((50, 70, 10), 0.5, 0.3, 8),            # clouds smaller than a query block: blocks straddle clouds
+        ((3000, 1, 2100, 4500), 0.25, 0.1, 16),  # a one-point cloud in the middle
+        ((2048, 2049), 0.1, 0.2, 64),
+        ((700,), 1.0, 0.5, 1000),
+    ],
+)
+def test_ball_query_partial_parity(tpk, oracle, dev, sizes, qfrac, r, ns):
+    x, y, bx, by = _packed_case(7 + len(sizes), sizes, qfrac, 0.0)
+    idx, dist = tpk.ball_query(r, ns, x.to(dev), y.to(dev), mode="partial_dense", batch_x=bx.to(dev), batch_y=by.to(dev))
+    wi, wd = oracle.ball_query_partial_dense(r, ns, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), wd)
+
+
+def test_ball_query_partial_missing_and_extra_clouds(tpk, oracle, dev):
+    # cloud ids with a gap (0, 2) and queries whose cloud has no support points (id 1, id 3)
+    g = torch.Generator().manual_seed(5)
+    x = torch.rand(300, 3, generator=g)
+    bx = torch.cat([torch.zeros(100), torch.full((200,), 2)]).long()
+    y = torch.rand(90, 3, generator=g)
+    by = torch.cat([torch.zeros(30), torch.ones(20), torch.full((30,), 2)]).long()
+    by = torch.cat([by, torch.full((10,), 3)]).long()
+    idx, dist = tpk.ball_query(0.4, 12, x.to(dev), y.to(dev), mode="partial_dense", batch_x=bx.to(dev), batch_y=by.to(dev))
+    got_idx, got_dist = _np(idx), _np(dist)
+    wi, wd = oracle.ball_query_partial_dense(0.4, 12, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+    # the oracle (like the reference) only walks clouds 0..batch_x[-1]; cloud 3 stays -1
+    np.testing.assert_array_equal(got_idx, wi)
+    np.testing.assert_array_equal(got_dist, wd)
+    assert (got_idx[30:50] == -1).all() and (got_idx[80:] == -1).all()
+
+
+def test_ball_query_full_config1(tpk, oracle, dev):
+    w = W.cfg1_ball_query_dense()
+    idx, dist = tpk.ball_query(w["radius"], w["nsample"], w["xyz"].to(dev), w["new_xyz"].to(dev), mode="dense")
+    wi, wd = oracle.ball_query_dense(w["radius"], w["nsample"], w["xyz"].numpy(), w["new_xyz"].numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), wd)
+    assert int(idx.min()) >= 0  # reference test/test_ballquerry.py:37-40
+
+
+def test_ball_query_full_config4(tpk, oracle, dev):
+    w = W.cfg4_ball_query_partial()
+    x, y, bx, by = (w[k].to(dev) for k in ("x", "y", "batch_x", "batch_y"))
+    idx, dist = tpk.ball_query(w["radius"], w["nsample"], x, y, mode="partial_dense", batch_x=bx, batch_y=by)
+    assert idx.shape == (y.shape[0], w["nsample"])
+    # Size-independent properties over the whole output, evaluated with torch on the GPU:
+    valid = idx >= 0
+    assert ((dist >= 0) == valid).all()
+    cnt = valid.sum(1)
+    pos = torch.arange(w["nsample"], device=dev).unsqueeze(0)
+    assert (valid == (pos < cnt.unsqueeze(1))).all()          # hits first, -1 padding after
+    safe = idx.clamp(min=0)
+    assert (bx[safe][valid] == by.unsqueeze(1).expand_as(idx)[valid]).all()  # own cloud only
+    d = x[safe] - y.unsqueeze(1)
+    d2 = d[..., 0] * d[..., 0] + d[..., 1] * d[..., 1] + d[..., 2] * d[..., 2]
+    assert (d2[valid] == dist[valid]).all()                    # stored distance = recomputed
+    r2 = torch.tensor(w["radius"], dtype=torch.float32) * torch.tensor(w["radius"], dtype=torch.float32)
+    assert (dist[valid] <= r2.item()).all()
+    inc = (idx[:, 1:] > idx[:, :-1]) | ~valid[:, 1:]
+    assert inc.all()                                           # ascending index order
+    # Bit-exact against the oracle on every 5th query (full scan of the whole packed support).
+    sel = torch.arange(0, y.shape[0], 5)
+    wi, wd = oracle.ball_query_partial_dense(
+        w["radius"], w["nsample"], w["x"].numpy(), w["y"][sel].numpy(), w["batch_x"].numpy(), w["batch_y"][sel].numpy())
+    np.testing.assert_array_equal(_np(idx[sel.to(dev)]), wi)
+    np.testing.assert_array_equal(_np(dist[sel.to(dev)]), wd)
+
+
+# ------------------------------------------------------------------ FPS
+
+
+@pytest.mark.parametrize(
+    "B,N,npoint",
+    [(2, 3, 3), (3, 100, 40), (2, 1024, 256), (2, 1500, 300), (2, 4096, 512), (1, 7000, 128), (2, 16384, 200)],
+)
+def test_fps_parity(tpk, oracle, dev, B, N, npoint):
+    g = torch.Generator().manual_seed(N)
+    xyz = torch.randn(B, N, 3, generator=g)
+    out = tpk.furthest_point_sample(xyz.to(dev), npoint)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), npoint))
+
+
+def test_fps_streaming_path_parity(tpk, oracle, dev):
+    # more points than one workgroup keeps in registers
+    g = torch.Generator().manual_seed(77)
+    xyz = torch.rand(2, 20000, 3, generator=g)
+    out = tpk.furthest_point_sample(xyz.to(dev), 150)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), 150))
+
+
+def test_fps_ties_origin_skip_and_exhaustion(tpk, oracle, dev):
+    # duplicated points (exact ties in every round), points near the origin (never eligible)
+    # and more samples than distinct points: all decided by the tie rule.
+    g = torch.Generator().manual_seed(9)
+    base = torch.rand(1, 40, 3, generator=g) + 0.5
+    xyz = torch.cat([base, base, base.flip(1), torch.full((1, 8, 3), 0.01)], 1)[:, torch.randperm(128, generator=g)]
+    for n in (128, 100, 8):
+        pts = xyz[:, :n].contiguous()
+        out = tpk.furthest_point_sample(pts.to(dev), n)
+        np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(pts.numpy(), n))
+    # lattice: many exactly equal distances, larger than one reference block
+    ax = torch.arange(12, dtype=torch.float32)
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3) + 1.0
+    out = tpk.furthest_point_sample(lattice.to(dev), 300)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(lattice.numpy(), 300))
+    # nothing eligible
+    tiny = torch.full((2, 50, 3), 0.001)
+    assert (tpk.furthest_point_sample(tiny.to(dev), 10) == 0).all()
+
+
+def test_fps_full_config2(tpk, oracle, dev):
+    w = W.cfg2_fps()
+    xyz = w["xyz"].to(dev)
+    out = tpk.furthest_point_sample(xyz, w["npoint"])
+    out2 = tpk.furthest_point_sample(xyz, w["npoint"])
+    assert (out == out2).all()  # deterministic
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(w["xyz"].numpy(), w["npoint"]))
+
+
+# ------------------------------------------------------------------ three_nn / three_interpolate
+
+
+@pytest.mark.parametrize("B,n,m", [(2, 3, 1), (2, 5, 2), (3, 70, 3), (2, 1000, 1025), (1, 2500, 4096), (4, 513, 300)])
+def test_three_nn_parity(tpk, oracle, dev, B, n, m):
+    g = torch.Generator().manual_seed(n * 7 + m)
+    unknown = torch.randn(B, n, 3, generator=g)
+    known = torch.randn(B, m, 3, generator=g)
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    dist2, idx = native.three_nn(unknown.to(dev), known.to(dev))
+    wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist2), wd)
+    dist, idx2 = tpk.three_nn(unknown.to(dev), known.to(dev))
+    np.testing.assert_array_equal(_np(dist), np.sqrt(wd))
+
+
+def test_three_nn_ties(tpk, oracle, dev):
+    # duplicated known points: equal distances must keep the lower index first
+    g = torch.Generator().manual_seed(3)
+    k = torch.rand(1, 300, 3, generator=g)
+    known = torch.cat([k, k, k], 1)
+    unknown = torch.rand(1, 257, 3, generator=g)
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    dist2, idx = native.three_nn(unknown.to(dev), known.to(dev))
+    wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist2), wd)
+
+
+def _interp_case(B, C, m, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    feats = torch.randn(B, C, m, generator=g)
+    idx = torch.randint(0, m, (B, n, 3), generator=g, dtype=torch.int32)
+    w = torch.rand(B, n, 3, generator=g)
+    w = w / w.sum(2, keepdim=True)
+    gout = torch.randn(B, C, n, generator=g)
+    return feats, idx, w, gout
+
+
+@pytest.mark.parametrize(
+    "B,C,m,n",
+    [(2, 5, 40, 70), (3, 30, 100, 500), (2, 19, 4096, 3000), (1, 3, 20000, 1500), (1, 4, 40000, 999)],
+)
+def test_three_interpolate_parity(tpk, oracle, dev, B, C, m, n):
+    # m = 20000 leaves room for one row in LDS, m = 40000 for none (direct path)
+    feats, idx, w, gout = _interp_case(B, C, m, n, m + n)
+    f = feats.to(dev).requires_grad_(True)
+    out = tpk.three_interpolate(f, idx.to(dev), w.to(dev))
+    np.testing.assert_array_equal(_np(out), oracle.three_interpolate(feats.numpy(), idx.numpy(), w.numpy()))
+    out.backward(gout.to(dev))
+    want = oracle.three_interpolate_grad(gout.numpy(), idx.numpy(), w.numpy(), m)
+    np.testing.assert_allclose(_np(f.grad), want, rtol=RTOL, atol=ATOL)
+
+
+def test_three_interpolate_colliding_indices(tpk, oracle, dev):
+    # every column points at the same few rows entries: worst case for the atomic accumulation
+    B, C, m, n = 1, 8, 64, 5000
+    feats, _, w, gout = _interp_case(B, C, m, n, 4)
+    idx = torch.zeros(B, n, 3, dtype=torch.int32)
+    idx[..., 1] = 1
+    idx[..., 2] = torch.arange(n) % 2
+    f = feats.to(dev).requires_grad_(True)
+    out = tpk.three_interpolate(f, idx.to(dev), w.to(dev))
+    np.testing.assert_array_equal(_np(out), oracle.three_interpolate(feats.numpy(), idx.numpy(), w.numpy()))
+    out.backward(gout.to(dev))
+    want = oracle.three_interpolate_grad(gout.numpy(), idx.numpy(), w.numpy(), m)
+    # sums of ~5000 terms in a different order: tolerance scaled to the magnitude of the sum
+    np.testing.assert_allclose(_np(f.grad), want, rtol=1e-4, atol=1e-3)
+
+
+def test_interpolate_full_config3a(tpk, oracle, dev):
+    w = W.cfg3a_interpolate()
+    unknown, known = w["unknown"].to(dev), w["known"].to(dev)
+    dist, idx = tpk.three_nn(unknown, known)
+    wd2, wi = oracle.three_nn(w["unknown"].numpy(), w["known"].numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), np.sqrt(wd2))
+    weight = W.inverse_distance_weights(dist)
+    feats = w["features"].to(dev).requires_grad_(True)
+    out = tpk.three_interpolate(feats, idx, weight)
+    np.testing.assert_array_equal(_np(out), oracle.three_interpolate(w["features"].numpy(), wi, _np(weight)))
+    out.backward(w["grad_out"].to(dev))
+    want = oracle.three_interpolate_grad(w["grad_out"].numpy(), wi, _np(weight), known.shape[1])
+    np.testing.assert_allclose(_np(feats.grad), want, rtol=RTOL, atol=ATOL)
+
+
+# ------------------------------------------------------------------ grouping
+
+
+@pytest.mark.parametrize("B,C,N,npoint,nsample", [(2, 3, 10, 4, 2), (2, 17, 1000, 129, 16), (1, 5, 30000, 64, 8), (1, 2, 50000, 40, 4)])
+def test_grouping_parity(tpk, oracle, dev, B, C, N, npoint, nsample):
+    g = torch.Generator().manual_seed(N + npoint)
+    feats = torch.randn(B, C, N, generator=g)
+    idx = torch.randint(0, N, (B, npoint, nsample), generator=g)
+    gout = torch.randn(B, C, npoint, nsample, generator=g)
+    f = feats.to(dev).requires_grad_(True)
+    out = tpk.grouping_operation(f, idx.to(dev))
+    np.testing.assert_array_equal(_np(out), oracle.grouping_operation(feats.numpy(), idx.numpy()))
+    out.backward(gout.to(dev))
+    want = oracle.grouping_operation_grad(gout.numpy(), idx.numpy(), N)
+    np.testing.assert_allclose(_np(f.grad), want, rtol=RTOL, atol=ATOL)
+
+
+def test_grouping_full_config3b(tpk, oracle, dev):
+    w = W.cfg3b_grouping()
+    f = w["features"].to(dev).requires_grad_(True)
+    idx = w["idx"].to(dev)
+    out = tpk.grouping_operation(f, idx)
+    # the reference implementation itself: torch.gather on the repeated index (torchpoints.py:129-146)
+    all_idx = idx.reshape(idx.shape[0], -1).unsqueeze(1).expand(-1, f.shape[1], -1)
+    assert (out == f.detach().gather(2, all_idx).reshape(out.shape)).all()
+    np.testing.assert_array_equal(_np(out[:2]), oracle.grouping_operation(w["features"][:2].numpy(), w["idx"][:2].numpy()))
+    out.backward(w["grad_out"].to(dev))
+    want = oracle.grouping_operation_grad(w["grad_out"].numpy(), w["idx"].numpy(), f.shape[2])
+    np.testing.assert_allclose(_np(f.grad), want, rtol=RTOL, atol=ATOL)
+
+
+# ------------------------------------------------------------------ chamfer
+
+
+@pytest.mark.parametrize("B,n,m", [(1, 3, 2), (2, 300, 515), (2, 1030, 700), (3, 64, 1), (1, 2500, 2047), (2, 1, 9)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_chamfer_parity(tpk, oracle, dev, B, n, m, dtype):
+    g = torch.Generator().manual_seed(n + 3 * m)
+    a = torch.rand(B, n, 3, generator=g, dtype=dtype)
+    b = torch.rand(B, m, 3, generator=g, dtype=dtype)
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    d1, d2, i1, i2 = native.chamfer_dist(a.to(dev), b.to(dev))
+    w1, w2, wi1, wi2 = oracle.chamfer_fwd(a.numpy(), b.numpy())
+    assert i1.dtype == torch.int32 and d1.dtype == dtype
+    np.testing.assert_array_equal(_np(i1), wi1)
+    np.testing.assert_array_equal(_np(i2), wi2)
+    np.testing.assert_array_equal(_np(d1), w1)
+    np.testing.assert_array_equal(_np(d2), w2)
+    g1 = torch.randn(B, n, generator=g, dtype=dtype)
+    g2 = torch.randn(B, m, generator=g, dtype=dtype)
+    ga, gb = native.chamfer_dist_grad(a.to(dev), b.to(dev), i1, i2, g1.to(dev), g2.to(dev))
+    wa, wb = oracle.chamfer_bwd(a.numpy(), b.numpy(), wi1, wi2, g1.numpy(), g2.numpy())
+    np.testing.assert_allclose(_np(ga), wa, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(_np(gb), wb, rtol=RTOL, atol=ATOL)
+
+
+def test_chamfer_ties_take_lowest_index(tpk, oracle, dev):
+    a = torch.zeros(1, 300, 3)
+    b = torch.full((1, 3000, 3), 5.0)
+    b[0, [3, 4, 600, 1100, 2999], 0] = 1.0
+    b[0, [3, 4, 600, 1100, 2999], 1:] = 0.0
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    d1, d2, i1, i2 = native.chamfer_dist(a.to(dev), b.to(dev))
+    w1, w2, wi1, wi2 = oracle.chamfer_fwd(a.numpy(), b.numpy())
+    assert (i1 == 3).all()
+    np.testing.assert_array_equal(_np(i1), wi1)
+    np.testing.assert_array_equal(_np(i2), wi2)  # every b point ties over all of a: index 0
+    np.testing.assert_array_equal(_np(d2), w2)
+
+
+def test_chamfer_gradcheck_double(tpk, dev):
+    # reference test/test_chamfer_dist.py:20-25
+    from torch.autograd import gradcheck
+    from torch_points_kernels.chamfer_dist import ChamferFunction
+
+    g = torch.Generator().manual_seed(1)
+    x = torch.rand(4, 64, 3, generator=g).double().to(dev).requires_grad_(True)
+    y = torch.rand(4, 128, 3, generator=g).double().to(dev).requires_grad_(True)
+    assert gradcheck(ChamferFunction.apply, [x, y])
+
+
+def test_chamfer_full_config5(tpk, oracle, dev):
+    w = W.cfg5_chamfer()
+    a, b = w["xyz1"].to(dev), w["xyz2"].to(dev)
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    d1, d2, i1, i2 = native.chamfer_dist(a, b)
+    # (1) stored distance == distance to the reported neighbour, recomputed with separately
+    #     rounded torch ops in the reference's operand order
+    for da, ia, p, q in ((d1, i1, a, b), (d2, i2, b, a)):
+        near = torch.gather(q, 1, ia.long().unsqueeze(-1).expand(-1, -1, 3))
+        diff = near - p
+        rec = diff[..., 0] * diff[..., 0] + diff[..., 1] * diff[..., 1] + diff[..., 2] * diff[..., 2]
+        assert (rec == da).all()
+    # (2) bit-exact against the oracle for a 512-point subset of the queries of every cloud
+    #     (each query's result depends on the whole other cloud, not on the other queries)
+    sel = torch.arange(5, a.shape[1], a.shape[1] // 512)[:512]
+    w1, _, wi1, _ = oracle.chamfer_fwd(w["xyz1"][:, sel].numpy(), w["xyz2"].numpy())
+    np.testing.assert_array_equal(_np(i1[:, sel.to(dev)]), wi1)
+    np.testing.assert_array_equal(_np(d1[:, sel.to(dev)]), w1)
+    w2, _, wi2, _ = oracle.chamfer_fwd(w["xyz2"][:, sel].numpy(), w["xyz1"].numpy())
+    np.testing.assert_array_equal(_np(i2[:, sel.to(dev)]), wi2)
+    np.testing.assert_array_equal(_np(d2[:, sel.to(dev)]), w2)
+    # (3) backward against the oracle on the full size (linear in the number of points)
+    ga, gb = native.chamfer_dist_grad(a, b, i1, i2, w["grad_dist1"].to(dev), w["grad_dist2"].to(dev))
+    wa, wb = oracle.chamfer_bwd(w["xyz1"].numpy(), w["xyz2"].numpy(), _np(i1), _np(i2),
+                                w["grad_dist1"].numpy(), w["grad_dist2"].numpy())
+    np.testing.assert_allclose(_np(ga), wa, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(_np(gb), wb, rtol=RTOL, atol=ATOL)
+    # (4) determinism of the integer outputs
+    _, _, j1, j2 = native.chamfer_dist(a, b)
+    assert (j1 == i1).all() and (j2 == i2).all()
+
+
+# ------------------------------------------------------------------ the C ABI called directly
+
+
+def test_c_abi_direct_call(oracle, dev):
+    """libtpk_hip.so used without the extension: ctypes + raw device pointers + a stream."""
+    import ctypes
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = ctypes.CDLL(os.path.join(root, "torch-points-kernels_amd", "torch_points_kernels", "libtpk_hip.so"))
+    g = torch.Generator().manual_seed(2)
+    unknown = torch.rand(2, 700, 3, generator=g)
+    known = torch.rand(2, 900, 3, generator=g)
+    u, k = unknown.to(dev), known.to(dev)
+    dist2 = torch.empty(2, 700, 3, device=dev)
+    idx = torch.empty(2, 700, 3, dtype=torch.int32, device=dev)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    st = lib.tpk_three_nn_f32(2, 700, 900, ctypes.c_void_p(u.data_ptr()), ctypes.c_void_p(k.data_ptr()),
+                              ctypes.c_void_p(dist2.data_ptr()), ctypes.c_void_p(idx.data_ptr()),
+                              ctypes.c_void_p(stream.cuda_stream))
+    assert st == 0
+    stream.synchronize()
+    wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist2), wd)
+    # an undersized FPS workspace is refused before any launch
+    pts = torch.rand(1, 20000, 3).to(dev)
+    out = torch.empty(1, 4, dtype=torch.int32, device=dev)
+    st = lib.tpk_fps_f32(1, 20000, 4, ctypes.c_void_p(pts.data_ptr()), None, ctypes.c_size_t(0),
+                         ctypes.c_void_p(out.data_ptr()), None)
+    assert st == -3
+
+
+def test_extension_rejects_bad_tensors(tpk, dev):
+    x = torch.rand(2, 16, 3, device=dev)
+    with pytest.raises(RuntimeError):
+        tpk.ball_query(0.1, 4, x.transpose(0, 1), x)  # not contiguous
+    with pytest.raises(RuntimeError):
+        tpk.ball_query(0.1, 4, x.double(), x.double())  # wrong dtype
+    with pytest.raises(RuntimeError):
+        tpk.three_interpolate(torch.rand(2, 4, 16, device=dev), torch.zeros(2, 8, 3, dtype=torch.int64, device=dev),
+                              torch.rand(2, 8, 3, device=dev))  # idx must be int32, as three_nn returns it

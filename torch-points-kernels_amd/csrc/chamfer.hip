@@ -1,0 +1,371 @@
+// Chamfer distance: nearest-neighbour distance and index in both directions, and the
+// gradient of those distances with respect to both clouds.
+//
+// Forward.  Both directions run in ONE launch (the first part of the grid scans cloud 2
+// for the points of cloud 1, the rest the other way round).  A lane owns Q query points;
+// the scanned cloud streams through LDS as tiles of (x, y, z, pad), read by all lanes at
+// the same address (broadcast).  The scan is a plain all-pairs fp32/fp64 VALU reduction;
+// the inner dimension is 3 and the products must round as the reference's do, so the
+// matrix cores are not used.
+//
+// Per pair the work is 8 flops for the distance; keeping "which candidate was it" next to
+// the minimum would add a compare and two selects per pair.  Instead the scan keeps only
+// the minimum of each group of CHUNK consecutive candidates (min3: half an operation per
+// pair), compares it once per group with the running best (strictly smaller replaces, so
+// the earliest group holding the minimum wins) and remembers the group.  After the scan
+// each lane re-evaluates the CHUNK candidates of its winning group and takes the first
+// whose distance equals the minimum: the same candidate a serial first-strictly-smaller
+// scan (cuda/src/chamfer_dist_gpu.cu:9-155) ends on.
+//
+// Backward (cuda/src/chamfer_dist_gpu.cu:187-245).  Each point's own term is stored
+// plainly by a first kernel (so the outputs need no zero fill), the terms scattered to the
+// matched points of the other cloud are added by a second kernel with hardware float
+// atomics.  The order of those additions is not fixed, exactly as in the reference.
+#include "tpk_device.h"
+
+namespace {
+
+constexpr int CH_THREADS = 256;
+constexpr int CH_TILE = 1024; // scanned points per LDS tile
+constexpr int CH_CHUNK = 8;   // candidates per "which group held the minimum" record
+
+template <typename T>
+struct Point4
+{
+    T x, y, z, w;
+};
+
+template <typename T>
+__device__ __forceinline__ T tpk_min(T a, T b);
+template <>
+__device__ __forceinline__ float tpk_min<float>(float a, float b)
+{
+    return fminf(a, b);
+}
+template <>
+__device__ __forceinline__ double tpk_min<double>(double a, double b)
+{
+    return fmin(a, b);
+}
+
+template <typename T>
+__device__ __forceinline__ T tpk_inf();
+template <>
+__device__ __forceinline__ float tpk_inf<float>()
+{
+    return __builtin_inff();
+}
+template <>
+__device__ __forceinline__ double tpk_inf<double>()
+{
+    return __builtin_inf();
+}
+
+template <typename T, int Q>
+__global__ __launch_bounds__(CH_THREADS) void chamfer_fwd_kernel(
+    int n, int m, int blocks_per_cloud1, int blocks_per_cloud2, int blocks_dir1,
+    const T* __restrict__ xyz1, const T* __restrict__ xyz2, T* __restrict__ dist1,
+    T* __restrict__ dist2, int32_t* __restrict__ idx1, int32_t* __restrict__ idx2)
+{
+    __shared__ Point4<T> tile[CH_TILE];
+
+    // Direction 1: queries = cloud 1 (n points), scanned = cloud 2 (m points); direction 2
+    // swaps the roles.
+    int bid = blockIdx.x;
+    const bool dir2 = bid >= blocks_dir1;
+    if (dir2)
+        bid -= blocks_dir1;
+    const int nq = dir2 ? m : n;
+    const int nc = dir2 ? n : m;
+    const int bpc = dir2 ? blocks_per_cloud2 : blocks_per_cloud1;
+    const int cloud = bid / bpc;
+    const int blk = bid - cloud * bpc;
+    const T* __restrict__ qs = (dir2 ? xyz2 : xyz1) + static_cast<int64_t>(cloud) * nq * 3;
+    const T* __restrict__ cs = (dir2 ? xyz1 : xyz2) + static_cast<int64_t>(cloud) * nc * 3;
+    T* __restrict__ dout = (dir2 ? dist2 : dist1) + static_cast<int64_t>(cloud) * nq;
+    int32_t* __restrict__ iout = (dir2 ? idx2 : idx1) + static_cast<int64_t>(cloud) * nq;
+
+    const int tid = threadIdx.x;
+    const int j0 = blk * (CH_THREADS * Q) + tid;
+
+    T qx[Q], qy[Q], qz[Q], best[Q];
+    int bgroup[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+    {
+        int j = j0 + q * CH_THREADS;
+        j = j < nq ? j : nq - 1; // lanes past the end shadow the last query and store nothing
+        qx[q] = qs[static_cast<int64_t>(j) * 3 + 0];
+        qy[q] = qs[static_cast<int64_t>(j) * 3 + 1];
+        qz[q] = qs[static_cast<int64_t>(j) * 3 + 2];
+        best[q] = tpk_inf<T>();
+        bgroup[q] = 0;
+    }
+
+    for (int base = 0; base < nc; base += CH_TILE)
+    {
+        const int cnt = min(CH_TILE, nc - base);
+        __syncthreads(); // the previous tile has been consumed by every wave
+        for (int t = tid; t < CH_TILE; t += CH_THREADS)
+        {
+            Point4<T> p;
+            if (t < cnt)
+            {
+                const T* src = cs + static_cast<int64_t>(base + t) * 3;
+                p.x = src[0];
+                p.y = src[1];
+                p.z = src[2];
+            }
+            else
+            {
+                // Padding: an infinitely distant point never lowers a minimum.
+                p.x = p.y = p.z = tpk_inf<T>();
+            }
+            p.w = 0;
+            tile[t] = p;
+        }
+        __syncthreads();
+
+        const int cnt_groups = (cnt + CH_CHUNK - 1) / CH_CHUNK;
+        for (int g = 0; g < cnt_groups; ++g)
+        {
+            T mn[Q];
+#pragma unroll
+            for (int c = 0; c < CH_CHUNK; ++c)
+            {
+                const Point4<T> p = tile[g * CH_CHUNK + c];
+#pragma unroll
+                for (int q = 0; q < Q; ++q)
+                {
+                    // Operand order of the reference: (scanned - query), squares summed x,y,z.
+                    const T d = tpk_dist2(p.x, p.y, p.z, qx[q], qy[q], qz[q]);
+                    mn[q] = c == 0 ? d : tpk_min(mn[q], d);
+                }
+            }
+            const int group = base / CH_CHUNK + g;
+#pragma unroll
+            for (int q = 0; q < Q; ++q)
+            {
+                const bool better = mn[q] < best[q];
+                best[q] = better ? mn[q] : best[q];
+                bgroup[q] = better ? group : bgroup[q];
+            }
+        }
+    }
+
+    // Recover the index: first candidate of the winning group whose distance equals the
+    // minimum (re-evaluated with the same operations, hence the same bits).
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+    {
+        const int j = j0 + q * CH_THREADS;
+        if (j >= nq)
+            continue;
+        T bd = best[q];
+        int bi = bgroup[q] * CH_CHUNK;
+        if (nc == 0)
+        {
+            bd = 0;
+            bi = 0;
+        }
+        else
+        {
+            const int k0 = bgroup[q] * CH_CHUNK;
+            bool found = false;
+#pragma unroll
+            for (int c = 0; c < CH_CHUNK; ++c)
+            {
+                const int k = k0 + c;
+                if (k < nc)
+                {
+                    const T* src = cs + static_cast<int64_t>(k) * 3;
+                    const T d = tpk_dist2(src[0], src[1], src[2], qx[q], qy[q], qz[q]);
+                    if (!found && d == bd)
+                    {
+                        found = true;
+                        bi = k;
+                    }
+                }
+            }
+        }
+        dout[j] = bd;
+        iout[j] = bi;
+    }
+}
+
+// Own term of every point: grad[j] = 2 * grad_dist[j] * (p[j] - other[idx[j]]), stored.
+template <typename T>
+__global__ __launch_bounds__(256) void chamfer_bwd_own_kernel(
+    int64_t total1, int64_t total2, int n, int m, const T* __restrict__ xyz1,
+    const T* __restrict__ xyz2, const int32_t* __restrict__ idx1,
+    const int32_t* __restrict__ idx2, const T* __restrict__ grad_dist1,
+    const T* __restrict__ grad_dist2, T* __restrict__ grad_xyz1, T* __restrict__ grad_xyz2)
+{
+    int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (; t < total1 + total2; t += stride)
+    {
+        const bool second = t >= total1;
+        const int64_t p = second ? t - total1 : t; // flat point number (cloud * npts + j)
+        const int npts = second ? m : n;
+        const int nother = second ? n : m;
+        const int64_t cloud = p / npts;
+        const T* a = (second ? xyz2 : xyz1) + p * 3;
+        const int j2 = (second ? idx2 : idx1)[p];
+        const T* o = (second ? xyz1 : xyz2) + (cloud * nother + j2) * 3;
+        const T g = (second ? grad_dist2 : grad_dist1)[p] * 2;
+        T* out = (second ? grad_xyz2 : grad_xyz1) + p * 3;
+        out[0] = g * (a[0] - o[0]);
+        out[1] = g * (a[1] - o[1]);
+        out[2] = g * (a[2] - o[2]);
+    }
+}
+
+// Scattered term: grad_other[idx[j]] += -(2 * grad_dist[j] * (p[j] - other[idx[j]])).
+template <typename T>
+__global__ __launch_bounds__(256) void chamfer_bwd_scatter_kernel(
+    int64_t total1, int64_t total2, int n, int m, const T* __restrict__ xyz1,
+    const T* __restrict__ xyz2, const int32_t* __restrict__ idx1,
+    const int32_t* __restrict__ idx2, const T* __restrict__ grad_dist1,
+    const T* __restrict__ grad_dist2, T* grad_xyz1, T* grad_xyz2)
+{
+    int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (; t < total1 + total2; t += stride)
+    {
+        const bool second = t >= total1;
+        const int64_t p = second ? t - total1 : t;
+        const int npts = second ? m : n;
+        const int nother = second ? n : m;
+        const int64_t cloud = p / npts;
+        const T* a = (second ? xyz2 : xyz1) + p * 3;
+        const int j2 = (second ? idx2 : idx1)[p];
+        const int64_t op = cloud * nother + j2;
+        const T* o = (second ? xyz1 : xyz2) + op * 3;
+        const T g = (second ? grad_dist2 : grad_dist1)[p] * 2;
+        T* out = (second ? grad_xyz1 : grad_xyz2) + op * 3;
+        unsafeAtomicAdd(out + 0, -(g * (a[0] - o[0])));
+        unsafeAtomicAdd(out + 1, -(g * (a[1] - o[1])));
+        unsafeAtomicAdd(out + 2, -(g * (a[2] - o[2])));
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void fill_zero_kernel(T* p, int64_t count)
+{
+    int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (; t < count; t += stride)
+        p[t] = 0;
+}
+
+template <typename T, int Q>
+int launch_fwd(int b, int n, int m, const T* xyz1, const T* xyz2, T* dist1, T* dist2,
+               int32_t* idx1, int32_t* idx2, hipStream_t s)
+{
+    const int64_t bpc1 = tpk_ceil_div(n, CH_THREADS * Q);
+    const int64_t bpc2 = tpk_ceil_div(m, CH_THREADS * Q);
+    const int64_t blocks1 = bpc1 * b;
+    const int64_t blocks2 = bpc2 * b;
+    if (blocks1 + blocks2 > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    if (blocks1 + blocks2 == 0)
+        return TPK_OK;
+    hipLaunchKernelGGL((chamfer_fwd_kernel<T, Q>), dim3(static_cast<unsigned>(blocks1 + blocks2)),
+                       dim3(CH_THREADS), 0, s, n, m, static_cast<int>(bpc1 ? bpc1 : 1),
+                       static_cast<int>(bpc2 ? bpc2 : 1), static_cast<int>(blocks1), xyz1, xyz2,
+                       dist1, dist2, idx1, idx2);
+    return tpk_launch_status();
+}
+
+template <typename T>
+int chamfer_fwd(int b, int n, int m, const T* xyz1, const T* xyz2, T* dist1, T* dist2,
+                int32_t* idx1, int32_t* idx2, void* stream)
+{
+    if (b < 0 || n < 0 || m < 0)
+        return TPK_ERR_INVALID_ARG;
+    if (b == 0 || (n == 0 && m == 0))
+        return TPK_OK;
+    if ((n > 0 && (!xyz1 || !dist1 || !idx1)) || (m > 0 && (!xyz2 || !dist2 || !idx2)))
+        return TPK_ERR_INVALID_ARG;
+    hipStream_t s = tpk_stream(stream);
+    const int64_t queries = static_cast<int64_t>(b) * (static_cast<int64_t>(n) + m);
+    if (queries >= 4LL * CH_THREADS * 1024)
+        return launch_fwd<T, 4>(b, n, m, xyz1, xyz2, dist1, dist2, idx1, idx2, s);
+    if (queries >= 2LL * CH_THREADS * 1024)
+        return launch_fwd<T, 2>(b, n, m, xyz1, xyz2, dist1, dist2, idx1, idx2, s);
+    return launch_fwd<T, 1>(b, n, m, xyz1, xyz2, dist1, dist2, idx1, idx2, s);
+}
+
+template <typename T>
+int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t* idx1,
+                const int32_t* idx2, const T* grad_dist1, const T* grad_dist2, T* grad_xyz1,
+                T* grad_xyz2, void* stream)
+{
+    if (b < 0 || n < 0 || m < 0)
+        return TPK_ERR_INVALID_ARG;
+    if (b == 0 || (n == 0 && m == 0))
+        return TPK_OK;
+    if ((n > 0 && (!xyz1 || !idx1 || !grad_dist1 || !grad_xyz1)) ||
+        (m > 0 && (!xyz2 || !idx2 || !grad_dist2 || !grad_xyz2)))
+        return TPK_ERR_INVALID_ARG;
+    hipStream_t s = tpk_stream(stream);
+    const int64_t total1 = static_cast<int64_t>(b) * n;
+    const int64_t total2 = static_cast<int64_t>(b) * m;
+    if (n == 0 || m == 0)
+    {
+        // One cloud is empty: no pairs exist; the reference returns its zero-initialised
+        // gradients.
+        const int64_t count = (total1 + total2) * 3;
+        T* p = n == 0 ? grad_xyz2 : grad_xyz1;
+        const unsigned blocks = static_cast<unsigned>(tpk_min64(tpk_ceil_div(count, 256), 4096));
+        hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(blocks), dim3(256), 0, s, p, count);
+        return tpk_launch_status();
+    }
+    const unsigned blocks =
+        static_cast<unsigned>(tpk_min64(tpk_ceil_div(total1 + total2, 256), 1 << 20));
+    hipLaunchKernelGGL(chamfer_bwd_own_kernel<T>, dim3(blocks), dim3(256), 0, s, total1, total2,
+                       n, m, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2, grad_xyz1,
+                       grad_xyz2);
+    int st = tpk_launch_status();
+    if (st != TPK_OK)
+        return st;
+    hipLaunchKernelGGL(chamfer_bwd_scatter_kernel<T>, dim3(blocks), dim3(256), 0, s, total1,
+                       total2, n, m, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2, grad_xyz1,
+                       grad_xyz2);
+    return tpk_launch_status();
+}
+
+} // namespace
+
+extern "C" int tpk_chamfer_fwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2,
+                                   float* dist1, float* dist2, int32_t* idx1, int32_t* idx2,
+                                   void* stream)
+{
+    return chamfer_fwd<float>(b, n, m, xyz1, xyz2, dist1, dist2, idx1, idx2, stream);
+}
+
+extern "C" int tpk_chamfer_fwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
+                                   double* dist1, double* dist2, int32_t* idx1, int32_t* idx2,
+                                   void* stream)
+{
+    return chamfer_fwd<double>(b, n, m, xyz1, xyz2, dist1, dist2, idx1, idx2, stream);
+}
+
+extern "C" int tpk_chamfer_bwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2,
+                                   const int32_t* idx1, const int32_t* idx2,
+                                   const float* grad_dist1, const float* grad_dist2,
+                                   float* grad_xyz1, float* grad_xyz2, void* stream)
+{
+    return chamfer_bwd<float>(b, n, m, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2, grad_xyz1,
+                              grad_xyz2, stream);
+}
+
+extern "C" int tpk_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
+                                   const int32_t* idx1, const int32_t* idx2,
+                                   const double* grad_dist1, const double* grad_dist2,
+                                   double* grad_xyz1, double* grad_xyz2, void* stream)
+{
+    return chamfer_bwd<double>(b, n, m, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2,
+                               grad_xyz1, grad_xyz2, stream);
+}

@@ -1,0 +1,423 @@
+// torch_points_kernels.points_cuda for AMD MI355X: the pybind11 module the Python layer
+// imports for tensors on the GPU.  It exports the names and signatures of the reference
+// module (cuda/src/bindings.cpp:11-29) for the spatial-search operators, checks and
+// allocates tensors the way the reference's host functions do, and hands raw pointers to
+// the C ABI of libtpk_hip.so (include/tpk.h) on PyTorch's current HIP stream.  It contains
+// no kernels and no CPU implementation: without a GPU tensor it raises.
+#include <torch/extension.h>
+
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <utility>
+#include <vector>
+
+#include "../../include/tpk.h"
+
+namespace {
+
+void check_status(int status, const char* what)
+{
+    TORCH_CHECK(status == TPK_OK, what, " failed: ", tpk_status_string(status), " (status ",
+                status, ")");
+}
+
+// The reference's checks (cuda/include/utils.h:5-27) made stricter where it would misread
+// memory: exact dtypes instead of "some float" / "some int".
+void check_gpu(const at::Tensor& t, const char* name)
+{
+    TORCH_CHECK(t.is_cuda(), name, " must be a CUDA tensor");
+}
+void check_contiguous(const at::Tensor& t, const char* name)
+{
+    TORCH_CHECK(t.is_contiguous(), name, " must be a contiguous tensor");
+}
+void check_f32(const at::Tensor& t, const char* name)
+{
+    TORCH_CHECK(t.scalar_type() == at::kFloat, name, " must be a float32 tensor");
+}
+void check_dtype(const at::Tensor& t, at::ScalarType st, const char* name)
+{
+    TORCH_CHECK(t.scalar_type() == st, name, " must be a ", c10::toString(st), " tensor");
+}
+void check_same_device(const at::Tensor& a, const at::Tensor& b, const char* names)
+{
+    TORCH_CHECK(a.device() == b.device(), names, " must be on the same device");
+}
+void check_points(const at::Tensor& t, int64_t dims, const char* name)
+{
+    TORCH_CHECK(t.dim() == dims && t.size(dims - 1) == 3, name, " must have shape (",
+                dims == 3 ? "B, N, 3)" : "N, 3)");
+}
+int as_int(int64_t v, const char* name)
+{
+    TORCH_CHECK(v >= 0 && v <= INT32_MAX, name, " is out of range: ", v);
+    return static_cast<int>(v);
+}
+
+void* current_stream(const at::Tensor& t)
+{
+    return static_cast<void*>(c10::hip::getCurrentHIPStream(t.get_device()).stream());
+}
+
+// cuda/src/sampling.cpp:8-25
+at::Tensor furthest_point_sampling(at::Tensor points, const int nsamples)
+{
+    check_contiguous(points, "points");
+    check_f32(points, "points");
+    check_gpu(points, "points");
+    check_points(points, 3, "points");
+    TORCH_CHECK(nsamples >= 0, "nsamples must be non-negative");
+    const c10::hip::HIPGuard guard(points.device());
+
+    at::Tensor output = torch::empty({points.size(0), nsamples},
+                                     at::device(points.device()).dtype(at::ScalarType::Int));
+    const int b = as_int(points.size(0), "batch size");
+    const int n = as_int(points.size(1), "number of points");
+    const size_t ws_bytes = tpk_fps_workspace_bytes(b, n);
+    at::Tensor ws;
+    if (ws_bytes)
+        ws = torch::empty({static_cast<int64_t>(ws_bytes)},
+                          at::device(points.device()).dtype(at::ScalarType::Byte));
+    check_status(tpk_fps_f32(b, n, nsamples, points.data_ptr<float>(),
+                             ws_bytes ? ws.data_ptr() : nullptr, ws_bytes,
+                             output.data_ptr<int32_t>(), current_stream(points)),
+                 "furthest_point_sampling");
+    return output;
+}
+
+// cuda/src/interpolate.cpp:12-32
+std::vector<at::Tensor> three_nn(at::Tensor unknowns, at::Tensor knows)
+{
+    check_contiguous(unknowns, "unknowns");
+    check_contiguous(knows, "knows");
+    check_f32(unknowns, "unknowns");
+    check_f32(knows, "knows");
+    check_gpu(knows, "knows");
+    check_gpu(unknowns, "unknowns");
+    check_same_device(unknowns, knows, "unknowns and knows");
+    check_points(unknowns, 3, "unknowns");
+    check_points(knows, 3, "knows");
+    TORCH_CHECK(unknowns.size(0) == knows.size(0), "unknowns and knows differ in batch size");
+    const c10::hip::HIPGuard guard(unknowns.device());
+
+    at::Tensor idx = torch::empty({unknowns.size(0), unknowns.size(1), 3},
+                                  at::device(unknowns.device()).dtype(at::ScalarType::Int));
+    at::Tensor dist2 = torch::empty({unknowns.size(0), unknowns.size(1), 3},
+                                    at::device(unknowns.device()).dtype(at::ScalarType::Float));
+    check_status(tpk_three_nn_f32(as_int(unknowns.size(0), "batch size"),
+                                  as_int(unknowns.size(1), "number of unknown points"),
+                                  as_int(knows.size(1), "number of known points"),
+                                  unknowns.data_ptr<float>(), knows.data_ptr<float>(),
+                                  dist2.data_ptr<float>(), idx.data_ptr<int32_t>(),
+                                  current_stream(unknowns)),
+                 "three_nn");
+    return {dist2, idx};
+}
+
+// cuda/src/interpolate.cpp:34-54
+at::Tensor three_interpolate(at::Tensor points, at::Tensor idx, at::Tensor weight)
+{
+    check_contiguous(points, "points");
+    check_contiguous(idx, "idx");
+    check_contiguous(weight, "weight");
+    check_f32(points, "points");
+    check_dtype(idx, at::kInt, "idx");
+    check_f32(weight, "weight");
+    check_gpu(points, "points");
+    check_gpu(idx, "idx");
+    check_gpu(weight, "weight");
+    check_same_device(points, idx, "points and idx");
+    check_same_device(points, weight, "points and weight");
+    TORCH_CHECK(points.dim() == 3, "points must have shape (B, c, m)");
+    TORCH_CHECK(idx.dim() == 3 && idx.size(2) == 3 && idx.size(0) == points.size(0),
+                "idx must have shape (B, n, 3)");
+    TORCH_CHECK(weight.sizes() == idx.sizes(), "weight must have the shape of idx");
+    const c10::hip::HIPGuard guard(points.device());
+
+    at::Tensor output = torch::empty({points.size(0), points.size(1), idx.size(1)},
+                                     at::device(points.device()).dtype(at::ScalarType::Float));
+    check_status(tpk_three_interpolate_f32(
+                     as_int(points.size(0), "batch size"), as_int(points.size(1), "channels"),
+                     as_int(points.size(2), "m"), as_int(idx.size(1), "n"),
+                     points.data_ptr<float>(), idx.data_ptr<int32_t>(), weight.data_ptr<float>(),
+                     output.data_ptr<float>(), current_stream(points)),
+                 "three_interpolate");
+    return output;
+}
+
+// cuda/src/interpolate.cpp:55-76
+at::Tensor three_interpolate_grad(at::Tensor grad_out, at::Tensor idx, at::Tensor weight,
+                                  const int m)
+{
+    check_contiguous(grad_out, "grad_out");
+    check_contiguous(idx, "idx");
+    check_contiguous(weight, "weight");
+    check_f32(grad_out, "grad_out");
+    check_dtype(idx, at::kInt, "idx");
+    check_f32(weight, "weight");
+    check_gpu(idx, "idx");
+    check_gpu(weight, "weight");
+    check_gpu(grad_out, "grad_out");
+    check_same_device(grad_out, idx, "grad_out and idx");
+    check_same_device(grad_out, weight, "grad_out and weight");
+    TORCH_CHECK(grad_out.dim() == 3, "grad_out must have shape (B, c, n)");
+    TORCH_CHECK(idx.dim() == 3 && idx.size(2) == 3 && idx.size(0) == grad_out.size(0) &&
+                    idx.size(1) == grad_out.size(2),
+                "idx must have shape (B, n, 3)");
+    TORCH_CHECK(weight.sizes() == idx.sizes(), "weight must have the shape of idx");
+    TORCH_CHECK(m >= 0, "m must be non-negative");
+    const c10::hip::HIPGuard guard(grad_out.device());
+
+    at::Tensor output = torch::empty({grad_out.size(0), grad_out.size(1), m},
+                                     at::device(grad_out.device()).dtype(at::ScalarType::Float));
+    check_status(tpk_three_interpolate_grad_f32(
+                     as_int(grad_out.size(0), "batch size"), as_int(grad_out.size(1), "channels"),
+                     as_int(grad_out.size(2), "n"), m, grad_out.data_ptr<float>(),
+                     idx.data_ptr<int32_t>(), weight.data_ptr<float>(), output.data_ptr<float>(),
+                     current_stream(grad_out)),
+                 "three_interpolate_grad");
+    return output;
+}
+
+// cuda/src/ball_query.cpp:15-36.  Query centres first, as in the reference.
+std::pair<at::Tensor, at::Tensor> ball_query_dense(at::Tensor new_xyz, at::Tensor xyz,
+                                                   const float radius, const int nsample)
+{
+    check_contiguous(new_xyz, "new_xyz");
+    check_contiguous(xyz, "xyz");
+    check_f32(new_xyz, "new_xyz");
+    check_f32(xyz, "xyz");
+    check_gpu(xyz, "xyz");
+    check_gpu(new_xyz, "new_xyz");
+    check_same_device(xyz, new_xyz, "xyz and new_xyz");
+    check_points(new_xyz, 3, "new_xyz");
+    check_points(xyz, 3, "xyz");
+    TORCH_CHECK(xyz.size(0) == new_xyz.size(0), "xyz and new_xyz differ in batch size");
+    TORCH_CHECK(nsample >= 0, "nsample must be non-negative");
+    const c10::hip::HIPGuard guard(new_xyz.device());
+
+    at::Tensor idx = torch::empty({new_xyz.size(0), new_xyz.size(1), nsample},
+                                  at::device(new_xyz.device()).dtype(at::ScalarType::Long));
+    at::Tensor dist = torch::empty({new_xyz.size(0), new_xyz.size(1), nsample},
+                                   at::device(new_xyz.device()).dtype(at::ScalarType::Float));
+    check_status(tpk_ball_query_dense_f32(
+                     as_int(xyz.size(0), "batch size"), as_int(xyz.size(1), "support points"),
+                     as_int(new_xyz.size(1), "query points"), radius, nsample,
+                     new_xyz.data_ptr<float>(), xyz.data_ptr<float>(), idx.data_ptr<int64_t>(),
+                     dist.data_ptr<float>(), current_stream(new_xyz)),
+                 "ball_query_dense");
+    return std::make_pair(idx, dist);
+}
+
+// cuda/src/ball_query.cpp:45-81.  Support first, as in the reference.  The cloud ranges
+// are found on the device from the sorted batch vectors; nothing is copied to the host.
+std::pair<at::Tensor, at::Tensor> ball_query_partial_dense(at::Tensor x, at::Tensor y,
+                                                           at::Tensor batch_x, at::Tensor batch_y,
+                                                           const float radius, const int nsample)
+{
+    check_contiguous(x, "x");
+    check_contiguous(y, "y");
+    check_f32(x, "x");
+    check_f32(y, "y");
+    check_gpu(x, "x");
+    check_gpu(y, "y");
+    check_gpu(batch_x, "batch_x");
+    check_gpu(batch_y, "batch_y");
+    check_same_device(x, y, "x and y");
+    check_same_device(x, batch_x, "x and batch_x");
+    check_same_device(x, batch_y, "x and batch_y");
+    check_points(x, 2, "x");
+    check_points(y, 2, "y");
+    check_dtype(batch_x, at::kLong, "batch_x");
+    check_dtype(batch_y, at::kLong, "batch_y");
+    TORCH_CHECK(batch_x.dim() == 1 && batch_x.size(0) == x.size(0),
+                "batch_x must have one entry per point of x");
+    TORCH_CHECK(batch_y.dim() == 1 && batch_y.size(0) == y.size(0),
+                "batch_y must have one entry per point of y");
+    TORCH_CHECK(nsample >= 0, "nsample must be non-negative");
+    const c10::hip::HIPGuard guard(x.device());
+    batch_x = batch_x.contiguous();
+    batch_y = batch_y.contiguous();
+
+    at::Tensor idx =
+        torch::empty({y.size(0), nsample}, at::device(y.device()).dtype(at::ScalarType::Long));
+    at::Tensor dist =
+        torch::empty({y.size(0), nsample}, at::device(y.device()).dtype(at::ScalarType::Float));
+    check_status(tpk_ball_query_partial_f32(x.size(0), y.size(0), radius, nsample,
+                                            x.data_ptr<float>(), y.data_ptr<float>(),
+                                            batch_x.data_ptr<int64_t>(),
+                                            batch_y.data_ptr<int64_t>(), idx.data_ptr<int64_t>(),
+                                            dist.data_ptr<float>(), current_stream(x)),
+                 "ball_query_partial_dense");
+    return std::make_pair(idx, dist);
+}
+
+// No counterpart in the reference's native module: its grouping_operation is
+// torch.gather on a repeated index (torch_points_kernels/torchpoints.py:129-146).
+at::Tensor grouping_operation(at::Tensor features, at::Tensor idx)
+{
+    check_contiguous(features, "features");
+    check_contiguous(idx, "idx");
+    check_f32(features, "features");
+    check_dtype(idx, at::kLong, "idx");
+    check_gpu(features, "features");
+    check_gpu(idx, "idx");
+    check_same_device(features, idx, "features and idx");
+    TORCH_CHECK(features.dim() == 3, "features must have shape (B, C, N)");
+    TORCH_CHECK(idx.dim() == 3 && idx.size(0) == features.size(0),
+                "idx must have shape (B, npoint, nsample)");
+    const c10::hip::HIPGuard guard(features.device());
+
+    at::Tensor out = torch::empty({features.size(0), features.size(1), idx.size(1), idx.size(2)},
+                                  at::device(features.device()).dtype(at::ScalarType::Float));
+    check_status(tpk_group_f32(as_int(features.size(0), "batch size"),
+                               as_int(features.size(1), "channels"), as_int(features.size(2), "N"),
+                               as_int(idx.size(1), "npoint"), as_int(idx.size(2), "nsample"),
+                               features.data_ptr<float>(), idx.data_ptr<int64_t>(),
+                               out.data_ptr<float>(), current_stream(features)),
+                 "grouping_operation");
+    return out;
+}
+
+at::Tensor grouping_operation_grad(at::Tensor grad_out, at::Tensor idx, const int n)
+{
+    check_contiguous(grad_out, "grad_out");
+    check_contiguous(idx, "idx");
+    check_f32(grad_out, "grad_out");
+    check_dtype(idx, at::kLong, "idx");
+    check_gpu(grad_out, "grad_out");
+    check_gpu(idx, "idx");
+    check_same_device(grad_out, idx, "grad_out and idx");
+    TORCH_CHECK(grad_out.dim() == 4, "grad_out must have shape (B, C, npoint, nsample)");
+    TORCH_CHECK(idx.dim() == 3 && idx.size(0) == grad_out.size(0) &&
+                    idx.size(1) == grad_out.size(2) && idx.size(2) == grad_out.size(3),
+                "idx must have shape (B, npoint, nsample)");
+    TORCH_CHECK(n >= 0, "n must be non-negative");
+    const c10::hip::HIPGuard guard(grad_out.device());
+
+    at::Tensor out = torch::empty({grad_out.size(0), grad_out.size(1), n},
+                                  at::device(grad_out.device()).dtype(at::ScalarType::Float));
+    check_status(tpk_group_grad_f32(as_int(grad_out.size(0), "batch size"),
+                                    as_int(grad_out.size(1), "channels"), n,
+                                    as_int(idx.size(1), "npoint"), as_int(idx.size(2), "nsample"),
+                                    grad_out.data_ptr<float>(), idx.data_ptr<int64_t>(),
+                                    out.data_ptr<float>(), current_stream(grad_out)),
+                 "grouping_operation_grad");
+    return out;
+}
+
+// cuda/src/chamfer_dist.cpp:3-6 -> cuda/src/chamfer_dist_gpu.cu:157-184
+std::vector<torch::Tensor> chamfer_dist(torch::Tensor xyz1, torch::Tensor xyz2)
+{
+    check_gpu(xyz1, "xyz1");
+    check_gpu(xyz2, "xyz2");
+    check_same_device(xyz1, xyz2, "xyz1 and xyz2");
+    check_points(xyz1, 3, "xyz1");
+    check_points(xyz2, 3, "xyz2");
+    TORCH_CHECK(xyz1.size(0) == xyz2.size(0), "xyz1 and xyz2 differ in batch size");
+    TORCH_CHECK(xyz1.scalar_type() == xyz2.scalar_type(), "xyz1 and xyz2 differ in dtype");
+    TORCH_CHECK(xyz1.scalar_type() == at::kFloat || xyz1.scalar_type() == at::kDouble,
+                "chamfer_dist supports float32 and float64");
+    const c10::hip::HIPGuard guard(xyz1.device());
+    xyz1 = xyz1.contiguous();
+    xyz2 = xyz2.contiguous();
+
+    const int b = as_int(xyz1.size(0), "batch size");
+    const int n = as_int(xyz1.size(1), "points of xyz1");
+    const int m = as_int(xyz2.size(1), "points of xyz2");
+    auto fopt = xyz1.options();
+    auto iopt = xyz1.options().dtype(torch::kInt);
+    torch::Tensor dist1 = torch::empty({b, n}, fopt);
+    torch::Tensor dist2 = torch::empty({b, m}, fopt);
+    torch::Tensor idx1 = torch::empty({b, n}, iopt);
+    torch::Tensor idx2 = torch::empty({b, m}, iopt);
+    void* s = current_stream(xyz1);
+    if (xyz1.scalar_type() == at::kFloat)
+        check_status(tpk_chamfer_fwd_f32(b, n, m, xyz1.data_ptr<float>(), xyz2.data_ptr<float>(),
+                                         dist1.data_ptr<float>(), dist2.data_ptr<float>(),
+                                         idx1.data_ptr<int32_t>(), idx2.data_ptr<int32_t>(), s),
+                     "chamfer_dist");
+    else
+        check_status(tpk_chamfer_fwd_f64(b, n, m, xyz1.data_ptr<double>(),
+                                         xyz2.data_ptr<double>(), dist1.data_ptr<double>(),
+                                         dist2.data_ptr<double>(), idx1.data_ptr<int32_t>(),
+                                         idx2.data_ptr<int32_t>(), s),
+                     "chamfer_dist");
+    return {dist1, dist2, idx1, idx2};
+}
+
+// cuda/src/chamfer_dist.cpp:8-13 -> cuda/src/chamfer_dist_gpu.cu:215-245
+std::vector<torch::Tensor> chamfer_dist_grad(torch::Tensor xyz1, torch::Tensor xyz2,
+                                             torch::Tensor idx1, torch::Tensor idx2,
+                                             torch::Tensor grad_dist1, torch::Tensor grad_dist2)
+{
+    check_gpu(xyz1, "xyz1");
+    check_gpu(xyz2, "xyz2");
+    check_gpu(idx1, "idx1");
+    check_gpu(idx2, "idx2");
+    check_gpu(grad_dist1, "grad_dist1");
+    check_gpu(grad_dist2, "grad_dist2");
+    check_points(xyz1, 3, "xyz1");
+    check_points(xyz2, 3, "xyz2");
+    check_dtype(idx1, at::kInt, "idx1");
+    check_dtype(idx2, at::kInt, "idx2");
+    TORCH_CHECK(xyz1.scalar_type() == xyz2.scalar_type() &&
+                    xyz1.scalar_type() == grad_dist1.scalar_type() &&
+                    xyz1.scalar_type() == grad_dist2.scalar_type(),
+                "clouds and gradients differ in dtype");
+    TORCH_CHECK(xyz1.scalar_type() == at::kFloat || xyz1.scalar_type() == at::kDouble,
+                "chamfer_dist_grad supports float32 and float64");
+    const int b = as_int(xyz1.size(0), "batch size");
+    const int n = as_int(xyz1.size(1), "points of xyz1");
+    const int m = as_int(xyz2.size(1), "points of xyz2");
+    TORCH_CHECK(xyz2.size(0) == b && idx1.numel() == static_cast<int64_t>(b) * n &&
+                    idx2.numel() == static_cast<int64_t>(b) * m &&
+                    grad_dist1.numel() == idx1.numel() && grad_dist2.numel() == idx2.numel(),
+                "shapes of clouds, indices and gradients do not match");
+    const c10::hip::HIPGuard guard(xyz1.device());
+    xyz1 = xyz1.contiguous();
+    xyz2 = xyz2.contiguous();
+    idx1 = idx1.contiguous();
+    idx2 = idx2.contiguous();
+    grad_dist1 = grad_dist1.contiguous();
+    grad_dist2 = grad_dist2.contiguous();
+
+    torch::Tensor grad_xyz1 = torch::empty_like(xyz1);
+    torch::Tensor grad_xyz2 = torch::empty_like(xyz2);
+    void* s = current_stream(xyz1);
+    if (xyz1.scalar_type() == at::kFloat)
+        check_status(tpk_chamfer_bwd_f32(b, n, m, xyz1.data_ptr<float>(), xyz2.data_ptr<float>(),
+                                         idx1.data_ptr<int32_t>(), idx2.data_ptr<int32_t>(),
+                                         grad_dist1.data_ptr<float>(),
+                                         grad_dist2.data_ptr<float>(),
+                                         grad_xyz1.data_ptr<float>(),
+                                         grad_xyz2.data_ptr<float>(), s),
+                     "chamfer_dist_grad");
+    else
+        check_status(tpk_chamfer_bwd_f64(b, n, m, xyz1.data_ptr<double>(),
+                                         xyz2.data_ptr<double>(), idx1.data_ptr<int32_t>(),
+                                         idx2.data_ptr<int32_t>(), grad_dist1.data_ptr<double>(),
+                                         grad_dist2.data_ptr<double>(),
+                                         grad_xyz1.data_ptr<double>(),
+                                         grad_xyz2.data_ptr<double>(), s),
+                     "chamfer_dist_grad");
+    return {grad_xyz1, grad_xyz2};
+}
+
+} // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("furthest_point_sampling", &furthest_point_sampling);
+    m.def("three_nn", &three_nn);
+    m.def("three_interpolate", &three_interpolate);
+    m.def("three_interpolate_grad", &three_interpolate_grad);
+    m.def("ball_query_dense", &ball_query_dense);
+    m.def("ball_query_partial_dense", &ball_query_partial_dense);
+    m.def("grouping_operation", &grouping_operation);
+    m.def("grouping_operation_grad", &grouping_operation_grad);
+    m.def("chamfer_dist", &chamfer_dist);
+    m.def("chamfer_dist_grad", &chamfer_dist_grad);
+    m.def("tpk_version", &tpk_version);
+}

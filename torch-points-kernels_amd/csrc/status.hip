@@ -1,0 +1,27 @@
+// Version and status text of the C ABI.
+#include "tpk_device.h"
+
+extern "C" int tpk_version(void)
+{
+    return 100; // 0.1.0
+}
+
+extern "C" const char* tpk_status_string(int status)
+{
+    switch (status)
+    {
+    case TPK_OK:
+        return "ok";
+    case TPK_ERR_INVALID_ARG:
+        return "invalid argument (negative size or missing pointer)";
+    case TPK_ERR_UNSUPPORTED:
+        return "size outside the supported range";
+    case TPK_ERR_WORKSPACE:
+        return "workspace missing or too small";
+    default:
+        break;
+    }
+    if (status > 0)
+        return hipGetErrorString(static_cast<hipError_t>(status));
+    return "unknown status";
+}

@@ -1,0 +1,152 @@
+// three_nn: for every "unknown" point the three nearest "known" points of the same cloud.
+//
+// Work split: one lane owns Q query points and keeps their running best three (distance,
+// index) in registers; the known points of the cloud stream through LDS in tiles of
+// float4 (x, y, z, pad), so every lane of a wavefront reads the same LDS address at the
+// same time (a broadcast read, no bank conflicts) and one LDS read feeds Q distance
+// evaluations.  Insertion into the sorted triple happens only in lanes whose distance
+// beats their current third best, which after the first few hundred candidates is rare.
+//
+// Semantics follow the reference kernel (cuda/src/interpolate_gpu.cu:9-65): candidates are
+// visited in index order and replace an entry only when strictly smaller, so equal
+// distances keep the lower index first.  The reference holds its running bests as doubles
+// initialised to 1e40; every distance is an fp32 value, so fp32 running bests initialised
+// to +inf select identically and store identical values.
+#include "tpk_device.h"
+
+namespace {
+
+constexpr int NN_THREADS = 256;
+constexpr int NN_TILE = 1024; // known points per LDS tile (16 KiB)
+
+template <int Q>
+__global__ __launch_bounds__(NN_THREADS) void three_nn_kernel(
+    int n, int m, int blocks_per_cloud, const float* __restrict__ unknown,
+    const float* __restrict__ known, float* __restrict__ dist2, int32_t* __restrict__ idx)
+{
+    __shared__ float4 tile[NN_TILE];
+
+    const int cloud = blockIdx.x / blocks_per_cloud;
+    const int blk = blockIdx.x - cloud * blocks_per_cloud;
+    unknown += static_cast<int64_t>(cloud) * n * 3;
+    known += static_cast<int64_t>(cloud) * m * 3;
+    dist2 += static_cast<int64_t>(cloud) * n * 3;
+    idx += static_cast<int64_t>(cloud) * n * 3;
+
+    const int tid = threadIdx.x;
+    const int j0 = blk * (NN_THREADS * Q) + tid;
+
+    float ux[Q], uy[Q], uz[Q];
+    float b1[Q], b2[Q], b3[Q];
+    int i1[Q], i2[Q], i3[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+    {
+        int j = j0 + q * NN_THREADS;
+        j = j < n ? j : n - 1; // lanes past the end shadow the last query and store nothing
+        ux[q] = unknown[j * 3 + 0];
+        uy[q] = unknown[j * 3 + 1];
+        uz[q] = unknown[j * 3 + 2];
+        b1[q] = b2[q] = b3[q] = __builtin_inff();
+        i1[q] = i2[q] = i3[q] = 0;
+    }
+
+    for (int base = 0; base < m; base += NN_TILE)
+    {
+        const int cnt = min(NN_TILE, m - base);
+        __syncthreads(); // the previous tile has been consumed by every wave
+        for (int t = tid; t < NN_TILE; t += NN_THREADS)
+        {
+            float4 p;
+            if (t < cnt)
+            {
+                const float* src = known + static_cast<int64_t>(base + t) * 3;
+                p = make_float4(src[0], src[1], src[2], 0.f);
+            }
+            else
+            {
+                // Padding: an infinitely distant point never beats a running best.
+                p = make_float4(__builtin_inff(), __builtin_inff(), __builtin_inff(), 0.f);
+            }
+            tile[t] = p;
+        }
+        __syncthreads();
+
+        const int cnt4 = (cnt + 3) & ~3;
+#pragma unroll 4
+        for (int k = 0; k < cnt4; ++k)
+        {
+            const float4 c = tile[k];
+            const int kk = base + k;
+#pragma unroll
+            for (int q = 0; q < Q; ++q)
+            {
+                const float d = tpk_dist2(ux[q], uy[q], uz[q], c.x, c.y, c.z);
+                if (d < b3[q])
+                {
+                    // Sorted insert written as selects: one short block, no nested divergence.
+                    const bool lt1 = d < b1[q];
+                    const bool lt2 = d < b2[q];
+                    b3[q] = lt2 ? b2[q] : d;
+                    i3[q] = lt2 ? i2[q] : kk;
+                    b2[q] = lt1 ? b1[q] : (lt2 ? d : b2[q]);
+                    i2[q] = lt1 ? i1[q] : (lt2 ? kk : i2[q]);
+                    b1[q] = lt1 ? d : b1[q];
+                    i1[q] = lt1 ? kk : i1[q];
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+    {
+        const int j = j0 + q * NN_THREADS;
+        if (j < n)
+        {
+            dist2[j * 3 + 0] = b1[q];
+            dist2[j * 3 + 1] = b2[q];
+            dist2[j * 3 + 2] = b3[q];
+            idx[j * 3 + 0] = i1[q];
+            idx[j * 3 + 1] = i2[q];
+            idx[j * 3 + 2] = i3[q];
+        }
+    }
+}
+
+template <int Q>
+int launch_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2,
+                    int32_t* idx, hipStream_t stream)
+{
+    const int64_t blocks_per_cloud = tpk_ceil_div(n, NN_THREADS * Q);
+    const int64_t blocks = blocks_per_cloud * b;
+    if (blocks > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(three_nn_kernel<Q>, dim3(static_cast<unsigned>(blocks)), dim3(NN_THREADS),
+                       0, stream, n, m, static_cast<int>(blocks_per_cloud), unknown, known, dist2,
+                       idx);
+    return tpk_launch_status();
+}
+
+} // namespace
+
+extern "C" int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* known,
+                                float* dist2, int32_t* idx, void* stream)
+{
+    if (b < 0 || n < 0 || m < 0)
+        return TPK_ERR_INVALID_ARG;
+    if (b == 0 || n == 0)
+        return TPK_OK;
+    if (!unknown || !dist2 || !idx || (m > 0 && !known))
+        return TPK_ERR_INVALID_ARG;
+    if (static_cast<int64_t>(n) * 3 > 0x7fffffffLL || static_cast<int64_t>(m) * 3 > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    hipStream_t s = tpk_stream(stream);
+    // Queries per lane: as many as still leave a few workgroups per compute unit.
+    const int64_t queries = static_cast<int64_t>(b) * n;
+    if (queries >= 4LL * NN_THREADS * 2048)
+        return launch_three_nn<4>(b, n, m, unknown, known, dist2, idx, s);
+    if (queries >= 2LL * NN_THREADS * 2048)
+        return launch_three_nn<2>(b, n, m, unknown, known, dist2, idx, s);
+    return launch_three_nn<1>(b, n, m, unknown, known, dist2, idx, s);
+}

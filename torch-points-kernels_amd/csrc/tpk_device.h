@@ -1,0 +1,75 @@
+// Shared pieces of the gfx950 kernels: launch bookkeeping and wavefront helpers.
+//
+// Arithmetic rule for every distance in this library: fp32 (or fp64), each product and
+// each sum rounded on its own, evaluated left to right.  The translation units are
+// compiled with -ffp-contract=off and additionally carry the pragma below, so no
+// multiply-add is ever fused; integer outputs (neighbour indices, sample indices) depend
+// on it.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tpk.h"
+
+#pragma clang fp contract(off)
+
+#define TPK_WAVE 64
+
+// LDS a workgroup may use on gfx950 (160 KiB); the kernels stay below it.
+#define TPK_LDS_BYTES 163840
+
+static inline hipStream_t tpk_stream(void* s)
+{
+    return reinterpret_cast<hipStream_t>(s);
+}
+
+// Status of the launch just made: 0, or the hipError_t it raised.
+static inline int tpk_launch_status()
+{
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TPK_OK : static_cast<int>(e);
+}
+
+static inline int64_t tpk_ceil_div(int64_t a, int64_t b)
+{
+    return (a + b - 1) / b;
+}
+
+__host__ __device__ __forceinline__ int64_t tpk_min64(int64_t a, int64_t b)
+{
+    return a < b ? a : b;
+}
+
+// Number of lanes below this one whose bit is set in `mask` (a wave64 ballot).
+__device__ __forceinline__ unsigned tpk_prefix_count(unsigned long long mask)
+{
+    return __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u));
+}
+
+__device__ __forceinline__ unsigned tpk_lane_id()
+{
+    return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// Value of `v` in lane `lane` (wave-uniform lane number), as a wave-uniform scalar.
+__device__ __forceinline__ float tpk_read_lane(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+__device__ __forceinline__ int tpk_read_lane(int v, int lane)
+{
+    return __builtin_amdgcn_readlane(v, lane);
+}
+
+// Squared distance, unfused, in the order ((dx*dx + dy*dy) + dz*dz).
+template <typename T>
+__device__ __forceinline__ T tpk_dist2(T ax, T ay, T az, T bx, T by, T bz)
+{
+    const T dx = ax - bx;
+    const T dy = ay - by;
+    const T dz = az - bz;
+    return dx * dx + dy * dy + dz * dz;
+}

@@ -1,0 +1,30 @@
+"""torch_points_kernels for AMD MI355X: the spatial-search operators of
+torch-points3d/torch-points-kernels (furthest point sampling, ball query, three_nn /
+three_interpolate, grouping, Chamfer distance) on hand-written HIP kernels.
+
+Same names and call signatures as the reference package (torch_points_kernels/__init__.py);
+GPU tensors only.
+"""
+from .torchpoints import (
+    ThreeInterpolate,
+    GroupingOperation,
+    ball_query,
+    ball_query_dense,
+    ball_query_partial_dense,
+    furthest_point_sample,
+    grouping_operation,
+    three_interpolate,
+    three_nn,
+)
+from .chamfer_dist import ChamferFunction
+from . import chamfer_dist  # the reference exports the submodule under this name
+
+__all__ = [
+    "ball_query",
+    "furthest_point_sample",
+    "grouping_operation",
+    "three_interpolate",
+    "three_nn",
+    "chamfer_dist",
+    "ChamferFunction",
+]
