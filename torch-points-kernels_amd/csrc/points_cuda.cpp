@@ -6,8 +6,8 @@
 // no kernels and no CPU implementation: without a GPU tensor it raises.
 #include <torch/extension.h>
 
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <utility>
 #include <vector>
@@ -57,7 +57,7 @@ int as_int(int64_t v, const char* name)
 
 void* current_stream(const at::Tensor& t)
 {
-    return static_cast<void*>(c10::hip::getCurrentHIPStream(t.get_device()).stream());
+    return static_cast<void*>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.get_device()).stream());
 }
 
 // cuda/src/sampling.cpp:8-25
@@ -68,7 +68,7 @@ at::Tensor furthest_point_sampling(at::Tensor points, const int nsamples)
     check_gpu(points, "points");
     check_points(points, 3, "points");
     TORCH_CHECK(nsamples >= 0, "nsamples must be non-negative");
-    const c10::hip::HIPGuard guard(points.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(points.device());
 
     at::Tensor output = torch::empty({points.size(0), nsamples},
                                      at::device(points.device()).dtype(at::ScalarType::Int));
@@ -99,7 +99,7 @@ std::vector<at::Tensor> three_nn(at::Tensor unknowns, at::Tensor knows)
     check_points(unknowns, 3, "unknowns");
     check_points(knows, 3, "knows");
     TORCH_CHECK(unknowns.size(0) == knows.size(0), "unknowns and knows differ in batch size");
-    const c10::hip::HIPGuard guard(unknowns.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(unknowns.device());
 
     at::Tensor idx = torch::empty({unknowns.size(0), unknowns.size(1), 3},
                                   at::device(unknowns.device()).dtype(at::ScalarType::Int));
@@ -133,7 +133,7 @@ at::Tensor three_interpolate(at::Tensor points, at::Tensor idx, at::Tensor weigh
     TORCH_CHECK(idx.dim() == 3 && idx.size(2) == 3 && idx.size(0) == points.size(0),
                 "idx must have shape (B, n, 3)");
     TORCH_CHECK(weight.sizes() == idx.sizes(), "weight must have the shape of idx");
-    const c10::hip::HIPGuard guard(points.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(points.device());
 
     at::Tensor output = torch::empty({points.size(0), points.size(1), idx.size(1)},
                                      at::device(points.device()).dtype(at::ScalarType::Float));
@@ -167,7 +167,7 @@ at::Tensor three_interpolate_grad(at::Tensor grad_out, at::Tensor idx, at::Tenso
                 "idx must have shape (B, n, 3)");
     TORCH_CHECK(weight.sizes() == idx.sizes(), "weight must have the shape of idx");
     TORCH_CHECK(m >= 0, "m must be non-negative");
-    const c10::hip::HIPGuard guard(grad_out.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_out.device());
 
     at::Tensor output = torch::empty({grad_out.size(0), grad_out.size(1), m},
                                      at::device(grad_out.device()).dtype(at::ScalarType::Float));
@@ -195,7 +195,7 @@ std::pair<at::Tensor, at::Tensor> ball_query_dense(at::Tensor new_xyz, at::Tenso
     check_points(xyz, 3, "xyz");
     TORCH_CHECK(xyz.size(0) == new_xyz.size(0), "xyz and new_xyz differ in batch size");
     TORCH_CHECK(nsample >= 0, "nsample must be non-negative");
-    const c10::hip::HIPGuard guard(new_xyz.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(new_xyz.device());
 
     at::Tensor idx = torch::empty({new_xyz.size(0), new_xyz.size(1), nsample},
                                   at::device(new_xyz.device()).dtype(at::ScalarType::Long));
@@ -236,7 +236,7 @@ std::pair<at::Tensor, at::Tensor> ball_query_partial_dense(at::Tensor x, at::Ten
     TORCH_CHECK(batch_y.dim() == 1 && batch_y.size(0) == y.size(0),
                 "batch_y must have one entry per point of y");
     TORCH_CHECK(nsample >= 0, "nsample must be non-negative");
-    const c10::hip::HIPGuard guard(x.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
     batch_x = batch_x.contiguous();
     batch_y = batch_y.contiguous();
 
@@ -267,7 +267,7 @@ at::Tensor grouping_operation(at::Tensor features, at::Tensor idx)
     TORCH_CHECK(features.dim() == 3, "features must have shape (B, C, N)");
     TORCH_CHECK(idx.dim() == 3 && idx.size(0) == features.size(0),
                 "idx must have shape (B, npoint, nsample)");
-    const c10::hip::HIPGuard guard(features.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(features.device());
 
     at::Tensor out = torch::empty({features.size(0), features.size(1), idx.size(1), idx.size(2)},
                                   at::device(features.device()).dtype(at::ScalarType::Float));
@@ -294,7 +294,7 @@ at::Tensor grouping_operation_grad(at::Tensor grad_out, at::Tensor idx, const in
                     idx.size(1) == grad_out.size(2) && idx.size(2) == grad_out.size(3),
                 "idx must have shape (B, npoint, nsample)");
     TORCH_CHECK(n >= 0, "n must be non-negative");
-    const c10::hip::HIPGuard guard(grad_out.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_out.device());
 
     at::Tensor out = torch::empty({grad_out.size(0), grad_out.size(1), n},
                                   at::device(grad_out.device()).dtype(at::ScalarType::Float));
@@ -319,7 +319,7 @@ std::vector<torch::Tensor> chamfer_dist(torch::Tensor xyz1, torch::Tensor xyz2)
     TORCH_CHECK(xyz1.scalar_type() == xyz2.scalar_type(), "xyz1 and xyz2 differ in dtype");
     TORCH_CHECK(xyz1.scalar_type() == at::kFloat || xyz1.scalar_type() == at::kDouble,
                 "chamfer_dist supports float32 and float64");
-    const c10::hip::HIPGuard guard(xyz1.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(xyz1.device());
     xyz1 = xyz1.contiguous();
     xyz2 = xyz2.contiguous();
 
@@ -375,7 +375,7 @@ std::vector<torch::Tensor> chamfer_dist_grad(torch::Tensor xyz1, torch::Tensor x
                     idx2.numel() == static_cast<int64_t>(b) * m &&
                     grad_dist1.numel() == idx1.numel() && grad_dist2.numel() == idx2.numel(),
                 "shapes of clouds, indices and gradients do not match");
-    const c10::hip::HIPGuard guard(xyz1.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(xyz1.device());
     xyz1 = xyz1.contiguous();
     xyz2 = xyz2.contiguous();
     idx1 = idx1.contiguous();
