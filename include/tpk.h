@@ -102,12 +102,18 @@ int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* kno
  *   points (b, c, m)   idx (b, n, 3) int32 in [0, m)   weight (b, n, 3)
  *   out (b, c, n) = sum_t points[b, c, idx[b, n, t]] * weight[b, n, t]
  *   grad_points (b, c, m) += grad_out (b, c, n) scattered back (fully written, no pre-zero)
+ * The backward pass inverts the index into per-target lists held in `workspace`
+ * (tpk_three_interpolate_grad_workspace_bytes() bytes, 256-byte aligned; contents need not
+ * be initialised and are garbage afterwards).  With workspace == NULL, or rows too long for
+ * the lists, it falls back to global float atomics - same result to rounding, much slower.
+ * Index values outside [0, m) are ignored by the list path.
  * ------------------------------------------------------------------------------------- */
 int tpk_three_interpolate_f32(int b, int c, int m, int n, const float* points,
                               const int32_t* idx, const float* weight, float* out, void* stream);
+size_t tpk_three_interpolate_grad_workspace_bytes(int b, int n, int m);
 int tpk_three_interpolate_grad_f32(int b, int c, int n, int m, const float* grad_out,
                                    const int32_t* idx, const float* weight, float* grad_points,
-                                   void* stream);
+                                   void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Grouping (gather of feature columns), forward and backward.
@@ -117,11 +123,14 @@ int tpk_three_interpolate_grad_f32(int b, int c, int n, int m, const float* grad
  *   features (b, c, n)   idx (b, npoint, nsample) int64 in [0, n)
  *   out (b, c, npoint, nsample) = features[b, c, idx[b, p, s]]
  *   grad_features (b, c, n) = scatter-add of grad_out (fully written, no pre-zero)
+ * `workspace`: as for tpk_three_interpolate_grad_f32 (tpk_group_grad_workspace_bytes()).
  * ------------------------------------------------------------------------------------- */
 int tpk_group_f32(int b, int c, int n, int npoint, int nsample, const float* features,
                   const int64_t* idx, float* out, void* stream);
+size_t tpk_group_grad_workspace_bytes(int b, int n, int npoint, int nsample);
 int tpk_group_grad_f32(int b, int c, int n, int npoint, int nsample, const float* grad_out,
-                       const int64_t* idx, float* grad_features, void* stream);
+                       const int64_t* idx, float* grad_features, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Chamfer distance, forward (both directions) and backward.

@@ -171,11 +171,15 @@ at::Tensor three_interpolate_grad(at::Tensor grad_out, at::Tensor idx, at::Tenso
 
     at::Tensor output = torch::empty({grad_out.size(0), grad_out.size(1), m},
                                      at::device(grad_out.device()).dtype(at::ScalarType::Float));
+    const int b = as_int(grad_out.size(0), "batch size");
+    const int n = as_int(grad_out.size(2), "n");
+    const size_t ws_bytes = tpk_three_interpolate_grad_workspace_bytes(b, n, m);
+    at::Tensor ws = torch::empty({static_cast<int64_t>(ws_bytes)},
+                                 at::device(grad_out.device()).dtype(at::ScalarType::Byte));
     check_status(tpk_three_interpolate_grad_f32(
-                     as_int(grad_out.size(0), "batch size"), as_int(grad_out.size(1), "channels"),
-                     as_int(grad_out.size(2), "n"), m, grad_out.data_ptr<float>(),
+                     b, as_int(grad_out.size(1), "channels"), n, m, grad_out.data_ptr<float>(),
                      idx.data_ptr<int32_t>(), weight.data_ptr<float>(), output.data_ptr<float>(),
-                     current_stream(grad_out)),
+                     ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, current_stream(grad_out)),
                  "three_interpolate_grad");
     return output;
 }
@@ -298,11 +302,16 @@ at::Tensor grouping_operation_grad(at::Tensor grad_out, at::Tensor idx, const in
 
     at::Tensor out = torch::empty({grad_out.size(0), grad_out.size(1), n},
                                   at::device(grad_out.device()).dtype(at::ScalarType::Float));
-    check_status(tpk_group_grad_f32(as_int(grad_out.size(0), "batch size"),
-                                    as_int(grad_out.size(1), "channels"), n,
-                                    as_int(idx.size(1), "npoint"), as_int(idx.size(2), "nsample"),
+    const int b = as_int(grad_out.size(0), "batch size");
+    const int npoint = as_int(idx.size(1), "npoint");
+    const int nsample = as_int(idx.size(2), "nsample");
+    const size_t ws_bytes = tpk_group_grad_workspace_bytes(b, n, npoint, nsample);
+    at::Tensor ws = torch::empty({static_cast<int64_t>(ws_bytes)},
+                                 at::device(grad_out.device()).dtype(at::ScalarType::Byte));
+    check_status(tpk_group_grad_f32(b, as_int(grad_out.size(1), "channels"), n, npoint, nsample,
                                     grad_out.data_ptr<float>(), idx.data_ptr<int64_t>(),
-                                    out.data_ptr<float>(), current_stream(grad_out)),
+                                    out.data_ptr<float>(), ws_bytes ? ws.data_ptr() : nullptr,
+                                    ws_bytes, current_stream(grad_out)),
                  "grouping_operation_grad");
     return out;
 }
