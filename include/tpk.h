@@ -143,20 +143,24 @@ int tpk_group_grad_f32(int b, int c, int n, int npoint, int nsample, const float
  *   int32 its index (lowest index on ties); dist2 (b, m), idx2 (b, m) the other direction.
  *   grad_xyz1 (b, n, 3), grad_xyz2 (b, m, 3): fully written, no pre-zero needed.
  * n == 0 or m == 0 yields zeros, as the reference's zero-initialised outputs do.
+ * The backward pass inverts idx1 / idx2 into per-point lists held in `workspace`
+ * (tpk_chamfer_bwd_workspace_bytes() bytes, 256-byte aligned, contents arbitrary before and
+ * after); with workspace == NULL it scatters with hardware float atomics instead (slower).
  * ------------------------------------------------------------------------------------- */
 int tpk_chamfer_fwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2, float* dist1,
                         float* dist2, int32_t* idx1, int32_t* idx2, void* stream);
 int tpk_chamfer_fwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
                         double* dist1, double* dist2, int32_t* idx1, int32_t* idx2,
                         void* stream);
+size_t tpk_chamfer_bwd_workspace_bytes(int b, int n, int m);
 int tpk_chamfer_bwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2,
                         const int32_t* idx1, const int32_t* idx2, const float* grad_dist1,
                         const float* grad_dist2, float* grad_xyz1, float* grad_xyz2,
-                        void* stream);
+                        void* workspace, size_t workspace_bytes, void* stream);
 int tpk_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
                         const int32_t* idx1, const int32_t* idx2, const double* grad_dist1,
                         const double* grad_dist2, double* grad_xyz1, double* grad_xyz2,
-                        void* stream);
+                        void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -17,11 +17,15 @@
 // whose distance equals the minimum: the same candidate a serial first-strictly-smaller
 // scan (cuda/src/chamfer_dist_gpu.cu:9-155) ends on.
 //
-// Backward (cuda/src/chamfer_dist_gpu.cu:187-245).  Each point's own term is stored
-// plainly by a first kernel (so the outputs need no zero fill), the terms scattered to the
-// matched points of the other cloud are added by a second kernel with hardware float
-// atomics.  The order of those additions is not fixed, exactly as in the reference.
-#include "tpk_device.h"
+// Backward (cuda/src/chamfer_dist_gpu.cu:187-245).  A point's gradient is its own term,
+// 2*g*(p - nearest), plus one term from every point of the other cloud that chose it as
+// nearest neighbour.  The reference scatters those with float atomics.  Here the two
+// nearest-neighbour index arrays are inverted into per-target lists (lists.h) and one
+// kernel, one lane per point, adds the own term and walks the point's list: no atomics, no
+// zero fill, every output written once.  Without workspace for the lists the scatter falls
+// back to hardware float atomics (own terms stored first by one kernel, scattered terms
+// added by a second).
+#include "lists.h"
 
 namespace {
 
@@ -250,6 +254,73 @@ __global__ __launch_bounds__(256) void chamfer_bwd_scatter_kernel(
     }
 }
 
+// One lane per point of either cloud: own term, then the terms of the points that chose it.
+// offs_a/ent_a: lists over the points of cloud 1 (built from idx2); offs_b/ent_b: lists over
+// the points of cloud 2 (built from idx1).
+template <typename T>
+__global__ __launch_bounds__(256) void chamfer_bwd_lists_kernel(
+    int n, int m, int clouds, const T* __restrict__ xyz1, const T* __restrict__ xyz2,
+    const int32_t* __restrict__ idx1, const int32_t* __restrict__ idx2,
+    const T* __restrict__ grad_dist1, const T* __restrict__ grad_dist2,
+    const int* __restrict__ offs_a, const ListEntry<false>* __restrict__ ent_a,
+    const int* __restrict__ offs_b, const ListEntry<false>* __restrict__ ent_b,
+    T* __restrict__ grad_xyz1, T* __restrict__ grad_xyz2)
+{
+    // blockIdx.y: cloud; blockIdx.x covers the n points of cloud 1 first, then the m of cloud 2
+    const int blocks1 = (n + 255) / 256;
+    for (int cloud = blockIdx.y; cloud < clouds; cloud += gridDim.y)
+    {
+        const bool second = static_cast<int>(blockIdx.x) >= blocks1;
+        const int k = (second ? blockIdx.x - blocks1 : blockIdx.x) * 256 + threadIdx.x;
+        const int npts = second ? m : n;
+        const int nother = second ? n : m;
+        if (k >= npts)
+            continue;
+        const T* __restrict__ own = (second ? xyz2 : xyz1) + static_cast<int64_t>(cloud) * npts * 3;
+        const T* __restrict__ other = (second ? xyz1 : xyz2) + static_cast<int64_t>(cloud) * nother * 3;
+        const int32_t* __restrict__ own_idx = (second ? idx2 : idx1) + static_cast<int64_t>(cloud) * npts;
+        const T* __restrict__ own_g = (second ? grad_dist2 : grad_dist1) + static_cast<int64_t>(cloud) * npts;
+        const T* __restrict__ other_g = (second ? grad_dist1 : grad_dist2) + static_cast<int64_t>(cloud) * nother;
+        const int* __restrict__ offs = (second ? offs_b : offs_a) + static_cast<int64_t>(cloud) * (npts + 1);
+        const ListEntry<false>* __restrict__ ent = (second ? ent_b : ent_a) + static_cast<int64_t>(cloud) * nother;
+        T* __restrict__ out = (second ? grad_xyz2 : grad_xyz1) + (static_cast<int64_t>(cloud) * npts + k) * 3;
+
+        const T px = own[k * 3 + 0], py = own[k * 3 + 1], pz = own[k * 3 + 2];
+        const int j2 = own_idx[k];
+        const T g = own_g[k] * 2;
+        T ax = g * (px - other[j2 * 3 + 0]);
+        T ay = g * (py - other[j2 * 3 + 1]);
+        T az = g * (pz - other[j2 * 3 + 2]);
+        const int beg = offs[k], end = offs[k + 1];
+        for (int p = beg; p < end; ++p)
+        {
+            const int j = ent[p].j;
+            const T gj = other_g[j] * 2;
+            ax = ax + -(gj * (other[j * 3 + 0] - px));
+            ay = ay + -(gj * (other[j * 3 + 1] - py));
+            az = az + -(gj * (other[j * 3 + 2] - pz));
+        }
+        out[0] = ax;
+        out[1] = ay;
+        out[2] = az;
+    }
+}
+
+size_t chamfer_lists_bytes(int b, int n, int m, size_t* off_a, size_t* off_b, size_t* ent_a, size_t* ent_b)
+{
+    auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    size_t pos = 0;
+    *off_a = pos;
+    pos = up(pos + static_cast<size_t>(b) * (static_cast<size_t>(n) + 1) * sizeof(int));
+    *off_b = pos;
+    pos = up(pos + static_cast<size_t>(b) * (static_cast<size_t>(m) + 1) * sizeof(int));
+    *ent_a = pos;
+    pos = up(pos + static_cast<size_t>(b) * static_cast<size_t>(m) * sizeof(ListEntry<false>));
+    *ent_b = pos;
+    pos = up(pos + static_cast<size_t>(b) * static_cast<size_t>(n) * sizeof(ListEntry<false>));
+    return pos;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void fill_zero_kernel(T* p, int64_t count)
 {
@@ -300,7 +371,7 @@ int chamfer_fwd(int b, int n, int m, const T* xyz1, const T* xyz2, T* dist1, T* 
 template <typename T>
 int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t* idx1,
                 const int32_t* idx2, const T* grad_dist1, const T* grad_dist2, T* grad_xyz1,
-                T* grad_xyz2, void* stream)
+                T* grad_xyz2, void* workspace, size_t workspace_bytes, void* stream)
 {
     if (b < 0 || n < 0 || m < 0)
         return TPK_ERR_INVALID_ARG;
@@ -321,6 +392,32 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
         const unsigned blocks = static_cast<unsigned>(tpk_min64(tpk_ceil_div(count, 256), 4096));
         hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(blocks), dim3(256), 0, s, p, count);
         return tpk_launch_status();
+    }
+    size_t off_a, off_b, ent_a, ent_b;
+    const size_t need = chamfer_lists_bytes(b, n, m, &off_a, &off_b, &ent_a, &ent_b);
+    if (workspace && workspace_bytes >= need && static_cast<int64_t>(n) * 3 <= 0x7fffffffLL &&
+        static_cast<int64_t>(m) * 3 <= 0x7fffffffLL)
+    {
+        char* ws = static_cast<char*>(workspace);
+        int* offs_a = reinterpret_cast<int*>(ws + off_a);
+        int* offs_b = reinterpret_cast<int*>(ws + off_b);
+        auto* ents_a = reinterpret_cast<ListEntry<false>*>(ws + ent_a);
+        auto* ents_b = reinterpret_cast<ListEntry<false>*>(ws + ent_b);
+        // lists over cloud-1 points: who in cloud 2 chose them (idx2); and the mirror image
+        int st = launch_build_lists<1, false, int32_t>(b, n, m, idx2, nullptr, offs_a, ents_a, s);
+        if (st == TPK_OK)
+            st = launch_build_lists<1, false, int32_t>(b, m, n, idx1, nullptr, offs_b, ents_b, s);
+        if (st == TPK_OK)
+        {
+            const unsigned bx = static_cast<unsigned>(tpk_ceil_div(n, 256) + tpk_ceil_div(m, 256));
+            const unsigned by = static_cast<unsigned>(b < 65535 ? b : 65535);
+            hipLaunchKernelGGL(chamfer_bwd_lists_kernel<T>, dim3(bx, by), dim3(256), 0, s, n, m, b, xyz1,
+                               xyz2, idx1, idx2, grad_dist1, grad_dist2, offs_a, ents_a, offs_b,
+                               ents_b, grad_xyz1, grad_xyz2);
+            return tpk_launch_status();
+        }
+        if (st != TPK_ERR_UNSUPPORTED)
+            return st;
     }
     const unsigned blocks =
         static_cast<unsigned>(tpk_min64(tpk_ceil_div(total1 + total2, 256), 1 << 20));
@@ -355,17 +452,27 @@ extern "C" int tpk_chamfer_fwd_f64(int b, int n, int m, const double* xyz1, cons
 extern "C" int tpk_chamfer_bwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2,
                                    const int32_t* idx1, const int32_t* idx2,
                                    const float* grad_dist1, const float* grad_dist2,
-                                   float* grad_xyz1, float* grad_xyz2, void* stream)
+                                   float* grad_xyz1, float* grad_xyz2, void* workspace,
+                                   size_t workspace_bytes, void* stream)
 {
     return chamfer_bwd<float>(b, n, m, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2, grad_xyz1,
-                              grad_xyz2, stream);
+                            grad_xyz2, workspace, workspace_bytes, stream);
 }
 
 extern "C" int tpk_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
                                    const int32_t* idx1, const int32_t* idx2,
                                    const double* grad_dist1, const double* grad_dist2,
-                                   double* grad_xyz1, double* grad_xyz2, void* stream)
+                                   double* grad_xyz1, double* grad_xyz2, void* workspace,
+                                   size_t workspace_bytes, void* stream)
 {
-    return chamfer_bwd<double>(b, n, m, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2,
-                               grad_xyz1, grad_xyz2, stream);
+    return chamfer_bwd<double>(b, n, m, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2, grad_xyz1,
+                            grad_xyz2, workspace, workspace_bytes, stream);
+}
+
+extern "C" size_t tpk_chamfer_bwd_workspace_bytes(int b, int n, int m)
+{
+    if (b <= 0 || n <= 0 || m <= 0)
+        return 0;
+    size_t a, bb, c, d;
+    return chamfer_lists_bytes(b, n, m, &a, &bb, &c, &d);
 }

@@ -394,6 +394,9 @@ std::vector<torch::Tensor> chamfer_dist_grad(torch::Tensor xyz1, torch::Tensor x
 
     torch::Tensor grad_xyz1 = torch::empty_like(xyz1);
     torch::Tensor grad_xyz2 = torch::empty_like(xyz2);
+    const size_t ws_bytes = tpk_chamfer_bwd_workspace_bytes(b, n, m);
+    torch::Tensor ws = torch::empty({static_cast<int64_t>(ws_bytes)}, xyz1.options().dtype(torch::kByte));
+    void* wsp = ws_bytes ? ws.data_ptr() : nullptr;
     void* s = current_stream(xyz1);
     if (xyz1.scalar_type() == at::kFloat)
         check_status(tpk_chamfer_bwd_f32(b, n, m, xyz1.data_ptr<float>(), xyz2.data_ptr<float>(),
@@ -401,7 +404,7 @@ std::vector<torch::Tensor> chamfer_dist_grad(torch::Tensor xyz1, torch::Tensor x
                                          grad_dist1.data_ptr<float>(),
                                          grad_dist2.data_ptr<float>(),
                                          grad_xyz1.data_ptr<float>(),
-                                         grad_xyz2.data_ptr<float>(), s),
+                                         grad_xyz2.data_ptr<float>(), wsp, ws_bytes, s),
                      "chamfer_dist_grad");
     else
         check_status(tpk_chamfer_bwd_f64(b, n, m, xyz1.data_ptr<double>(),
@@ -409,7 +412,7 @@ std::vector<torch::Tensor> chamfer_dist_grad(torch::Tensor xyz1, torch::Tensor x
                                          idx2.data_ptr<int32_t>(), grad_dist1.data_ptr<double>(),
                                          grad_dist2.data_ptr<double>(),
                                          grad_xyz1.data_ptr<double>(),
-                                         grad_xyz2.data_ptr<double>(), s),
+                                         grad_xyz2.data_ptr<double>(), wsp, ws_bytes, s),
                      "chamfer_dist_grad");
     return {grad_xyz1, grad_xyz2};
 }
