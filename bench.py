@@ -34,11 +34,11 @@ PEAK_FP32_TFLOPS = 157.3  # vector == matrix fp32 figure; counts packed FMA (4 f
 # scaled by the same counter's reading for a 256 MiB device copy); see profiles/*pmc*.txt.
 # None = not measured yet.
 MEASURED_TRAFFIC_BYTES = {
-    "fps": None,
-    "three_interpolate_fwd": None,
-    "three_interpolate_bwd": None,
-    "grouping_fwd": None,
-    "grouping_bwd": None,
+    "fps": 3561000,                    # 3.30 MB read (the clouds) + 0.26 MB written (the indices)
+    "three_interpolate_fwd": 174130000,  # = algorithmic bytes: nothing is read twice from HBM
+    "three_interpolate_bwd": 299500000,  # list build 79 MB + list walk 220 MB (lists re-read per row block)
+    "grouping_fwd": 352500000,         # rows staged twice (two column halves per row block)
+    "grouping_bwd": 373400000,
     "chamfer_bwd": None,
 }
 
