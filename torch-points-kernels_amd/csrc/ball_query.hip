@@ -186,9 +186,10 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
         const int j = jq0 + q;
         const bool ok = j < m;
         const int jj = ok ? j : m - 1;
-        qx[q] = new_xyz[jj * 3 + 0];
-        qy[q] = new_xyz[jj * 3 + 1];
-        qz[q] = new_xyz[jj * 3 + 2];
+        // wave-uniform values, kept in vector registers (double-rate fp32 arithmetic)
+        qx[q] = to_vector_register(new_xyz[jj * 3 + 0]);
+        qy[q] = to_vector_register(new_xyz[jj * 3 + 1]);
+        qz[q] = to_vector_register(new_xyz[jj * 3 + 2]);
         in_run |= ok ? (1u << q) : 0u;
     }
     scan_run<false>(tile, xyz, 0, n, in_run, qx, qy, qz, radius2, nsample,
@@ -213,9 +214,9 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_partial_kernel(
     {
         const int64_t j = jq0 + q;
         const int64_t jj = j < size_y ? j : size_y - 1;
-        qx[q] = y[jj * 3 + 0];
-        qy[q] = y[jj * 3 + 1];
-        qz[q] = y[jj * 3 + 2];
+        qx[q] = to_vector_register(y[jj * 3 + 0]);
+        qy[q] = to_vector_register(y[jj * 3 + 1]);
+        qz[q] = to_vector_register(y[jj * 3 + 2]);
         qc[q] = batch_y[jj];
     }
 
