@@ -28,7 +28,7 @@ for _p in (ROOT, os.path.join(ROOT, "torch-points-kernels_amd")):
 
 # Published MI355X peaks used for the roofline fractions.
 PEAK_HBM_GBS = 8000.0
-PEAK_FP32_TFLOPS = 157.3  # vector == matrix fp32 figure; counts packed FMA (4 flop/lane/clk)
+PEAK_FP32_TFLOPS = 157.3  # published fp32 figure (vector = matrix); it counts every lane-op as an FMA (2 flop)
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE run + WRITE_SIZE run, each
 # scaled by the same counter's reading for a 256 MiB device copy); see profiles/*pmc*.txt.
@@ -68,7 +68,7 @@ def _roof_flops(pairs_or_updates, flops_each, ms):
     return {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
             "frac": achieved / PEAK_FP32_TFLOPS, "traffic": None,
             "note": "fp32 VALU kernel (inner dimension 3, unfused arithmetic: no MFMA, no FMA, no packed "
-                    "fp32); peak is the published fp32 figure, which assumes packed FMA"}
+                    "fp32); peak is the published fp32 figure, which assumes FMA: without FMA the ceiling is 0.5"}
 
 
 def _roof_bytes(nbytes, ms, key):
