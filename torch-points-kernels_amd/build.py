@@ -23,9 +23,13 @@ HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
 # -ffp-contract=off: products and sums round separately (integer outputs depend on it).
 # -packed-fp32-ops: packed fp32 VALU instructions are not to be generated.
+# -simplifycfg-sink-common=false: keeps the arms of wave-uniform branches that pick one element
+#   of a register-resident array from being merged into one indexed access, which would move
+#   the whole array to scratch memory (fps.hip).
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-simplifycfg-sink-common=false",
     "-Wall", "-Wno-unused-function", "-I" + INCLUDE,
 ]
 

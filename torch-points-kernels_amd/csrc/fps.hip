@@ -103,10 +103,11 @@ __device__ __forceinline__ int winning_lane(int val, unsigned tk, int& wave_val)
 template <int WAVES>
 __device__ __forceinline__ void reduce_records(const WaveRecord* __restrict__ rec, int lane,
                                                float p0x, float p0y, float p0z, int& k,
-                                               float& sx, float& sy, float& sz)
+                                               float& sx, float& sy, float& sz, int& gv_out)
 {
     const WaveRecord e = rec[lane & (WAVES - 1)];
     const int gv = __builtin_amdgcn_readfirstlane(row_all_max_i32(e.val));
+    gv_out = gv;
     constexpr unsigned wave_bits = (1u << WAVES) - 1u;
     const unsigned top = static_cast<unsigned>(__ballot(e.val == gv)) & wave_bits;
     int w;
@@ -287,9 +288,424 @@ __global__ __launch_bounds__(THREADS) void fps_resident_kernel(
 
         // 3. all wavefronts reduce the records
         int k;
-        reduce_records<WAVES>(records[j & 1], lane, p0x, p0y, p0z, k, sx, sy, sz);
+        int gv_unused;
+        reduce_records<WAVES>(records[j & 1], lane, p0x, p0y, p0z, k, sx, sy, sz, gv_unused);
         if (tid == 0)
             out[j] = k;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Register-resident kernel with exact pruning, for clouds of a few thousand to 16384 points.
+//
+// A point's running minimum changes in a round only if its distance to the new sample is
+// smaller than that minimum, and no minimum exceeds the value that won the previous round.
+// So a set of points whose bounding box is further from the new sample than the square root
+// of the previous winning value cannot change, and its update can be skipped without
+// changing any result.  To make such sets exist, the kernel first sorts the cloud along a
+// Z-order curve (18-bit Morton code, bitonic sort in LDS) and gives every lane GS points of
+// each of NG consecutive curve segments ("groups"): group g is slots g*GS.. of ALL lanes,
+// so skipping it is a wave-uniform decision shared by all wavefronts (no load imbalance).
+// The skip test of all groups is evaluated at once, lane g testing the box of group g.
+// The fp32 box distance is compared with a relative margin of 2e-6, several times the
+// rounding error of either side, so a skipped update is provably a no-op.
+//
+// Because slots are no longer in index order, the original index of every point is kept in
+// a register and equal maxima are resolved explicitly by the reference's tie key.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned spread_bits_6(unsigned v) // abcdef -> a00b00c00d00e00f
+{
+    v &= 0x3Fu;
+    v = (v | (v << 8)) & 0x300Fu;
+    v = (v | (v << 4)) & 0x30C3u;
+    v = (v | (v << 2)) & 0x9249u;
+    return v;
+}
+
+// Order-preserving map of a float to a signed integer (for integer atomic min / max).
+__device__ __forceinline__ int float_to_ordered_int(float f)
+{
+    const int b = __float_as_int(f);
+    return b >= 0 ? b : b ^ 0x7FFFFFFF;
+}
+__device__ __forceinline__ float ordered_int_to_float(int b)
+{
+    return __int_as_float(b >= 0 ? b : b ^ 0x7FFFFFFF);
+}
+
+__device__ __forceinline__ unsigned tie_key(int k, int log2_bs, int ref_groups)
+{
+    const unsigned bs_mask = (1u << log2_bs) - 1u;
+    const unsigned rev = log2_bs ? (__brev(static_cast<unsigned>(k) & bs_mask) >> (32 - log2_bs)) : 0u;
+    return rev * static_cast<unsigned>(ref_groups) + (static_cast<unsigned>(k) >> log2_bs);
+}
+
+// Every lane selects, among the GS members of its group `grp` (wave-uniform, reached through
+// a binary tree of scalar branches), the one whose running minimum equals `value`; `hits`
+// counts the members that equal it.
+template <int PPT, int GS, int LO, int HI>
+struct GroupSelect
+{
+    __device__ __forceinline__ static void run(const float (&x)[PPT], const float (&y)[PPT],
+                                               const float (&z)[PPT], const int (&t)[PPT], int grp,
+                                               int value, int& hits, float& cx, float& cy,
+                                               float& cz, int& ce)
+    {
+        if constexpr (HI - LO == 1)
+        {
+#pragma unroll
+            for (int e = GS - 1; e >= 0; --e)
+            {
+                const int i = LO * GS + e;
+                const bool match = t[i] == value;
+                hits += match ? 1 : 0;
+                cx = match ? x[i] : cx;
+                cy = match ? y[i] : cy;
+                cz = match ? z[i] : cz;
+                ce = match ? e : ce;
+            }
+        }
+        else
+        {
+            constexpr int MID = (LO + HI) / 2;
+            if (grp < MID)
+                GroupSelect<PPT, GS, LO, MID>::run(x, y, z, t, grp, value, hits, cx, cy, cz, ce);
+            else
+                GroupSelect<PPT, GS, MID, HI>::run(x, y, z, t, grp, value, hits, cx, cy, cz, ce);
+        }
+    }
+};
+
+// The words of LDS through which the wavefronts of a workgroup agree on a round's winner.
+struct RoundWords
+{
+    int max_val;      // atomic max of the running minima (bit patterns), starts at INT_MIN
+    int winners;      // 1 when exactly one point holds max_val, more when several may
+    unsigned min_tie; // atomic min of the tie keys of the points holding max_val (ties only)
+    int pad;
+};
+
+// Workgroup barrier that orders LDS traffic only (outstanding global stores of sample
+// indices need not complete before the next round).
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): also covers the LDS atomics issued below
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// LDS atomics without return value, issued as written: one instruction for the active lanes
+// (the compiler would otherwise wrap a same-address atomic in a loop over those lanes).
+__device__ __forceinline__ unsigned lds_offset(const void* p)
+{
+    return static_cast<unsigned>(reinterpret_cast<unsigned long long>(
+        (const __attribute__((address_space(3))) char*)p));
+}
+__device__ __forceinline__ void lds_atomic_max_i32(int* p, int v)
+{
+    asm volatile("ds_max_i32 %0, %1" ::"v"(lds_offset(p)), "v"(v) : "memory");
+}
+__device__ __forceinline__ void lds_atomic_add_u32(int* p, int v)
+{
+    asm volatile("ds_add_u32 %0, %1" ::"v"(lds_offset(p)), "v"(v) : "memory");
+}
+
+template <int PPT, int THREADS, int GS>
+__global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
+    int n, int npoint, int log2_bs, int ref_groups, int sort_n, const float* __restrict__ xyz,
+    int32_t* __restrict__ out)
+{
+    constexpr int WAVES = THREADS / TPK_WAVE;
+    constexpr int NG = PPT / GS;
+    static_assert(NG <= 16, "one DPP row of lanes tests the group boxes");
+    static_assert(WAVES >= 2, "a cloud without eligible points must count several winners");
+    // sort_n keys (morton << 14) | index, kept for the whole kernel, then PPT * THREADS words
+    // into which the running minima are copied when equal maxima have to be resolved
+    extern __shared__ unsigned sort_keys[];
+    int* const t_copy = reinterpret_cast<int*>(sort_keys + sort_n);
+    __shared__ RoundWords words[2];
+    __shared__ float4 record[2];      // x, y, z of the round's winner and its sorted position
+    __shared__ int cloud_box[6];      // ordered ints: min x,y,z then max x,y,z
+    __shared__ int group_box[16 * 6]; // the same per group
+
+    xyz += static_cast<int64_t>(blockIdx.x) * n * 3;
+    out += static_cast<int64_t>(blockIdx.x) * npoint;
+    const int tid = threadIdx.x;
+    const int lane = tid & (TPK_WAVE - 1);
+
+    // ---- set-up 1: box of the cloud (only to quantise coordinates for the curve)
+    const int empty_lo = float_to_ordered_int(__builtin_inff());
+    const int empty_hi = float_to_ordered_int(-__builtin_inff());
+    if (tid < 6)
+        cloud_box[tid] = tid < 3 ? empty_lo : empty_hi;
+    for (int i = tid; i < NG * 6; i += THREADS)
+        group_box[i] = (i % 6) < 3 ? empty_lo : empty_hi;
+    if (tid < 2)
+        words[tid] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
+    __syncthreads();
+    {
+        float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
+        float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};
+        for (int k = tid; k < n; k += THREADS)
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+            {
+                const float v = xyz[k * 3 + a];
+                lo[a] = fminf(lo[a], v);
+                hi[a] = fmaxf(hi[a], v);
+            }
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+        {
+            atomicMin(&cloud_box[a], float_to_ordered_int(lo[a]));
+            atomicMax(&cloud_box[3 + a], float_to_ordered_int(hi[a]));
+        }
+    }
+    __syncthreads();
+
+    // ---- set-up 2: sort keys = position on the Z-order curve, then the index
+    {
+        float lo[3], scale[3];
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+        {
+            lo[a] = ordered_int_to_float(cloud_box[a]);
+            const float ext = ordered_int_to_float(cloud_box[3 + a]) - lo[a];
+            scale[a] = ext > 0.f ? 63.999f / ext : 0.f;
+        }
+        for (int k = tid; k < sort_n; k += THREADS)
+        {
+            unsigned key = 0xFFFFFFFFu; // padding sorts last
+            if (k < n)
+            {
+                unsigned code = 0;
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                {
+                    float q = (xyz[k * 3 + a] - lo[a]) * scale[a];
+                    q = q >= 0.f ? q : 0.f; // also maps NaN to cell 0
+                    const unsigned cell = q < 63.f ? static_cast<unsigned>(q) : 63u;
+                    code |= spread_bits_6(cell) << a;
+                }
+                key = (code << 14) | static_cast<unsigned>(k);
+            }
+            sort_keys[k] = key;
+        }
+    }
+    __syncthreads();
+    for (int size = 2; size <= sort_n; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1)
+        {
+            for (int i0 = tid; i0 < (sort_n >> 1); i0 += THREADS)
+            {
+                const int i = ((i0 & ~(stride - 1)) << 1) | (i0 & (stride - 1));
+                const int p = i | stride;
+                const unsigned a = sort_keys[i], b = sort_keys[p];
+                const bool ascending = (i & size) == 0;
+                if ((a > b) == ascending)
+                {
+                    sort_keys[i] = b;
+                    sort_keys[p] = a;
+                }
+            }
+            __syncthreads();
+        }
+
+    // ---- set-up 3: this lane's points.  Slot i = group (i / GS), member (i % GS); group g
+    // holds the curve positions [g * THREADS * GS, (g + 1) * THREADS * GS).
+    float x[PPT], y[PPT], z[PPT];
+    int t[PPT];
+#pragma unroll
+    for (int gi = 0; gi < NG; ++gi)
+    {
+        float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
+        float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};
+#pragma unroll
+        for (int e = 0; e < GS; ++e)
+        {
+            const int i = gi * GS + e;
+            const int q = gi * (THREADS * GS) + e * THREADS + tid;
+            const int k = static_cast<int>(sort_keys[q < n ? q : 0] & 0x3FFFu);
+            const float px = xyz[k * 3 + 0], py = xyz[k * 3 + 1], pz = xyz[k * 3 + 2];
+            const bool ok = q < n && eligible(px, py, pz);
+            x[i] = ok ? px : 0.f;
+            y[i] = ok ? py : 0.f;
+            z[i] = ok ? pz : 0.f;
+            t[i] = ordered_bits(ok ? 1e10f : -1.0f);
+            lo[0] = ok ? fminf(lo[0], px) : lo[0];
+            lo[1] = ok ? fminf(lo[1], py) : lo[1];
+            lo[2] = ok ? fminf(lo[2], pz) : lo[2];
+            hi[0] = ok ? fmaxf(hi[0], px) : hi[0];
+            hi[1] = ok ? fmaxf(hi[1], py) : hi[1];
+            hi[2] = ok ? fmaxf(hi[2], pz) : hi[2];
+        }
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+        {
+            atomicMin(&group_box[gi * 6 + a], float_to_ordered_int(lo[a]));
+            atomicMax(&group_box[gi * 6 + 3 + a], float_to_ordered_int(hi[a]));
+        }
+    }
+    __syncthreads();
+    // lane g of every 16-lane row tests group g; lanes beyond NG hold an empty box
+    const int my_group = lane & 15;
+    float blo[3], bhi[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+    {
+        blo[a] = my_group < NG ? ordered_int_to_float(group_box[my_group * 6 + a]) : __builtin_inff();
+        bhi[a] = my_group < NG ? ordered_int_to_float(group_box[my_group * 6 + 3 + a]) : -__builtin_inff();
+    }
+
+    int g[NG]; // per-lane maximum of each group, kept across rounds
+#pragma unroll
+    for (int gi = 0; gi < NG; ++gi)
+    {
+        g[gi] = t[gi * GS];
+#pragma unroll
+        for (int e = 1; e < GS; ++e)
+            g[gi] = max(g[gi], t[gi * GS + e]);
+    }
+
+    const float p0x = xyz[0], p0y = xyz[1], p0z = xyz[2];
+    float vx = p0x, vy = p0y, vz = p0z;         // the last sample (the same in every lane)
+    int bound = ordered_bits(__builtin_inff()); // no running minimum exceeds this
+    const bool row_head = (lane & 15) == 0;
+    if (tid == 0)
+        out[0] = 0;
+
+    for (int j = 1; j < npoint; ++j)
+    {
+        const int par = j & 1;
+
+        // 1. which groups can change?  squared distance from the sample to the group's box
+        unsigned live; // bit g set: group g must be updated
+        {
+            const float dx = fmaxf(fmaxf(blo[0] - vx, vx - bhi[0]), 0.f);
+            const float dy = fmaxf(fmaxf(blo[1] - vy, vy - bhi[1]), 0.f);
+            const float dz = fmaxf(fmaxf(blo[2] - vz, vz - bhi[2]), 0.f);
+            const float lb = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz)) * 0.999998f;
+            // an empty box gives lb = +inf (never live); NaN compares false -> live
+            const bool skip = lb >= __int_as_float(bound);
+            live = static_cast<unsigned>(__ballot(!skip)) & ((1u << NG) - 1u);
+        }
+
+        // 2. distance update of the live groups
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi)
+        {
+            if ((live >> gi) & 1u) // wave-uniform
+            {
+#pragma unroll
+                for (int e = 0; e < GS; ++e)
+                {
+                    const int i = gi * GS + e;
+                    const float d = tpk_dist2(x[i], y[i], z[i], vx, vy, vz);
+                    t[i] = min(t[i], ordered_bits(d));
+                    g[gi] = e == 0 ? t[i] : max(g[gi], t[i]);
+                }
+            }
+        }
+        int best = g[0];
+#pragma unroll
+        for (int gi = 1; gi < NG; ++gi)
+            best = max(best, g[gi]);
+
+        // 3. workgroup maximum: DPP reduction over each 16-lane row, then one LDS atomic per row
+        const int row_val = row_all_max_i32(best);
+        if (row_head)
+            lds_atomic_max_i32(&words[par].max_val, row_val);
+        lds_barrier();
+        const int gv_lanes = words[par].max_val;
+        const int gv = __builtin_amdgcn_readfirstlane(gv_lanes);
+
+        // 4. only a wavefront holding the maximum looks for the slot and publishes the point
+        const unsigned long long top = __ballot(best == gv);
+        if (top != 0)
+        {
+            int my_grp = 0, my_hits = 0;
+#pragma unroll
+            for (int gi = NG - 1; gi >= 0; --gi)
+            {
+                const bool m = g[gi] == best;
+                my_grp = m ? gi : my_grp;
+                my_hits += m ? 1 : 0;
+            }
+            const int wl = __builtin_ctzll(top);
+            const int grp = __builtin_amdgcn_readlane(my_grp, wl);
+            int hits = 0, ce = 0;
+            float cx = 0.f, cy = 0.f, cz = 0.f;
+            GroupSelect<PPT, GS, 0, NG>::run(x, y, z, t, grp, gv, hits, cx, cy, cz, ce);
+            const bool single = __builtin_popcountll(top) == 1 &&
+                                __builtin_amdgcn_readlane(my_hits, wl) == 1 &&
+                                __builtin_amdgcn_readlane(hits, wl) == 1;
+            if (lane == wl)
+            {
+                const int pos = grp * (THREADS * GS) + ce * THREADS + tid;
+                record[par] = make_float4(cx, cy, cz, __int_as_float(pos));
+                lds_atomic_add_u32(&words[par].winners, single ? 1 : 2);
+                words[par ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0}; // for the next round
+                if (single)
+                    out[j] = static_cast<int>(sort_keys[pos] & 0x3FFFu);
+            }
+        }
+        lds_barrier();
+        float4 rec = record[par];
+        const int winners = __builtin_amdgcn_readfirstlane(words[par].winners);
+
+        if (winners != 1)
+        {
+            // Rare: several points hold the maximum (or none is eligible).
+            if (gv < 0)
+            {
+                // No eligible point in the whole cloud: the reference's reduction yields index 0.
+                rec = make_float4(p0x, p0y, p0z, 0.f);
+                if (tid == 0)
+                    out[j] = 0;
+            }
+            else
+            {
+                // The smallest tie key decides.  The running minima go through LDS so that
+                // this path can loop over the slots without indexing registers dynamically.
+#pragma unroll
+                for (int i = 0; i < PPT; ++i)
+                    t_copy[i * THREADS + tid] = t[i];
+                unsigned my_tk = 0xFFFFFFFFu;
+                int my_q = 0;
+#pragma clang loop unroll(disable)
+                for (int i = 0; i < PPT; ++i)
+                {
+                    const int q = (i / GS) * (THREADS * GS) + (i % GS) * THREADS + tid;
+                    if (t_copy[i * THREADS + tid] == gv && q < n)
+                    {
+                        const unsigned tk =
+                            tie_key(static_cast<int>(sort_keys[q] & 0x3FFFu), log2_bs, ref_groups);
+                        if (tk < my_tk)
+                        {
+                            my_tk = tk;
+                            my_q = q;
+                        }
+                    }
+                }
+                if (my_tk != 0xFFFFFFFFu)
+                    atomicMin(&words[par].min_tie, my_tk);
+                lds_barrier();
+                if (my_tk == words[par].min_tie) // tie keys are distinct: exactly one lane
+                {
+                    const int k = static_cast<int>(sort_keys[my_q] & 0x3FFFu);
+                    record[par] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2],
+                                              __int_as_float(my_q));
+                    out[j] = k;
+                }
+                lds_barrier();
+                rec = record[par];
+            }
+        }
+        vx = rec.x;
+        vy = rec.y;
+        vz = rec.z;
+        bound = gv_lanes;
     }
 }
 
@@ -350,7 +766,8 @@ __global__ __launch_bounds__(FPS_THREADS) void fps_streaming_kernel(
         __syncthreads();
 
         int k;
-        reduce_records<FPS_WAVES>(records[j & 1], lane, p0x, p0y, p0z, k, sx, sy, sz);
+        int gv_unused;
+        reduce_records<FPS_WAVES>(records[j & 1], lane, p0x, p0y, p0z, k, sx, sy, sz, gv_unused);
         if (tid == 0)
             out[j] = k;
     }
@@ -388,6 +805,25 @@ void launch_resident(int b, int n, int npoint, int log2_bs, int groups, const fl
 }
 
 } // namespace
+
+template <int PPT, int THREADS, int GS>
+int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float* xyz,
+                  int32_t* out, hipStream_t s)
+{
+    int sort_n = 1;
+    while (sort_n < n)
+        sort_n <<= 1;
+    const size_t lds = (static_cast<size_t>(sort_n) + static_cast<size_t>(PPT) * THREADS) * sizeof(unsigned);
+    auto kernel = fps_pruned_kernel<PPT, THREADS, GS>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       static_cast<int>(lds));
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    hipLaunchKernelGGL(kernel, dim3(b), dim3(THREADS), lds, s, n, npoint, log2_bs, groups, sort_n,
+                       xyz, out);
+    return tpk_launch_status();
+}
 
 extern "C" size_t tpk_fps_workspace_bytes(int b, int n)
 {
@@ -431,9 +867,8 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
     else if (n <= FPS_THREADS * 8)
         launch_resident<8, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_THREADS * 16)
-        // 8 wavefronts x 32 points per lane: the per-round selection work is paid by half as
-        // many wavefronts as with 16 x 16 (measured 6.20 ms against 6.35 ms per batch of 16 clouds)
-        launch_resident<32, 512>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        // 8 wavefronts x 32 points per lane, Z-order groups with exact pruning
+        return launch_pruned<32, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else
     {
         const size_t need = tpk_fps_workspace_bytes(b, n);
