@@ -272,6 +272,31 @@ def test_fps_ties_origin_skip_and_exhaustion(tpk, oracle, dev):
     assert (tpk.furthest_point_sample(tiny.to(dev), 10) == 0).all()
 
 
+def test_fps_ties_large_cloud(tpk, oracle, dev):
+    # the same tie cases at cloud sizes served by the kernel that sorts the cloud along a space
+    # filling curve (slots no longer in index order: the tie key has to be applied explicitly)
+    ax = torch.arange(24, dtype=torch.float32)
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3) + 1.0
+    g = torch.Generator().manual_seed(5)
+    shuffled = lattice[:, torch.randperm(lattice.shape[1], generator=g)]
+    for pts in (lattice, shuffled):
+        out = tpk.furthest_point_sample(pts.contiguous().to(dev), 400)
+        np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(pts.numpy(), 400))
+    # every point three times, some points never eligible, 2 clouds
+    base = torch.rand(2, 3000, 3, generator=g) * 4.0 - 2.0
+    base[:, :37] *= 0.004
+    xyz = torch.cat([base, base.flip(1), base], 1)[:, torch.randperm(9000, generator=g)].contiguous()
+    out = tpk.furthest_point_sample(xyz.to(dev), 3100)  # more samples than distinct points
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), 3100))
+    # nothing eligible
+    tiny = torch.full((2, 9000, 3), 0.001)
+    assert (tpk.furthest_point_sample(tiny.to(dev), 10) == 0).all()
+    # a single eligible point
+    tiny[1, 8123] = 1.0
+    out = _np(tpk.furthest_point_sample(tiny.to(dev), 5))
+    np.testing.assert_array_equal(out, oracle.furthest_point_sample(tiny.numpy(), 5))
+
+
 def test_fps_full_config2(tpk, oracle, dev):
     w = W.cfg2_fps()
     xyz = w["xyz"].to(dev)
