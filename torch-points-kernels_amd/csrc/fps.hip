@@ -411,6 +411,13 @@ __device__ __forceinline__ void lds_atomic_add_u32(int* p, int v)
     asm volatile("ds_add_u32 %0, %1" ::"v"(lds_offset(p)), "v"(v) : "memory");
 }
 
+// Position on the sorted curve of member `e` of group `g` held by lane `lane` of wavefront `wave`.
+template <int WAVES, int GS>
+__device__ __forceinline__ int sorted_position(int g, int wave, int e, int lane)
+{
+    return ((g * WAVES + wave) * GS + e) * TPK_WAVE + lane;
+}
+
 template <int PPT, int THREADS, int GS>
 __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     int n, int npoint, int log2_bs, int ref_groups, int sort_n, const float* __restrict__ xyz,
@@ -427,19 +434,20 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     __shared__ RoundWords words[2];
     __shared__ float4 record[2];      // x, y, z of the round's winner and its sorted position
     __shared__ int cloud_box[6];      // ordered ints: min x,y,z then max x,y,z
-    __shared__ int group_box[16 * 6]; // the same per group
+    __shared__ int group_box[WAVES * NG * 6]; // the same per (wavefront, group) cell
 
     xyz += static_cast<int64_t>(blockIdx.x) * n * 3;
     out += static_cast<int64_t>(blockIdx.x) * npoint;
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
 
     // ---- set-up 1: box of the cloud (only to quantise coordinates for the curve)
     const int empty_lo = float_to_ordered_int(__builtin_inff());
     const int empty_hi = float_to_ordered_int(-__builtin_inff());
     if (tid < 6)
         cloud_box[tid] = tid < 3 ? empty_lo : empty_hi;
-    for (int i = tid; i < NG * 6; i += THREADS)
+    for (int i = tid; i < WAVES * NG * 6; i += THREADS)
         group_box[i] = (i % 6) < 3 ? empty_lo : empty_hi;
     if (tid < 2)
         words[tid] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
@@ -512,8 +520,10 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             __syncthreads();
         }
 
-    // ---- set-up 3: this lane's points.  Slot i = group (i / GS), member (i % GS); group g
-    // holds the curve positions [g * THREADS * GS, (g + 1) * THREADS * GS).
+    // ---- set-up 3: this lane's points.  The curve is cut into cells of 64 * GS consecutive
+    // points; cell c belongs to wavefront c % WAVES as its group c / WAVES (neighbouring cells
+    // go to different wavefronts, which spreads the work around a sample).  Slot i of a lane =
+    // group (i / GS), member (i % GS); see sorted_position().
     float x[PPT], y[PPT], z[PPT];
     int t[PPT];
 #pragma unroll
@@ -525,7 +535,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         for (int e = 0; e < GS; ++e)
         {
             const int i = gi * GS + e;
-            const int q = gi * (THREADS * GS) + e * THREADS + tid;
+            const int q = sorted_position<WAVES, GS>(gi, wave, e, lane);
             const int k = static_cast<int>(sort_keys[q < n ? q : 0] & 0x3FFFu);
             const float px = xyz[k * 3 + 0], py = xyz[k * 3 + 1], pz = xyz[k * 3 + 2];
             const bool ok = q < n && eligible(px, py, pz);
@@ -543,19 +553,19 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
 #pragma unroll
         for (int a = 0; a < 3; ++a)
         {
-            atomicMin(&group_box[gi * 6 + a], float_to_ordered_int(lo[a]));
-            atomicMax(&group_box[gi * 6 + 3 + a], float_to_ordered_int(hi[a]));
+            atomicMin(&group_box[(wave * NG + gi) * 6 + a], float_to_ordered_int(lo[a]));
+            atomicMax(&group_box[(wave * NG + gi) * 6 + 3 + a], float_to_ordered_int(hi[a]));
         }
     }
     __syncthreads();
-    // lane g of every 16-lane row tests group g; lanes beyond NG hold an empty box
+    // lane g of every 16-lane row tests this wavefront's group g; lanes beyond NG hold an empty box
     const int my_group = lane & 15;
     float blo[3], bhi[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a)
     {
-        blo[a] = my_group < NG ? ordered_int_to_float(group_box[my_group * 6 + a]) : __builtin_inff();
-        bhi[a] = my_group < NG ? ordered_int_to_float(group_box[my_group * 6 + 3 + a]) : -__builtin_inff();
+        blo[a] = my_group < NG ? ordered_int_to_float(group_box[(wave * NG + my_group) * 6 + a]) : __builtin_inff();
+        bhi[a] = my_group < NG ? ordered_int_to_float(group_box[(wave * NG + my_group) * 6 + 3 + a]) : -__builtin_inff();
     }
 
     int g[NG]; // per-lane maximum of each group, kept across rounds
@@ -595,7 +605,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
 #pragma unroll
         for (int gi = 0; gi < NG; ++gi)
         {
-            if ((live >> gi) & 1u) // wave-uniform
+            if ((live >> gi) & 1u) // uniform over the wavefront
             {
 #pragma unroll
                 for (int e = 0; e < GS; ++e)
@@ -642,7 +652,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                                 __builtin_amdgcn_readlane(hits, wl) == 1;
             if (lane == wl)
             {
-                const int pos = grp * (THREADS * GS) + ce * THREADS + tid;
+                const int pos = sorted_position<WAVES, GS>(grp, wave, ce, lane);
                 record[par] = make_float4(cx, cy, cz, __int_as_float(pos));
                 lds_atomic_add_u32(&words[par].winners, single ? 1 : 2);
                 words[par ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0}; // for the next round
@@ -676,7 +686,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
 #pragma clang loop unroll(disable)
                 for (int i = 0; i < PPT; ++i)
                 {
-                    const int q = (i / GS) * (THREADS * GS) + (i % GS) * THREADS + tid;
+                    const int q = sorted_position<WAVES, GS>(i / GS, wave, i % GS, lane);
                     if (t_copy[i * THREADS + tid] == gv && q < n)
                     {
                         const unsigned tk =
