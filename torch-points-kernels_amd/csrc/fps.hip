@@ -582,6 +582,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     float vx = p0x, vy = p0y, vz = p0z;         // the last sample (the same in every lane)
     int bound = ordered_bits(__builtin_inff()); // no running minimum exceeds this
     const bool row_head = (lane & 15) == 0;
+    int pending = -1; // sorted position of the previous round's sample while its index is unstored
     if (tid == 0)
         out[0] = 0;
 
@@ -632,7 +633,19 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
 
         // 4. only a wavefront holding the maximum looks for the slot and publishes the point
         const unsigned long long top = __ballot(best == gv);
-        if (top != 0)
+        if (top == 0)
+        {
+            // Nothing to publish: the wait for the winner is used to prepare the words of the
+            // next round and to store the previous round's index.  Two wavefronts are in charge
+            // of the store; with a single winner at least one of them comes through here.
+            if (lane == 0)
+            {
+                words[par ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
+                if (pending >= 0 && (wave == (j & (WAVES - 1)) || wave == ((j + 1) & (WAVES - 1))))
+                    out[j - 1] = static_cast<int>(sort_keys[pending] & 0x3FFFu);
+            }
+        }
+        else
         {
             int my_grp = 0, my_hits = 0;
 #pragma unroll
@@ -647,32 +660,41 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             int hits = 0, ce = 0;
             float cx = 0.f, cy = 0.f, cz = 0.f;
             GroupSelect<PPT, GS, 0, NG>::run(x, y, z, t, grp, gv, hits, cx, cy, cz, ce);
+            // one group and one member of it hold the maximum in lane wl, and no other lane does
             const bool single = __builtin_popcountll(top) == 1 &&
-                                __builtin_amdgcn_readlane(my_hits, wl) == 1 &&
-                                __builtin_amdgcn_readlane(hits, wl) == 1;
+                                __builtin_amdgcn_readlane(my_hits + hits, wl) == 2;
             if (lane == wl)
             {
                 const int pos = sorted_position<WAVES, GS>(grp, wave, ce, lane);
                 record[par] = make_float4(cx, cy, cz, __int_as_float(pos));
                 lds_atomic_add_u32(&words[par].winners, single ? 1 : 2);
-                words[par ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0}; // for the next round
-                if (single)
-                    out[j] = static_cast<int>(sort_keys[pos] & 0x3FFFu);
             }
         }
         lds_barrier();
         float4 rec = record[par];
         const int winners = __builtin_amdgcn_readfirstlane(words[par].winners);
 
+        // The index of a single winner is stored during the next round (see above).
+        const int previous = pending;
+        pending = __builtin_amdgcn_readfirstlane(__float_as_int(rec.w));
         if (winners != 1)
         {
-            // Rare: several points hold the maximum (or none is eligible).
+            // Rare: several points hold the maximum (or none is eligible).  Every wavefront
+            // may have been busy publishing, so what the waiting ones do is done here.
+            pending = -1; // this round's index is stored below
+            if (tid == 0)
+            {
+                words[par ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
+                if (previous >= 0)
+                    out[j - 1] = static_cast<int>(sort_keys[previous] & 0x3FFFu);
+            }
             if (gv < 0)
             {
                 // No eligible point in the whole cloud: the reference's reduction yields index 0.
                 rec = make_float4(p0x, p0y, p0z, 0.f);
                 if (tid == 0)
                     out[j] = 0;
+                lds_barrier();
             }
             else
             {
@@ -717,6 +739,8 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         vz = rec.z;
         bound = gv_lanes;
     }
+    if (tid == 0 && pending >= 0)
+        out[npoint - 1] = static_cast<int>(sort_keys[pending] & 0x3FFFu);
 }
 
 // Clouds too large for registers: points and running minima stream from global memory.
