@@ -72,6 +72,11 @@ __device__ __forceinline__ int wave_max_i32(int v)
     return max(max(a, b), max(c, d));
 }
 
+__device__ __forceinline__ int wave_min_i32(int v)
+{
+    return ~wave_max_i32(~v);
+}
+
 __device__ __forceinline__ unsigned wave_min_u32(unsigned v)
 {
     v = row_all_min_u32(v);
@@ -340,40 +345,14 @@ __device__ __forceinline__ unsigned tie_key(int k, int log2_bs, int ref_groups)
     return rev * static_cast<unsigned>(ref_groups) + (static_cast<unsigned>(k) >> log2_bs);
 }
 
-// Every lane selects, among the GS members of its group `grp` (wave-uniform, reached through
-// a binary tree of scalar branches), the one whose running minimum equals `value`; `hits`
-// counts the members that equal it.
-template <int PPT, int GS, int LO, int HI>
-struct GroupSelect
+// Register arrays of the sorted kernel are vector types: the winner's slot is a wave-uniform
+// number known only at run time, and indexing a vector register tuple with a uniform index
+// is one move in GPR-index mode (an array would be indexed through scratch memory).
+template <int N>
+struct RegisterVector
 {
-    __device__ __forceinline__ static void run(const float (&x)[PPT], const float (&y)[PPT],
-                                               const float (&z)[PPT], const int (&t)[PPT], int grp,
-                                               int value, int& hits, float& cx, float& cy,
-                                               float& cz, int& ce)
-    {
-        if constexpr (HI - LO == 1)
-        {
-#pragma unroll
-            for (int e = GS - 1; e >= 0; --e)
-            {
-                const int i = LO * GS + e;
-                const bool match = t[i] == value;
-                hits += match ? 1 : 0;
-                cx = match ? x[i] : cx;
-                cy = match ? y[i] : cy;
-                cz = match ? z[i] : cz;
-                ce = match ? e : ce;
-            }
-        }
-        else
-        {
-            constexpr int MID = (LO + HI) / 2;
-            if (grp < MID)
-                GroupSelect<PPT, GS, LO, MID>::run(x, y, z, t, grp, value, hits, cx, cy, cz, ce);
-            else
-                GroupSelect<PPT, GS, MID, HI>::run(x, y, z, t, grp, value, hits, cx, cy, cz, ce);
-        }
-    }
+    typedef float floats __attribute__((ext_vector_type(N)));
+    typedef int ints __attribute__((ext_vector_type(N)));
 };
 
 // The words of LDS through which the wavefronts of a workgroup agree on a round's winner.
@@ -420,17 +399,25 @@ __device__ __forceinline__ int sorted_position(int g, int wave, int e, int lane)
 
 template <int PPT, int THREADS, int GS>
 __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
-    int n, int npoint, int log2_bs, int ref_groups, int sort_n, const float* __restrict__ xyz,
-    int32_t* __restrict__ out)
+    int n, int npoint, int log2_bs, int ref_groups, int key_capacity,
+    const float* __restrict__ xyz, int32_t* __restrict__ out)
 {
     constexpr int WAVES = THREADS / TPK_WAVE;
     constexpr int NG = PPT / GS;
     static_assert(NG <= 16, "one DPP row of lanes tests the group boxes");
     static_assert(WAVES >= 2, "a cloud without eligible points must count several winners");
-    // sort_n keys (morton << 14) | index, kept for the whole kernel, then PPT * THREADS words
-    // into which the running minima are copied when equal maxima have to be resolved
+    // key_capacity keys (morton << 14) | index in curve order, kept for the whole kernel; then
+    // PPT * THREADS words (the unsorted keys during set-up, later the copy of the running minima
+    // made when equal maxima have to be resolved); then the bins of the counting sort
+    constexpr int BINS = 4096;
+    constexpr int SETUP_BATCH = 16;
+    constexpr int BINS_PER_THREAD = BINS / THREADS;
+    static_assert(BINS % THREADS == 0, "every thread scans the same number of bins");
     extern __shared__ unsigned sort_keys[];
-    int* const t_copy = reinterpret_cast<int*>(sort_keys + sort_n);
+    int* const t_copy = reinterpret_cast<int*>(sort_keys + key_capacity);
+    unsigned* const unsorted = sort_keys + key_capacity;
+    int* const bins = t_copy + PPT * THREADS;
+    __shared__ int wave_totals[WAVES];
     __shared__ RoundWords words[2];
     __shared__ float4 record[2];      // x, y, z of the round's winner and its sorted position
     __shared__ int cloud_box[6];      // ordered ints: min x,y,z then max x,y,z
@@ -447,32 +434,54 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     const int empty_hi = float_to_ordered_int(-__builtin_inff());
     if (tid < 6)
         cloud_box[tid] = tid < 3 ? empty_lo : empty_hi;
-    for (int i = tid; i < WAVES * NG * 6; i += THREADS)
-        group_box[i] = (i % 6) < 3 ? empty_lo : empty_hi;
     if (tid < 2)
         words[tid] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
+    for (int i = tid; i < BINS; i += THREADS)
+        bins[i] = 0;
     __syncthreads();
     {
         float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
         float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};
-        for (int k = tid; k < n; k += THREADS)
+        // (loads in batches of SETUP_BATCH points: the first touch of the cloud pays the full
+        // memory latency, which must not be paid once per point)
+        for (int k0 = tid; k0 < n; k0 += THREADS * SETUP_BATCH)
+        {
+            float v[SETUP_BATCH][3];
 #pragma unroll
-            for (int a = 0; a < 3; ++a)
+            for (int u = 0; u < SETUP_BATCH; ++u)
             {
-                const float v = xyz[k * 3 + a];
-                lo[a] = fminf(lo[a], v);
-                hi[a] = fmaxf(hi[a], v);
+                const int k = min(k0 + u * THREADS, n - 1);
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                    v[u][a] = xyz[k * 3 + a];
             }
+#pragma unroll
+            for (int u = 0; u < SETUP_BATCH; ++u)
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                {
+                    lo[a] = fminf(lo[a], v[u][a]);
+                    hi[a] = fmaxf(hi[a], v[u][a]);
+                }
+        }
 #pragma unroll
         for (int a = 0; a < 3; ++a)
         {
-            atomicMin(&cloud_box[a], float_to_ordered_int(lo[a]));
-            atomicMax(&cloud_box[3 + a], float_to_ordered_int(hi[a]));
+            const int wave_lo = wave_min_i32(float_to_ordered_int(lo[a]));
+            const int wave_hi = wave_max_i32(float_to_ordered_int(hi[a]));
+            if (lane == 0)
+            {
+                atomicMin(&cloud_box[a], wave_lo);
+                atomicMax(&cloud_box[3 + a], wave_hi);
+            }
         }
     }
     __syncthreads();
 
-    // ---- set-up 2: sort keys = position on the Z-order curve, then the index
+    // ---- set-up 2: sort keys = position on the Z-order curve, then the index.  Counting sort
+    // on the leading 12 bits of the code: histogram, prefix sum, scatter through LDS atomics.
+    // Inside a bin (1/16 of the cloud's extent per axis) the order is that in which the atomics
+    // were served; it decides which lane holds which point, never which point is sampled.
     {
         float lo[3], scale[3];
 #pragma unroll
@@ -482,50 +491,82 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             const float ext = ordered_int_to_float(cloud_box[3 + a]) - lo[a];
             scale[a] = ext > 0.f ? 63.999f / ext : 0.f;
         }
-        for (int k = tid; k < sort_n; k += THREADS)
+        for (int k0 = tid; k0 < n; k0 += THREADS * SETUP_BATCH)
         {
-            unsigned key = 0xFFFFFFFFu; // padding sorts last
-            if (k < n)
+            float v[SETUP_BATCH][3];
+#pragma unroll
+            for (int u = 0; u < SETUP_BATCH; ++u)
             {
+                const int k = min(k0 + u * THREADS, n - 1);
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                    v[u][a] = xyz[k * 3 + a];
+            }
+#pragma unroll
+            for (int u = 0; u < SETUP_BATCH; ++u)
+            {
+                const int k = k0 + u * THREADS;
                 unsigned code = 0;
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
                 {
-                    float q = (xyz[k * 3 + a] - lo[a]) * scale[a];
+                    float q = (v[u][a] - lo[a]) * scale[a];
                     q = q >= 0.f ? q : 0.f; // also maps NaN to cell 0
                     const unsigned cell = q < 63.f ? static_cast<unsigned>(q) : 63u;
                     code |= spread_bits_6(cell) << a;
                 }
-                key = (code << 14) | static_cast<unsigned>(k);
+                const unsigned key = (code << 14) | static_cast<unsigned>(k);
+                if (k < n)
+                {
+                    unsorted[k] = key;
+                    atomicAdd(&bins[key >> 20], 1);
+                }
             }
-            sort_keys[k] = key;
         }
     }
     __syncthreads();
-    for (int size = 2; size <= sort_n; size <<= 1)
-        for (int stride = size >> 1; stride > 0; stride >>= 1)
+    {
+        int count[BINS_PER_THREAD];
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < BINS_PER_THREAD; ++i)
         {
-            for (int i0 = tid; i0 < (sort_n >> 1); i0 += THREADS)
-            {
-                const int i = ((i0 & ~(stride - 1)) << 1) | (i0 & (stride - 1));
-                const int p = i | stride;
-                const unsigned a = sort_keys[i], b = sort_keys[p];
-                const bool ascending = (i & size) == 0;
-                if ((a > b) == ascending)
-                {
-                    sort_keys[i] = b;
-                    sort_keys[p] = a;
-                }
-            }
-            __syncthreads();
+            count[i] = bins[tid * BINS_PER_THREAD + i];
+            sum += count[i];
         }
-
+        int scan = sum; // inclusive prefix sum over the wavefront
+#pragma unroll
+        for (int d = 1; d < TPK_WAVE; d <<= 1)
+        {
+            const int below = __shfl_up(scan, d);
+            scan += lane >= d ? below : 0;
+        }
+        if (lane == TPK_WAVE - 1)
+            wave_totals[wave] = scan;
+        __syncthreads();
+        int run = scan - sum;
+        for (int w = 0; w < wave; ++w)
+            run += wave_totals[w];
+#pragma unroll
+        for (int i = 0; i < BINS_PER_THREAD; ++i)
+        {
+            bins[tid * BINS_PER_THREAD + i] = run; // start of the bin
+            run += count[i];
+        }
+    }
+    __syncthreads();
+    for (int k = tid; k < n; k += THREADS)
+    {
+        const unsigned key = unsorted[k];
+        sort_keys[atomicAdd(&bins[key >> 20], 1)] = key;
+    }
+    __syncthreads();
     // ---- set-up 3: this lane's points.  The curve is cut into cells of 64 * GS consecutive
     // points; cell c belongs to wavefront c % WAVES as its group c / WAVES (neighbouring cells
     // go to different wavefronts, which spreads the work around a sample).  Slot i of a lane =
     // group (i / GS), member (i % GS); see sorted_position().
-    float x[PPT], y[PPT], z[PPT];
-    int t[PPT];
+    typename RegisterVector<PPT>::floats x, y, z;
+    typename RegisterVector<PPT>::ints t;
 #pragma unroll
     for (int gi = 0; gi < NG; ++gi)
     {
@@ -550,11 +591,17 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             hi[1] = ok ? fmaxf(hi[1], py) : hi[1];
             hi[2] = ok ? fmaxf(hi[2], pz) : hi[2];
         }
+        // the cell belongs to this wavefront alone: reduce over its lanes, plain store
 #pragma unroll
         for (int a = 0; a < 3; ++a)
         {
-            atomicMin(&group_box[(wave * NG + gi) * 6 + a], float_to_ordered_int(lo[a]));
-            atomicMax(&group_box[(wave * NG + gi) * 6 + 3 + a], float_to_ordered_int(hi[a]));
+            const int cell_lo = wave_min_i32(float_to_ordered_int(lo[a]));
+            const int cell_hi = wave_max_i32(float_to_ordered_int(hi[a]));
+            if (lane == 0)
+            {
+                group_box[(wave * NG + gi) * 6 + a] = cell_lo;
+                group_box[(wave * NG + gi) * 6 + 3 + a] = cell_hi;
+            }
         }
     }
     __syncthreads();
@@ -582,6 +629,11 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     float vx = p0x, vy = p0y, vz = p0z;         // the last sample (the same in every lane)
     int bound = ordered_bits(__builtin_inff()); // no running minimum exceeds this
     const bool row_head = (lane & 15) == 0;
+    int best = g[0]; // this lane's largest running minimum and that of its row of 16 lanes
+#pragma unroll
+    for (int gi = 1; gi < NG; ++gi)
+        best = max(best, g[gi]);
+    int row_val = row_all_max_i32(best);
     int pending = -1; // sorted position of the previous round's sample while its index is unstored
     if (tid == 0)
         out[0] = 0;
@@ -602,29 +654,32 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             live = static_cast<unsigned>(__ballot(!skip)) & ((1u << NG) - 1u);
         }
 
-        // 2. distance update of the live groups
-#pragma unroll
-        for (int gi = 0; gi < NG; ++gi)
+        // 2. distance update of the live groups; a wavefront without any keeps its maxima
+        if (live != 0)
         {
-            if ((live >> gi) & 1u) // uniform over the wavefront
-            {
 #pragma unroll
-                for (int e = 0; e < GS; ++e)
+            for (int gi = 0; gi < NG; ++gi)
+            {
+                if ((live >> gi) & 1u) // uniform over the wavefront
                 {
-                    const int i = gi * GS + e;
-                    const float d = tpk_dist2(x[i], y[i], z[i], vx, vy, vz);
-                    t[i] = min(t[i], ordered_bits(d));
-                    g[gi] = e == 0 ? t[i] : max(g[gi], t[i]);
+#pragma unroll
+                    for (int e = 0; e < GS; ++e)
+                    {
+                        const int i = gi * GS + e;
+                        const float d = tpk_dist2(x[i], y[i], z[i], vx, vy, vz);
+                        t[i] = min(t[i], ordered_bits(d));
+                        g[gi] = e == 0 ? t[i] : max(g[gi], t[i]);
+                    }
                 }
             }
-        }
-        int best = g[0];
+            best = g[0];
 #pragma unroll
-        for (int gi = 1; gi < NG; ++gi)
-            best = max(best, g[gi]);
+            for (int gi = 1; gi < NG; ++gi)
+                best = max(best, g[gi]);
+            row_val = row_all_max_i32(best); // DPP reduction over each 16-lane row
+        }
 
-        // 3. workgroup maximum: DPP reduction over each 16-lane row, then one LDS atomic per row
-        const int row_val = row_all_max_i32(best);
+        // 3. workgroup maximum: one LDS atomic per row
         if (row_head)
             lds_atomic_max_i32(&words[par].max_val, row_val);
         lds_barrier();
@@ -657,12 +712,21 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             }
             const int wl = __builtin_ctzll(top);
             const int grp = __builtin_amdgcn_readlane(my_grp, wl);
-            int hits = 0, ce = 0;
-            float cx = 0.f, cy = 0.f, cz = 0.f;
-            GroupSelect<PPT, GS, 0, NG>::run(x, y, z, t, grp, gv, hits, cx, cy, cz, ce);
+            // members of that group (uniform index into the registers), first match per lane
+            int hits = 0, my_e = 0;
+#pragma unroll
+            for (int e = GS - 1; e >= 0; --e)
+            {
+                const bool m = t[grp * GS + e] == gv;
+                my_e = m ? e : my_e;
+                hits += m ? 1 : 0;
+            }
+            const int ce = __builtin_amdgcn_readlane(my_e, wl);
             // one group and one member of it hold the maximum in lane wl, and no other lane does
             const bool single = __builtin_popcountll(top) == 1 &&
                                 __builtin_amdgcn_readlane(my_hits + hits, wl) == 2;
+            const int slot = grp * GS + ce;
+            const float cx = x[slot], cy = y[slot], cz = z[slot];
             if (lane == wl)
             {
                 const int pos = sorted_position<WAVES, GS>(grp, wave, ce, lane);
@@ -844,17 +908,15 @@ template <int PPT, int THREADS, int GS>
 int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float* xyz,
                   int32_t* out, hipStream_t s)
 {
-    int sort_n = 1;
-    while (sort_n < n)
-        sort_n <<= 1;
-    const size_t lds = (static_cast<size_t>(sort_n) + static_cast<size_t>(PPT) * THREADS) * sizeof(unsigned);
+    const int key_capacity = (n + 63) & ~63;
+    const size_t lds = (static_cast<size_t>(key_capacity) + static_cast<size_t>(PPT) * THREADS + 4096) * sizeof(unsigned);
     auto kernel = fps_pruned_kernel<PPT, THREADS, GS>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        static_cast<int>(lds));
     if (e != hipSuccess)
         return static_cast<int>(e);
-    hipLaunchKernelGGL(kernel, dim3(b), dim3(THREADS), lds, s, n, npoint, log2_bs, groups, sort_n,
+    hipLaunchKernelGGL(kernel, dim3(b), dim3(THREADS), lds, s, n, npoint, log2_bs, groups, key_capacity,
                        xyz, out);
     return tpk_launch_status();
 }
