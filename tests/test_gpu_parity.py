@@ -235,7 +235,8 @@ def test_ball_query_full_config4(tpk, oracle, dev):
 
 @pytest.mark.parametrize(
     "B,N,npoint",
-    [(2, 3, 3), (3, 100, 40), (2, 1024, 256), (2, 1500, 300), (2, 4096, 512), (1, 7000, 128), (2, 16384, 200)],
+    [(2, 3, 3), (3, 100, 40), (2, 512, 100), (2, 513, 513), (2, 1024, 256), (2, 1500, 300), (2, 4096, 512),
+     (1, 4097, 90), (1, 7000, 128), (3, 8193, 70), (2, 16384, 200)],
 )
 def test_fps_parity(tpk, oracle, dev, B, N, npoint):
     g = torch.Generator().manual_seed(N)
@@ -267,6 +268,12 @@ def test_fps_ties_origin_skip_and_exhaustion(tpk, oracle, dev):
     lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3) + 1.0
     out = tpk.furthest_point_sample(lattice.to(dev), 300)
     np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(lattice.numpy(), 300))
+    # lattices of 729 and 2197 points: the cloud sizes of the other register layouts
+    for side in (9, 13):
+        ax = torch.arange(side, dtype=torch.float32)
+        lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3) + 1.0
+        out = tpk.furthest_point_sample(lattice.to(dev), 200)
+        np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(lattice.numpy(), 200))
     # nothing eligible
     tiny = torch.full((2, 50, 3), 0.001)
     assert (tpk.furthest_point_sample(tiny.to(dev), 10) == 0).all()

@@ -1,22 +1,20 @@
 // Furthest point sampling: npoint-1 dependent rounds of "update every point's distance to
 // the chosen set, pick the point whose distance is largest".
 //
-// One 1024-lane workgroup (16 wavefronts, one compute unit) owns a cloud for the whole
-// call.  Up to 16 points per lane (16384 per cloud) stay in registers for all rounds -
-// coordinates and running minimum distance - so a round touches no memory except one
-// 24-byte LDS record per wavefront:
-//   1. every lane updates its points against the last chosen point and keeps its first
-//      largest value (strict >, points in ascending index order);
-//   2. the wavefront finds its largest value with DPP row reductions + four lane reads,
-//      picks the owning lane (ballot; the tie key below only when two lanes tie), and
-//      lane 0 publishes (value, tie key, point index, x, y, z) of the winner to LDS;
-//   3. after the round's single barrier every wavefront reduces the 16 records the same
-//      way (16 records = one DPP row) and continues with the winner's coordinates taken
-//      from the record: the chosen point is never re-read from memory.
-// Records are double buffered so that one barrier per round suffices.
-//
-// Clouds that do not fit in registers use the same selection code over points streamed
-// from global memory with the running minima in a caller-provided workspace.
+// One workgroup (one compute unit) owns a cloud for the whole call; the rounds of a cloud
+// depend on each other, so a call runs as many workgroups as there are clouds.  Three kernels
+// by cloud size:
+//   up to 512 points     fps_resident_kernel: one point per lane in registers, every point
+//                        updated every round, one 24-byte LDS record per wavefront and one
+//                        barrier per round (records double buffered);
+//   up to 16384 points   fps_pruned_kernel: up to 32 points per lane in registers, cloud
+//                        ordered along a space filling curve so that most updates can be
+//                        skipped exactly (described at the kernel);
+//   larger clouds        fps_streaming_kernel: the selection code of the first kernel over
+//                        points streamed from global memory, running minima in a workspace
+//                        provided by the caller.
+// In all of them the chosen point's coordinates travel through LDS with the selection: the
+// chosen point is never re-read from memory.
 //
 // Semantics follow the reference kernel (cuda/src/sampling_gpu.cu:17-144): start at point
 // 0; squared distances; points whose squared norm is <= 1e-3 are neither updated nor
@@ -34,7 +32,7 @@ namespace {
 
 constexpr int FPS_THREADS = 1024;
 constexpr int FPS_WAVES = FPS_THREADS / TPK_WAVE;
-constexpr int FPS_MAX_PPT = 16; // points per lane kept in registers
+constexpr int FPS_REGISTER_POINTS = 16384; // largest cloud kept in registers
 
 struct WaveRecord
 {
@@ -303,20 +301,33 @@ __global__ __launch_bounds__(THREADS) void fps_resident_kernel(
 // ---------------------------------------------------------------------------------------
 // Register-resident kernel with exact pruning, for clouds of a few thousand to 16384 points.
 //
-// A point's running minimum changes in a round only if its distance to the new sample is
-// smaller than that minimum, and no minimum exceeds the value that won the previous round.
-// So a set of points whose bounding box is further from the new sample than the square root
-// of the previous winning value cannot change, and its update can be skipped without
-// changing any result.  To make such sets exist, the kernel first sorts the cloud along a
-// Z-order curve (18-bit Morton code, bitonic sort in LDS) and gives every lane GS points of
-// each of NG consecutive curve segments ("groups"): group g is slots g*GS.. of ALL lanes,
-// so skipping it is a wave-uniform decision shared by all wavefronts (no load imbalance).
-// The skip test of all groups is evaluated at once, lane g testing the box of group g.
-// The fp32 box distance is compared with a relative margin of 2e-6, several times the
-// rounding error of either side, so a skipped update is provably a no-op.
+// Pruning.  A point's running minimum changes in a round only if its distance to the new
+// sample is smaller than that minimum, and no minimum exceeds the value that won the previous
+// round.  So a set of points whose bounding box is further from the new sample than the square
+// root of the previous winning value cannot change, and its update can be skipped without
+// changing any result.  To make such sets exist, the kernel first orders the cloud along a
+// Z-order curve (18-bit Morton code, counting sort in LDS) and cuts the curve into cells of
+// 64 * GS consecutive points.  A cell is GS registers of the 64 lanes of one wavefront; every
+// wavefront holds NG cells, taken round-robin along the curve so that the cells around a
+// sample belong to different wavefronts.  A wavefront tests its NG boxes at once, lane g
+// testing the box of its group g, and updates only the live groups (wave-uniform branches).
+// The fp32 box distance is compared with a relative margin of 2e-6, several times the rounding
+// error of either side, so a skipped update is provably a no-op.
 //
-// Because slots are no longer in index order, the original index of every point is kept in
-// a register and equal maxima are resolved explicitly by the reference's tie key.
+// Selection.  Each lane keeps the maximum of every group and of all its points; a wavefront
+// whose groups were all skipped keeps these from the round before.  The workgroup maximum is
+// one LDS atomic max per 16-lane row (after a DPP reduction) and a barrier.  Only a wavefront
+// that holds the maximum then looks for the slot: group per lane by compare/select, the
+// winning lane's group and member through wave-uniform (GPR-indexed) register reads.  It
+// publishes the point's coordinates and sorted position in LDS and counts itself as winner;
+// after the second barrier every wavefront reads the new sample from there.  The wavefronts
+// that wait for the winner reset the words of the next round and store the previous round's
+// index, which keeps both off the critical path.
+//
+// Equal maxima.  When the winners' count is not exactly one (several points hold the maximum,
+// or no point is eligible) the round is resolved by the reference's tie key over all points
+// holding the maximum, through a copy of the running minima in LDS (slots are not in index
+// order here, so the key is computed from the original index kept in the sort keys).
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ unsigned spread_bits_6(unsigned v) // abcdef -> a00b00c00d00e00f
 {
@@ -923,7 +934,7 @@ int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float
 
 extern "C" size_t tpk_fps_workspace_bytes(int b, int n)
 {
-    if (b <= 0 || n <= FPS_THREADS * FPS_MAX_PPT)
+    if (b <= 0 || n <= FPS_REGISTER_POINTS)
         return 0;
     return static_cast<size_t>(b) * static_cast<size_t>(n) * sizeof(float);
 }
@@ -954,16 +965,19 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
     const int log2_bs = reference_log2_block(n);
     const int groups = static_cast<int>(tpk_ceil_div(n, 1 << log2_bs));
 
-    if (n <= FPS_THREADS * 1)
+    // Tiny clouds: one point per lane, no sorting.  Up to 16384 points: registers of a
+    // 512-lane workgroup, curve order and pruning (cells of 64, 128 or 256 points).
+    if (n <= 512)
         launch_resident<1, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
-    else if (n <= FPS_THREADS * 2)
-        launch_resident<2, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
-    else if (n <= FPS_THREADS * 4)
-        launch_resident<4, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
-    else if (n <= FPS_THREADS * 8)
-        launch_resident<8, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
-    else if (n <= FPS_THREADS * 16)
-        // 8 wavefronts x 32 points per lane, Z-order groups with exact pruning
+    else if (n <= 512 * 2)
+        return launch_pruned<2, 512, 1>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+    else if (n <= 512 * 4)
+        return launch_pruned<4, 512, 1>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+    else if (n <= 512 * 8)
+        return launch_pruned<8, 512, 2>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+    else if (n <= 512 * 16)
+        return launch_pruned<16, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+    else if (n <= FPS_REGISTER_POINTS)
         return launch_pruned<32, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else
     {
