@@ -34,12 +34,12 @@ PEAK_FP32_TFLOPS = 157.3  # published fp32 figure (vector = matrix); it counts e
 # scaled by the same counter's reading for a 256 MiB device copy); see profiles/*pmc*.txt.
 # None = not measured yet.
 MEASURED_TRAFFIC_BYTES = {
-    "fps": 3561000,                    # 3.30 MB read (the clouds) + 0.26 MB written (the indices)
+    "fps": 3871000,                    # 3.61 MB read (the clouds; set-up passes mostly hit L2) + 0.26 MB written (the indices)
     "three_interpolate_fwd": 174130000,  # = algorithmic bytes: nothing is read twice from HBM
     "three_interpolate_bwd": 299500000,  # list build 79 MB + list walk 220 MB (lists re-read per row block)
     "grouping_fwd": 352500000,         # rows staged twice (two column halves per row block)
     "grouping_bwd": 373400000,
-    "chamfer_bwd": None,
+    "chamfer_bwd": 223400000,          # list build 25.4 MB + list walk 198.0 MB (random 12-byte gathers fetch whole lines)
 }
 
 
@@ -100,8 +100,11 @@ def bench_fps(dev, steps, warmup, with_cpu):
     updates = W.fps_point_updates()
     roof = _roof_flops(updates, 10, ev)
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get("fps")
-    roof["note"] += "; one workgroup per cloud: 16 of 256 compute units are occupied by design, " \
-                    "fraction of those 16 CUs' peak = %.4f" % (roof["frac"] * 256 / 16)
+    roof["note"] += "; algorithmic work = every point updated in every round (10 flop each), as the reference " \
+                    "does; the kernel skips updates it proves to be no-ops, so the achieved figure is a rate of " \
+                    "algorithmic, not executed, flops; the rounds of a cloud are sequential and one workgroup " \
+                    "owns a cloud: 16 of 256 compute units are occupied by design, fraction of those 16 CUs' " \
+                    "peak = %.4f" % (roof["frac"] * 256 / 16)
     res = {"wall_ms": wall, "kernel_ms": ev, "roofline": roof, "point_updates": updates}
     if with_cpu:
         import oracle
