@@ -266,12 +266,18 @@ __global__ __launch_bounds__(256) void chamfer_bwd_lists_kernel(
     const int* __restrict__ offs_b, const ListEntry<false>* __restrict__ ent_b,
     T* __restrict__ grad_xyz1, T* __restrict__ grad_xyz2)
 {
-    // blockIdx.y: cloud; blockIdx.x covers the n points of cloud 1 first, then the m of cloud 2
+    // A cloud pair takes blocks1 + blocks2 consecutive logical blocks: the n points of cloud 1
+    // first, then the m of cloud 2.  Logical blocks are numbered so that those of a pair run on
+    // one die: its L2 then serves the random reads into the pair's points and gradients.
     const int blocks1 = (n + 255) / 256;
-    for (int cloud = blockIdx.y; cloud < clouds; cloud += gridDim.y)
+    const int per_cloud = blocks1 + (m + 255) / 256;
+    const int64_t total = static_cast<int64_t>(per_cloud) * clouds;
+    for (int64_t lin = xcd_local_block(blockIdx.x, gridDim.x); lin < total; lin += gridDim.x)
     {
-        const bool second = static_cast<int>(blockIdx.x) >= blocks1;
-        const int k = (second ? blockIdx.x - blocks1 : blockIdx.x) * 256 + threadIdx.x;
+        const int cloud = static_cast<int>(lin / per_cloud);
+        const int bx = static_cast<int>(lin % per_cloud);
+        const bool second = bx >= blocks1;
+        const int k = (second ? bx - blocks1 : bx) * 256 + threadIdx.x;
         const int npts = second ? m : n;
         const int nother = second ? n : m;
         if (k >= npts)
@@ -409,9 +415,9 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
             st = launch_build_lists<1, false, int32_t>(b, m, n, idx1, nullptr, offs_b, ents_b, s);
         if (st == TPK_OK)
         {
-            const unsigned bx = static_cast<unsigned>(tpk_ceil_div(n, 256) + tpk_ceil_div(m, 256));
-            const unsigned by = static_cast<unsigned>(b < 65535 ? b : 65535);
-            hipLaunchKernelGGL(chamfer_bwd_lists_kernel<T>, dim3(bx, by), dim3(256), 0, s, n, m, b, xyz1,
+            const int64_t blocks = (tpk_ceil_div(n, 256) + tpk_ceil_div(m, 256)) * static_cast<int64_t>(b);
+            hipLaunchKernelGGL(chamfer_bwd_lists_kernel<T>,
+                               dim3(static_cast<unsigned>(tpk_min64(blocks, 1 << 24))), dim3(256), 0, s, n, m, b, xyz1,
                                xyz2, idx1, idx2, grad_dist1, grad_dist2, offs_a, ents_a, offs_b,
                                ents_b, grad_xyz1, grad_xyz2);
             return tpk_launch_status();

@@ -68,17 +68,6 @@ struct Column
     }
 };
 
-// Workgroups are handed to the 8 accelerator dies (XCDs) round-robin, and each die has its own
-// L2.  This turns the hardware block number into a logical one such that consecutive logical
-// blocks - which work on the same cloud and re-read the same index / list data - run on the
-// same die, so that data is served by one L2 instead of being fetched into all eight.
-__device__ __forceinline__ unsigned xcd_local_block(unsigned bid, unsigned blocks)
-{
-    constexpr unsigned XCDS = 8;
-    const unsigned even = blocks - blocks % XCDS;
-    return bid < even ? (bid % XCDS) * (even / XCDS) + bid / XCDS : bid;
-}
-
 // Cooperative copy of `count` floats from global memory into LDS by the whole workgroup.
 // Loads are issued in batches of eight per thread before any is written (one memory
 // latency per batch, not per element), 16 bytes per lane when both sides are 16-byte

@@ -85,3 +85,13 @@ __device__ __forceinline__ float to_vector_register(float uniform_value)
     return v;
 }
 
+// Workgroups are handed to the 8 accelerator dies (XCDs) round-robin, and each die has its own
+// L2.  This turns the hardware block number into a logical one such that consecutive logical
+// blocks - which work on the same cloud and re-read the same index / list data - run on the
+// same die, so that data is served by one L2 instead of being fetched into all eight.
+__device__ __forceinline__ unsigned xcd_local_block(unsigned bid, unsigned blocks)
+{
+    constexpr unsigned XCDS = 8;
+    const unsigned even = blocks - blocks % XCDS;
+    return bid < even ? (bid % XCDS) * (even / XCDS) + bid / XCDS : bid;
+}
