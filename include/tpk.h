@@ -143,12 +143,18 @@ int tpk_group_grad_f32(int b, int c, int n, int npoint, int nsample, const float
  *   int32 its index (lowest index on ties); dist2 (b, m), idx2 (b, m) the other direction.
  *   grad_xyz1 (b, n, 3), grad_xyz2 (b, m, 3): fully written, no pre-zero needed.
  * n == 0 or m == 0 yields zeros, as the reference's zero-initialised outputs do.
+ * The float32 forward pass orders both clouds along a space filling curve into `workspace`
+ * (tpk_chamfer_fwd_workspace_bytes() bytes - 0 for shapes it does not serve that way -, 256-byte
+ * aligned, contents arbitrary before and after) and searches only nearby cells; with
+ * workspace == NULL, and always in float64, it tests all pairs (same results, slower).
  * The backward pass inverts idx1 / idx2 into per-point lists held in `workspace`
  * (tpk_chamfer_bwd_workspace_bytes() bytes, 256-byte aligned, contents arbitrary before and
  * after); with workspace == NULL it scatters with hardware float atomics instead (slower).
  * ------------------------------------------------------------------------------------- */
+size_t tpk_chamfer_fwd_workspace_bytes(int b, int n, int m);
 int tpk_chamfer_fwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2, float* dist1,
-                        float* dist2, int32_t* idx1, int32_t* idx2, void* stream);
+                        float* dist2, int32_t* idx1, int32_t* idx2, void* workspace,
+                        size_t workspace_bytes, void* stream);
 int tpk_chamfer_fwd_f64(int b, int n, int m, const double* xyz1, const double* xyz2,
                         double* dist1, double* dist2, int32_t* idx1, int32_t* idx2,
                         void* stream);

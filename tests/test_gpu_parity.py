@@ -473,6 +473,53 @@ def test_chamfer_ties_take_lowest_index(tpk, oracle, dev):
     np.testing.assert_array_equal(_np(d2), w2)
 
 
+def _clustered(g, B, n):
+    centres = torch.rand(B, 6, 3, generator=g) * 4.0 - 2.0
+    which = torch.randint(0, 6, (B, n), generator=g)
+    pts = torch.gather(centres, 1, which.unsqueeze(-1).expand(B, n, 3)) + 0.1 * torch.randn(B, n, 3, generator=g)
+    pts[:, : n // 10] = torch.rand(B, n // 10, 3, generator=g) * 6.0 - 3.0
+    return pts.contiguous()
+
+
+@pytest.mark.parametrize("B,n,m", [(2, 512, 512), (3, 1000, 777), (2, 4099, 513), (1, 16384, 16384), (2, 9000, 16000)])
+def test_chamfer_cell_search_parity(tpk, oracle, dev, B, n, m):
+    # cloud sizes served by the search over curve-ordered cells (float32, 512..16384 points)
+    from torch_points_kernels._native import native
+    g = torch.Generator().manual_seed(n + m)
+    for a, b in ((torch.rand(B, n, 3, generator=g), torch.rand(B, m, 3, generator=g)),
+                 (_clustered(g, B, n), _clustered(g, B, m))):
+        d1, d2, i1, i2 = native().chamfer_dist(a.to(dev), b.to(dev))
+        w1, w2, wi1, wi2 = oracle.chamfer_fwd(a.numpy(), b.numpy())
+        np.testing.assert_array_equal(_np(i1), wi1)
+        np.testing.assert_array_equal(_np(i2), wi2)
+        np.testing.assert_array_equal(_np(d1), w1)
+        np.testing.assert_array_equal(_np(d2), w2)
+
+
+def test_chamfer_cell_search_ties(tpk, oracle, dev):
+    # equal distances everywhere: lattices against shifted lattices, every point duplicated,
+    # identical clouds, one cloud collapsed to a single location
+    from torch_points_kernels._native import native
+    g = torch.Generator().manual_seed(3)
+    ax = torch.arange(10, dtype=torch.float32)
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3)
+    shifted = lattice + torch.tensor([0.5, 0.5, 0.0])
+    base = torch.rand(1, 700, 3, generator=g)
+    doubled = torch.cat([base, base, base.flip(1)], 1)[:, torch.randperm(2100, generator=g)]
+    collapsed = torch.full((1, 600, 3), 0.25)
+    cases = [(lattice, shifted[:, torch.randperm(1000, generator=g)]),
+             (lattice[:, torch.randperm(1000, generator=g)], lattice),
+             (doubled, base[:, :640]), (doubled, doubled.flip(1)), (base, collapsed), (collapsed, collapsed)]
+    for a, b in cases:
+        a, b = a.contiguous(), b.contiguous()
+        d1, d2, i1, i2 = native().chamfer_dist(a.to(dev), b.to(dev))
+        w1, w2, wi1, wi2 = oracle.chamfer_fwd(a.numpy(), b.numpy())
+        np.testing.assert_array_equal(_np(i1), wi1)
+        np.testing.assert_array_equal(_np(i2), wi2)
+        np.testing.assert_array_equal(_np(d1), w1)
+        np.testing.assert_array_equal(_np(d2), w2)
+
+
 def test_chamfer_gradcheck_double(tpk, dev):
     # reference test/test_chamfer_dist.py:20-25
     from torch.autograd import gradcheck

@@ -26,6 +26,7 @@
 // back to hardware float atomics (own terms stored first by one kernel, scattered terms
 // added by a second).
 #include "lists.h"
+#include "nn_grid.h"
 
 namespace {
 
@@ -441,10 +442,23 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
 
 } // namespace
 
+extern "C" size_t tpk_chamfer_fwd_workspace_bytes(int b, int n, int m)
+{
+    return tpk_grid_chamfer_workspace_bytes(b, n, m);
+}
+
 extern "C" int tpk_chamfer_fwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2,
                                    float* dist1, float* dist2, int32_t* idx1, int32_t* idx2,
-                                   void* stream)
+                                   void* workspace, size_t workspace_bytes, void* stream)
 {
+    if (workspace && b > 0 && n > 0 && m > 0 && xyz1 && xyz2 && dist1 && dist2 && idx1 && idx2)
+    {
+        // Search over curve-ordered cells where it applies; otherwise all pairs.
+        const int st = tpk_grid_chamfer_fwd(b, n, m, xyz1, xyz2, dist1, dist2, idx1, idx2, workspace,
+                                            workspace_bytes, tpk_stream(stream));
+        if (st != TPK_ERR_UNSUPPORTED)
+            return st;
+    }
     return chamfer_fwd<float>(b, n, m, xyz1, xyz2, dist1, dist2, idx1, idx2, stream);
 }
 

@@ -1,0 +1,223 @@
+// Ordering of a point cloud along a Z-order (Morton) curve by one workgroup, in LDS, and the
+// wavefront reductions it uses.  Shared by the kernels that cut a cloud into spatially compact
+// cells so that whole cells can be skipped exactly (furthest point sampling, nearest-neighbour
+// searches).
+#pragma once
+
+#include "tpk_device.h"
+
+namespace {
+
+// DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_ror:4, row_ror:8.  After the
+// four steps every lane of a 16-lane row holds the row's result.
+__device__ __forceinline__ int row_all_max_i32(int v)
+{
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true));
+    return v;
+}
+
+__device__ __forceinline__ unsigned row_all_min_u32(unsigned v)
+{
+    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true)));
+    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true)));
+    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true)));
+    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true)));
+    return v;
+}
+
+__device__ __forceinline__ int wave_max_i32(int v)
+{
+    v = row_all_max_i32(v);
+    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return max(max(a, b), max(c, d));
+}
+
+__device__ __forceinline__ int wave_min_i32(int v)
+{
+    return ~wave_max_i32(~v);
+}
+
+__device__ __forceinline__ unsigned wave_min_u32(unsigned v)
+{
+    v = row_all_min_u32(v);
+    const unsigned a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const unsigned c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return min(min(a, b), min(c, d));
+}
+
+__device__ __forceinline__ unsigned spread_bits_6(unsigned v) // abcdef -> a00b00c00d00e00f
+{
+    v &= 0x3Fu;
+    v = (v | (v << 8)) & 0x300Fu;
+    v = (v | (v << 4)) & 0x30C3u;
+    v = (v | (v << 2)) & 0x9249u;
+    return v;
+}
+
+// Order-preserving map of a float to a signed integer (for integer atomic min / max).
+__device__ __forceinline__ int float_to_ordered_int(float f)
+{
+    const int b = __float_as_int(f);
+    return b >= 0 ? b : b ^ 0x7FFFFFFF;
+}
+__device__ __forceinline__ float ordered_int_to_float(int b)
+{
+    return __int_as_float(b >= 0 ? b : b ^ 0x7FFFFFFF);
+}
+
+constexpr int CURVE_BINS = 4096;        // bins of the counting sort: leading 12 bits of the 18-bit code
+constexpr int CURVE_MAX_POINTS = 16384; // the index of a point takes the low 14 bits of its sort key
+constexpr int CURVE_LOAD_BATCH = 16;    // global loads in flight per thread
+
+// Orders the n points (1 <= n <= CURVE_MAX_POINTS) of the cloud at `xyz` along the curve.  On
+// return sort_keys[0..n) holds (code << 14) | index, ascending in the leading 12 bits of the code
+// and visible to the whole workgroup.  All arrays are LDS: sort_keys and unsorted n words each,
+// bins CURVE_BINS words, cloud_box 6 words, wave_totals one word per wavefront.  Called by every
+// thread of a workgroup of THREADS lanes (contains barriers).
+template <int THREADS>
+__device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n, unsigned* sort_keys,
+                                            unsigned* unsorted, int* bins, int* cloud_box,
+                                            int* wave_totals)
+{
+    static_assert(CURVE_BINS % THREADS == 0, "every thread scans the same number of bins");
+    const int tid = threadIdx.x;
+    const int lane = tid & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
+
+    // box of the cloud (only to quantise coordinates for the curve)
+    const int empty_lo = float_to_ordered_int(__builtin_inff());
+    const int empty_hi = float_to_ordered_int(-__builtin_inff());
+    if (tid < 6)
+        cloud_box[tid] = tid < 3 ? empty_lo : empty_hi;
+    for (int i = tid; i < CURVE_BINS; i += THREADS)
+        bins[i] = 0;
+    __syncthreads();
+    {
+        float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
+        float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};
+        // (loads in batches of CURVE_LOAD_BATCH points: the first touch of the cloud pays the full
+        // memory latency, which must not be paid once per point)
+        for (int k0 = tid; k0 < n; k0 += THREADS * CURVE_LOAD_BATCH)
+        {
+            float v[CURVE_LOAD_BATCH][3];
+#pragma unroll
+            for (int u = 0; u < CURVE_LOAD_BATCH; ++u)
+            {
+                const int k = min(k0 + u * THREADS, n - 1);
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                    v[u][a] = xyz[k * 3 + a];
+            }
+#pragma unroll
+            for (int u = 0; u < CURVE_LOAD_BATCH; ++u)
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                {
+                    lo[a] = fminf(lo[a], v[u][a]);
+                    hi[a] = fmaxf(hi[a], v[u][a]);
+                }
+        }
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+        {
+            const int wave_lo = wave_min_i32(float_to_ordered_int(lo[a]));
+            const int wave_hi = wave_max_i32(float_to_ordered_int(hi[a]));
+            if (lane == 0)
+            {
+                atomicMin(&cloud_box[a], wave_lo);
+                atomicMax(&cloud_box[3 + a], wave_hi);
+            }
+        }
+    }
+    __syncthreads();
+
+    // sort keys = position on the Z-order curve, then the index.  Counting sort
+    // on the leading 12 bits of the code: histogram, prefix sum, scatter through LDS atomics.
+    // Inside a bin (1/16 of the cloud's extent per axis) the order is that in which the atomics
+    // were served; it decides which lane holds which point, never which point is sampled.
+    {
+        float lo[3], scale[3];
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+        {
+            lo[a] = ordered_int_to_float(cloud_box[a]);
+            const float ext = ordered_int_to_float(cloud_box[3 + a]) - lo[a];
+            scale[a] = ext > 0.f ? 63.999f / ext : 0.f;
+        }
+        for (int k0 = tid; k0 < n; k0 += THREADS * CURVE_LOAD_BATCH)
+        {
+            float v[CURVE_LOAD_BATCH][3];
+#pragma unroll
+            for (int u = 0; u < CURVE_LOAD_BATCH; ++u)
+            {
+                const int k = min(k0 + u * THREADS, n - 1);
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                    v[u][a] = xyz[k * 3 + a];
+            }
+#pragma unroll
+            for (int u = 0; u < CURVE_LOAD_BATCH; ++u)
+            {
+                const int k = k0 + u * THREADS;
+                unsigned code = 0;
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                {
+                    float q = (v[u][a] - lo[a]) * scale[a];
+                    q = q >= 0.f ? q : 0.f; // also maps NaN to cell 0
+                    const unsigned cell = q < 63.f ? static_cast<unsigned>(q) : 63u;
+                    code |= spread_bits_6(cell) << a;
+                }
+                const unsigned key = (code << 14) | static_cast<unsigned>(k);
+                if (k < n)
+                {
+                    unsorted[k] = key;
+                    atomicAdd(&bins[key >> 20], 1);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    {
+        int count[CURVE_BINS / THREADS];
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < CURVE_BINS / THREADS; ++i)
+        {
+            count[i] = bins[tid * CURVE_BINS / THREADS + i];
+            sum += count[i];
+        }
+        int scan = sum; // inclusive prefix sum over the wavefront
+#pragma unroll
+        for (int d = 1; d < TPK_WAVE; d <<= 1)
+        {
+            const int below = __shfl_up(scan, d);
+            scan += lane >= d ? below : 0;
+        }
+        if (lane == TPK_WAVE - 1)
+            wave_totals[wave] = scan;
+        __syncthreads();
+        int run = scan - sum;
+        for (int w = 0; w < wave; ++w)
+            run += wave_totals[w];
+#pragma unroll
+        for (int i = 0; i < CURVE_BINS / THREADS; ++i)
+        {
+            bins[tid * CURVE_BINS / THREADS + i] = run; // start of the bin
+            run += count[i];
+        }
+    }
+    __syncthreads();
+    for (int k = tid; k < n; k += THREADS)
+    {
+        const unsigned key = unsorted[k];
+        sort_keys[atomicAdd(&bins[key >> 20], 1)] = key;
+    }
+    __syncthreads();
+}
+
+} // namespace

@@ -24,7 +24,7 @@
 // k among its own equal maxima, and the halving tree then prefers the thread whose number
 // has the smaller bit-reversal.  Both rules together are "smallest tie key", with
 //   key(k) = bitrev(k mod BS) * ceil(n / BS) + floor(k / BS).
-#include "tpk_device.h"
+#include "curve_order.h"
 
 #include <cmath>
 
@@ -41,47 +41,6 @@ struct WaveRecord
     int k;       // its index in the cloud
     float x, y, z;
 };
-
-// DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_ror:4, row_ror:8.  After the
-// four steps every lane of a 16-lane row holds the row's result.
-__device__ __forceinline__ int row_all_max_i32(int v)
-{
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true));
-    return v;
-}
-
-__device__ __forceinline__ unsigned row_all_min_u32(unsigned v)
-{
-    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true)));
-    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true)));
-    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true)));
-    v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true)));
-    return v;
-}
-
-__device__ __forceinline__ int wave_max_i32(int v)
-{
-    v = row_all_max_i32(v);
-    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
-    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
-    return max(max(a, b), max(c, d));
-}
-
-__device__ __forceinline__ int wave_min_i32(int v)
-{
-    return ~wave_max_i32(~v);
-}
-
-__device__ __forceinline__ unsigned wave_min_u32(unsigned v)
-{
-    v = row_all_min_u32(v);
-    const unsigned a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
-    const unsigned c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
-    return min(min(a, b), min(c, d));
-}
 
 // Distances are >= 0 and the "nothing eligible" marker is -1.0f, so the bit patterns order
 // like signed integers.
@@ -329,26 +288,6 @@ __global__ __launch_bounds__(THREADS) void fps_resident_kernel(
 // holding the maximum, through a copy of the running minima in LDS (slots are not in index
 // order here, so the key is computed from the original index kept in the sort keys).
 // ---------------------------------------------------------------------------------------
-__device__ __forceinline__ unsigned spread_bits_6(unsigned v) // abcdef -> a00b00c00d00e00f
-{
-    v &= 0x3Fu;
-    v = (v | (v << 8)) & 0x300Fu;
-    v = (v | (v << 4)) & 0x30C3u;
-    v = (v | (v << 2)) & 0x9249u;
-    return v;
-}
-
-// Order-preserving map of a float to a signed integer (for integer atomic min / max).
-__device__ __forceinline__ int float_to_ordered_int(float f)
-{
-    const int b = __float_as_int(f);
-    return b >= 0 ? b : b ^ 0x7FFFFFFF;
-}
-__device__ __forceinline__ float ordered_int_to_float(int b)
-{
-    return __int_as_float(b >= 0 ? b : b ^ 0x7FFFFFFF);
-}
-
 __device__ __forceinline__ unsigned tie_key(int k, int log2_bs, int ref_groups)
 {
     const unsigned bs_mask = (1u << log2_bs) - 1u;
@@ -420,14 +359,10 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     // key_capacity keys (morton << 14) | index in curve order, kept for the whole kernel; then
     // PPT * THREADS words (the unsorted keys during set-up, later the copy of the running minima
     // made when equal maxima have to be resolved); then the bins of the counting sort
-    constexpr int BINS = 4096;
-    constexpr int SETUP_BATCH = 16;
-    constexpr int BINS_PER_THREAD = BINS / THREADS;
-    static_assert(BINS % THREADS == 0, "every thread scans the same number of bins");
     extern __shared__ unsigned sort_keys[];
     int* const t_copy = reinterpret_cast<int*>(sort_keys + key_capacity);
     unsigned* const unsorted = sort_keys + key_capacity;
-    int* const bins = t_copy + PPT * THREADS;
+    int* const bins = t_copy + PPT * THREADS; // CURVE_BINS words
     __shared__ int wave_totals[WAVES];
     __shared__ RoundWords words[2];
     __shared__ float4 record[2];      // x, y, z of the round's winner and its sorted position
@@ -440,138 +375,11 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     const int lane = tid & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
 
-    // ---- set-up 1: box of the cloud (only to quantise coordinates for the curve)
-    const int empty_lo = float_to_ordered_int(__builtin_inff());
-    const int empty_hi = float_to_ordered_int(-__builtin_inff());
-    if (tid < 6)
-        cloud_box[tid] = tid < 3 ? empty_lo : empty_hi;
+    // ---- set-up 1 and 2: order the cloud along the curve (curve_order.h)
     if (tid < 2)
         words[tid] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
-    for (int i = tid; i < BINS; i += THREADS)
-        bins[i] = 0;
-    __syncthreads();
-    {
-        float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
-        float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};
-        // (loads in batches of SETUP_BATCH points: the first touch of the cloud pays the full
-        // memory latency, which must not be paid once per point)
-        for (int k0 = tid; k0 < n; k0 += THREADS * SETUP_BATCH)
-        {
-            float v[SETUP_BATCH][3];
-#pragma unroll
-            for (int u = 0; u < SETUP_BATCH; ++u)
-            {
-                const int k = min(k0 + u * THREADS, n - 1);
-#pragma unroll
-                for (int a = 0; a < 3; ++a)
-                    v[u][a] = xyz[k * 3 + a];
-            }
-#pragma unroll
-            for (int u = 0; u < SETUP_BATCH; ++u)
-#pragma unroll
-                for (int a = 0; a < 3; ++a)
-                {
-                    lo[a] = fminf(lo[a], v[u][a]);
-                    hi[a] = fmaxf(hi[a], v[u][a]);
-                }
-        }
-#pragma unroll
-        for (int a = 0; a < 3; ++a)
-        {
-            const int wave_lo = wave_min_i32(float_to_ordered_int(lo[a]));
-            const int wave_hi = wave_max_i32(float_to_ordered_int(hi[a]));
-            if (lane == 0)
-            {
-                atomicMin(&cloud_box[a], wave_lo);
-                atomicMax(&cloud_box[3 + a], wave_hi);
-            }
-        }
-    }
-    __syncthreads();
+    curve_order<THREADS>(xyz, n, sort_keys, unsorted, bins, cloud_box, wave_totals);
 
-    // ---- set-up 2: sort keys = position on the Z-order curve, then the index.  Counting sort
-    // on the leading 12 bits of the code: histogram, prefix sum, scatter through LDS atomics.
-    // Inside a bin (1/16 of the cloud's extent per axis) the order is that in which the atomics
-    // were served; it decides which lane holds which point, never which point is sampled.
-    {
-        float lo[3], scale[3];
-#pragma unroll
-        for (int a = 0; a < 3; ++a)
-        {
-            lo[a] = ordered_int_to_float(cloud_box[a]);
-            const float ext = ordered_int_to_float(cloud_box[3 + a]) - lo[a];
-            scale[a] = ext > 0.f ? 63.999f / ext : 0.f;
-        }
-        for (int k0 = tid; k0 < n; k0 += THREADS * SETUP_BATCH)
-        {
-            float v[SETUP_BATCH][3];
-#pragma unroll
-            for (int u = 0; u < SETUP_BATCH; ++u)
-            {
-                const int k = min(k0 + u * THREADS, n - 1);
-#pragma unroll
-                for (int a = 0; a < 3; ++a)
-                    v[u][a] = xyz[k * 3 + a];
-            }
-#pragma unroll
-            for (int u = 0; u < SETUP_BATCH; ++u)
-            {
-                const int k = k0 + u * THREADS;
-                unsigned code = 0;
-#pragma unroll
-                for (int a = 0; a < 3; ++a)
-                {
-                    float q = (v[u][a] - lo[a]) * scale[a];
-                    q = q >= 0.f ? q : 0.f; // also maps NaN to cell 0
-                    const unsigned cell = q < 63.f ? static_cast<unsigned>(q) : 63u;
-                    code |= spread_bits_6(cell) << a;
-                }
-                const unsigned key = (code << 14) | static_cast<unsigned>(k);
-                if (k < n)
-                {
-                    unsorted[k] = key;
-                    atomicAdd(&bins[key >> 20], 1);
-                }
-            }
-        }
-    }
-    __syncthreads();
-    {
-        int count[BINS_PER_THREAD];
-        int sum = 0;
-#pragma unroll
-        for (int i = 0; i < BINS_PER_THREAD; ++i)
-        {
-            count[i] = bins[tid * BINS_PER_THREAD + i];
-            sum += count[i];
-        }
-        int scan = sum; // inclusive prefix sum over the wavefront
-#pragma unroll
-        for (int d = 1; d < TPK_WAVE; d <<= 1)
-        {
-            const int below = __shfl_up(scan, d);
-            scan += lane >= d ? below : 0;
-        }
-        if (lane == TPK_WAVE - 1)
-            wave_totals[wave] = scan;
-        __syncthreads();
-        int run = scan - sum;
-        for (int w = 0; w < wave; ++w)
-            run += wave_totals[w];
-#pragma unroll
-        for (int i = 0; i < BINS_PER_THREAD; ++i)
-        {
-            bins[tid * BINS_PER_THREAD + i] = run; // start of the bin
-            run += count[i];
-        }
-    }
-    __syncthreads();
-    for (int k = tid; k < n; k += THREADS)
-    {
-        const unsigned key = unsorted[k];
-        sort_keys[atomicAdd(&bins[key >> 20], 1)] = key;
-    }
-    __syncthreads();
     // ---- set-up 3: this lane's points.  The curve is cut into cells of 64 * GS consecutive
     // points; cell c belongs to wavefront c % WAVES as its group c / WAVES (neighbouring cells
     // go to different wavefronts, which spreads the work around a sample).  Slot i of a lane =
@@ -920,7 +728,7 @@ int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float
                   int32_t* out, hipStream_t s)
 {
     const int key_capacity = (n + 63) & ~63;
-    const size_t lds = (static_cast<size_t>(key_capacity) + static_cast<size_t>(PPT) * THREADS + 4096) * sizeof(unsigned);
+    const size_t lds = (static_cast<size_t>(key_capacity) + static_cast<size_t>(PPT) * THREADS + CURVE_BINS) * sizeof(unsigned);
     auto kernel = fps_pruned_kernel<PPT, THREADS, GS>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,

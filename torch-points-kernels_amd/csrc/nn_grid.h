@@ -1,0 +1,15 @@
+// Nearest-neighbour searches over curve-ordered cells (nn_grid.hip), as seen by the entry
+// points of the all-pairs kernels, which hand suitable problems over when a workspace is given.
+#pragma once
+
+#include "tpk_device.h"
+
+// Bytes of workspace tpk_grid_chamfer_fwd needs for b pairs of n- and m-point clouds; 0 when it
+// does not serve that shape (callers then use the all-pairs scan).
+size_t tpk_grid_chamfer_workspace_bytes(int b, int n, int m);
+
+// Chamfer forward, both directions, float32.  TPK_ERR_UNSUPPORTED when the shape is not served,
+// TPK_ERR_WORKSPACE when the workspace is missing, too small or not 256-byte aligned.
+int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xyz2, float* dist1,
+                         float* dist2, int32_t* idx1, int32_t* idx2, void* workspace,
+                         size_t workspace_bytes, hipStream_t stream);

@@ -343,10 +343,17 @@ std::vector<torch::Tensor> chamfer_dist(torch::Tensor xyz1, torch::Tensor xyz2)
     torch::Tensor idx2 = torch::empty({b, m}, iopt);
     void* s = current_stream(xyz1);
     if (xyz1.scalar_type() == at::kFloat)
+    {
+        const size_t ws_bytes = tpk_chamfer_fwd_workspace_bytes(b, n, m);
+        torch::Tensor ws;
+        if (ws_bytes)
+            ws = torch::empty({static_cast<int64_t>(ws_bytes)}, xyz1.options().dtype(torch::kUInt8));
         check_status(tpk_chamfer_fwd_f32(b, n, m, xyz1.data_ptr<float>(), xyz2.data_ptr<float>(),
                                          dist1.data_ptr<float>(), dist2.data_ptr<float>(),
-                                         idx1.data_ptr<int32_t>(), idx2.data_ptr<int32_t>(), s),
+                                         idx1.data_ptr<int32_t>(), idx2.data_ptr<int32_t>(),
+                                         ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, s),
                      "chamfer_dist");
+    }
     else
         check_status(tpk_chamfer_fwd_f64(b, n, m, xyz1.data_ptr<double>(),
                                          xyz2.data_ptr<double>(), dist1.data_ptr<double>(),
