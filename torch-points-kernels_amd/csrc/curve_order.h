@@ -1,4 +1,4 @@
-// Ordering of a point cloud along a Z-order (Morton) curve by one workgroup, in LDS, and the
+// Ordering of a point cloud along a Hilbert curve by one workgroup, in LDS, and the
 // wavefront reductions it uses.  Shared by the kernels that cut a cloud into spatially compact
 // cells so that whole cells can be skipped exactly (furthest point sampling, nearest-neighbour
 // searches).
@@ -56,6 +56,37 @@ __device__ __forceinline__ unsigned spread_bits_6(unsigned v) // abcdef -> a00b0
     v = (v | (v << 4)) & 0x30C3u;
     v = (v | (v << 2)) & 0x9249u;
     return v;
+}
+
+// Position of grid cell (x0, x1, x2), 6 bits per axis, on the 3-D Hilbert curve through the 64^3
+// grid (18 bits; Skilling's transposition: undo the excess rotations level by level, Gray-encode,
+// interleave).  Consecutive positions are always adjacent cells, so a run of consecutive points
+// is a compact blob - a Z-order run can straddle a jump across the whole cloud.
+__device__ __forceinline__ unsigned hilbert_code_6(unsigned x0, unsigned x1, unsigned x2)
+{
+    unsigned x[3] = {x0, x1, x2};
+#pragma unroll
+    for (unsigned q = 32u; q > 1u; q >>= 1)
+    {
+        const unsigned p = q - 1u;
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+        {
+            const bool high = (x[i] & q) != 0;
+            const unsigned t = (x[0] ^ x[i]) & p;
+            const unsigned first = high ? x[0] ^ p : x[0] ^ t;
+            if (i)
+                x[i] = high ? x[i] : x[i] ^ t;
+            x[0] = first;
+        }
+    }
+    x[1] ^= x[0];
+    x[2] ^= x[1];
+    unsigned t = 0;
+#pragma unroll
+    for (unsigned q = 32u; q > 1u; q >>= 1)
+        t ^= (x[2] & q) ? q - 1u : 0u;
+    return (spread_bits_6(x[0] ^ t) << 2) | (spread_bits_6(x[1] ^ t) << 1) | spread_bits_6(x[2] ^ t);
 }
 
 // Order-preserving map of a float to a signed integer (for integer atomic min / max).
@@ -135,7 +166,7 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
     }
     __syncthreads();
 
-    // sort keys = position on the Z-order curve, then the index.  Counting sort
+    // sort keys = position on the curve, then the index.  Counting sort
     // on the leading 12 bits of the code: histogram, prefix sum, scatter through LDS atomics.
     // Inside a bin (1/16 of the cloud's extent per axis) the order is that in which the atomics
     // were served; it decides which lane holds which point, never which point is sampled.
@@ -163,15 +194,15 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
             for (int u = 0; u < CURVE_LOAD_BATCH; ++u)
             {
                 const int k = k0 + u * THREADS;
-                unsigned code = 0;
+                unsigned cell[3];
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
                 {
                     float q = (v[u][a] - lo[a]) * scale[a];
                     q = q >= 0.f ? q : 0.f; // also maps NaN to cell 0
-                    const unsigned cell = q < 63.f ? static_cast<unsigned>(q) : 63u;
-                    code |= spread_bits_6(cell) << a;
+                    cell[a] = q < 63.f ? static_cast<unsigned>(q) : 63u;
                 }
+                const unsigned code = hilbert_code_6(cell[0], cell[1], cell[2]);
                 const unsigned key = (code << 14) | static_cast<unsigned>(k);
                 if (k < n)
                 {

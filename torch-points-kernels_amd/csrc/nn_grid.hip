@@ -1,7 +1,7 @@
 // Nearest-neighbour search over clouds cut into spatially compact cells.
 //
 // The all-pairs scans (chamfer.hip, three_nn.hip) test every query against every candidate.
-// Here both clouds are first ordered along a Z-order curve (curve_order.h) and cut into cells
+// Here both clouds are first ordered along a Hilbert curve (curve_order.h) and cut into cells
 // of 64 consecutive points, each with its bounding box.  A wavefront then serves the 64
 // queries of one cell: it measures the distance from its cell's box to every candidate cell's
 // box (one lane per candidate cell), scans the nearest candidate cell to get a first answer,
