@@ -90,9 +90,15 @@ int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int
  *   dist2 (b, n, 3) float32 squared distances, ascending   idx (b, n, 3) int32
  * Equal distances keep the lower index first; with m < 3 the missing entries are
  * (+inf, 0).
+ * With a `workspace` (tpk_three_nn_workspace_bytes() bytes - 0 for shapes not served that way -,
+ * 256-byte aligned, contents arbitrary before and after) both clouds are ordered along a space
+ * filling curve and only nearby cells are searched; with workspace == NULL all pairs are tested
+ * (same results, slower).
  * ------------------------------------------------------------------------------------- */
+size_t tpk_three_nn_workspace_bytes(int b, int n, int m);
 int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* known,
-                     float* dist2, int32_t* idx, void* stream);
+                     float* dist2, int32_t* idx, void* workspace, size_t workspace_bytes,
+                     void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Three-point interpolation, forward and backward.

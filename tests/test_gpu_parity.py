@@ -40,6 +40,14 @@ def _assert_scatter_sum_close(got, want, abs_sum):
     assert not bad.any(), "%d of %d elements differ, worst %g" % (bad.sum(), bad.size, np.abs(got - want).max())
 
 
+def _clustered(g, B, n):
+    centres = torch.rand(B, 6, 3, generator=g) * 4.0 - 2.0
+    which = torch.randint(0, 6, (B, n), generator=g)
+    pts = torch.gather(centres, 1, which.unsqueeze(-1).expand(B, n, 3)) + 0.1 * torch.randn(B, n, 3, generator=g)
+    pts[:, : n // 10] = torch.rand(B, n // 10, 3, generator=g) * 6.0 - 3.0
+    return pts.contiguous()
+
+
 # ------------------------------------------------------------------ known answers on the GPU
 
 
@@ -330,6 +338,39 @@ def test_three_nn_parity(tpk, oracle, dev, B, n, m):
     np.testing.assert_array_equal(_np(dist), np.sqrt(wd))
 
 
+@pytest.mark.parametrize("B,n,m", [(2, 512, 512), (3, 1000, 777), (2, 5000, 515), (1, 16384, 4096), (2, 700, 16384)])
+def test_three_nn_cell_search_parity(tpk, oracle, dev, B, n, m):
+    # cloud sizes served by the search over curve-ordered cells (512..16384 points each side)
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    g = torch.Generator().manual_seed(n * 3 + m)
+    for unknown, known in ((torch.rand(B, n, 3, generator=g), torch.rand(B, m, 3, generator=g)),
+                           (_clustered(g, B, n), _clustered(g, B, m))):
+        dist2, idx = native.three_nn(unknown.to(dev), known.to(dev))
+        wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist2), wd)
+
+
+def test_three_nn_cell_search_ties(tpk, oracle, dev):
+    # equal distances in every triple: tripled known points, lattices, a collapsed cloud
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    g = torch.Generator().manual_seed(4)
+    k = torch.rand(1, 400, 3, generator=g)
+    tripled = torch.cat([k, k.flip(1), k], 1)[:, torch.randperm(1200, generator=g)]
+    ax = torch.arange(10, dtype=torch.float32)
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3)
+    cases = [(torch.rand(1, 600, 3, generator=g), tripled),
+             (lattice + 0.5, lattice[:, torch.randperm(1000, generator=g)]),
+             (lattice, lattice),
+             (torch.rand(1, 520, 3, generator=g), torch.full((1, 600, 3), 0.5))]
+    for unknown, known in cases:
+        unknown, known = unknown.contiguous(), known.contiguous()
+        dist2, idx = native.three_nn(unknown.to(dev), known.to(dev))
+        wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist2), wd)
+
+
 def test_three_nn_ties(tpk, oracle, dev):
     # duplicated known points: equal distances must keep the lower index first
     g = torch.Generator().manual_seed(3)
@@ -473,14 +514,6 @@ def test_chamfer_ties_take_lowest_index(tpk, oracle, dev):
     np.testing.assert_array_equal(_np(d2), w2)
 
 
-def _clustered(g, B, n):
-    centres = torch.rand(B, 6, 3, generator=g) * 4.0 - 2.0
-    which = torch.randint(0, 6, (B, n), generator=g)
-    pts = torch.gather(centres, 1, which.unsqueeze(-1).expand(B, n, 3)) + 0.1 * torch.randn(B, n, 3, generator=g)
-    pts[:, : n // 10] = torch.rand(B, n // 10, 3, generator=g) * 6.0 - 3.0
-    return pts.contiguous()
-
-
 @pytest.mark.parametrize("B,n,m", [(2, 512, 512), (3, 1000, 777), (2, 4099, 513), (1, 16384, 16384), (2, 9000, 16000)])
 def test_chamfer_cell_search_parity(tpk, oracle, dev, B, n, m):
     # cloud sizes served by the search over curve-ordered cells (float32, 512..16384 points)
@@ -581,14 +614,28 @@ def test_c_abi_direct_call(oracle, dev):
     idx = torch.empty(2, 700, 3, dtype=torch.int32, device=dev)
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
+    wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
+    lib.tpk_three_nn_workspace_bytes.restype = ctypes.c_size_t
+    ws_bytes = lib.tpk_three_nn_workspace_bytes(2, 700, 900)
+    assert ws_bytes > 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    # without workspace (all pairs), then with it (search over cells): same answers
+    for ws_ptr, nbytes in ((None, 0), (ctypes.c_void_p(ws.data_ptr()), ws_bytes)):
+        dist2.fill_(-1.0)
+        idx.fill_(-1)
+        stream.wait_stream(torch.cuda.current_stream())
+        st = lib.tpk_three_nn_f32(2, 700, 900, ctypes.c_void_p(u.data_ptr()), ctypes.c_void_p(k.data_ptr()),
+                                  ctypes.c_void_p(dist2.data_ptr()), ctypes.c_void_p(idx.data_ptr()),
+                                  ws_ptr, ctypes.c_size_t(nbytes), ctypes.c_void_p(stream.cuda_stream))
+        assert st == 0
+        stream.synchronize()
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist2), wd)
+    # a workspace that is too small is refused before any launch
     st = lib.tpk_three_nn_f32(2, 700, 900, ctypes.c_void_p(u.data_ptr()), ctypes.c_void_p(k.data_ptr()),
                               ctypes.c_void_p(dist2.data_ptr()), ctypes.c_void_p(idx.data_ptr()),
-                              ctypes.c_void_p(stream.cuda_stream))
-    assert st == 0
-    stream.synchronize()
-    wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
-    np.testing.assert_array_equal(_np(idx), wi)
-    np.testing.assert_array_equal(_np(dist2), wd)
+                              ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(1024), ctypes.c_void_p(stream.cuda_stream))
+    assert st == -3
     # an undersized FPS workspace is refused before any launch
     pts = torch.rand(1, 20000, 3).to(dev)
     out = torch.empty(1, 4, dtype=torch.int32, device=dev)

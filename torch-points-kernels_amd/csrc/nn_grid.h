@@ -13,3 +13,8 @@ size_t tpk_grid_chamfer_workspace_bytes(int b, int n, int m);
 int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xyz2, float* dist1,
                          float* dist2, int32_t* idx1, int32_t* idx2, void* workspace,
                          size_t workspace_bytes, hipStream_t stream);
+
+// three_nn, float32: same conventions.
+size_t tpk_grid_three_nn_workspace_bytes(int b, int n, int m);
+int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2,
+                      int32_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);

@@ -298,6 +298,157 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// three_nn over cells: the three nearest known points of every unknown point.
+//
+// The running answer of a lane is a triple sorted by (distance, original index); a candidate
+// enters where it is smaller in that order.  This is the order a serial scan in index order with
+// strictly-smaller replacement (cuda/src/interpolate_gpu.cu:9-65) ends with, whatever order the
+// candidates are visited in.  A cell is skipped when its box is further away than the third
+// best of every lane.
+// ---------------------------------------------------------------------------------------
+struct Nearest3
+{
+    float b1, b2, b3;
+    int i1, i2, i3;
+};
+
+__device__ __forceinline__ bool pair_less(float d, int ci, float b, int i)
+{
+    return d < b || (d == b && ci < i);
+}
+
+__device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, int cell, float4* stage,
+                                           int lane, float qx, float qy, float qz, Nearest3& s)
+{
+    stage[lane] = cand[cell * NG_CELL + lane];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
+    {
+        float mn = 0.f;
+#pragma unroll
+        for (int c = 0; c < NG_CHUNK; ++c)
+        {
+            const float4 p = stage[ch * NG_CHUNK + c];
+            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            mn = c == 0 ? d : fminf(mn, d);
+        }
+        if (__ballot(mn <= s.b3) == 0)
+            continue; // no candidate of this group enters any lane's triple
+#pragma unroll
+        for (int c = 0; c < NG_CHUNK; ++c)
+        {
+            const float4 p = stage[ch * NG_CHUNK + c];
+            // Operand order of the reference: (query - scanned).
+            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            const int ci = __float_as_int(p.w);
+            const bool l3 = pair_less(d, ci, s.b3, s.i3);
+            if (__ballot(l3) == 0)
+                continue;
+            const bool l2 = pair_less(d, ci, s.b2, s.i2);
+            const bool l1 = pair_less(d, ci, s.b1, s.i1);
+            s.b3 = l2 ? s.b2 : (l3 ? d : s.b3);
+            s.i3 = l2 ? s.i2 : (l3 ? ci : s.i3);
+            s.b2 = l1 ? s.b1 : (l2 ? d : s.b2);
+            s.i2 = l1 ? s.i1 : (l2 ? ci : s.i2);
+            s.b1 = l1 ? d : s.b1;
+            s.i1 = l1 ? ci : s.i1;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One wavefront = the 64 unknown points of one cell; logical wavefront = cloud * qcells + cell.
+__global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
+    int n, int m, int clouds, const float4* __restrict__ sorted_unknown,
+    const float4* __restrict__ sorted_known, const float4* __restrict__ boxes_unknown,
+    const float4* __restrict__ boxes_known, float* __restrict__ dist2, int32_t* __restrict__ idx)
+{
+    __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
+    __shared__ float lows_all[NG_SCAN_THREADS / TPK_WAVE][NG_MAX_CELLS];
+
+    const int lane = threadIdx.x & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
+    const int qcells = (n + NG_CELL - 1) / NG_CELL, ccells = (m + NG_CELL - 1) / NG_CELL;
+    const int64_t task = static_cast<int64_t>(xcd_local_block(blockIdx.x, gridDim.x)) *
+                             (NG_SCAN_THREADS / TPK_WAVE) + wave;
+    if (task >= static_cast<int64_t>(qcells) * clouds)
+        return; // (no workgroup barrier anywhere in this kernel)
+    const int cloud = static_cast<int>(task / qcells);
+    const int qcell = static_cast<int>(task - static_cast<int64_t>(cloud) * qcells);
+    const float4* __restrict__ qpts = sorted_unknown + static_cast<int64_t>(cloud) * qcells * NG_CELL;
+    const float4* __restrict__ qbox = boxes_unknown + static_cast<int64_t>(cloud) * qcells * 2;
+    const float4* __restrict__ cpts = sorted_known + static_cast<int64_t>(cloud) * ccells * NG_CELL;
+    const float4* __restrict__ cbox = boxes_known + static_cast<int64_t>(cloud) * ccells * 2;
+    dist2 += static_cast<int64_t>(cloud) * n * 3;
+    idx += static_cast<int64_t>(cloud) * n * 3;
+    float4* const stage = stages[wave];
+    float* const lows = lows_all[wave];
+
+    const float4 query = qpts[qcell * NG_CELL + lane];
+    const float qx = query.x, qy = query.y, qz = query.z;
+    const int qindex = __float_as_int(query.w); // 0x7FFFFFFF: padding, nothing to store
+    const float4 qlo = qbox[qcell * 2 + 0], qhi = qbox[qcell * 2 + 1];
+
+    const int groups = (ccells + NG_CELL - 1) / NG_CELL;
+    unsigned seed_key = 0xFFFFFFFFu;
+    for (int g = 0; g < groups; ++g)
+    {
+        const int c = g * NG_CELL + lane;
+        const bool valid = c < ccells;
+        const int cc = valid ? c : 0;
+        const float lb = box_box_dist2(qlo, qhi, cbox[cc * 2 + 0], cbox[cc * 2 + 1]);
+        lows[c] = valid ? lb : __builtin_inff();
+        const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~3u) | static_cast<unsigned>(g);
+        seed_key = valid && key < seed_key ? key : seed_key;
+    }
+    Nearest3 s;
+    s.b1 = s.b2 = s.b3 = __builtin_inff();
+    s.i1 = s.i2 = s.i3 = 0;
+    {
+        const unsigned lowest = wave_min_u32(seed_key);
+        int seed = static_cast<int>(lowest & 3u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
+        if (seed >= ccells)
+            seed = 0;
+        scan_cell3(cpts, seed, stage, lane, qx, qy, qz, s);
+        if (lane == (seed & (NG_CELL - 1)))
+            lows[seed] = __builtin_inff();
+    }
+    for (int phase = 0; phase < 2; ++phase)
+        for (int g = 0; g < groups; ++g)
+        {
+            const float lw = lows[g * NG_CELL + lane];
+            float bound = __int_as_float(wave_max_i32(__float_as_int(s.b3)));
+            unsigned long long live =
+                __ballot(lw < __builtin_inff() && (phase == 0 ? lw == 0.f : lw * NG_MARGIN <= bound));
+            while (live != 0)
+            {
+                const int bit = __builtin_ctzll(live);
+                const int c = g * NG_CELL + bit;
+                live &= live - 1;
+                const float lb = point_box_dist2(qx, qy, qz, cbox[c * 2 + 0], cbox[c * 2 + 1]);
+                if (__ballot(lb * NG_MARGIN <= s.b3) != 0)
+                    scan_cell3(cpts, c, stage, lane, qx, qy, qz, s);
+                if (lane == bit)
+                    lows[c] = __builtin_inff(); // scanned, or useless now and ever after
+                if (phase)
+                {
+                    bound = __int_as_float(wave_max_i32(__float_as_int(s.b3)));
+                    live &= __ballot(lw * NG_MARGIN <= bound);
+                }
+            }
+        }
+    if (qindex != 0x7FFFFFFF)
+    {
+        dist2[qindex * 3 + 0] = s.b1;
+        dist2[qindex * 3 + 1] = s.b2;
+        dist2[qindex * 3 + 2] = s.b3;
+        idx[qindex * 3 + 0] = s.i1;
+        idx[qindex * 3 + 1] = s.i2;
+        idx[qindex * 3 + 2] = s.i3;
+    }
+}
+
 struct GridLayout
 {
     size_t sorted_a, sorted_b, boxes_a, boxes_b, total;
@@ -371,5 +522,33 @@ int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xy
         return TPK_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(chamfer_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, n,
                        m, b, a.sorted, c.sorted, a.boxes, c.boxes, dist1, dist2, idx1, idx2);
+    return tpk_launch_status();
+}
+
+size_t tpk_grid_three_nn_workspace_bytes(int b, int n, int m)
+{
+    return grid_supported(b, n, m) ? grid_layout(b, n, m).total : 0;
+}
+
+int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2,
+                      int32_t* idx, void* workspace, size_t workspace_bytes, hipStream_t s)
+{
+    if (!grid_supported(b, n, m) || static_cast<int64_t>(b) * 2 > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    const GridLayout l = grid_layout(b, n, m);
+    if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return TPK_ERR_WORKSPACE;
+    char* w = static_cast<char*>(workspace);
+    CloudSet a{unknown, n, reinterpret_cast<float4*>(w + l.sorted_a), reinterpret_cast<float4*>(w + l.boxes_a)};
+    CloudSet c{known, m, reinterpret_cast<float4*>(w + l.sorted_b), reinterpret_cast<float4*>(w + l.boxes_b)};
+    int st = launch_curve_cells(b, a, c, s);
+    if (st != TPK_OK)
+        return st;
+    const int64_t waves = static_cast<int64_t>((n + NG_CELL - 1) / NG_CELL) * b;
+    const int64_t blocks = tpk_ceil_div(waves, NG_SCAN_THREADS / TPK_WAVE);
+    if (blocks > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(three_nn_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, n,
+                       m, b, a.sorted, c.sorted, a.boxes, c.boxes, dist2, idx);
     return tpk_launch_status();
 }

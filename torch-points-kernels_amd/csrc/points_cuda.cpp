@@ -105,11 +105,16 @@ std::vector<at::Tensor> three_nn(at::Tensor unknowns, at::Tensor knows)
                                   at::device(unknowns.device()).dtype(at::ScalarType::Int));
     at::Tensor dist2 = torch::empty({unknowns.size(0), unknowns.size(1), 3},
                                     at::device(unknowns.device()).dtype(at::ScalarType::Float));
-    check_status(tpk_three_nn_f32(as_int(unknowns.size(0), "batch size"),
-                                  as_int(unknowns.size(1), "number of unknown points"),
-                                  as_int(knows.size(1), "number of known points"),
-                                  unknowns.data_ptr<float>(), knows.data_ptr<float>(),
+    const int b = as_int(unknowns.size(0), "batch size");
+    const int n = as_int(unknowns.size(1), "number of unknown points");
+    const int m = as_int(knows.size(1), "number of known points");
+    const size_t ws_bytes = tpk_three_nn_workspace_bytes(b, n, m);
+    at::Tensor ws;
+    if (ws_bytes)
+        ws = torch::empty({static_cast<int64_t>(ws_bytes)}, unknowns.options().dtype(torch::kUInt8));
+    check_status(tpk_three_nn_f32(b, n, m, unknowns.data_ptr<float>(), knows.data_ptr<float>(),
                                   dist2.data_ptr<float>(), idx.data_ptr<int32_t>(),
+                                  ws_bytes ? ws.data_ptr() : nullptr, ws_bytes,
                                   current_stream(unknowns)),
                  "three_nn");
     return {dist2, idx};

@@ -12,7 +12,7 @@
 // distances keep the lower index first.  The reference holds its running bests as doubles
 // initialised to 1e40; every distance is an fp32 value, so fp32 running bests initialised
 // to +inf select identically and store identical values.
-#include "tpk_device.h"
+#include "nn_grid.h"
 
 namespace {
 
@@ -130,8 +130,14 @@ int launch_three_nn(int b, int n, int m, const float* unknown, const float* know
 
 } // namespace
 
+extern "C" size_t tpk_three_nn_workspace_bytes(int b, int n, int m)
+{
+    return tpk_grid_three_nn_workspace_bytes(b, n, m);
+}
+
 extern "C" int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* known,
-                                float* dist2, int32_t* idx, void* stream)
+                                float* dist2, int32_t* idx, void* workspace, size_t workspace_bytes,
+                                void* stream)
 {
     if (b < 0 || n < 0 || m < 0)
         return TPK_ERR_INVALID_ARG;
@@ -142,6 +148,13 @@ extern "C" int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const
     if (static_cast<int64_t>(n) * 3 > 0x7fffffffLL || static_cast<int64_t>(m) * 3 > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     hipStream_t s = tpk_stream(stream);
+    if (workspace)
+    {
+        // Search over curve-ordered cells where it applies; otherwise all pairs.
+        const int st = tpk_grid_three_nn(b, n, m, unknown, known, dist2, idx, workspace, workspace_bytes, s);
+        if (st != TPK_ERR_UNSUPPORTED)
+            return st;
+    }
     // Queries per lane: as many as still leave a few workgroups per compute unit.
     const int64_t queries = static_cast<int64_t>(b) * n;
     if (queries >= 4LL * NN_THREADS * 2048)
