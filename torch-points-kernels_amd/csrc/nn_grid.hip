@@ -26,7 +26,7 @@ namespace {
 
 constexpr int NG_CELL = 64;                  // points per cell = lanes of a wavefront
 constexpr int NG_MAX_CELLS = 256;            // candidate cells per cloud (their box distances sit in LDS)
-constexpr int NG_SORT_THREADS = 512;
+constexpr int NG_SORT_THREADS = 1024;
 constexpr int NG_SCAN_THREADS = 256;         // 4 wavefronts, each searching on its own
 constexpr float NG_MARGIN = 0.999998f;
 constexpr int NG_CHUNK = 8;
