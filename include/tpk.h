@@ -77,10 +77,17 @@ int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int nsample,
  *   idx (size_y, nsample) int64 (indices into x)    dist (size_y, nsample) float32
  * First `nsample` points of the query's own cloud in index order with d2 <= radius*radius;
  * unused slots are -1 in both outputs.
+ * With a `workspace` (tpk_ball_query_partial_workspace_bytes() bytes - 0 for sizes not served
+ * that way -, 256-byte aligned, contents arbitrary before and after) both arrays are ordered
+ * along a space filling curve and a query only visits cells within its radius; queries with
+ * more than 16 neighbours in the radius are then answered by a scan in index order that stops
+ * after nsample hits.  With workspace == NULL every query scans its whole cloud (same results).
  * ------------------------------------------------------------------------------------- */
+size_t tpk_ball_query_partial_workspace_bytes(int64_t size_x, int64_t size_y, int nsample);
 int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int nsample,
                                const float* x, const float* y, const int64_t* batch_x,
-                               const int64_t* batch_y, int64_t* idx, float* dist, void* stream);
+                               const int64_t* batch_y, int64_t* idx, float* dist,
+                               void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Three nearest neighbours.

@@ -22,7 +22,7 @@ def _declared_symbols():
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
     for want in (
-        "tpk_fps_f32", "tpk_fps_workspace_bytes", "tpk_ball_query_dense_f32", "tpk_ball_query_partial_f32",
+        "tpk_fps_f32", "tpk_fps_workspace_bytes", "tpk_ball_query_dense_f32", "tpk_ball_query_partial_workspace_bytes", "tpk_ball_query_partial_f32",
         "tpk_three_nn_workspace_bytes", "tpk_three_nn_f32", "tpk_three_interpolate_f32", "tpk_three_interpolate_grad_f32", "tpk_group_f32",
         "tpk_group_grad_f32", "tpk_chamfer_fwd_workspace_bytes", "tpk_chamfer_fwd_f32", "tpk_chamfer_fwd_f64", "tpk_chamfer_bwd_f32",
         "tpk_chamfer_bwd_f64", "tpk_status_string", "tpk_version",

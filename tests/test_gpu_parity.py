@@ -238,6 +238,42 @@ def test_ball_query_full_config4(tpk, oracle, dev):
     np.testing.assert_array_equal(_np(dist[sel.to(dev)]), wd)
 
 
+@pytest.mark.parametrize(
+    "sizes,qfrac,r,ns",
+    [
+        ((20000, 30000), 0.25, 0.03, 64),          # sparse neighbourhoods, clouds across window boundaries
+        ((9000, 500, 12000), 0.5, 0.06, 8),         # more neighbours than nsample for many queries
+        ((16384, 16384), 0.1, 0.05, 1),
+        (tuple([50] * 200), 1.0, 0.3, 16),          # many tiny clouds in one window
+        ((40000,), 0.3, 0.012, 32),                 # most balls hold the query point only
+    ],
+)
+def test_ball_query_partial_cell_search_parity(tpk, oracle, dev, sizes, qfrac, r, ns):
+    # packed arrays large enough for the search over curve-ordered cells
+    x, y, bx, by = _packed_case(11 + len(sizes), sizes, qfrac, 0.0)
+    idx, dist = tpk.ball_query(r, ns, x.to(dev), y.to(dev), mode="partial_dense", batch_x=bx.to(dev), batch_y=by.to(dev))
+    wi, wd = oracle.ball_query_partial_dense(r, ns, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), wd)
+
+
+def test_ball_query_partial_cell_search_edges(tpk, oracle, dev):
+    g = torch.Generator().manual_seed(21)
+    # points exactly on the sphere count (<=); duplicated support points; a query cloud without support
+    lattice_ax = torch.arange(22, dtype=torch.float32) * 0.25
+    lattice = torch.stack(torch.meshgrid(lattice_ax, lattice_ax, lattice_ax, indexing="ij"), -1).reshape(-1, 3)
+    x = torch.cat([lattice, lattice[:3000], torch.rand(5000, 3, generator=g) * 5.0])
+    bx = torch.cat([torch.zeros(lattice.shape[0] + 3000, dtype=torch.long), torch.full((5000,), 2, dtype=torch.long)])
+    y = torch.cat([lattice[::7], torch.rand(300, 3, generator=g), torch.rand(400, 3, generator=g) * 5.0])
+    by = torch.cat([torch.zeros(lattice[::7].shape[0], dtype=torch.long), torch.ones(300, dtype=torch.long),
+                    torch.full((400,), 2, dtype=torch.long)])
+    for r, ns in ((0.25, 10), (0.25, 40), (0.5, 16), (0.3, 3)):
+        idx, dist = tpk.ball_query(r, ns, x.to(dev), y.to(dev), mode="partial_dense", batch_x=bx.to(dev), batch_y=by.to(dev))
+        wi, wd = oracle.ball_query_partial_dense(r, ns, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist), wd)
+
+
 # ------------------------------------------------------------------ FPS
 
 

@@ -19,7 +19,7 @@
 // the equal range of c in batch_x, found by binary search on the device.  A workgroup
 // owns a block of consecutive queries; where the block straddles clouds it processes one
 // run of equal cloud id at a time.  Nothing is copied to the host.
-#include "tpk_device.h"
+#include "nn_grid.h"
 
 namespace {
 
@@ -269,10 +269,16 @@ extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int n
     return tpk_launch_status();
 }
 
+extern "C" size_t tpk_ball_query_partial_workspace_bytes(int64_t size_x, int64_t size_y, int nsample)
+{
+    return tpk_grid_ball_query_workspace_bytes(size_x, size_y, nsample);
+}
+
 extern "C" int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius,
                                           int nsample, const float* x, const float* y,
                                           const int64_t* batch_x, const int64_t* batch_y,
-                                          int64_t* idx, float* dist, void* stream)
+                                          int64_t* idx, float* dist, void* workspace,
+                                          size_t workspace_bytes, void* stream)
 {
     if (size_x < 0 || size_y < 0 || nsample < 0)
         return TPK_ERR_INVALID_ARG;
@@ -284,6 +290,14 @@ extern "C" int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float 
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     const float radius2 = radius * radius;
+    if (workspace)
+    {
+        // Search over curve-ordered cells where it applies; otherwise all pairs.
+        const int st = tpk_grid_ball_query_partial(size_x, size_y, radius2, nsample, x, y, batch_x, batch_y, idx,
+                                                   dist, workspace, workspace_bytes, tpk_stream(stream));
+        if (st != TPK_ERR_UNSUPPORTED)
+            return st;
+    }
     hipLaunchKernelGGL(ball_query_partial_kernel, dim3(static_cast<unsigned>(blocks)),
                        dim3(BQ_THREADS), 0, tpk_stream(stream), size_x, size_y, radius2, nsample,
                        x, y, batch_x, batch_y, idx, dist);

@@ -109,10 +109,13 @@ constexpr int CURVE_LOAD_BATCH = 16;    // global loads in flight per thread
 // and visible to the whole workgroup.  All arrays are LDS: sort_keys and unsorted n words each,
 // bins CURVE_BINS words, cloud_box 6 words, wave_totals one word per wavefront.  Called by every
 // thread of a workgroup of THREADS lanes (contains barriers).
+// With `group` != nullptr (one sorted id per point: several clouds packed in one array) the points
+// of the first 7 distinct-id offsets (group[k] - group[0] = 0..6) come first, one id after the
+// other, each in curve order; the rest follow together.  Only the order changes, never its use.
 template <int THREADS>
 __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n, unsigned* sort_keys,
                                             unsigned* unsorted, int* bins, int* cloud_box,
-                                            int* wave_totals)
+                                            int* wave_totals, const int64_t* __restrict__ group = nullptr)
 {
     static_assert(CURVE_BINS % THREADS == 0, "every thread scans the same number of bins");
     const int tid = threadIdx.x;
@@ -202,7 +205,12 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
                     q = q >= 0.f ? q : 0.f; // also maps NaN to cell 0
                     cell[a] = q < 63.f ? static_cast<unsigned>(q) : 63u;
                 }
-                const unsigned code = hilbert_code_6(cell[0], cell[1], cell[2]);
+                unsigned code = hilbert_code_6(cell[0], cell[1], cell[2]);
+                if (group && k < n)
+                {
+                    const int64_t offset = group[k] - group[0];
+                    code = (static_cast<unsigned>(offset < 7 ? offset : 7) << 15) | (code >> 3);
+                }
                 const unsigned key = (code << 14) | static_cast<unsigned>(k);
                 if (k < n)
                 {

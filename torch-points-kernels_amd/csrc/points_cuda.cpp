@@ -253,11 +253,16 @@ std::pair<at::Tensor, at::Tensor> ball_query_partial_dense(at::Tensor x, at::Ten
         torch::empty({y.size(0), nsample}, at::device(y.device()).dtype(at::ScalarType::Long));
     at::Tensor dist =
         torch::empty({y.size(0), nsample}, at::device(y.device()).dtype(at::ScalarType::Float));
+    const size_t ws_bytes = tpk_ball_query_partial_workspace_bytes(x.size(0), y.size(0), nsample);
+    at::Tensor ws;
+    if (ws_bytes)
+        ws = torch::empty({static_cast<int64_t>(ws_bytes)}, x.options().dtype(torch::kUInt8));
     check_status(tpk_ball_query_partial_f32(x.size(0), y.size(0), radius, nsample,
                                             x.data_ptr<float>(), y.data_ptr<float>(),
                                             batch_x.data_ptr<int64_t>(),
                                             batch_y.data_ptr<int64_t>(), idx.data_ptr<int64_t>(),
-                                            dist.data_ptr<float>(), current_stream(x)),
+                                            dist.data_ptr<float>(), ws_bytes ? ws.data_ptr() : nullptr,
+                                            ws_bytes, current_stream(x)),
                  "ball_query_partial_dense");
     return std::make_pair(idx, dist);
 }
