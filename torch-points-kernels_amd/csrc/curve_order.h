@@ -58,15 +58,16 @@ __device__ __forceinline__ unsigned spread_bits_6(unsigned v) // abcdef -> a00b0
     return v;
 }
 
-// Position of grid cell (x0, x1, x2), 6 bits per axis, on the 3-D Hilbert curve through the 64^3
-// grid (18 bits; Skilling's transposition: undo the excess rotations level by level, Gray-encode,
+// Position of grid cell (x0, x1, x2), BITS (<= 6) bits per axis, on the 3-D Hilbert curve through
+// the grid (3 * BITS bits; Skilling's transposition: undo the excess rotations level by level, Gray-encode,
 // interleave).  Consecutive positions are always adjacent cells, so a run of consecutive points
 // is a compact blob - a Z-order run can straddle a jump across the whole cloud.
-__device__ __forceinline__ unsigned hilbert_code_6(unsigned x0, unsigned x1, unsigned x2)
+template <int BITS>
+__device__ __forceinline__ unsigned hilbert_code(unsigned x0, unsigned x1, unsigned x2)
 {
     unsigned x[3] = {x0, x1, x2};
 #pragma unroll
-    for (unsigned q = 32u; q > 1u; q >>= 1)
+    for (unsigned q = 1u << (BITS - 1); q > 1u; q >>= 1)
     {
         const unsigned p = q - 1u;
 #pragma unroll
@@ -84,9 +85,20 @@ __device__ __forceinline__ unsigned hilbert_code_6(unsigned x0, unsigned x1, uns
     x[2] ^= x[1];
     unsigned t = 0;
 #pragma unroll
-    for (unsigned q = 32u; q > 1u; q >>= 1)
+    for (unsigned q = 1u << (BITS - 1); q > 1u; q >>= 1)
         t ^= (x[2] & q) ? q - 1u : 0u;
     return (spread_bits_6(x[0] ^ t) << 2) | (spread_bits_6(x[1] ^ t) << 1) | spread_bits_6(x[2] ^ t);
+}
+__device__ __forceinline__ unsigned hilbert_code_6(unsigned x0, unsigned x1, unsigned x2)
+{
+    return hilbert_code<6>(x0, x1, x2);
+}
+// Bin of the counting sort (leading 12 bits of the 18-bit position) that holds the points of
+// cell (bx, by, bz) of the 16^3 grid: the position of that cell on the 4-bit curve, because the
+// leading bits of a Hilbert position are the position of the enclosing coarser cell.
+__device__ __forceinline__ unsigned curve_bin_of_cell(unsigned bx, unsigned by, unsigned bz)
+{
+    return hilbert_code<4>(bx, by, bz);
 }
 
 // Order-preserving map of a float to a signed integer (for integer atomic min / max).
@@ -98,6 +110,34 @@ __device__ __forceinline__ int float_to_ordered_int(float f)
 __device__ __forceinline__ float ordered_int_to_float(int b)
 {
     return __int_as_float(b >= 0 ? b : b ^ 0x7FFFFFFF);
+}
+
+// The 64^3 grid over a cloud's bounding box in which curve positions are computed.
+struct CurveGrid
+{
+    float lo[3], scale[3];
+};
+
+// From the box as the ordering left it in LDS (ordered ints: min x, y, z, then max x, y, z).
+__device__ __forceinline__ CurveGrid curve_grid(const int* cloud_box)
+{
+    CurveGrid g;
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+    {
+        g.lo[a] = ordered_int_to_float(cloud_box[a]);
+        const float ext = ordered_int_to_float(cloud_box[3 + a]) - g.lo[a];
+        g.scale[a] = ext > 0.f ? 63.999f / ext : 0.f;
+    }
+    return g;
+}
+
+// Grid cell (0..63) of coordinate v along one axis; monotone in v; NaN goes to cell 0.
+__device__ __forceinline__ unsigned curve_grid_cell(float v, float lo, float scale)
+{
+    float q = (v - lo) * scale;
+    q = q >= 0.f ? q : 0.f;
+    return q < 63.f ? static_cast<unsigned>(q) : 63u;
 }
 
 constexpr int CURVE_BINS = 4096;        // bins of the counting sort: leading 12 bits of the 18-bit code
@@ -174,14 +214,7 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
     // Inside a bin (1/16 of the cloud's extent per axis) the order is that in which the atomics
     // were served; it decides which lane holds which point, never which point is sampled.
     {
-        float lo[3], scale[3];
-#pragma unroll
-        for (int a = 0; a < 3; ++a)
-        {
-            lo[a] = ordered_int_to_float(cloud_box[a]);
-            const float ext = ordered_int_to_float(cloud_box[3 + a]) - lo[a];
-            scale[a] = ext > 0.f ? 63.999f / ext : 0.f;
-        }
+        const CurveGrid grid = curve_grid(cloud_box);
         for (int k0 = tid; k0 < n; k0 += THREADS * CURVE_LOAD_BATCH)
         {
             float v[CURVE_LOAD_BATCH][3];
@@ -200,11 +233,7 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
                 unsigned cell[3];
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
-                {
-                    float q = (v[u][a] - lo[a]) * scale[a];
-                    q = q >= 0.f ? q : 0.f; // also maps NaN to cell 0
-                    cell[a] = q < 63.f ? static_cast<unsigned>(q) : 63u;
-                }
+                    cell[a] = curve_grid_cell(v[u][a], grid.lo[a], grid.scale[a]);
                 unsigned code = hilbert_code_6(cell[0], cell[1], cell[2]);
                 if (group && k < n)
                 {

@@ -19,10 +19,11 @@ size_t tpk_grid_three_nn_workspace_bytes(int b, int n, int m);
 int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2,
                       int32_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
-// Ball query, packed layout (squared radius; a hit has squared distance <= radius2): same
-// conventions.  Queries with many hits are answered by a scan in index order (part of the call).
+// Ball query, packed layout (a hit has squared distance <= radius2 = radius * radius as the caller
+// rounds it): same conventions.  Queries with dense neighbourhoods are answered by a scan in
+// index order inside the same kernel.
 size_t tpk_grid_ball_query_workspace_bytes(int64_t size_x, int64_t size_y, int nsample);
-int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius2, int nsample, const float* x,
-                                const float* y, const int64_t* batch_x, const int64_t* batch_y,
-                                int64_t* idx, float* dist, void* workspace, size_t workspace_bytes,
-                                hipStream_t stream);
+int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample,
+                                const float* x, const float* y, const int64_t* batch_x,
+                                const int64_t* batch_y, int64_t* idx, float* dist, void* workspace,
+                                size_t workspace_bytes, hipStream_t stream);

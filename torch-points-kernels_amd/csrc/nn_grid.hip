@@ -20,6 +20,8 @@
 // Workspace per cloud: 16 bytes per point (x, y, z, original index) padded to whole cells, and
 // 32 bytes per cell (box).  Clouds of up to 16384 points (the curve ordering works in LDS).
 #include "curve_order.h"
+
+#include <cmath>
 #include "nn_grid.h"
 
 namespace {
@@ -44,7 +46,9 @@ struct PointSet
     int64_t total;
     int stride;
     float4* sorted;       // [windows][cells * 64]
-    float4* boxes;        // [windows][cells][2]: (lo.xyz, -), (hi.xyz, -)
+    float4* boxes;        // [windows][cells][2]: (lo.xyz, -), (hi.xyz, -); or nullptr
+    int* bin_ends;        // optional [windows][CURVE_BINS]: end of every bin of the counting sort
+    float4* grid;         // optional [windows][2]: origin and scale of the window's 64^3 grid
 };
 
 __host__ __device__ inline int set_cells(const PointSet& s)
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     const int cells = set_cells(set);
     const float* __restrict__ xyz = set.xyz + start * 3;
     float4* __restrict__ sorted = set.sorted + window * cells * NG_CELL;
-    float4* __restrict__ boxes = set.boxes + window * cells * 2;
+    float4* __restrict__ boxes = set.boxes ? set.boxes + window * cells * 2 : nullptr;
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
     if (zero_word && blockIdx.x == 0 && tid == 0)
@@ -112,6 +116,8 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
             const float inf = __builtin_inff();
             sorted[q] = real ? make_float4(v[u][0], v[u][1], v[u][2], __int_as_float(k[u]))
                              : make_float4(inf, inf, inf, __int_as_float(0x7FFFFFFF));
+            if (!boxes) // uniform
+                continue;
             float lo[3], hi[3];
 #pragma unroll
             for (int a = 0; a < 3; ++a)
@@ -124,6 +130,19 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
                 boxes[(q / NG_CELL) * 2 + 0] = make_float4(lo[0], lo[1], lo[2], 0.f);
                 boxes[(q / NG_CELL) * 2 + 1] = make_float4(hi[0], hi[1], hi[2], 0.f);
             }
+        }
+    }
+    if (set.bin_ends)
+    {
+        // bins[i] is the end of bin i on the curve; the bin of a point is the leading 12 bits of
+        // its position: the cell of the 16^3 grid it lies in (curve_bin_of_cell()).
+        for (int i = tid; i < CURVE_BINS; i += NG_SORT_THREADS)
+            set.bin_ends[window * CURVE_BINS + i] = bins[i];
+        if (tid == 0)
+        {
+            const CurveGrid grid = curve_grid(cloud_box);
+            set.grid[window * 2 + 0] = make_float4(grid.lo[0], grid.lo[1], grid.lo[2], 0.f);
+            set.grid[window * 2 + 1] = make_float4(grid.scale[0], grid.scale[1], grid.scale[2], 0.f);
         }
     }
 }
@@ -473,24 +492,23 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// Ball query over cells, packed layout (several clouds back to back, sorted cloud id per point).
+// Ball query over bins, packed layout (several clouds back to back, sorted cloud id per point).
 //
-// Both packed arrays are cut into windows of CURVE_MAX_POINTS consecutive rows, each ordered on
-// its own (curve_cells_kernel; inside a window the clouds come one after the other).  A
-// wavefront serves the 64 queries of one cell: it looks up the support rows of its queries'
-// clouds, walks the windows that hold them, and scans the cells whose box is within the radius
-// of its own cell's box and of at least one of its queries.  A candidate is a hit when its
-// squared distance is <= radius^2 and its row lies in the query's cloud.
-// The result rows must hold the hits with the LOWEST rows, in ascending order (a serial scan in
-// index order that stops after nsample hits, cuda/src/ball_query_gpu.cu:54-95).  A lane collects
-// up to BQG_KEEP hits in LDS, sorts them, and the wavefront writes the rows (hits, then -1)
-// with coalesced stores.  A query with more hits than that - or than nsample - is put on a
-// list and answered by ball_query_overflow_kernel, one wavefront per query scanning its cloud
-// in index order with early exit: dense neighbourhoods are exactly where that scan is short.
+// The support array is cut into windows of CURVE_MAX_POINTS consecutive rows, each ordered on its
+// own (curve_cells_kernel), which groups a window's points by the cell of a 16^3 grid over the
+// window's bounding box; the ordering kernel also leaves where each such bin ends.  One
+// wavefront serves one query: it finds the support rows of the query's cloud (the windows they
+// lie in), and in every window the bins that the cube around the ball touches - a handful
+// when the radius is small against the cloud - and tests their points, 64 per step, one per
+// lane.  A candidate is a hit when its squared distance is <= radius^2 and its row lies in the
+// query's cloud.  The hits (at most 64) are collected in LDS, ranked by row, and written in
+// ascending row order, then -1: the rows a serial scan in index order that stops after nsample
+// hits (cuda/src/ball_query_gpu.cu:54-95) would have produced.
+// A query whose ball touches more than 64 bins of a window, or that has more than 64 hits, is
+// answered by that serial scan itself, 64 rows per step with early exit: those are the dense
+// neighbourhoods, where the scan ends soon.
 // ---------------------------------------------------------------------------------------
-constexpr int BQG_KEEP = 16;          // hits a lane keeps in LDS
-constexpr int BQG_PITCH = NG_CELL + 1; // LDS row pitch of the hit buffers (conflict-free both ways)
-constexpr int BQG_LIST = 64;           // overflow list: word 0 = count, queries from word BQG_LIST on
+constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
 
 // First position of sorted a[0..len) whose value is >= v, found by the whole wavefront:
 // 64 samples per round instead of one.
@@ -513,211 +531,151 @@ __device__ __forceinline__ int wave_lower_bound(const int64_t* __restrict__ a, i
     return lo;
 }
 
-__global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_grid_kernel(
-    int size_x, int size_y, float radius2, int nsample, const float4* __restrict__ sorted_x,
-    const float4* __restrict__ boxes_x, const float4* __restrict__ sorted_y,
-    const float4* __restrict__ boxes_y, const int64_t* __restrict__ batch_x,
-    const int64_t* __restrict__ batch_y, int64_t* __restrict__ idx, float* __restrict__ dist,
-    int* __restrict__ overflow)
+// Range of 16^3-grid cells along one axis that [v - r, v + r] can touch.  The interval is widened
+// by a few ulps of its ends so that a point the fp32 radius test accepts is never left out.
+__device__ __forceinline__ void bin_range(float v, float r, float lo, float scale, int& first, int& last)
 {
-    constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
-    constexpr int CELLS = CURVE_MAX_POINTS / NG_CELL; // cells per window
-    __shared__ float4 stages[WAVES][NG_CELL];
-    __shared__ int hit_rows[WAVES][BQG_KEEP * BQG_PITCH];
-    __shared__ float hit_dists[WAVES][BQG_KEEP * BQG_PITCH];
-
-    const int lane = threadIdx.x & (TPK_WAVE - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
-    const int windows_y = (size_y + CURVE_MAX_POINTS - 1) / CURVE_MAX_POINTS;
-    const int64_t task = static_cast<int64_t>(xcd_local_block(blockIdx.x, gridDim.x)) * WAVES + wave;
-    if (task >= static_cast<int64_t>(windows_y) * CELLS)
-        return; // (no workgroup barrier anywhere in this kernel)
-    const int wy = static_cast<int>(task / CELLS);
-    const int qcell = static_cast<int>(task - static_cast<int64_t>(wy) * CELLS);
-    float4* const stage = stages[wave];
-    int* const my_rows = hit_rows[wave];
-    float* const my_dists = hit_dists[wave];
-
-    const float4 query = sorted_y[(static_cast<int64_t>(wy) * CELLS + qcell) * NG_CELL + lane];
-    const float qx = query.x, qy = query.y, qz = query.z;
-    const bool valid = __float_as_int(query.w) != 0x7FFFFFFF;
-    if (__ballot(valid) == 0)
-        return; // a cell past the end of its window
-    const int qrow = wy * CURVE_MAX_POINTS + (valid ? __float_as_int(query.w) : 0);
-    const float4 qlo = boxes_y[(static_cast<int64_t>(wy) * CELLS + qcell) * 2 + 0];
-    const float4 qhi = boxes_y[(static_cast<int64_t>(wy) * CELLS + qcell) * 2 + 1];
-
-    // Support rows [lo, hi) of every lane's cloud; usually all lanes share one cloud.
-    const int64_t cloud = valid ? batch_y[qrow] : -1;
-    int lo = 0, hi = 0;
-    for (unsigned long long todo = __ballot(valid); todo != 0;)
-    {
-        const int l = __builtin_ctzll(todo);
-        const int64_t c = (static_cast<int64_t>(__builtin_amdgcn_readlane(static_cast<int>(cloud >> 32), l)) << 32) |
-                          static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(cloud), l));
-        const int s0 = wave_lower_bound(batch_x, size_x, c, lane);
-        const int s1 = wave_lower_bound(batch_x, size_x, c + 1, lane);
-        const bool mine = valid && cloud == c;
-        lo = mine ? s0 : lo;
-        hi = mine ? s1 : hi;
-        todo &= ~__ballot(mine);
-    }
-    const bool has_support = valid && hi > lo;
-    const int first_row = wave_min_i32(has_support ? lo : 0x7FFFFFFF);
-    const int last_row = wave_max_i32(has_support ? hi : 0);
-
-    const int keep = nsample < BQG_KEEP ? nsample : BQG_KEEP;
-    int cnt = 0;         // hits so far; keep + 1 = too many for this kernel
-    bool active = has_support;
-    if (last_row > first_row)
-    {
-        for (int wx = first_row / CURVE_MAX_POINTS; wx <= (last_row - 1) / CURVE_MAX_POINTS; ++wx)
-        {
-            const float4* __restrict__ cpts = sorted_x + static_cast<int64_t>(wx) * CELLS * NG_CELL;
-            const float4* __restrict__ cbox = boxes_x + static_cast<int64_t>(wx) * CELLS * 2;
-            const int row_base = wx * CURVE_MAX_POINTS;
-            // box tests of the window's 256 cells first (their loads in flight together)
-            static_assert(CELLS / NG_CELL == 4, "four groups of 64 cells per window");
-            unsigned long long live_of[4];
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-            {
-                const int cc = g * NG_CELL + lane;
-                const float lw = box_box_dist2(qlo, qhi, cbox[cc * 2 + 0], cbox[cc * 2 + 1]);
-                live_of[g] = __ballot(lw * NG_MARGIN <= radius2); // empty boxes: +inf
-            }
-            for (int g = 0; g < 4; ++g)
-            {
-                unsigned long long live = g == 0 ? live_of[0] : g == 1 ? live_of[1] : g == 2 ? live_of[2] : live_of[3];
-                while (live != 0)
-                {
-                    const int c = g * NG_CELL + __builtin_ctzll(live);
-                    live &= live - 1;
-                    const float lb = point_box_dist2(qx, qy, qz, cbox[c * 2 + 0], cbox[c * 2 + 1]);
-                    if (__ballot(active && lb * NG_MARGIN <= radius2) == 0)
-                        continue;
-                    stage[lane] = cpts[c * NG_CELL + lane];
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    for (int k = 0; k < NG_CELL; ++k)
-                    {
-                        const float4 p = stage[k];
-                        const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-                        // (a padding record has index 0x7FFFFFFF: its row wraps out of every range)
-                        const int row = static_cast<int>(static_cast<unsigned>(row_base) +
-                                                         static_cast<unsigned>(__float_as_int(p.w)));
-                        const bool hit = active && d <= radius2 && row >= lo && row < hi;
-                        if (__ballot(hit) != 0 && hit)
-                        {
-                            if (cnt < keep)
-                            {
-                                my_rows[cnt * BQG_PITCH + lane] = row;
-                                my_dists[cnt * BQG_PITCH + lane] = d;
-                            }
-                            ++cnt;
-                            active = cnt <= keep;
-                        }
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                }
-            }
-            if (__ballot(active) == 0)
-                break;
-        }
-    }
-
-    // Lanes with too many hits hand their query over; the others sort their hits by row.
-    const bool handed_over = valid && cnt > keep;
-    if (handed_over)
-        overflow[BQG_LIST + atomicAdd(&overflow[0], 1)] = qrow;
-    if (valid && !handed_over)
-        for (int a = 1; a < cnt; ++a)
-        {
-            const int key = my_rows[a * BQG_PITCH + lane];
-            const float kd = my_dists[a * BQG_PITCH + lane];
-            int b = a - 1;
-            while (b >= 0 && my_rows[b * BQG_PITCH + lane] > key)
-            {
-                my_rows[(b + 1) * BQG_PITCH + lane] = my_rows[b * BQG_PITCH + lane];
-                my_dists[(b + 1) * BQG_PITCH + lane] = my_dists[b * BQG_PITCH + lane];
-                --b;
-            }
-            my_rows[(b + 1) * BQG_PITCH + lane] = key;
-            my_dists[(b + 1) * BQG_PITCH + lane] = kd;
-        }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    // Rows are written by the whole wavefront, one query after the other: hits, then -1.
-    const unsigned long long writers = __ballot(valid && !handed_over);
-    for (unsigned long long todo = writers; todo != 0; todo &= todo - 1)
-    {
-        const int q = __builtin_ctzll(todo);
-        const int64_t out = static_cast<int64_t>(__builtin_amdgcn_readlane(qrow, q)) * nsample;
-        const int c = __builtin_amdgcn_readlane(cnt, q);
-        for (int s = lane; s < nsample; s += TPK_WAVE)
-        {
-            const bool is_hit = s < c;
-            const int at = (is_hit ? s : 0) * BQG_PITCH + q;
-            idx[out + s] = is_hit ? static_cast<int64_t>(my_rows[at]) : -1;
-            dist[out + s] = is_hit ? my_dists[at] : -1.0f;
-        }
-    }
+    const float slack = (fabsf(v) + r) * 1e-6f + 1e-30f;
+    first = static_cast<int>(curve_grid_cell((v - r) - slack, lo, scale) >> 2);
+    last = static_cast<int>(curve_grid_cell((v + r) + slack, lo, scale) >> 2);
 }
 
-// The queries handed over by ball_query_grid_kernel: one wavefront per query, the lanes hold 64
-// consecutive support rows of the query's cloud; ballot + prefix count give the hits their slots
-// in index order; the scan stops after nsample hits.
-__global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_overflow_kernel(
-    int size_x, float radius2, int nsample, const float* __restrict__ x, const float* __restrict__ y,
-    const int64_t* __restrict__ batch_x, const int64_t* __restrict__ batch_y,
-    int64_t* __restrict__ idx, float* __restrict__ dist, const int* __restrict__ overflow)
+__global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
+    int size_x, int size_y, float radius, float radius2, int nsample, const float* __restrict__ x,
+    const float* __restrict__ y, const float4* __restrict__ sorted_x, const int* __restrict__ bin_ends,
+    const float4* __restrict__ grids, const int64_t* __restrict__ batch_x,
+    const int64_t* __restrict__ batch_y, int64_t* __restrict__ idx, float* __restrict__ dist)
 {
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
+    __shared__ int hit_rows[WAVES][BQB_HITS];
+    __shared__ float hit_dists[WAVES][BQB_HITS];
+
     const int lane = threadIdx.x & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
-    const int listed = overflow[0];
-    for (int t = blockIdx.x * WAVES + wave; t < listed; t += gridDim.x * WAVES)
+    const int64_t q = static_cast<int64_t>(blockIdx.x) * WAVES + wave;
+    if (q >= size_y)
+        return; // (no workgroup barrier anywhere in this kernel)
+    int* const rows = hit_rows[wave];
+    float* const dists = hit_dists[wave];
+
+    const float ux = y[q * 3 + 0], uy = y[q * 3 + 1], uz = y[q * 3 + 2];
+    const float qx = to_vector_register(ux), qy = to_vector_register(uy), qz = to_vector_register(uz);
+    const int64_t cloud = batch_y[q];
+    const int s0 = wave_lower_bound(batch_x, size_x, cloud, lane);
+    const int s1 = wave_lower_bound(batch_x, size_x, cloud + 1, lane);
+    const int64_t out = q * nsample;
+
+    int cnt = 0;
+    bool serial = false; // answer by the scan in index order instead
+    for (int wx = s0 / CURVE_MAX_POINTS; !serial && s1 > s0 && wx * CURVE_MAX_POINTS < s1; ++wx)
     {
-        const int q = overflow[BQG_LIST + t];
-        const float qx = to_vector_register(y[static_cast<int64_t>(q) * 3 + 0]);
-        const float qy = to_vector_register(y[static_cast<int64_t>(q) * 3 + 1]);
-        const float qz = to_vector_register(y[static_cast<int64_t>(q) * 3 + 2]);
-        const int64_t c = batch_y[q];
-        const int s0 = wave_lower_bound(batch_x, size_x, c, lane);
-        const int s1 = wave_lower_bound(batch_x, size_x, c + 1, lane);
-        const int64_t out = static_cast<int64_t>(q) * nsample;
-        int cnt = 0;
-        constexpr int BATCH = 4; // loads of four steps in flight
-        for (int base = s0; base < s1 && cnt < nsample; base += BATCH * TPK_WAVE)
+        const float4 origin = grids[wx * 2 + 0], scale = grids[wx * 2 + 1];
+        int fx, lx, fy, ly, fz, lz;
+        bin_range(ux, radius, origin.x, scale.x, fx, lx);
+        bin_range(uy, radius, origin.y, scale.y, fy, ly);
+        bin_range(uz, radius, origin.z, scale.z, fz, lz);
+        const int nx = lx - fx + 1, ny = ly - fy + 1, nz = lz - fz + 1;
+        const int nbins = nx * ny * nz;
+        if (nbins > TPK_WAVE)
         {
-            float px[BATCH], py[BATCH], pz[BATCH];
-#pragma unroll
-            for (int u = 0; u < BATCH; ++u)
+            serial = true;
+            break;
+        }
+        // lane l looks up bin l of the block of bins
+        int start = 0, size = 0;
+        if (lane < nbins)
+        {
+            const int bx = fx + lane % nx, by = fy + (lane / nx) % ny, bz = fz + lane / (nx * ny);
+            const unsigned bin = curve_bin_of_cell(bx, by, bz);
+            const int* __restrict__ ends = bin_ends + static_cast<int64_t>(wx) * CURVE_BINS;
+            start = bin ? ends[bin - 1] : 0;
+            size = ends[bin] - start;
+        }
+        const float4* __restrict__ cpts = sorted_x + static_cast<int64_t>(wx) * CURVE_MAX_POINTS;
+        const int row_base = wx * CURVE_MAX_POINTS;
+        for (int b = 0; b < nbins; ++b)
+        {
+            const int bstart = __builtin_amdgcn_readlane(start, b);
+            const int bsize = __builtin_amdgcn_readlane(size, b);
+            for (int t0 = 0; t0 < bsize; t0 += TPK_WAVE)
             {
-                const int64_t pos = min(base + u * TPK_WAVE + lane, s1 - 1);
-                px[u] = x[pos * 3 + 0];
-                py[u] = x[pos * 3 + 1];
-                pz[u] = x[pos * 3 + 2];
-            }
-#pragma unroll
-            for (int u = 0; u < BATCH; ++u)
-            {
-                const int pos = base + u * TPK_WAVE + lane;
-                const float d = tpk_dist2(qx, qy, qz, px[u], py[u], pz[u]);
-                const bool hit = pos < s1 && d <= radius2;
+                const bool has = t0 + lane < bsize;
+                const float4 p = cpts[bstart + (has ? t0 + lane : 0)];
+                const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+                const int row = row_base + __float_as_int(p.w);
+                const bool hit = has && d <= radius2 && row >= s0 && row < s1;
                 const unsigned long long mask = __ballot(hit);
-                const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
-                if (hit && slot < nsample)
+                if (mask == 0)
+                    continue;
+                const int at = cnt + static_cast<int>(tpk_prefix_count(mask));
+                if (hit && at < BQB_HITS)
                 {
-                    idx[out + slot] = pos;
-                    dist[out + slot] = d;
+                    rows[at] = row;
+                    dists[at] = d;
                 }
                 cnt += __builtin_popcountll(mask);
             }
+        }
+        serial = cnt > BQB_HITS;
+    }
+
+    if (!serial)
+    {
+        // rank of every hit among the hits (rows are distinct), then hits in order, then -1
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        const int my_row = rows[lane < cnt ? lane : 0];
+        const float my_dist = dists[lane < cnt ? lane : 0];
+        int rank = 0;
+        for (int j = 0; j < cnt; ++j)
+            rank += rows[j] < my_row ? 1 : 0;
+        if (lane < cnt && rank < nsample)
+        {
+            idx[out + rank] = my_row;
+            dist[out + rank] = my_dist;
         }
         for (int s = cnt + lane; s < nsample; s += TPK_WAVE)
         {
             idx[out + s] = -1;
             dist[out + s] = -1.0f;
         }
+        return;
+    }
+
+    // Serial semantics directly: lanes hold 64 consecutive support rows; ballot + prefix count
+    // give the hits their slots in index order; stop after nsample hits.
+    cnt = 0;
+    constexpr int BATCH = 4; // loads of four steps in flight
+    for (int base = s0; base < s1 && cnt < nsample; base += BATCH * TPK_WAVE)
+    {
+        float px[BATCH], py[BATCH], pz[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+        {
+            const int64_t pos = min(base + u * TPK_WAVE + lane, s1 - 1);
+            px[u] = x[pos * 3 + 0];
+            py[u] = x[pos * 3 + 1];
+            pz[u] = x[pos * 3 + 2];
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+        {
+            const int pos = base + u * TPK_WAVE + lane;
+            const float d = tpk_dist2(qx, qy, qz, px[u], py[u], pz[u]);
+            const bool hit = pos < s1 && d <= radius2;
+            const unsigned long long mask = __ballot(hit);
+            const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
+            if (hit && slot < nsample)
+            {
+                idx[out + slot] = pos;
+                dist[out + slot] = d;
+            }
+            cnt += __builtin_popcountll(mask);
+        }
+    }
+    for (int s = cnt + lane; s < nsample; s += TPK_WAVE)
+    {
+        idx[out + s] = -1;
+        dist[out + s] = -1.0f;
     }
 }
 
@@ -788,9 +746,9 @@ int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xy
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
     PointSet a{xyz1, nullptr, static_cast<int64_t>(b) * n, n, reinterpret_cast<float4*>(w + l.sorted_a),
-               reinterpret_cast<float4*>(w + l.boxes_a)};
+               reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
     PointSet c{xyz2, nullptr, static_cast<int64_t>(b) * m, m, reinterpret_cast<float4*>(w + l.sorted_b),
-               reinterpret_cast<float4*>(w + l.boxes_b)};
+               reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
     int st = launch_curve_cells(a, c, nullptr, s);
     if (st != TPK_OK)
         return st;
@@ -818,9 +776,9 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
     PointSet a{unknown, nullptr, static_cast<int64_t>(b) * n, n, reinterpret_cast<float4*>(w + l.sorted_a),
-               reinterpret_cast<float4*>(w + l.boxes_a)};
+               reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
     PointSet c{known, nullptr, static_cast<int64_t>(b) * m, m, reinterpret_cast<float4*>(w + l.sorted_b),
-               reinterpret_cast<float4*>(w + l.boxes_b)};
+               reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
     int st = launch_curve_cells(a, c, nullptr, s);
     if (st != TPK_OK)
         return st;
@@ -837,74 +795,62 @@ namespace {
 
 struct BallLayout
 {
-    size_t sorted_x, sorted_y, boxes_x, boxes_y, overflow, total;
+    size_t sorted_x, bin_ends, grids, total;
 };
 
-BallLayout ball_layout(int64_t size_x, int64_t size_y)
+BallLayout ball_layout(int64_t size_x)
 {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
     const size_t wx = static_cast<size_t>((size_x + CURVE_MAX_POINTS - 1) / CURVE_MAX_POINTS);
-    const size_t wy = static_cast<size_t>((size_y + CURVE_MAX_POINTS - 1) / CURVE_MAX_POINTS);
-    const size_t cells = CURVE_MAX_POINTS / NG_CELL;
     BallLayout l;
     size_t pos = 0;
     l.sorted_x = pos;
     pos = up(pos + wx * CURVE_MAX_POINTS * sizeof(float4));
-    l.sorted_y = pos;
-    pos = up(pos + wy * CURVE_MAX_POINTS * sizeof(float4));
-    l.boxes_x = pos;
-    pos = up(pos + wx * cells * 2 * sizeof(float4));
-    l.boxes_y = pos;
-    pos = up(pos + wy * cells * 2 * sizeof(float4));
-    l.overflow = pos;
-    pos = up(pos + (static_cast<size_t>(size_y) + BQG_LIST) * sizeof(int));
+    l.bin_ends = pos;
+    pos = up(pos + wx * CURVE_BINS * sizeof(int));
+    l.grids = pos;
+    pos = up(pos + wx * 2 * sizeof(float4));
     l.total = pos;
     return l;
 }
 
-bool ball_grid_supported(int64_t size_x, int64_t size_y, int nsample)
+bool ball_bins_supported(int64_t size_x, int64_t size_y, int nsample)
 {
     // Small problems are served as fast by the all-pairs scan; rows are 32-bit here.
-    return size_x >= 8192 && size_y >= 64 && nsample > 0 && size_x < (1LL << 30) && size_y < (1LL << 30);
+    return size_x >= 8192 && size_y > 0 && nsample > 0 && size_x < (1LL << 30);
 }
 
 } // namespace
 
 size_t tpk_grid_ball_query_workspace_bytes(int64_t size_x, int64_t size_y, int nsample)
 {
-    return ball_grid_supported(size_x, size_y, nsample) ? ball_layout(size_x, size_y).total : 0;
+    return ball_bins_supported(size_x, size_y, nsample) ? ball_layout(size_x).total : 0;
 }
 
-int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius2, int nsample, const float* x,
-                                const float* y, const int64_t* batch_x, const int64_t* batch_y,
-                                int64_t* idx, float* dist, void* workspace, size_t workspace_bytes,
-                                hipStream_t s)
+int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample,
+                                const float* x, const float* y, const int64_t* batch_x,
+                                const int64_t* batch_y, int64_t* idx, float* dist, void* workspace,
+                                size_t workspace_bytes, hipStream_t s)
 {
-    if (!ball_grid_supported(size_x, size_y, nsample))
+    if (!ball_bins_supported(size_x, size_y, nsample))
         return TPK_ERR_UNSUPPORTED;
-    const BallLayout l = ball_layout(size_x, size_y);
+    const BallLayout l = ball_layout(size_x);
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
-    PointSet px{x, batch_x, size_x, CURVE_MAX_POINTS, reinterpret_cast<float4*>(w + l.sorted_x),
-                reinterpret_cast<float4*>(w + l.boxes_x)};
-    PointSet py{y, batch_y, size_y, CURVE_MAX_POINTS, reinterpret_cast<float4*>(w + l.sorted_y),
-                reinterpret_cast<float4*>(w + l.boxes_y)};
-    int* overflow = reinterpret_cast<int*>(w + l.overflow);
-    int st = launch_curve_cells(px, py, overflow, s);
+    // (cloud ids are not used for the order: bins may mix the clouds of a window, rows tell them apart)
+    PointSet px{x, nullptr, size_x, CURVE_MAX_POINTS, reinterpret_cast<float4*>(w + l.sorted_x), nullptr,
+                reinterpret_cast<int*>(w + l.bin_ends), reinterpret_cast<float4*>(w + l.grids)};
+    PointSet none{nullptr, nullptr, 0, CURVE_MAX_POINTS, nullptr, nullptr, nullptr, nullptr};
+    int st = launch_curve_cells(px, none, nullptr, s);
     if (st != TPK_OK)
         return st;
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
-    const int64_t waves = set_windows(py) * (CURVE_MAX_POINTS / NG_CELL);
-    hipLaunchKernelGGL(ball_query_grid_kernel, dim3(static_cast<unsigned>(tpk_ceil_div(waves, WAVES))),
-                       dim3(NG_SCAN_THREADS), 0, s, static_cast<int>(size_x), static_cast<int>(size_y), radius2,
-                       nsample, px.sorted, px.boxes, py.sorted, py.boxes, batch_x, batch_y, idx, dist, overflow);
-    st = tpk_launch_status();
-    if (st != TPK_OK)
-        return st;
-    // The number of handed-over queries is known on the device only: a fixed grid walks the list.
-    const unsigned blocks = static_cast<unsigned>(tpk_min64(tpk_ceil_div(size_y, WAVES), 2048));
-    hipLaunchKernelGGL(ball_query_overflow_kernel, dim3(blocks), dim3(NG_SCAN_THREADS), 0, s,
-                       static_cast<int>(size_x), radius2, nsample, x, y, batch_x, batch_y, idx, dist, overflow);
+    const int64_t blocks = tpk_ceil_div(size_y, WAVES);
+    if (blocks > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(ball_query_bins_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+                       static_cast<int>(size_x), static_cast<int>(size_y), std::fabs(radius), radius2, nsample, x, y,
+                       px.sorted, px.bin_ends, px.grid, batch_x, batch_y, idx, dist);
     return tpk_launch_status();
 }
