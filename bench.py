@@ -173,6 +173,7 @@ def bench_others(dev, steps, warmup, with_cpu):
     e = {"workload": "configs[3]: ball_query partial_dense clouds 20k/45k/70k/100k, 25% queries, r=0.05 nsample=64",
          "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
          "roofline": _roof_flops(pairs, 8, ev), "pairs_upper_bound": pairs}
+    e["roofline"]["note"] += PRUNED_NOTE
     if ref is not None:
         secs = _cpu_time(lambda: ref.batch_ball_query(w["x"], w["y"], w["batch_x"], w["batch_y"], w["radius"],
                                                       w["nsample"], 0, False))
