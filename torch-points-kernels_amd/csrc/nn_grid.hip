@@ -510,25 +510,54 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
 // ---------------------------------------------------------------------------------------
 constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
 
-// First position of sorted a[0..len) whose value is >= v, found by the whole wavefront:
-// 64 samples per round instead of one.
-__device__ __forceinline__ int wave_lower_bound(const int64_t* __restrict__ a, int len, int64_t v, int lane)
+// The equal range [first, last) of value v in sorted a[0..len), found by the whole wavefront: 64
+// samples per round instead of one, and both ends in the same rounds, so that their loads
+// travel together.
+__device__ __forceinline__ void wave_equal_range(const int64_t* __restrict__ a, int len, int64_t v, int lane,
+                                                 int& first, int& last)
 {
-    int lo = 0, hi = len; // the answer lies in [lo, hi]
-    while (hi > lo)
+    int lo0 = 0, hi0 = len, lo1 = 0, hi1 = len;
+    while (hi0 > lo0 || hi1 > lo1)
     {
-        const int step = (hi - lo + TPK_WAVE - 1) / TPK_WAVE;
-        const int pos = lo + lane * step;
-        const bool in = pos < hi;
-        const int64_t sample = a[in ? pos : lo];
-        const unsigned long long ge = __ballot(!in || sample >= v);
-        const int f = ge ? __builtin_ctzll(ge) : TPK_WAVE; // first lane whose sample is >= v
-        const int next_lo = f > 0 ? lo + (f - 1) * step + 1 : lo;
-        const int next_hi = f < TPK_WAVE ? min(lo + f * step, hi) : hi;
-        lo = next_lo;
-        hi = next_hi;
+        const int step0 = (hi0 - lo0 + TPK_WAVE - 1) / TPK_WAVE, step1 = (hi1 - lo1 + TPK_WAVE - 1) / TPK_WAVE;
+        const int pos0 = lo0 + lane * step0, pos1 = lo1 + lane * step1;
+        const bool in0 = pos0 < hi0, in1 = pos1 < hi1;
+        const int64_t sample0 = a[in0 ? pos0 : 0], sample1 = a[in1 ? pos1 : 0];
+        const unsigned long long ge0 = __ballot(!in0 || sample0 >= v);
+        const unsigned long long ge1 = __ballot(!in1 || sample1 > v);
+        if (hi0 > lo0)
+        {
+            const int f = ge0 ? __builtin_ctzll(ge0) : TPK_WAVE;
+            const int next_lo = f > 0 ? lo0 + (f - 1) * step0 + 1 : lo0;
+            hi0 = f < TPK_WAVE ? min(lo0 + f * step0, hi0) : hi0;
+            lo0 = next_lo;
+        }
+        if (hi1 > lo1)
+        {
+            const int f = ge1 ? __builtin_ctzll(ge1) : TPK_WAVE;
+            const int next_lo = f > 0 ? lo1 + (f - 1) * step1 + 1 : lo1;
+            hi1 = f < TPK_WAVE ? min(lo1 + f * step1, hi1) : hi1;
+            lo1 = next_lo;
+        }
     }
-    return lo;
+    first = lo0;
+    last = lo1;
+}
+
+// Sum of v over the lanes below this one (DPP prefix sum inside every row of 16 lanes, then
+// the totals of the rows before).
+__device__ __forceinline__ int wave_exclusive_sum(int v)
+{
+    int s = v;
+    s += __builtin_amdgcn_update_dpp(0, s, 0x111, 0xF, 0xF, false); // row_shr:1
+    s += __builtin_amdgcn_update_dpp(0, s, 0x112, 0xF, 0xF, false); // row_shr:2
+    s += __builtin_amdgcn_update_dpp(0, s, 0x114, 0xF, 0xF, false); // row_shr:4
+    s += __builtin_amdgcn_update_dpp(0, s, 0x118, 0xF, 0xF, false); // row_shr:8
+    const int r0 = __builtin_amdgcn_readlane(s, 15), r1 = __builtin_amdgcn_readlane(s, 31);
+    const int r2 = __builtin_amdgcn_readlane(s, 47);
+    const int row = (threadIdx.x & (TPK_WAVE - 1)) >> 4;
+    s += (row > 0 ? r0 : 0) + (row > 1 ? r1 : 0) + (row > 2 ? r2 : 0);
+    return s - v;
 }
 
 // Range of 16^3-grid cells along one axis that [v - r, v + r] can touch.  The interval is widened
@@ -549,6 +578,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
     __shared__ int hit_rows[WAVES][BQB_HITS];
     __shared__ float hit_dists[WAVES][BQB_HITS];
+    __shared__ int slot_rows[WAVES][TPK_WAVE]; // pair descriptors, then candidate addresses
 
     const int lane = threadIdx.x & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
@@ -557,52 +587,74 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
         return; // (no workgroup barrier anywhere in this kernel)
     int* const rows = hit_rows[wave];
     float* const dists = hit_dists[wave];
+    int* const slots = slot_rows[wave];
 
     const float ux = y[q * 3 + 0], uy = y[q * 3 + 1], uz = y[q * 3 + 2];
     const float qx = to_vector_register(ux), qy = to_vector_register(uy), qz = to_vector_register(uz);
     const int64_t cloud = batch_y[q];
-    const int s0 = wave_lower_bound(batch_x, size_x, cloud, lane);
-    const int s1 = wave_lower_bound(batch_x, size_x, cloud + 1, lane);
+    int s0, s1;
+    wave_equal_range(batch_x, size_x, cloud, lane, s0, s1);
     const int64_t out = q * nsample;
 
+    // The walk is laid out so that dependent loads are few: all windows at once (one lane each),
+    // then all (window, bin) pairs at once, then the candidates 64 at a time.
     int cnt = 0;
-    bool serial = false; // answer by the scan in index order instead
-    for (int wx = s0 / CURVE_MAX_POINTS; !serial && s1 > s0 && wx * CURVE_MAX_POINTS < s1; ++wx)
+    const int wx0 = s0 / CURVE_MAX_POINTS;
+    const int windows = s1 > s0 ? (s1 - 1) / CURVE_MAX_POINTS - wx0 + 1 : 0;
+    bool serial = windows > TPK_WAVE; // answer by the scan in index order instead
+    if (!serial && windows > 0)
     {
-        const float4 origin = grids[wx * 2 + 0], scale = grids[wx * 2 + 1];
-        int fx, lx, fy, ly, fz, lz;
-        bin_range(ux, radius, origin.x, scale.x, fx, lx);
-        bin_range(uy, radius, origin.y, scale.y, fy, ly);
-        bin_range(uz, radius, origin.z, scale.z, fz, lz);
-        const int nx = lx - fx + 1, ny = ly - fy + 1, nz = lz - fz + 1;
-        const int nbins = nx * ny * nz;
-        if (nbins > TPK_WAVE)
+        // lane w: the block of bins that the ball's cube touches in window wx0 + w
+        int nbins = 0, block = 0;
+        if (lane < windows)
         {
-            serial = true;
-            break;
+            const float4 origin = grids[(wx0 + lane) * 2 + 0], scale = grids[(wx0 + lane) * 2 + 1];
+            int fx, lx, fy, ly, fz, lz;
+            bin_range(ux, radius, origin.x, scale.x, fx, lx);
+            bin_range(uy, radius, origin.y, scale.y, fy, ly);
+            bin_range(uz, radius, origin.z, scale.z, fz, lz);
+            const int nx = lx - fx + 1, ny = ly - fy + 1;
+            nbins = nx * ny * (lz - fz + 1);
+            block = fx | (fy << 4) | (fz << 8) | ((nx - 1) << 12) | ((ny - 1) << 16) | (lane << 26);
         }
-        // lane l looks up bin l of the block of bins
-        int start = 0, size = 0;
-        if (lane < nbins)
+        const int pairs_before = wave_exclusive_sum(nbins);
+        const int pairs = __builtin_amdgcn_readlane(pairs_before + nbins, TPK_WAVE - 1);
+        serial = pairs > TPK_WAVE;
+        if (!serial)
         {
-            const int bx = fx + lane % nx, by = fy + (lane / nx) % ny, bz = fz + lane / (nx * ny);
-            const unsigned bin = curve_bin_of_cell(bx, by, bz);
-            const int* __restrict__ ends = bin_ends + static_cast<int64_t>(wx) * CURVE_BINS;
-            start = bin ? ends[bin - 1] : 0;
-            size = ends[bin] - start;
-        }
-        const float4* __restrict__ cpts = sorted_x + static_cast<int64_t>(wx) * CURVE_MAX_POINTS;
-        const int row_base = wx * CURVE_MAX_POINTS;
-        for (int b = 0; b < nbins; ++b)
-        {
-            const int bstart = __builtin_amdgcn_readlane(start, b);
-            const int bsize = __builtin_amdgcn_readlane(size, b);
-            for (int t0 = 0; t0 < bsize; t0 += TPK_WAVE)
+            // one descriptor per (window, bin) pair, written by the window's lane
+            for (int i = 0; i < nbins; ++i)
+                slots[pairs_before + i] = block | (i << 20);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            // lane p: where the points of pair p start in the ordered array, and how many
+            int start = 0, size = 0;
+            if (lane < pairs)
             {
-                const bool has = t0 + lane < bsize;
-                const float4 p = cpts[bstart + (has ? t0 + lane : 0)];
+                const int d = slots[lane];
+                const int fx = d & 15, fy = (d >> 4) & 15, fz = (d >> 8) & 15;
+                const int nx = ((d >> 12) & 15) + 1, ny = ((d >> 16) & 15) + 1;
+                const int i = (d >> 20) & 63, wx = wx0 + ((d >> 26) & 63);
+                const unsigned bin = curve_bin_of_cell(fx + i % nx, fy + (i / nx) % ny, fz + i / (nx * ny));
+                const int* __restrict__ ends = bin_ends + static_cast<int64_t>(wx) * CURVE_BINS;
+                start = bin ? ends[bin - 1] : 0;
+                size = ends[bin] - start;
+                start += wx * CURVE_MAX_POINTS;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int before = wave_exclusive_sum(size);
+            const int total = __builtin_amdgcn_readlane(before + size, TPK_WAVE - 1);
+            for (int c0 = 0; c0 < total && !serial; c0 += TPK_WAVE)
+            {
+                // the pairs' lanes hand out the addresses of candidates c0 .. c0 + 63
+                for (int i = max(0, c0 - before); i < size && before + i < c0 + TPK_WAVE; ++i)
+                    slots[before + i - c0] = start + i;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                const bool has = c0 + lane < total;
+                const int at_x = has ? slots[lane] : start;
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const float4 p = sorted_x[has ? at_x : 0];
                 const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-                const int row = row_base + __float_as_int(p.w);
+                const int row = (at_x & ~(CURVE_MAX_POINTS - 1)) + __float_as_int(p.w);
                 const bool hit = has && d <= radius2 && row >= s0 && row < s1;
                 const unsigned long long mask = __ballot(hit);
                 if (mask == 0)
@@ -614,9 +666,9 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                     dists[at] = d;
                 }
                 cnt += __builtin_popcountll(mask);
+                serial = cnt > BQB_HITS;
             }
         }
-        serial = cnt > BQB_HITS;
     }
 
     if (!serial)
