@@ -89,13 +89,9 @@ __device__ __forceinline__ unsigned hilbert_code(unsigned x0, unsigned x1, unsig
         t ^= (x[2] & q) ? q - 1u : 0u;
     return (spread_bits_6(x[0] ^ t) << 2) | (spread_bits_6(x[1] ^ t) << 1) | spread_bits_6(x[2] ^ t);
 }
-__device__ __forceinline__ unsigned hilbert_code_6(unsigned x0, unsigned x1, unsigned x2)
-{
-    return hilbert_code<6>(x0, x1, x2);
-}
-// Bin of the counting sort (leading 12 bits of the 18-bit position) that holds the points of
-// cell (bx, by, bz) of the 16^3 grid: the position of that cell on the 4-bit curve, because the
-// leading bits of a Hilbert position are the position of the enclosing coarser cell.
+// Bin of the counting sort that holds the points of cell (bx, by, bz) of the 16^3 grid: the
+// position of that cell on the 4-bit curve (which is also the leading 12 bits of the position of
+// any finer cell inside it: a Hilbert position starts with that of the enclosing coarser cell).
 __device__ __forceinline__ unsigned curve_bin_of_cell(unsigned bx, unsigned by, unsigned bz)
 {
     return hilbert_code<4>(bx, by, bz);
@@ -140,13 +136,13 @@ __device__ __forceinline__ unsigned curve_grid_cell(float v, float lo, float sca
     return q < 63.f ? static_cast<unsigned>(q) : 63u;
 }
 
-constexpr int CURVE_BINS = 4096;        // bins of the counting sort: leading 12 bits of the 18-bit code
+constexpr int CURVE_BINS = 4096;        // bins of the counting sort: the cells of a 16^3 grid, in curve order
 constexpr int CURVE_MAX_POINTS = 16384; // the index of a point takes the low 14 bits of its sort key
 constexpr int CURVE_LOAD_BATCH = 16;    // global loads in flight per thread
 
 // Orders the n points (1 <= n <= CURVE_MAX_POINTS) of the cloud at `xyz` along the curve.  On
-// return sort_keys[0..n) holds (code << 14) | index, ascending in the leading 12 bits of the code
-// and visible to the whole workgroup.  All arrays are LDS: sort_keys and unsorted n words each,
+// return sort_keys[0..n) holds (bin << 20) | index, ascending in the bin - the position on the curve
+// of the point's cell in a 16^3 grid over the cloud's box - and visible to the whole workgroup.  All arrays are LDS: sort_keys and unsorted n words each,
 // bins CURVE_BINS words, cloud_box 6 words, wave_totals one word per wavefront.  Called by every
 // thread of a workgroup of THREADS lanes (contains barriers).
 // With `group` != nullptr (one sorted id per point: several clouds packed in one array) the points
@@ -234,13 +230,14 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
                     cell[a] = curve_grid_cell(v[u][a], grid.lo[a], grid.scale[a]);
-                unsigned code = hilbert_code_6(cell[0], cell[1], cell[2]);
+                // the bin: position on the curve of the cell of the 16^3 grid
+                unsigned bin = curve_bin_of_cell(cell[0] >> 2, cell[1] >> 2, cell[2] >> 2);
                 if (group && k < n)
                 {
                     const int64_t offset = group[k] - group[0];
-                    code = (static_cast<unsigned>(offset < 7 ? offset : 7) << 15) | (code >> 3);
+                    bin = (static_cast<unsigned>(offset < 7 ? offset : 7) << 9) | (bin >> 3);
                 }
-                const unsigned key = (code << 14) | static_cast<unsigned>(k);
+                const unsigned key = (bin << 20) | static_cast<unsigned>(k);
                 if (k < n)
                 {
                     unsorted[k] = key;

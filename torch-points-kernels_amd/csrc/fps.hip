@@ -265,7 +265,7 @@ __global__ __launch_bounds__(THREADS) void fps_resident_kernel(
 // round.  So a set of points whose bounding box is further from the new sample than the square
 // root of the previous winning value cannot change, and its update can be skipped without
 // changing any result.  To make such sets exist, the kernel first orders the cloud along a
-// Hilbert curve (18-bit position, counting sort in LDS) and cuts the curve into cells of
+// Hilbert curve (12-bit position of its cell in a 16^3 grid, counting sort in LDS) and cuts the curve into cells of
 // 64 * GS consecutive points.  A cell is GS registers of the 64 lanes of one wavefront; every
 // wavefront holds NG cells, taken round-robin along the curve so that the cells around a
 // sample belong to different wavefronts.  A wavefront tests its NG boxes at once, lane g
@@ -356,7 +356,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     constexpr int NG = PPT / GS;
     static_assert(NG <= 16, "one DPP row of lanes tests the group boxes");
     static_assert(WAVES >= 2, "a cloud without eligible points must count several winners");
-    // key_capacity keys (curve position << 14) | index in curve order, kept for the whole kernel; then
+    // key_capacity keys (curve position << 20) | index in curve order, kept for the whole kernel; then
     // PPT * THREADS words (the unsorted keys during set-up, later the copy of the running minima
     // made when equal maxima have to be resolved); then the bins of the counting sort
     extern __shared__ unsigned sort_keys[];
