@@ -42,13 +42,13 @@ def test_library_exports_every_declared_symbol():
     lib.tpk_fps_workspace_bytes.restype = ctypes.c_size_t
     assert lib.tpk_fps_workspace_bytes(4, 16384) == 0
     assert lib.tpk_fps_workspace_bytes(4, 50000) == 4 * 50000 * 4
-    # searches over curve-ordered cells: 16 bytes per point padded to cells of 64, 32 bytes per cell;
+    # searches over curve-ordered cells: 16 bytes per point padded to cells of 64, 160 bytes per cell;
     # 0 = the shape is served by the all-pairs scan, no workspace wanted
     for name in ("tpk_three_nn_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_size_t
         assert fn(2, 100, 100) == 0 and fn(2, 20000, 1000) == 0 and fn(0, 1000, 1000) == 0
-        want = sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((11, 1024), (15, 1024), (11, 32), (15, 32)))
+        want = sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((11, 1024), (15, 1024), (11, 160), (15, 160)))
         assert fn(2, 700, 900) == want
     lib.tpk_ball_query_partial_workspace_bytes.restype = ctypes.c_size_t
     lib.tpk_ball_query_partial_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]

@@ -32,6 +32,7 @@ constexpr int NG_SORT_THREADS = 1024;
 constexpr int NG_SCAN_THREADS = 256;         // 4 wavefronts, each searching on its own
 constexpr float NG_MARGIN = 0.999998f;
 constexpr int NG_CHUNK = 8;
+constexpr int NG_BOX = 10;                   // float4 per cell: box of the cell, then of its four runs of 16 points
 
 // A set of points to be ordered: `total` points cut into windows of `stride` consecutive points
 // (a batch of equal clouds: stride = points per cloud; a packed array: windows of at most
@@ -46,7 +47,7 @@ struct PointSet
     int64_t total;
     int stride;
     float4* sorted;       // [windows][cells * 64]
-    float4* boxes;        // [windows][cells][2]: (lo.xyz, -), (hi.xyz, -); or nullptr
+    float4* boxes;        // [windows][cells][NG_BOX]: (lo.xyz, -), (hi.xyz, -) of the cell and of its quarters; or nullptr
     int* bin_ends;        // optional [windows][CURVE_BINS]: end of every bin of the counting sort
     float4* grid;         // optional [windows][2]: origin and scale of the window's 64^3 grid
 };
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     const int cells = set_cells(set);
     const float* __restrict__ xyz = set.xyz + start * 3;
     float4* __restrict__ sorted = set.sorted + window * cells * NG_CELL;
-    float4* __restrict__ boxes = set.boxes ? set.boxes + window * cells * 2 : nullptr;
+    float4* __restrict__ boxes = set.boxes ? set.boxes + window * cells * NG_BOX : nullptr;
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
     if (zero_word && blockIdx.x == 0 && tid == 0)
@@ -118,17 +119,36 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
                              : make_float4(inf, inf, inf, __int_as_float(0x7FFFFFFF));
             if (!boxes) // uniform
                 continue;
-            float lo[3], hi[3];
+            // boxes of the four runs of 16 points (DPP row reductions), then of the whole cell
+            float4* const cell_box = boxes + (q / NG_CELL) * NG_BOX;
+            int lo[3], hi[3];
 #pragma unroll
             for (int a = 0; a < 3; ++a)
             {
-                lo[a] = ordered_int_to_float(wave_min_i32(float_to_ordered_int(real ? v[u][a] : inf)));
-                hi[a] = ordered_int_to_float(wave_max_i32(float_to_ordered_int(real ? v[u][a] : -inf)));
+                lo[a] = ~row_all_max_i32(~float_to_ordered_int(real ? v[u][a] : inf));
+                hi[a] = row_all_max_i32(float_to_ordered_int(real ? v[u][a] : -inf));
+            }
+            if ((lane & 15) == 0)
+            {
+                cell_box[2 + (lane >> 4) * 2 + 0] = make_float4(ordered_int_to_float(lo[0]), ordered_int_to_float(lo[1]),
+                                                                ordered_int_to_float(lo[2]), 0.f);
+                cell_box[2 + (lane >> 4) * 2 + 1] = make_float4(ordered_int_to_float(hi[0]), ordered_int_to_float(hi[1]),
+                                                                ordered_int_to_float(hi[2]), 0.f);
+            }
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+            {
+                lo[a] = min(min(__builtin_amdgcn_readlane(lo[a], 0), __builtin_amdgcn_readlane(lo[a], 16)),
+                            min(__builtin_amdgcn_readlane(lo[a], 32), __builtin_amdgcn_readlane(lo[a], 48)));
+                hi[a] = max(max(__builtin_amdgcn_readlane(hi[a], 0), __builtin_amdgcn_readlane(hi[a], 16)),
+                            max(__builtin_amdgcn_readlane(hi[a], 32), __builtin_amdgcn_readlane(hi[a], 48)));
             }
             if (lane == 0)
             {
-                boxes[(q / NG_CELL) * 2 + 0] = make_float4(lo[0], lo[1], lo[2], 0.f);
-                boxes[(q / NG_CELL) * 2 + 1] = make_float4(hi[0], hi[1], hi[2], 0.f);
+                cell_box[0] = make_float4(ordered_int_to_float(lo[0]), ordered_int_to_float(lo[1]),
+                                          ordered_int_to_float(lo[2]), 0.f);
+                cell_box[1] = make_float4(ordered_int_to_float(hi[0]), ordered_int_to_float(hi[1]),
+                                          ordered_int_to_float(hi[2]), 0.f);
             }
         }
     }
@@ -173,14 +193,25 @@ struct Nearest
 
 // Scans candidate cell `cell` for the 64 queries of the wavefront.  `stage` is the wavefront's
 // own 64-entry LDS buffer, through which every lane sees every candidate (broadcast reads).
-__device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, int cell, float4* stage,
-                                          int lane, float qx, float qy, float qz, Nearest& s)
+__device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, const float4* __restrict__ boxes,
+                                          int cell, float4* stage, int lane, float qx, float qy, float qz,
+                                          Nearest& s)
 {
     stage[lane] = cand[cell * NG_CELL + lane];
+    const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); // LDS serves a wavefront's requests in order
-#pragma unroll 2
     for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
     {
+        // a run of 16 candidates whose box no lane's answer reaches is passed over
+        if ((ch & 1) == 0)
+        {
+            const float lb = point_box_dist2(qx, qy, qz, quarter[ch], quarter[ch + 1]);
+            if (__ballot(lb * NG_MARGIN <= s.best) == 0)
+            {
+                ++ch;
+                continue;
+            }
+        }
         float mn = 0.f;
 #pragma unroll
         for (int c = 0; c < NG_CHUNK; ++c)
@@ -227,9 +258,9 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
     const int ccells = second ? cells1 : cells2;
     const int qcount = second ? m : n;
     const float4* __restrict__ qpts = (second ? sorted2 : sorted1) + static_cast<int64_t>(cloud) * qcells * NG_CELL;
-    const float4* __restrict__ qbox = (second ? boxes2 : boxes1) + static_cast<int64_t>(cloud) * qcells * 2;
+    const float4* __restrict__ qbox = (second ? boxes2 : boxes1) + static_cast<int64_t>(cloud) * qcells * NG_BOX;
     const float4* __restrict__ cpts = (second ? sorted1 : sorted2) + static_cast<int64_t>(cloud) * ccells * NG_CELL;
-    const float4* __restrict__ cbox = (second ? boxes1 : boxes2) + static_cast<int64_t>(cloud) * ccells * 2;
+    const float4* __restrict__ cbox = (second ? boxes1 : boxes2) + static_cast<int64_t>(cloud) * ccells * NG_BOX;
     float* __restrict__ dout = (second ? dist2 : dist1) + static_cast<int64_t>(cloud) * qcount;
     int32_t* __restrict__ iout = (second ? idx2 : idx1) + static_cast<int64_t>(cloud) * qcount;
     float4* const stage = stages[wave];
@@ -238,7 +269,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
     const float4 query = qpts[qcell * NG_CELL + lane];
     const float qx = query.x, qy = query.y, qz = query.z;
     const int qindex = __float_as_int(query.w); // 0x7FFFFFFF: padding, nothing to store
-    const float4 qlo = qbox[qcell * 2 + 0], qhi = qbox[qcell * 2 + 1];
+    const float4 qlo = qbox[qcell * NG_BOX + 0], qhi = qbox[qcell * NG_BOX + 1];
 
     // Box distances to all candidate cells, kept in the wavefront's LDS row (lane l computes
     // cells l, 64 + l, ...); +inf marks a cell that does not exist or has been scanned.
@@ -249,7 +280,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
         const int c = g * NG_CELL + lane;
         const bool valid = c < ccells;
         const int cc = valid ? c : 0;
-        const float lb = box_box_dist2(qlo, qhi, cbox[cc * 2 + 0], cbox[cc * 2 + 1]);
+        const float lb = box_box_dist2(qlo, qhi, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
         lows[c] = valid ? lb : __builtin_inff();
         // approximately the nearest cell (the two lowest bits of the distance carry g)
         const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~3u) | static_cast<unsigned>(g);
@@ -264,7 +295,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
         int seed = static_cast<int>(lowest & 3u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
         if (seed >= ccells) // no lane had a usable key (NaN boxes)
             seed = 0;
-        scan_cell(cpts, seed, stage, lane, qx, qy, qz, s);
+        scan_cell(cpts, cbox, seed, stage, lane, qx, qy, qz, s);
         if (lane == (seed & (NG_CELL - 1)))
             lows[seed] = __builtin_inff();
     }
@@ -283,7 +314,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
                 const int bit = __builtin_ctzll(live);
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
-                const float lb = point_box_dist2(qx, qy, qz, cbox[c * 2 + 0], cbox[c * 2 + 1]);
+                const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
                 if (__ballot(lb * NG_MARGIN <= s.best) == 0)
                 {
                     // no lane can improve here now, and answers only get better: never again
@@ -291,7 +322,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
                         lows[c] = __builtin_inff();
                     continue;
                 }
-                scan_cell(cpts, c, stage, lane, qx, qy, qz, s);
+                scan_cell(cpts, cbox, c, stage, lane, qx, qy, qz, s);
                 if (lane == bit)
                     lows[c] = __builtin_inff();
                 if (phase)
@@ -318,7 +349,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
         // Several groups reached the minimum (rare): lowest index over all cells that can hold it.
         for (int c = 0; c < ccells; ++c)
         {
-            const float lb = point_box_dist2(qx, qy, qz, cbox[c * 2 + 0], cbox[c * 2 + 1]);
+            const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
             if (__ballot(s.tie && lb * NG_MARGIN <= s.best) == 0)
                 continue;
             stage[lane] = cpts[c * NG_CELL + lane];
@@ -360,13 +391,25 @@ __device__ __forceinline__ bool pair_less(float d, int ci, float b, int i)
     return d < b || (d == b && ci < i);
 }
 
-__device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, int cell, float4* stage,
-                                           int lane, float qx, float qy, float qz, Nearest3& s)
+__device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, const float4* __restrict__ boxes,
+                                           int cell, float4* stage, int lane, float qx, float qy, float qz,
+                                           Nearest3& s)
 {
     stage[lane] = cand[cell * NG_CELL + lane];
+    const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
     {
+        // a run of 16 candidates whose box no lane's third best reaches is passed over
+        if ((ch & 1) == 0)
+        {
+            const float lb = point_box_dist2(qx, qy, qz, quarter[ch], quarter[ch + 1]);
+            if (__ballot(lb * NG_MARGIN <= s.b3) == 0)
+            {
+                ++ch;
+                continue;
+            }
+        }
         float mn = 0.f;
 #pragma unroll
         for (int c = 0; c < NG_CHUNK; ++c)
@@ -419,9 +462,9 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     const int cloud = static_cast<int>(task / qcells);
     const int qcell = static_cast<int>(task - static_cast<int64_t>(cloud) * qcells);
     const float4* __restrict__ qpts = sorted_unknown + static_cast<int64_t>(cloud) * qcells * NG_CELL;
-    const float4* __restrict__ qbox = boxes_unknown + static_cast<int64_t>(cloud) * qcells * 2;
+    const float4* __restrict__ qbox = boxes_unknown + static_cast<int64_t>(cloud) * qcells * NG_BOX;
     const float4* __restrict__ cpts = sorted_known + static_cast<int64_t>(cloud) * ccells * NG_CELL;
-    const float4* __restrict__ cbox = boxes_known + static_cast<int64_t>(cloud) * ccells * 2;
+    const float4* __restrict__ cbox = boxes_known + static_cast<int64_t>(cloud) * ccells * NG_BOX;
     dist2 += static_cast<int64_t>(cloud) * n * 3;
     idx += static_cast<int64_t>(cloud) * n * 3;
     float4* const stage = stages[wave];
@@ -430,7 +473,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     const float4 query = qpts[qcell * NG_CELL + lane];
     const float qx = query.x, qy = query.y, qz = query.z;
     const int qindex = __float_as_int(query.w); // 0x7FFFFFFF: padding, nothing to store
-    const float4 qlo = qbox[qcell * 2 + 0], qhi = qbox[qcell * 2 + 1];
+    const float4 qlo = qbox[qcell * NG_BOX + 0], qhi = qbox[qcell * NG_BOX + 1];
 
     const int groups = (ccells + NG_CELL - 1) / NG_CELL;
     unsigned seed_key = 0xFFFFFFFFu;
@@ -439,7 +482,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
         const int c = g * NG_CELL + lane;
         const bool valid = c < ccells;
         const int cc = valid ? c : 0;
-        const float lb = box_box_dist2(qlo, qhi, cbox[cc * 2 + 0], cbox[cc * 2 + 1]);
+        const float lb = box_box_dist2(qlo, qhi, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
         lows[c] = valid ? lb : __builtin_inff();
         const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~3u) | static_cast<unsigned>(g);
         seed_key = valid && key < seed_key ? key : seed_key;
@@ -452,7 +495,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
         int seed = static_cast<int>(lowest & 3u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
         if (seed >= ccells)
             seed = 0;
-        scan_cell3(cpts, seed, stage, lane, qx, qy, qz, s);
+        scan_cell3(cpts, cbox, seed, stage, lane, qx, qy, qz, s);
         if (lane == (seed & (NG_CELL - 1)))
             lows[seed] = __builtin_inff();
     }
@@ -468,9 +511,9 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
                 const int bit = __builtin_ctzll(live);
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
-                const float lb = point_box_dist2(qx, qy, qz, cbox[c * 2 + 0], cbox[c * 2 + 1]);
+                const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
                 if (__ballot(lb * NG_MARGIN <= s.b3) != 0)
-                    scan_cell3(cpts, c, stage, lane, qx, qy, qz, s);
+                    scan_cell3(cpts, cbox, c, stage, lane, qx, qy, qz, s);
                 if (lane == bit)
                     lows[c] = __builtin_inff(); // scanned, or useless now and ever after
                 if (phase)
@@ -748,9 +791,9 @@ GridLayout grid_layout(int b, int n, int m)
     l.sorted_b = pos;
     pos = up(pos + static_cast<size_t>(b) * cells_b * NG_CELL * sizeof(float4));
     l.boxes_a = pos;
-    pos = up(pos + static_cast<size_t>(b) * cells_a * 2 * sizeof(float4));
+    pos = up(pos + static_cast<size_t>(b) * cells_a * NG_BOX * sizeof(float4));
     l.boxes_b = pos;
-    pos = up(pos + static_cast<size_t>(b) * cells_b * 2 * sizeof(float4));
+    pos = up(pos + static_cast<size_t>(b) * cells_b * NG_BOX * sizeof(float4));
     l.total = pos;
     return l;
 }
