@@ -142,9 +142,10 @@ constexpr int CURVE_LOAD_BATCH = 16;    // global loads in flight per thread
 
 // Orders the n points (1 <= n <= CURVE_MAX_POINTS) of the cloud at `xyz` along the curve.  On
 // return sort_keys[0..n) holds (bin << 20) | index, ascending in the bin - the position on the curve
-// of the point's cell in a 16^3 grid over the cloud's box - and visible to the whole workgroup.  All arrays are LDS: sort_keys and unsorted n words each,
-// bins CURVE_BINS words, cloud_box 6 words, wave_totals one word per wavefront.  Called by every
-// thread of a workgroup of THREADS lanes (contains barriers).
+// of the point's cell in a 16^3 grid over the cloud's box - and visible to the whole workgroup.
+// All arrays are LDS: sort_keys max(n, CURVE_BINS) words, unsorted n words, bins CURVE_BINS words,
+// cloud_box 6 words, wave_totals one word per wavefront.  Called by every thread of a workgroup
+// of THREADS lanes (contains barriers).
 // With `group` != nullptr (one sorted id per point: several clouds packed in one array) the points
 // of the first 7 distinct-id offsets (group[k] - group[0] = 0..6) come first, one id after the
 // other, each in curve order; the rest follow together.  Only the order changes, never its use.
@@ -164,7 +165,12 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
     if (tid < 6)
         cloud_box[tid] = tid < 3 ? empty_lo : empty_hi;
     for (int i = tid; i < CURVE_BINS; i += THREADS)
+    {
         bins[i] = 0;
+        // curve position of every cell of the 16^3 grid, computed once per cell instead of once
+        // per point; the table borrows sort_keys, which the scatter fills only later
+        sort_keys[i] = curve_bin_of_cell(i & 15, (i >> 4) & 15, i >> 8);
+    }
     __syncthreads();
     {
         float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
@@ -231,7 +237,7 @@ __device__ __forceinline__ void curve_order(const float* __restrict__ xyz, int n
                 for (int a = 0; a < 3; ++a)
                     cell[a] = curve_grid_cell(v[u][a], grid.lo[a], grid.scale[a]);
                 // the bin: position on the curve of the cell of the 16^3 grid
-                unsigned bin = curve_bin_of_cell(cell[0] >> 2, cell[1] >> 2, cell[2] >> 2);
+                unsigned bin = sort_keys[(cell[0] >> 2) | ((cell[1] >> 2) << 4) | ((cell[2] >> 2) << 8)];
                 if (group && k < n)
                 {
                     const int64_t offset = group[k] - group[0];

@@ -727,7 +727,7 @@ template <int PPT, int THREADS, int GS>
 int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float* xyz,
                   int32_t* out, hipStream_t s)
 {
-    const int key_capacity = (n + 63) & ~63;
+    const int key_capacity = n > CURVE_BINS ? (n + 63) & ~63 : CURVE_BINS; // (the ordering borrows CURVE_BINS words)
     const size_t lds = (static_cast<size_t>(key_capacity) + static_cast<size_t>(PPT) * THREADS + CURVE_BINS) * sizeof(unsigned);
     auto kernel = fps_pruned_kernel<PPT, THREADS, GS>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),

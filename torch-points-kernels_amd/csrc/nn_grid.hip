@@ -808,7 +808,7 @@ bool grid_supported(int b, int n, int m)
 int launch_curve_cells(const PointSet& a, const PointSet& c, int* zero_word, hipStream_t s)
 {
     const int largest = a.stride > c.stride ? a.stride : c.stride;
-    const int key_capacity = (largest + 63) & ~63;
+    const int key_capacity = largest > CURVE_BINS ? (largest + 63) & ~63 : CURVE_BINS; // (the ordering borrows CURVE_BINS words)
     const int64_t windows_a = set_windows(a), windows_c = set_windows(c);
     if (windows_a + windows_c > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
