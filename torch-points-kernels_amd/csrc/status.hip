@@ -3,7 +3,7 @@
 
 extern "C" int tpk_version(void)
 {
-    return 100; // 0.1.0
+    return 200; // 0.2.0: three_nn, the Chamfer forward and the packed ball query take a workspace
 }
 
 extern "C" const char* tpk_status_string(int status)
