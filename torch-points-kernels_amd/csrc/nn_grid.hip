@@ -91,6 +91,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
                                  set.group ? set.group + start : nullptr);
 
     // Every wavefront writes whole cells; a batch of gathers is issued before any is used.
+    int* const run_boxes = reinterpret_cast<int*>(unsorted); // (free now) [cells * 4][6] ordered ints
     constexpr int BATCH = 4;
     const int padded = cells * NG_CELL;
     for (int q0 = tid; q0 < padded; q0 += NG_SORT_THREADS * BATCH)
@@ -119,8 +120,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
                              : make_float4(inf, inf, inf, __int_as_float(0x7FFFFFFF));
             if (!boxes) // uniform
                 continue;
-            // boxes of the four runs of 16 points (DPP row reductions), then of the whole cell
-            float4* const cell_box = boxes + (q / NG_CELL) * NG_BOX;
+            // boxes of the four runs of 16 points (DPP row reductions), left in LDS
             int lo[3], hi[3];
 #pragma unroll
             for (int a = 0; a < 3; ++a)
@@ -130,26 +130,44 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
             }
             if ((lane & 15) == 0)
             {
-                cell_box[2 + (lane >> 4) * 2 + 0] = make_float4(ordered_int_to_float(lo[0]), ordered_int_to_float(lo[1]),
-                                                                ordered_int_to_float(lo[2]), 0.f);
-                cell_box[2 + (lane >> 4) * 2 + 1] = make_float4(ordered_int_to_float(hi[0]), ordered_int_to_float(hi[1]),
-                                                                ordered_int_to_float(hi[2]), 0.f);
-            }
+                int* const run_box = run_boxes + (q / 16) * 6;
 #pragma unroll
-            for (int a = 0; a < 3; ++a)
-            {
-                lo[a] = min(min(__builtin_amdgcn_readlane(lo[a], 0), __builtin_amdgcn_readlane(lo[a], 16)),
-                            min(__builtin_amdgcn_readlane(lo[a], 32), __builtin_amdgcn_readlane(lo[a], 48)));
-                hi[a] = max(max(__builtin_amdgcn_readlane(hi[a], 0), __builtin_amdgcn_readlane(hi[a], 16)),
-                            max(__builtin_amdgcn_readlane(hi[a], 32), __builtin_amdgcn_readlane(hi[a], 48)));
+                for (int a = 0; a < 3; ++a)
+                {
+                    run_box[a] = lo[a];
+                    run_box[3 + a] = hi[a];
+                }
             }
-            if (lane == 0)
+        }
+    }
+    if (boxes)
+    {
+        // one thread per cell: the boxes of its four runs, and their union, to memory
+        __syncthreads();
+        for (int c = tid; c < cells; c += NG_SORT_THREADS)
+        {
+            int lo[3] = {0x7FFFFFFF, 0x7FFFFFFF, 0x7FFFFFFF}, hi[3] = {INT_MIN, INT_MIN, INT_MIN};
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
             {
-                cell_box[0] = make_float4(ordered_int_to_float(lo[0]), ordered_int_to_float(lo[1]),
-                                          ordered_int_to_float(lo[2]), 0.f);
-                cell_box[1] = make_float4(ordered_int_to_float(hi[0]), ordered_int_to_float(hi[1]),
-                                          ordered_int_to_float(hi[2]), 0.f);
+                const int* const run_box = run_boxes + (c * 4 + r) * 6;
+                boxes[c * NG_BOX + 2 + r * 2 + 0] =
+                    make_float4(ordered_int_to_float(run_box[0]), ordered_int_to_float(run_box[1]),
+                                ordered_int_to_float(run_box[2]), 0.f);
+                boxes[c * NG_BOX + 2 + r * 2 + 1] =
+                    make_float4(ordered_int_to_float(run_box[3]), ordered_int_to_float(run_box[4]),
+                                ordered_int_to_float(run_box[5]), 0.f);
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                {
+                    lo[a] = min(lo[a], run_box[a]);
+                    hi[a] = max(hi[a], run_box[3 + a]);
+                }
             }
+            boxes[c * NG_BOX + 0] = make_float4(ordered_int_to_float(lo[0]), ordered_int_to_float(lo[1]),
+                                                ordered_int_to_float(lo[2]), 0.f);
+            boxes[c * NG_BOX + 1] = make_float4(ordered_int_to_float(hi[0]), ordered_int_to_float(hi[1]),
+                                                ordered_int_to_float(hi[2]), 0.f);
         }
     }
     if (set.bin_ends)
