@@ -256,16 +256,16 @@ __global__ __launch_bounds__(256) void chamfer_bwd_scatter_kernel(
 }
 
 // One lane per point of either cloud: own term, then the terms of the points that chose it.
-// offs_a/ent_a: lists over the points of cloud 1 (built from idx2); offs_b/ent_b: lists over
-// the points of cloud 2 (built from idx1).
+// lists_a: lists over the points of cloud 1 (built from idx2); lists_b: lists over the points
+// of cloud 2 (built from idx1).  A wavefront serves one block of lists, one lane per point:
+// in step i the lanes read slot i of their lists
+// (consecutive entries; padding entries carry an index past the other cloud and are skipped).
 template <typename T>
 __global__ __launch_bounds__(256) void chamfer_bwd_lists_kernel(
     int n, int m, int clouds, const T* __restrict__ xyz1, const T* __restrict__ xyz2,
     const int32_t* __restrict__ idx1, const int32_t* __restrict__ idx2,
     const T* __restrict__ grad_dist1, const T* __restrict__ grad_dist2,
-    const int* __restrict__ offs_a, const ListEntry<false>* __restrict__ ent_a,
-    const int* __restrict__ offs_b, const ListEntry<false>* __restrict__ ent_b,
-    T* __restrict__ grad_xyz1, T* __restrict__ grad_xyz2)
+    Lists<false> lists_a, Lists<false> lists_b, T* __restrict__ grad_xyz1, T* __restrict__ grad_xyz2)
 {
     // A cloud pair takes blocks1 + blocks2 consecutive logical blocks: the n points of cloud 1
     // first, then the m of cloud 2.  Logical blocks are numbered so that those of a pair run on
@@ -273,59 +273,93 @@ __global__ __launch_bounds__(256) void chamfer_bwd_lists_kernel(
     const int blocks1 = (n + 255) / 256;
     const int per_cloud = blocks1 + (m + 255) / 256;
     const int64_t total = static_cast<int64_t>(per_cloud) * clouds;
+    const int lane = threadIdx.x & (TPK_WAVE - 1);
     for (int64_t lin = xcd_local_block(blockIdx.x, gridDim.x); lin < total; lin += gridDim.x)
     {
         const int cloud = static_cast<int>(lin / per_cloud);
         const int bx = static_cast<int>(lin % per_cloud);
         const bool second = bx >= blocks1;
-        const int k = (second ? bx - blocks1 : bx) * 256 + threadIdx.x;
+        const int pos = (second ? bx - blocks1 : bx) * 256 + threadIdx.x;
         const int npts = second ? m : n;
         const int nother = second ? n : m;
-        if (k >= npts)
+        if (pos - lane >= npts) // the whole wavefront lies past the cloud
             continue;
+        const Lists<false>& lists = second ? lists_b : lists_a;
+        const int64_t nblocks = (npts + L_BLOCK - 1) / L_BLOCK;
+        const int k = pos;
+        const bool live = k < npts;
+        const int kk = live ? k : 0;
         const T* __restrict__ own = (second ? xyz2 : xyz1) + static_cast<int64_t>(cloud) * npts * 3;
         const T* __restrict__ other = (second ? xyz1 : xyz2) + static_cast<int64_t>(cloud) * nother * 3;
         const int32_t* __restrict__ own_idx = (second ? idx2 : idx1) + static_cast<int64_t>(cloud) * npts;
         const T* __restrict__ own_g = (second ? grad_dist2 : grad_dist1) + static_cast<int64_t>(cloud) * npts;
         const T* __restrict__ other_g = (second ? grad_dist1 : grad_dist2) + static_cast<int64_t>(cloud) * nother;
-        const int* __restrict__ offs = (second ? offs_b : offs_a) + static_cast<int64_t>(cloud) * (npts + 1);
-        const ListEntry<false>* __restrict__ ent = (second ? ent_b : ent_a) + static_cast<int64_t>(cloud) * nother;
-        T* __restrict__ out = (second ? grad_xyz2 : grad_xyz1) + (static_cast<int64_t>(cloud) * npts + k) * 3;
+        const ListEntry<false>* __restrict__ ent = lists.entries + static_cast<int64_t>(cloud) * lists.capacity;
+        const ListBlock lb = list_block(lists.blocks + cloud * nblocks, pos / L_BLOCK);
 
-        const T px = own[k * 3 + 0], py = own[k * 3 + 1], pz = own[k * 3 + 2];
-        const int j2 = own_idx[k];
-        const T g = own_g[k] * 2;
+        const T px = own[kk * 3 + 0], py = own[kk * 3 + 1], pz = own[kk * 3 + 2];
+        const int j2 = own_idx[kk];
+        const T g = own_g[kk] * 2;
         T ax = g * (px - other[j2 * 3 + 0]);
         T ay = g * (py - other[j2 * 3 + 1]);
         T az = g * (pz - other[j2 * 3 + 2]);
-        const int beg = offs[k], end = offs[k + 1];
-        for (int p = beg; p < end; ++p)
-        {
-            const int j = ent[p].j;
+        auto add_entry = [&](int j) {
             const T gj = other_g[j] * 2;
             ax = ax + -(gj * (other[j * 3 + 0] - px));
             ay = ay + -(gj * (other[j * 3 + 1] - py));
             az = az + -(gj * (other[j * 3 + 2] - pz));
+        };
+        // Slots are fetched eight at a time, then the points they name (widths are multiples of 4).
+        for (int i = 0; i < lb.width; i += 8)
+        {
+            int j[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                j[u] = i + u < lb.width ? ent[lb.start + (i + u) * L_BLOCK + lane].j : nother;
+            T gj[8], ox[8], oy[8], oz[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+            {
+                const int jj = j[u] < nother ? j[u] : 0;
+                gj[u] = other_g[jj];
+                ox[u] = other[jj * 3 + 0];
+                oy[u] = other[jj * 3 + 1];
+                oz[u] = other[jj * 3 + 2];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (j[u] < nother)
+                {
+                    const T g2 = gj[u] * 2;
+                    ax = ax + -(g2 * (ox[u] - px));
+                    ay = ay + -(g2 * (oy[u] - py));
+                    az = az + -(g2 * (oz[u] - pz));
+                }
         }
-        out[0] = ax;
-        out[1] = ay;
-        out[2] = az;
+        if (lb.longer)
+        {
+            const int count = lists.counts[cloud * nblocks * L_BLOCK + pos];
+            int extra, extra_at;
+            list_extra(count, lb.width, extra, extra_at);
+            const ListEntry<false>* __restrict__ rest = ent + lb.start + lb.width * L_BLOCK + extra_at;
+            for (int p = 0; p < extra; ++p)
+                add_entry(rest[p].j);
+        }
+        if (live)
+        {
+            T* __restrict__ out = (second ? grad_xyz2 : grad_xyz1) + (static_cast<int64_t>(cloud) * npts + k) * 3;
+            out[0] = ax;
+            out[1] = ay;
+            out[2] = az;
+        }
     }
 }
 
-size_t chamfer_lists_bytes(int b, int n, int m, size_t* off_a, size_t* off_b, size_t* ent_a, size_t* ent_b)
+// Workspace of the list-based backward: lists over cloud 1, then lists over cloud 2.
+size_t chamfer_lists_bytes(int b, int n, int m, size_t* second)
 {
-    auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
-    size_t pos = 0;
-    *off_a = pos;
-    pos = up(pos + static_cast<size_t>(b) * (static_cast<size_t>(n) + 1) * sizeof(int));
-    *off_b = pos;
-    pos = up(pos + static_cast<size_t>(b) * (static_cast<size_t>(m) + 1) * sizeof(int));
-    *ent_a = pos;
-    pos = up(pos + static_cast<size_t>(b) * static_cast<size_t>(m) * sizeof(ListEntry<false>));
-    *ent_b = pos;
-    pos = up(pos + static_cast<size_t>(b) * static_cast<size_t>(n) * sizeof(ListEntry<false>));
-    return pos;
+    *second = lists_bytes<false>(b, n, m);
+    return *second + lists_bytes<false>(b, m, n);
 }
 
 template <typename T>
@@ -400,27 +434,27 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
         hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(blocks), dim3(256), 0, s, p, count);
         return tpk_launch_status();
     }
-    size_t off_a, off_b, ent_a, ent_b;
-    const size_t need = chamfer_lists_bytes(b, n, m, &off_a, &off_b, &ent_a, &ent_b);
+    size_t second;
+    const size_t need = chamfer_lists_bytes(b, n, m, &second);
     if (workspace && workspace_bytes >= need && static_cast<int64_t>(n) * 3 <= 0x7fffffffLL &&
         static_cast<int64_t>(m) * 3 <= 0x7fffffffLL)
     {
-        char* ws = static_cast<char*>(workspace);
-        int* offs_a = reinterpret_cast<int*>(ws + off_a);
-        int* offs_b = reinterpret_cast<int*>(ws + off_b);
-        auto* ents_a = reinterpret_cast<ListEntry<false>*>(ws + ent_a);
-        auto* ents_b = reinterpret_cast<ListEntry<false>*>(ws + ent_b);
         // lists over cloud-1 points: who in cloud 2 chose them (idx2); and the mirror image
-        int st = launch_build_lists<1, false, int32_t>(b, n, m, idx2, nullptr, offs_a, ents_a, s);
+        const Lists<false> lists_a = lists_at<false>(workspace, b, n, m);
+        const Lists<false> lists_b = lists_at<false>(static_cast<char*>(workspace) + second, b, m, n);
+        ListJob<false, int32_t> job_a, job_b;
+        int st = make_list_job<1, false, int32_t>(b, n, m, m, m, idx2, nullptr, lists_a, &job_a);
         if (st == TPK_OK)
-            st = launch_build_lists<1, false, int32_t>(b, m, n, idx1, nullptr, offs_b, ents_b, s);
+            st = make_list_job<1, false, int32_t>(b, m, n, n, n, idx1, nullptr, lists_b, &job_b);
+        if (st == TPK_OK)
+            st = launch_list_jobs<1, false, int32_t>(job_a, job_b, s);
         if (st == TPK_OK)
         {
             const int64_t blocks = (tpk_ceil_div(n, 256) + tpk_ceil_div(m, 256)) * static_cast<int64_t>(b);
             hipLaunchKernelGGL(chamfer_bwd_lists_kernel<T>,
                                dim3(static_cast<unsigned>(tpk_min64(blocks, 1 << 24))), dim3(256), 0, s, n, m, b, xyz1,
-                               xyz2, idx1, idx2, grad_dist1, grad_dist2, offs_a, ents_a, offs_b,
-                               ents_b, grad_xyz1, grad_xyz2);
+                               xyz2, idx1, idx2, grad_dist1, grad_dist2, lists_a, lists_b,
+                               grad_xyz1, grad_xyz2);
             return tpk_launch_status();
         }
         if (st != TPK_ERR_UNSUPPORTED)
@@ -493,6 +527,6 @@ extern "C" size_t tpk_chamfer_bwd_workspace_bytes(int b, int n, int m)
 {
     if (b <= 0 || n <= 0 || m <= 0)
         return 0;
-    size_t a, bb, c, d;
-    return chamfer_lists_bytes(b, n, m, &a, &bb, &c, &d);
+    size_t second;
+    return chamfer_lists_bytes(b, n, m, &second);
 }

@@ -8,17 +8,7 @@
 
 namespace {
 
-// DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_ror:4, row_ror:8.  After the
-// four steps every lane of a 16-lane row holds the row's result.
-__device__ __forceinline__ int row_all_max_i32(int v)
-{
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true));
-    return v;
-}
-
+// Row and wavefront minima, built like row_all_max_i32 / wave_max_i32.
 __device__ __forceinline__ unsigned row_all_min_u32(unsigned v)
 {
     v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true)));
@@ -26,14 +16,6 @@ __device__ __forceinline__ unsigned row_all_min_u32(unsigned v)
     v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true)));
     v = min(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true)));
     return v;
-}
-
-__device__ __forceinline__ int wave_max_i32(int v)
-{
-    v = row_all_max_i32(v);
-    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
-    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
-    return max(max(a, b), max(c, d));
 }
 
 __device__ __forceinline__ int wave_min_i32(int v)

@@ -314,16 +314,6 @@ struct RoundWords
     int pad;
 };
 
-// Workgroup barrier that orders LDS traffic only (outstanding global stores of sample
-// indices need not complete before the next round).
-__device__ __forceinline__ void lds_barrier()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): also covers the LDS atomics issued below
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 // LDS atomics without return value, issued as written: one instruction for the active lanes
 // (the compiler would otherwise wrap a same-address atomic in a loop over those lanes).
 __device__ __forceinline__ unsigned lds_offset(const void* p)

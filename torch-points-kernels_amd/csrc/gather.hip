@@ -15,18 +15,18 @@
 // about 190 cycles whatever the address pattern, against 8 for a random LDS read), so the
 // scatter is turned into a gather: a first kernel inverts the index of each cloud into
 // per-target lists (for target position i the columns j that reference it, with their
-// weights) using LDS *integer* atomics, which are fast, and an LDS prefix sum; the main
-// kernel then stages R rows of grad_out in LDS (rows of n floats) and sums, for every
-// target, the listed columns - 16 lanes share one target, read 16 list entries at a time
-// (one contiguous 128-byte piece) and combine with a DPP row reduction.  No float atomics,
-// no zero fill, each output written once.  The lists cost 8 bytes (4 unweighted) per index
-// entry of workspace, passed in by the caller.  The order in which a target's terms are
-// added differs from run to run only through the order of its list, as with the
-// reference's global atomics (cuda/src/interpolate_gpu.cu:122-152): results agree to
-// rounding.
+// weights) using LDS *integer* atomics, which are fast, and an LDS prefix sum, laid out so that
+// one lane per target can walk them with coalesced reads (lists.h); the main kernel then
+// stages rows of grad_out in LDS - whole rows when up to 128 KiB of them fit, else one row in
+// pieces of 64 KiB with lists per piece - and every lane sums the listed columns of its
+// target.  No float atomics, no zero fill, each output written by one lane.  The lists cost
+// about 3 entries of 8 bytes (4 unweighted) per index entry of workspace, passed in by the
+// caller.  The order in which a target's terms are added differs from run to run only through
+// the order of its list, as with the reference's global atomics
+// (cuda/src/interpolate_gpu.cu:122-152): results agree to rounding.
 //
-// Rows too long for LDS, or a call without workspace, take a direct path: gathers from
-// global memory (forward), zero fill + global float atomics (backward).
+// Forward rows too long for LDS, or a backward call without workspace, take a direct path:
+// gathers from global memory (forward), zero fill + global float atomics (backward).
 //
 // Forward arithmetic follows cuda/src/interpolate_gpu.cu:78-107: ((p1*w1) + (p2*w2)) +
 // (p3*w3), every operation rounded on its own.  The grouping forward is a pure copy
@@ -68,52 +68,67 @@ struct Column
     }
 };
 
-// Cooperative copy of `count` floats from global memory into LDS by the whole workgroup.
-// Loads are issued in batches of eight per thread before any is written (one memory
-// latency per batch, not per element), 16 bytes per lane when both sides are 16-byte
-// aligned.
-__device__ __forceinline__ void stage_copy(float* dst, const float* __restrict__ src, unsigned count)
+// Cooperative copy of `rows` pieces of `count` floats each from global memory into LDS by T
+// threads (`tid` = 0..T-1); consecutive pieces lie src_stride / dst_stride floats apart.  The
+// pieces are treated as one run of elements: loads are issued in batches of BATCH per thread
+// before any is written (one memory latency per batch, not per element or per piece), 16 bytes
+// per lane when everything is 16-byte aligned.
+template <unsigned T, int BATCH>
+__device__ __forceinline__ void stage_rows_by(float* dst, unsigned dst_stride, const float* __restrict__ src,
+                                              int64_t src_stride, unsigned rows, unsigned count, unsigned tid)
 {
-    const unsigned tid = threadIdx.x;
-    constexpr unsigned T = G_THREADS;
-    const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0 &&
+                         ((src_stride | dst_stride | count) & 3) == 0;
     if (aligned)
     {
-        const unsigned n4 = count >> 2;
-        const float4* __restrict__ s4 = reinterpret_cast<const float4*>(src);
-        float4* d4 = reinterpret_cast<float4*>(dst);
-        unsigned t = tid;
-        for (; t + 7 * T < n4; t += 8 * T)
+        const unsigned per_row = count >> 2;
+        const unsigned total = per_row * rows;
+        for (unsigned base = tid; base < total; base += BATCH * T)
         {
-            float4 v[8];
+            float4 v[BATCH];
+            unsigned at[BATCH];
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                v[u] = s4[t + u * T];
+            for (int u = 0; u < BATCH; ++u)
+            {
+                // (every load is issued, out-of-range ones at the last element: no branches
+                // between the loads)
+                const unsigned i = min(base + u * T, total - 1u);
+                const unsigned r = rows > 1u ? i / per_row : 0u, col = i - r * per_row;
+                at[u] = base + u * T < total ? r * dst_stride + col * 4u : ~0u;
+                v[u] = *reinterpret_cast<const float4*>(src + r * src_stride + col * 4u);
+            }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                d4[t + u * T] = v[u];
+            for (int u = 0; u < BATCH; ++u)
+                if (at[u] != ~0u)
+                    *reinterpret_cast<float4*>(dst + at[u]) = v[u];
         }
-        for (; t < n4; t += T)
-            d4[t] = s4[t];
-        for (t = (n4 << 2) + tid; t < count; t += T)
-            dst[t] = src[t];
     }
     else
     {
-        unsigned t = tid;
-        for (; t + 7 * T < count; t += 8 * T)
+        const unsigned total = count * rows;
+        for (unsigned base = tid; base < total; base += BATCH * T)
         {
-            float v[8];
+            float v[BATCH];
+            unsigned at[BATCH];
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                v[u] = src[t + u * T];
+            for (int u = 0; u < BATCH; ++u)
+            {
+                const unsigned i = min(base + u * T, total - 1u);
+                const unsigned r = rows > 1u ? i / count : 0u, col = i - r * count;
+                at[u] = base + u * T < total ? r * dst_stride + col : ~0u;
+                v[u] = src[r * src_stride + col];
+            }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                dst[t + u * T] = v[u];
+            for (int u = 0; u < BATCH; ++u)
+                if (at[u] != ~0u)
+                    dst[at[u]] = v[u];
         }
-        for (; t < count; t += T)
-            dst[t] = src[t];
     }
+}
+
+__device__ __forceinline__ void stage_copy(float* dst, const float* __restrict__ src, unsigned count)
+{
+    stage_rows_by<G_THREADS, 8>(dst, count, src, count, 1u, count, threadIdx.x);
 }
 
 // grid: (clouds * row_blocks * jsplit).  dynamic LDS: R * m floats.
@@ -154,201 +169,140 @@ __global__ __launch_bounds__(G_THREADS) void gather_fwd_lds_kernel(
     }
 }
 
-// DPP helpers on 16-lane rows.
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v)
-{
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
-}
-template <int CTRL>
-__device__ __forceinline__ int dpp_i32(int v)
-{
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
-}
+constexpr int GB_BUFFER_FLOATS = 16384; // floats of grad_out a workgroup stages at a time (64 KiB)
+constexpr int GB_STEPS = L_WIDTH_STEP;  // list slots per request group (widths are multiples of it)
 
-// Transposing reduction over a 16-lane row: every lane brings 16 partial sums t[0..15]
-// (t[s] = its share of target s of the row); lane l leaves with the row-wide sum of target
-// l.  Four exchange steps with the lanes l^15, l^7, l^3, l^1 (DPP row_mirror,
-// row_half_mirror and two quad permutations); in each step a lane keeps the half of its
-// values whose target agrees with its own lane number in the bit being resolved and
-// receives the partner's partials of exactly those targets: 15 additions instead of the 64
-// that 16 separate row reductions take.
-__device__ __forceinline__ float row_transpose_sum(float (&t)[16], int l)
-{
-    const bool b3 = l & 8, b2 = l & 4, b1 = l & 2, b0 = l & 1;
-    float u[8];
-#pragma unroll
-    for (int s = 0; s < 8; ++s)
-    {
-        const float keepv = b3 ? t[s + 8] : t[s];
-        const float send = b3 ? t[s] : t[s + 8];
-        u[s] = keepv + dpp_f32<0x140>(send); // row_mirror: partner l ^ 15
-    }
-    float v[4];
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-    {
-        const float keepv = b2 ? u[s + 4] : u[s];
-        const float send = b2 ? u[s] : u[s + 4];
-        v[s] = keepv + dpp_f32<0x141>(send); // row_half_mirror: partner l ^ 7
-    }
-    float w[2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-    {
-        const float keepv = b1 ? v[s + 2] : v[s];
-        const float send = b1 ? v[s] : v[s + 2];
-        w[s] = keepv + dpp_f32<0x1B>(send); // quad_perm [3,2,1,0]: partner l ^ 3
-    }
-    const float keepv = b0 ? w[1] : w[0];
-    const float send = b0 ? w[0] : w[1];
-    return keepv + dpp_f32<0xB1>(send); // quad_perm [1,0,3,2]: partner l ^ 1
-}
-
-// Value of lane S of the caller's 16-lane row (DPP row_newbcast).
-template <int S>
-__device__ __forceinline__ int row_broadcast(int v)
-{
-    return dpp_i32<0x150 + S>(v);
-}
-
-template <int K, bool WEIGHTED, int R, int S>
-struct ListRound
-{
-    // Loads entry (round*16 + l) of target S of the row for every S (recursively unrolled,
-    // so that the 16 loads are independent and issued together).
-    __device__ __forceinline__ static void load(const ListEntry<WEIGHTED>* __restrict__ entries,
-                                                int my_beg, int my_end, int first, int l,
-                                                ListEntry<WEIGHTED> (&e)[16], bool (&ok)[16])
-    {
-        const int beg = row_broadcast<S>(my_beg);
-        const int end = row_broadcast<S>(my_end);
-        const unsigned p = static_cast<unsigned>(beg + first + l);
-        ok[S] = static_cast<int>(p) < end;
-        e[S] = entries[ok[S] ? p : 0u];
-        if constexpr (S + 1 < 16)
-            ListRound<K, WEIGHTED, R, S + 1>::load(entries, my_beg, my_end, first, l, e, ok);
-    }
-};
-
-// grid: (clouds * row_blocks).  dynamic LDS: R rows of grad_out, n floats each.
-// A wavefront takes 64 consecutive targets at a time.  Lane L first fetches the list bounds
-// of target base+L (one coalesced read).  Then each of the wavefront's four 16-lane rows
-// serves its 16 targets: for target s of the row, lane l reads list entry l (a contiguous
-// 128-byte piece per row; the reads of the 16 targets are independent and issued
-// together) and multiplies the staged grad_out value; the transposing row reduction above
-// leaves the sum of target l in lane l, so the 64 results leave as one contiguous store per
-// feature row.  Lists longer than 16 take further rounds.
+// grid: (clouds * row_groups).  A workgroup takes R feature rows of one cloud and goes through
+// the parts of `part_len` columns (the lists are built per part, lists.h): it stages the piece
+// of grad_out in LDS, then every wavefront takes the lists of 64 consecutive targets at a time,
+// one target per lane: in step i the lanes read slot i of their lists - consecutive entries -
+// and the staged values these refer to; padding entries refer to a staged zero (slot part_len
+// of every row).  The few lists longer than the block's padded part are then summed by the
+// whole wavefront, 64 entries at a time.  Results leave as one contiguous store per feature
+// row; parts after the first add to what the same lane stored for the part before.
+// Two workgroups share a compute unit (64 KiB of LDS and 64 registers each): one stages while
+// the other walks its lists, and 32 wavefronts hide the latency of the entry reads.
+// dynamic LDS: R * (part_len + 4) floats.
 template <int K, bool WEIGHTED, int R>
-__global__ __launch_bounds__(G_THREADS) void gather_bwd_lists_kernel(
-    int c, int m, int64_t n, int row_blocks, const float* __restrict__ grad_out,
-    const int* __restrict__ offsets, const ListEntry<WEIGHTED>* __restrict__ entries,
-    float* __restrict__ grad_src)
+__global__ __launch_bounds__(G_THREADS, 2) void gather_bwd_lists_kernel(
+    int c, int m, int64_t n, int parts, int part_len, int row_groups, const float* __restrict__ grad_out,
+    Lists<WEIGHTED> lists, float* __restrict__ grad_src)
 {
     extern __shared__ float rows[];
-    const int bid = blockIdx.x;
-    const int rb = bid % row_blocks;
-    const int cloud = bid / row_blocks;
-    const int c0 = rb * R;
-    const int nrows = min(R, c - c0);
-    const unsigned ni = static_cast<unsigned>(n);
-
+    const unsigned stride = static_cast<unsigned>(part_len) + 4u;
     const int lane = threadIdx.x & (TPK_WAVE - 1);
-    const int wave = threadIdx.x / TPK_WAVE;
-    const int l = lane & 15;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE); // (a scalar for the compiler)
     constexpr int WAVES = G_THREADS / TPK_WAVE;
+    constexpr int STEPS = WEIGHTED ? GB_STEPS : 2 * GB_STEPS; // list slots requested per block at a time
+    const int nblocks = (m + L_BLOCK - 1) / L_BLOCK;
 
-    offsets += static_cast<int64_t>(cloud) * (m + 1);
-    entries += static_cast<int64_t>(cloud) * n * K;
+    // consecutive workgroups of a die work on consecutive row groups: one cloud's lists per L2
+    const int group = static_cast<int>(xcd_local_block(blockIdx.x, gridDim.x));
+    const int cloud = group / row_groups;
+    const int c0 = (group % row_groups) * R;
+    const int nrows = min(R, c - c0);
     float* __restrict__ d = grad_src + (static_cast<int64_t>(cloud) * c + c0) * m;
 
-    // list bounds of the first block of targets: requested before the rows are staged
-    int base = wave * TPK_WAVE;
-    int my_beg = 0, my_end = 0;
-    if (base + lane < m)
-    {
-        my_beg = offsets[base + lane];
-        my_end = offsets[base + lane + 1];
-    }
+    for (unsigned t = threadIdx.x; t < R * 4u; t += G_THREADS)
+        rows[(t >> 2) * stride + static_cast<unsigned>(part_len) + (t & 3u)] = 0.f;
 
-    // Staged rows have a stride of a little more than n floats: slot n of every row holds 0
-    // and is what lanes without a list entry read, so that no read in the loop below is
-    // conditional.  Rows beyond the last feature row are all zeros.
-    const unsigned stride = (ni + 4u) & ~3u;
-    const float* __restrict__ g = grad_out + (static_cast<int64_t>(cloud) * c + c0) * n;
-    for (int r = 0; r < R; ++r)
+    for (int part = 0; part < parts; ++part)
     {
-        if (r < nrows)
-        {
-            stage_copy(rows + r * stride, g + static_cast<int64_t>(r) * n, ni);
-            for (unsigned t = ni + threadIdx.x; t < stride; t += G_THREADS)
-                rows[r * stride + t] = 0.f;
-        }
-        else
-        {
-            for (unsigned t = threadIdx.x; t < stride; t += G_THREADS)
-                rows[r * stride + t] = 0.f;
-        }
-    }
-    __syncthreads();
+        const int64_t col0 = static_cast<int64_t>(part) * part_len;
+        const unsigned len = static_cast<unsigned>(tpk_min64(part_len, n - col0));
+        if (part > 0)
+            __syncthreads(); // everybody is done with the piece before
+        stage_rows_by<G_THREADS, 4>(rows, stride, grad_out + (static_cast<int64_t>(cloud) * c + c0) * n + col0, n,
+                                    static_cast<unsigned>(nrows), len, threadIdx.x);
+        __syncthreads();
 
-    for (; base < m; base += WAVES * TPK_WAVE)
-    {
-        const int tgt = base + lane;
-        // bounds of the next block, in flight while this one is processed
-        const int next = tgt + WAVES * TPK_WAVE;
-        int next_beg = 0, next_end = 0;
-        if (next < m)
-        {
-            next_beg = offsets[next];
-            next_end = offsets[next + 1];
-        }
-
-        float keep[R];
+        const int64_t cloud_part = static_cast<int64_t>(cloud) * parts + part;
+        const int* __restrict__ counts = lists.counts + cloud_part * nblocks * L_BLOCK;
+        const int2* __restrict__ blocks = lists.blocks + cloud_part * nblocks;
+        const ListEntry<WEIGHTED>* __restrict__ entries = lists.entries + cloud_part * lists.capacity;
+        auto add_entry = [&](const ListEntry<WEIGHTED>& e, float (&sum)[R]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-            keep[r] = 0.f;
-
-        const int longest = my_end - my_beg;
-        for (int first = 0; __any(longest > first); first += 16)
-        {
-            ListEntry<WEIGHTED> e[16];
-            bool ok[16];
-            ListRound<K, WEIGHTED, R, 0>::load(entries, my_beg, my_end, first, l, e, ok);
-            unsigned col[16];
-            float wv[16];
-#pragma unroll
-            for (int s = 0; s < 16; ++s)
+            for (int r = 0; r < R; ++r)
             {
-                col[s] = ok[s] ? static_cast<unsigned>(e[s].j) : ni; // ni = the zero slot
+                const float v = rows[static_cast<unsigned>(r) * stride + static_cast<unsigned>(e.j)];
                 if constexpr (WEIGHTED)
-                    wv[s] = ok[s] ? e[s].w : 0.f;
+                    sum[r] += v * e.w;
+                else
+                    sum[r] += v;
             }
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-            {
-                float t[16];
-#pragma unroll
-                for (int s = 0; s < 16; ++s)
-                {
-                    const float v = rows[static_cast<unsigned>(r) * stride + col[s]];
-                    if constexpr (WEIGHTED)
-                        t[s] = v * wv[s];
-                    else
-                        t[s] = v;
-                }
-                keep[r] += row_transpose_sum(t, l);
-            }
-        }
-        if (tgt < m)
+        };
+
+        ListBlock lb = list_block(blocks, min(wave, nblocks - 1));
+        for (int blk = wave; blk < nblocks; blk += WAVES)
         {
+            // (the next block's description is requested before this block's work starts)
+            const ListBlock next_lb = list_block(blocks, min(blk + WAVES, nblocks - 1));
+            const ListEntry<WEIGHTED>* __restrict__ e = entries + lb.start + lane;
+            const int tgt = blk * L_BLOCK + lane;
+            float acc[R];
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                if (r < nrows)
-                    d[static_cast<int64_t>(r) * m + tgt] = keep[r];
+                acc[r] = 0.f;
+            for (int i = 0; i < lb.width; i += STEPS)
+            {
+                // all requests of this round, then all the sums (widths are multiples of
+                // GB_STEPS: a round is one or two whole groups of that many slots)
+                ListEntry<WEIGHTED> ent[STEPS];
+#pragma unroll
+                for (int h = 0; h < STEPS; h += GB_STEPS)
+                    if (i + h < lb.width)
+                    {
+#pragma unroll
+                        for (int u = h; u < h + GB_STEPS; ++u)
+                            ent[u] = e[(i + u) * L_BLOCK];
+                    }
+#pragma unroll
+                for (int h = 0; h < STEPS; h += GB_STEPS)
+                    if (i + h < lb.width)
+                    {
+#pragma unroll
+                        for (int u = h; u < h + GB_STEPS; ++u)
+                            add_entry(ent[u], acc);
+                    }
+            }
+            if (lb.longer)
+            {
+                int extra, extra_at;
+                list_extra(counts[tgt], lb.width, extra, extra_at);
+                const ListEntry<WEIGHTED>* __restrict__ rest = entries + lb.start + lb.width * L_BLOCK;
+                for (unsigned long long todo = __ballot(extra > 0); todo; todo &= todo - 1)
+                {
+                    const int owner = __builtin_ctzll(todo);
+                    const int count = __builtin_amdgcn_readlane(extra, owner);
+                    const int at = __builtin_amdgcn_readlane(extra_at, owner);
+                    float rest_sum[R];
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        rest_sum[r] = 0.f;
+                    for (int p = lane; p < count; p += TPK_WAVE)
+                        add_entry(rest[at + p], rest_sum);
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                    {
+                        const float total = wave_sum_f32(rest_sum[r]);
+                        if (lane == owner)
+                            acc[r] += total;
+                    }
+                }
+            }
+            // (an empty block has nothing to add after the first part)
+            if (tgt < m && (part == 0 || lb.width > 0 || lb.longer))
+            {
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    if (r < nrows)
+                    {
+                        float* const out = d + static_cast<int64_t>(r) * m + tgt;
+                        *out = part == 0 ? acc[r] : *out + acc[r];
+                    }
+            }
+            lb = next_lb;
         }
-        my_beg = next_beg;
-        my_end = next_end;
     }
 }
 
@@ -461,32 +415,52 @@ int gather_fwd(int b, int c, int m, int64_t n, const float* src, const IdxT* idx
     return tpk_launch_status();
 }
 
-// Workspace of the list-based backward: offsets (b, m+1) ints, then the list entries.
+// Rows of grad_out staged together and columns per part, for rows of n floats.
+struct BwdShape
+{
+    int rows;
+    int part_len;
+    int parts;
+};
+BwdShape bwd_shape(int64_t n)
+{
+    BwdShape sh;
+    // Whole rows while up to 128 KiB of them fit (lists over whole rows have the least padding);
+    // longer rows go one at a time in pieces of 64 KiB, two workgroups to a compute unit.
+    sh.rows = n <= GB_BUFFER_FLOATS / 2 ? 4 : n <= GB_BUFFER_FLOATS ? 2 : 1;
+    const int64_t n4 = (n + 3) & ~static_cast<int64_t>(3);
+    sh.part_len = static_cast<int>(tpk_min64(n4, GB_BUFFER_FLOATS));
+    sh.parts = static_cast<int>(tpk_min64(tpk_ceil_div(n, sh.part_len), 0x7fffffff));
+    return sh;
+}
+
+// Workspace of the list-based backward: the lists of every (cloud, part) (lists.h).
 template <int K, bool WEIGHTED>
 size_t lists_workspace_bytes(int b, int m, int64_t n)
 {
     if (b <= 0 || m <= 0 || n <= 0)
         return 0;
-    const size_t off = (static_cast<size_t>(b) * (static_cast<size_t>(m) + 1) * sizeof(int) + 255) &
-                       ~static_cast<size_t>(255);
-    return off + static_cast<size_t>(b) * static_cast<size_t>(n) * K * sizeof(ListEntry<WEIGHTED>);
+    const BwdShape sh = bwd_shape(n);
+    if (static_cast<int64_t>(b) * sh.parts > 0x7fffffffLL)
+        return 0;
+    return lists_bytes<WEIGHTED>(b * sh.parts, m, static_cast<int64_t>(sh.part_len) * K);
 }
 
 template <int K, bool WEIGHTED, int R>
-int launch_bwd_lists(int b, int c, int m, int64_t n, const float* grad_out, const int* offsets,
-                     const ListEntry<WEIGHTED>* entries, float* grad_src, hipStream_t s)
+int launch_bwd_lists(int b, int c, int m, int64_t n, const BwdShape& sh, const float* grad_out,
+                     const Lists<WEIGHTED>& lists, float* grad_src, hipStream_t s)
 {
-    const int row_blocks = static_cast<int>(tpk_ceil_div(c, R));
-    const int64_t blocks = static_cast<int64_t>(b) * row_blocks;
-    if (blocks > 0x7fffffffLL)
+    const int row_groups = static_cast<int>(tpk_ceil_div(c, R));
+    const int64_t groups_total = static_cast<int64_t>(b) * row_groups;
+    if (groups_total > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    const size_t lds = static_cast<size_t>(R) * ((n + 4) & ~static_cast<int64_t>(3)) * sizeof(float);
+    const size_t lds = static_cast<size_t>(R) * (sh.part_len + 4) * sizeof(float);
     auto kernel = gather_bwd_lists_kernel<K, WEIGHTED, R>;
     int st = allow_lds(kernel, lds);
     if (st != TPK_OK)
         return st;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(G_THREADS), lds, s, c, m, n,
-                       row_blocks, grad_out, offsets, entries, grad_src);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups_total)), dim3(G_THREADS), lds, s, c, m, n,
+                       sh.parts, sh.part_len, row_groups, grad_out, lists, grad_src);
     return tpk_launch_status();
 }
 
@@ -501,27 +475,26 @@ int gather_bwd(int b, int c, int m, int64_t n, const float* grad_out, const IdxT
         return TPK_OK;
     if (!grad_src || (n > 0 && (!grad_out || !idx || (WEIGHTED && !weight))))
         return TPK_ERR_INVALID_ARG;
-    // The list path needs: a row of grad_out (n floats) in LDS, the counters of one cloud
-    // (m ints) in LDS, entry positions that fit an int, and the workspace.
-    const int64_t row_bytes = n * static_cast<int64_t>(sizeof(float));
-    const bool fits = n > 0 && row_bytes <= G_LDS_BUDGET &&
-                      m <= 16 * static_cast<int64_t>(L_MAX_TARGETS) && n * K <= 0x7fffffffLL;
+    // The list path needs entry positions that fit an int, and the workspace.
+    const BwdShape sh = bwd_shape(n > 0 ? n : 1);
+    const bool fits = n > 0 && n * K <= 0x7fffffffLL &&
+                      static_cast<int64_t>(b) * sh.parts <= 0x7fffffffLL;
     const size_t need = lists_workspace_bytes<K, WEIGHTED>(b, m, n);
-    if (fits && workspace && workspace_bytes >= need)
+    if (fits && workspace && need > 0 && workspace_bytes >= need)
     {
-        int* offsets = static_cast<int*>(workspace);
-        const size_t off = (static_cast<size_t>(b) * (static_cast<size_t>(m) + 1) * sizeof(int) + 255) &
-                           ~static_cast<size_t>(255);
-        auto* entries = reinterpret_cast<ListEntry<WEIGHTED>*>(static_cast<char*>(workspace) + off);
-        int st = launch_build_lists<K, WEIGHTED, IdxT>(b, m, n * K, idx, weight, offsets, entries, s);
-        if (st != TPK_OK)
+        const int64_t part_total = static_cast<int64_t>(sh.part_len) * K;
+        const Lists<WEIGHTED> lists = lists_at<WEIGHTED>(workspace, b * sh.parts, m, part_total);
+        int st = launch_build_lists<K, WEIGHTED, IdxT>(b, m, n * K, part_total, sh.part_len, idx, weight, lists, s);
+        if (st == TPK_OK)
+        {
+            if (sh.rows == 4)
+                return launch_bwd_lists<K, WEIGHTED, 4>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+            if (sh.rows == 2)
+                return launch_bwd_lists<K, WEIGHTED, 2>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+            return launch_bwd_lists<K, WEIGHTED, 1>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+        }
+        if (st != TPK_ERR_UNSUPPORTED)
             return st;
-        const int r = static_cast<int>(G_LDS_BUDGET / row_bytes);
-        if (r >= 4 && c >= 4)
-            return launch_bwd_lists<K, WEIGHTED, 4>(b, c, m, n, grad_out, offsets, entries, grad_src, s);
-        if (r >= 2 && c >= 2)
-            return launch_bwd_lists<K, WEIGHTED, 2>(b, c, m, n, grad_out, offsets, entries, grad_src, s);
-        return launch_bwd_lists<K, WEIGHTED, 1>(b, c, m, n, grad_out, offsets, entries, grad_src, s);
     }
     const int64_t count = static_cast<int64_t>(b) * c * m;
     hipLaunchKernelGGL(fill_zero_f32_kernel,

@@ -33,41 +33,160 @@ struct ListEntry<false>
     int j;
 };
 
-constexpr int L_MAX_TARGETS = 30720; // target positions whose counters fit in LDS (120 KiB)
+constexpr int L_MAX_TARGETS = 15360; // targets whose bookkeeping fits in LDS (2 ints each)
+constexpr int L_BLOCK = TPK_WAVE;    // targets per block of lists: one per lane
+constexpr int L_SLACK = 576;         // entry slots a block owns beyond three per entry
+constexpr int L_WIDTH_STEP = 4;      // widths of the padded parts are multiples of this
 
-// Inverts the index of one cloud.  grid: (clouds * splits); a workgroup builds the lists of
-// the targets [split * span, (split + 1) * span) of its cloud: it reads every index entry of
-// the cloud, counts those inside its span (LDS integer atomics) and those below it (their
-// number is where its lists start), prefix-sums the counts and fills the lists in a second
-// pass.  Workgroups never wait for each other.  dynamic LDS: (span + 1 + G_THREADS) ints.
-//   offsets[cloud][0..m]  start of each target's list (exclusive prefix sum of the counts)
-//   entries[cloud][...]   the lists, back to back
-// Index values outside [0, m) are dropped.
-template <int K, bool WEIGHTED, typename IdxT>
-__global__ __launch_bounds__(G_THREADS) void build_lists_kernel(
-    int m, int total, int splits, int span, const IdxT* __restrict__ idx,
-    const float* __restrict__ weight, int* __restrict__ offsets,
-    ListEntry<WEIGHTED>* __restrict__ entries)
+// Layout of the lists of one cloud ("sliced": made to be walked by one lane per target).
+// Targets are taken in blocks of 64; `counts` holds the length of every target's list (0 in the
+// unused positions of the last block).  Block b owns the entry slots from
+//   start_b = 3 * (entries of all earlier targets) + L_SLACK * b
+// and stores slot i of its target L at start_b + i * 64 + L for i < width_b, so that the 64
+// lanes read consecutive entries in every step.  width_b = min(longest list of the block,
+// 2 * ceil(entries of the block / 64) + 4), rounded up to a multiple of 4; shorter lists are
+// padded with (pad_j, 0) entries.  The entries of a list beyond width_b follow the padded part,
+// list after list in target order.  Padded part <= 2 * entries + 574 slots, the rest <= entries:
+// a block never leaves its own slots, whatever the index looks like.
+//   counts[cloud][64 * blocks]
+//   blocks[cloud][b]         (start_b, width_b; bit 31 of the width: some list is longer)
+//   entries[cloud][capacity]
+template <bool WEIGHTED>
+struct Lists
 {
-    extern __shared__ int counters[];
-    int* scan = counters + span + 1;
+    int* counts;
+    int2* blocks;
+    ListEntry<WEIGHTED>* entries;
+    int64_t capacity; // entry slots per cloud
+};
+
+inline int64_t list_blocks(int m)
+{
+    return (static_cast<int64_t>(m) + L_BLOCK - 1) / L_BLOCK;
+}
+inline int64_t list_capacity(int m, int64_t total)
+{
+    return 3 * total + L_SLACK * list_blocks(m);
+}
+inline size_t list_align(size_t v)
+{
+    return (v + 255) & ~static_cast<size_t>(255);
+}
+// Workspace bytes of the lists of `clouds` clouds with m targets and `total` index entries each.
+template <bool WEIGHTED>
+size_t lists_bytes(int clouds, int m, int64_t total)
+{
+    const size_t c = static_cast<size_t>(clouds);
+    const size_t positions = static_cast<size_t>(list_blocks(m)) * L_BLOCK;
+    return list_align(c * positions * sizeof(int)) +
+           list_align(c * static_cast<size_t>(list_blocks(m)) * sizeof(int2)) +
+           list_align(c * static_cast<size_t>(list_capacity(m, total)) * sizeof(ListEntry<WEIGHTED>));
+}
+template <bool WEIGHTED>
+Lists<WEIGHTED> lists_at(void* workspace, int clouds, int m, int64_t total)
+{
+    const size_t c = static_cast<size_t>(clouds);
+    const size_t positions = static_cast<size_t>(list_blocks(m)) * L_BLOCK;
+    char* p = static_cast<char*>(workspace);
+    Lists<WEIGHTED> l;
+    l.counts = reinterpret_cast<int*>(p);
+    p += list_align(c * positions * sizeof(int));
+    l.blocks = reinterpret_cast<int2*>(p);
+    p += list_align(c * static_cast<size_t>(list_blocks(m)) * sizeof(int2));
+    l.entries = reinterpret_cast<ListEntry<WEIGHTED>*>(p);
+    l.capacity = list_capacity(m, total);
+    return l;
+}
+
+// What a wavefront needs to walk the lists of block `block` of a cloud, lane L serving the
+// target block * 64 + L: start and width of the padded part, and whether longer
+// lists exist.
+struct ListBlock
+{
+    int start;
+    int width;
+    bool longer;
+};
+__device__ __forceinline__ ListBlock list_block(const int2* __restrict__ cloud_blocks, int block)
+{
+    const int2 d = cloud_blocks[__builtin_amdgcn_readfirstlane(block)];
+    return ListBlock{d.x, d.y & 0x7fffffff, d.y < 0};
+}
+// For a block with longer lists: how many entries of this lane's target lie beyond the padded
+// part (`extra`), and where they start relative to the end of the padded part (`extra_at`).
+// Every lane of the wavefront calls it; `count` is the length of the lane's list (0 for
+// lanes beyond the last target).
+__device__ __forceinline__ void list_extra(int count, int width, int& extra, int& extra_at)
+{
+    extra = max(count - width, 0);
+    extra_at = wave_exclusive_sum(extra);
+}
+
+// Inverts the index of one part of one cloud: the cloud's `cloud_total` index entries are cut
+// into `parts` runs of `part_total` (a multiple of K; the last may be shorter), and every
+// (cloud, part) gets lists of its own, stored as cloud number cloud * parts + part; the columns
+// in its entries count from the first column of the part.  grid: (clouds * parts * splits); a
+// workgroup builds the lists of the targets [split * span, (split + 1) * span) (span is a
+// multiple of 64): it reads every index entry of its part, counts those inside its span (LDS
+// integer atomics) and those below it (their number fixes where its blocks start), prefix-sums
+// the lengths, lays out its blocks and fills the lists in a second pass.  Workgroups never wait
+// for each other.  dynamic LDS: (2 * span + span / 32 + G_THREADS) ints.  Index values outside [0, m) are dropped.
+// One launch can carry two such jobs (the two directions of the Chamfer backward): the first
+// `workgroups` workgroups serve the first job, the rest the second.
+template <bool WEIGHTED, typename IdxT>
+struct ListJob
+{
+    int m, cloud_total, parts, part_total, splits, span, pad_j, workgroups;
+    const IdxT* idx;
+    const float* weight;
+    Lists<WEIGHTED> lists;
+};
+
+template <int K, bool WEIGHTED, typename IdxT>
+__global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED, IdxT> first_job,
+                                                                ListJob<WEIGHTED, IdxT> second_job)
+{
+    const bool second = static_cast<int>(blockIdx.x) >= first_job.workgroups;
+    const ListJob<WEIGHTED, IdxT>& job = second ? second_job : first_job;
+    const int workgroup = second ? blockIdx.x - first_job.workgroups : blockIdx.x;
+    const int m = job.m, cloud_total = job.cloud_total, parts = job.parts, part_total = job.part_total;
+    const int splits = job.splits, span = job.span, pad_j = job.pad_j;
+    const IdxT* __restrict__ idx = job.idx;
+    const float* __restrict__ weight = job.weight;
+    const Lists<WEIGHTED>& lists = job.lists;
+
+    extern __shared__ int counters[];            // [span] list lengths, later fill cursors
+    int* const aux = counters + span;            // [span] list starts, later starts of the long parts
+    int* const block_start = aux + span;         // [span / 64]
+    int* const block_width = block_start + span / L_BLOCK;
+    int* const scan = block_width + span / L_BLOCK; // [G_THREADS]
+    __shared__ int below_total;
     const int tid = threadIdx.x;
-    const int cloud = blockIdx.x / splits;
-    const int split = blockIdx.x - cloud * splits;
+    const int lane = tid & (TPK_WAVE - 1);
+    const int wave = tid / TPK_WAVE;
+    const int cloud_part = workgroup / splits;
+    const int split = workgroup - cloud_part * splits;
+    const int part = cloud_part % parts;
+    const int total = min(part_total, cloud_total - part * part_total);
     const int i0 = split * span;
     const int i1 = min(i0 + span, m);
     const int width = i1 - i0;
-    idx += static_cast<int64_t>(cloud) * total;
+    const int64_t first_entry = static_cast<int64_t>(cloud_part / parts) * cloud_total + static_cast<int64_t>(part) * part_total;
+    idx += first_entry;
     if (WEIGHTED)
-        weight += static_cast<int64_t>(cloud) * total;
-    offsets += static_cast<int64_t>(cloud) * (m + 1);
-    entries += static_cast<int64_t>(cloud) * total;
+        weight += first_entry;
+    const int64_t cloud_blocks = (m + L_BLOCK - 1) / L_BLOCK;
+    int* __restrict__ counts = lists.counts + cloud_part * cloud_blocks * L_BLOCK;
+    int2* __restrict__ blocks = lists.blocks + cloud_part * cloud_blocks;
+    ListEntry<WEIGHTED>* __restrict__ entries = lists.entries + static_cast<int64_t>(cloud_part) * lists.capacity;
 
-    for (int t = tid; t < width; t += G_THREADS)
+    for (int t = tid; t < span; t += G_THREADS)
         counters[t] = 0;
+    if (tid == 0)
+        below_total = 0;
     __syncthreads();
     int below = 0; // valid entries whose target lies before this span
-    constexpr int BATCH = 8; // index loads in flight per thread
+    constexpr int BATCH = 16; // index loads in flight per thread
     for (int e0 = tid; e0 < total; e0 += BATCH * G_THREADS)
     {
         int64_t iv[BATCH];
@@ -88,19 +207,16 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(
     }
     __syncthreads();
 
-    // prefix sums over the threads: of `below` (gives the start of the span's lists) and of
-    // the counters (every thread owns a run of `per` consecutive counters)
+    // Prefix sum of the list lengths (every thread owns a run of `per` consecutive targets):
+    // where the entries of every target would start.
+    atomicAdd(&below_total, below);
     const int per = (width + G_THREADS - 1) / G_THREADS;
     const int lo = min(tid * per, width), hi = min(lo + per, width);
     int sum = 0;
     for (int t = lo; t < hi; ++t)
         sum += counters[t];
-    __shared__ int below_total;
-    if (tid == 0)
-        below_total = 0;
     scan[tid] = sum;
     __syncthreads();
-    atomicAdd(&below_total, below);
     for (int step = 1; step < G_THREADS; step <<= 1)
     {
         const int add = tid >= step ? scan[tid - step] : 0;
@@ -111,13 +227,47 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(
     int run = below_total + scan[tid] - sum;
     for (int t = lo; t < hi; ++t)
     {
-        const int c = counters[t];
-        counters[t] = run; // becomes the fill cursor of target i0 + t
-        offsets[i0 + t] = run;
-        run += c;
+        aux[t] = run;
+        run += counters[t];
     }
-    if (split == splits - 1 && tid == G_THREADS - 1)
-        offsets[m] = below_total + scan[tid];
+    __syncthreads();
+
+    // Layout of the blocks, one wavefront per block at a time; the padding entries are written
+    // here, the real ones in the second pass.
+    ListEntry<WEIGHTED> pad;
+    pad.j = pad_j;
+    if constexpr (WEIGHTED)
+        pad.w = 0.f;
+    const int nblocks = (width + L_BLOCK - 1) / L_BLOCK;
+    for (int blk = wave; blk < nblocks; blk += G_THREADS / TPK_WAVE)
+    {
+        const int t = blk * L_BLOCK + lane;
+        const int count = t < width ? counters[t] : 0;
+        const int first = aux[blk * L_BLOCK];
+        const int before = wave_exclusive_sum(count);
+        const int block_entries = __builtin_amdgcn_readlane(before + count, TPK_WAVE - 1);
+        const int longest = wave_max_i32(count);
+        const int w = (min(longest, 2 * ((block_entries + L_BLOCK - 1) / L_BLOCK) + 4) + L_WIDTH_STEP - 1) &
+                      ~(L_WIDTH_STEP - 1);
+        const int start = 3 * first + L_SLACK * (i0 / L_BLOCK + blk);
+        int extra, extra_at;
+        list_extra(count, w, extra, extra_at);
+        if (t < width)
+        {
+            aux[t] = extra_at;
+            counters[t] = 0;
+        }
+        counts[i0 + t] = count;
+        if (lane == 0)
+        {
+            block_start[blk] = start;
+            block_width[blk] = w;
+            blocks[i0 / L_BLOCK + blk] = make_int2(start, longest > w ? w | static_cast<int>(0x80000000u) : w);
+        }
+        for (int i = 0; i < w; ++i)
+            if (i >= count)
+                entries[start + i * L_BLOCK + lane] = pad;
+    }
     __syncthreads();
 
     // Second pass: all loads of a batch are issued unconditionally (clamped index) before
@@ -140,46 +290,87 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(
             const bool mine = iv[u] >= i0 && iv[u] < i1 && e0 + u * G_THREADS < total;
             if (mine)
             {
-                const int pos = atomicAdd(&counters[static_cast<int>(iv[u]) - i0], 1);
+                const int t = static_cast<int>(iv[u]) - i0;
+                const int slot = atomicAdd(&counters[t], 1);
+                const int blk = t / L_BLOCK;
+                const int w = block_width[blk];
+                const int at = block_start[blk] +
+                               (slot < w ? slot * L_BLOCK + (t & (L_BLOCK - 1)) : w * L_BLOCK + aux[t] + (slot - w));
                 ListEntry<WEIGHTED> entry;
                 entry.j = (e0 + u * G_THREADS) / K;
                 if constexpr (WEIGHTED)
                     entry.w = wv[u];
-                entries[pos] = entry;
+                entries[at] = entry;
             }
         }
     }
 }
 
-
-// Launches build_lists_kernel for `clouds` clouds of `m` targets and `total` index entries
-// each.  Returns TPK_ERR_UNSUPPORTED when a span of targets would not fit in LDS.
+// Describes the job of building the lists of `clouds` clouds of `m` targets and `cloud_total`
+// index entries each, in parts of `part_total` entries (`lists` sized for clouds * parts clouds
+// of part_total entries); padding entries refer to column `pad_j`.  Returns TPK_ERR_UNSUPPORTED
+// when a span of targets would not fit in LDS or entry positions would not fit an int.
 template <int K, bool WEIGHTED, typename IdxT>
-int launch_build_lists(int clouds, int m, int64_t total, const IdxT* idx, const float* weight,
-                       int* offsets, ListEntry<WEIGHTED>* entries, hipStream_t s)
+int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, int pad_j, const IdxT* idx,
+                  const float* weight, const Lists<WEIGHTED>& lists, ListJob<WEIGHTED, IdxT>* job)
 {
-    if (clouds <= 0 || m <= 0 || total <= 0)
-        return TPK_OK;
-    if (total > 0x7fffffffLL)
+    *job = ListJob<WEIGHTED, IdxT>{};
+    if (clouds <= 0 || m <= 0 || cloud_total <= 0)
+        return TPK_OK; // nothing to build: no workgroups
+    if (part_total <= 0 || part_total % K != 0)
+        return TPK_ERR_INVALID_ARG;
+    const int64_t parts = tpk_ceil_div(cloud_total, part_total);
+    if (list_capacity(m, part_total) > 0x7fffffffLL || cloud_total > 0x7fffffffLL ||
+        clouds * parts > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     // Enough workgroups to occupy a good part of the chip; spans of a multiple of 64 targets.
-    int splits = static_cast<int>(tpk_ceil_div(128, clouds));
+    int splits = static_cast<int>(tpk_ceil_div(128, clouds * parts));
     if (splits > 16)
         splits = 16;
     if (splits < tpk_ceil_div(m, L_MAX_TARGETS))
         splits = static_cast<int>(tpk_ceil_div(m, L_MAX_TARGETS));
-    const int span = static_cast<int>(tpk_ceil_div(tpk_ceil_div(m, splits), 64) * 64);
+    const int span = static_cast<int>(tpk_ceil_div(tpk_ceil_div(m, splits), L_BLOCK) * L_BLOCK);
     splits = static_cast<int>(tpk_ceil_div(m, span));
-    if (span > L_MAX_TARGETS || static_cast<int64_t>(clouds) * splits > 0x7fffffffLL)
+    if (span > L_MAX_TARGETS || clouds * parts * splits > 0x3fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    const size_t lds = (static_cast<size_t>(span) + 1 + G_THREADS) * sizeof(int);
+    job->m = m;
+    job->cloud_total = static_cast<int>(cloud_total);
+    job->parts = static_cast<int>(parts);
+    job->part_total = static_cast<int>(part_total);
+    job->splits = splits;
+    job->span = span;
+    job->pad_j = pad_j;
+    job->workgroups = static_cast<int>(clouds * parts * splits);
+    job->idx = idx;
+    job->weight = weight;
+    job->lists = lists;
+    return TPK_OK;
+}
+
+// Launches build_lists_kernel for one or two jobs.
+template <int K, bool WEIGHTED, typename IdxT>
+int launch_list_jobs(const ListJob<WEIGHTED, IdxT>& first, const ListJob<WEIGHTED, IdxT>& second, hipStream_t s)
+{
+    const int workgroups = first.workgroups + second.workgroups;
+    if (workgroups == 0)
+        return TPK_OK;
+    const int span = first.span > second.span ? first.span : second.span;
+    const size_t lds = (2 * static_cast<size_t>(span) + 2 * (span / L_BLOCK) + G_THREADS) * sizeof(int);
     auto build = build_lists_kernel<K, WEIGHTED, IdxT>;
     int st = allow_lds(build, lds);
     if (st != TPK_OK)
         return st;
-    hipLaunchKernelGGL(build, dim3(static_cast<unsigned>(clouds) * splits), dim3(G_THREADS), lds, s, m,
-                       static_cast<int>(total), splits, span, idx, weight, offsets, entries);
+    hipLaunchKernelGGL(build, dim3(static_cast<unsigned>(workgroups)), dim3(G_THREADS), lds, s, first, second);
     return tpk_launch_status();
+}
+
+template <int K, bool WEIGHTED, typename IdxT>
+int launch_build_lists(int clouds, int m, int64_t cloud_total, int64_t part_total, int pad_j, const IdxT* idx,
+                       const float* weight, const Lists<WEIGHTED>& lists, hipStream_t s)
+{
+    ListJob<WEIGHTED, IdxT> job, none{};
+    const int st = make_list_job<K, WEIGHTED, IdxT>(clouds, m, cloud_total, part_total, pad_j, idx, weight, lists, &job);
+    return st == TPK_OK ? launch_list_jobs<K, WEIGHTED, IdxT>(job, none, s) : st;
 }
 
 } // namespace

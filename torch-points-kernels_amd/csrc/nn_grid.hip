@@ -435,22 +435,6 @@ __device__ __forceinline__ void wave_equal_range(const int64_t* __restrict__ a, 
     last = lo1;
 }
 
-// Sum of v over the lanes below this one (DPP prefix sum inside every row of 16 lanes, then
-// the totals of the rows before).
-__device__ __forceinline__ int wave_exclusive_sum(int v)
-{
-    int s = v;
-    s += __builtin_amdgcn_update_dpp(0, s, 0x111, 0xF, 0xF, false); // row_shr:1
-    s += __builtin_amdgcn_update_dpp(0, s, 0x112, 0xF, 0xF, false); // row_shr:2
-    s += __builtin_amdgcn_update_dpp(0, s, 0x114, 0xF, 0xF, false); // row_shr:4
-    s += __builtin_amdgcn_update_dpp(0, s, 0x118, 0xF, 0xF, false); // row_shr:8
-    const int r0 = __builtin_amdgcn_readlane(s, 15), r1 = __builtin_amdgcn_readlane(s, 31);
-    const int r2 = __builtin_amdgcn_readlane(s, 47);
-    const int row = (threadIdx.x & (TPK_WAVE - 1)) >> 4;
-    s += (row > 0 ? r0 : 0) + (row > 1 ? r1 : 0) + (row > 2 ? r2 : 0);
-    return s - v;
-}
-
 // Range of 16^3-grid cells along one axis that [v - r, v + r] can touch.  The interval is widened
 // by a few ulps of its ends so that a point the fp32 radius test accepts is never left out.
 __device__ __forceinline__ void bin_range(float v, float r, float lo, float scale, int& first, int& last)

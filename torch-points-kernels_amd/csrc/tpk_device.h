@@ -95,3 +95,61 @@ __device__ __forceinline__ unsigned xcd_local_block(unsigned bid, unsigned block
     const unsigned even = blocks - blocks % XCDS;
     return bid < even ? (bid % XCDS) * (even / XCDS) + bid / XCDS : bid;
 }
+
+// DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_ror:4, row_ror:8.  After the
+// four steps every lane of a 16-lane row holds the row's result.
+__device__ __forceinline__ int row_all_max_i32(int v)
+{
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true));
+    return v;
+}
+
+__device__ __forceinline__ int wave_max_i32(int v)
+{
+    v = row_all_max_i32(v);
+    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return max(max(a, b), max(c, d));
+}
+
+// Sum of v over the lanes below this one (DPP prefix sum inside every row of 16 lanes, then
+// the totals of the rows before).
+__device__ __forceinline__ int wave_exclusive_sum(int v)
+{
+    int s = v;
+    s += __builtin_amdgcn_update_dpp(0, s, 0x111, 0xF, 0xF, false); // row_shr:1
+    s += __builtin_amdgcn_update_dpp(0, s, 0x112, 0xF, 0xF, false); // row_shr:2
+    s += __builtin_amdgcn_update_dpp(0, s, 0x114, 0xF, 0xF, false); // row_shr:4
+    s += __builtin_amdgcn_update_dpp(0, s, 0x118, 0xF, 0xF, false); // row_shr:8
+    const int r0 = __builtin_amdgcn_readlane(s, 15), r1 = __builtin_amdgcn_readlane(s, 31);
+    const int r2 = __builtin_amdgcn_readlane(s, 47);
+    const int row = (threadIdx.x & (TPK_WAVE - 1)) >> 4;
+    s += (row > 0 ? r0 : 0) + (row > 1 ? r1 : 0) + (row > 2 ? r2 : 0);
+    return s - v;
+}
+
+
+// Sum of v over the wavefront, the same value in every lane (row rotations, then the four row
+// totals added in lane order: the result does not depend on which lanes call it).
+__device__ __forceinline__ float wave_sum_f32(float v)
+{
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, true));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true));
+    return ((tpk_read_lane(v, 0) + tpk_read_lane(v, 16)) + tpk_read_lane(v, 32)) + tpk_read_lane(v, 48);
+}
+
+// Workgroup barrier that orders LDS traffic only: global loads and stores a wavefront has in
+// flight stay in flight across it.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): also covers LDS atomics without return value
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
