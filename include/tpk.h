@@ -117,8 +117,8 @@ int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* kno
  *   grad_points (b, c, m) += grad_out (b, c, n) scattered back (fully written, no pre-zero)
  * The backward pass inverts the index into per-target lists held in `workspace`
  * (tpk_three_interpolate_grad_workspace_bytes() bytes, 256-byte aligned; contents need not
- * be initialised and are garbage afterwards).  With workspace == NULL, or rows too long for
- * the lists, it falls back to global float atomics - same result to rounding, much slower.
+ * be initialised and are garbage afterwards).  With workspace == NULL, or for shapes
+ * the lists do not serve, it falls back to global float atomics - same result to rounding, much slower.
  * Index values outside [0, m) are ignored by the list path.
  * ------------------------------------------------------------------------------------- */
 int tpk_three_interpolate_f32(int b, int c, int m, int n, const float* points,

@@ -309,7 +309,7 @@ __global__ __launch_bounds__(256) void chamfer_bwd_lists_kernel(
             ay = ay + -(gj * (other[j * 3 + 1] - py));
             az = az + -(gj * (other[j * 3 + 2] - pz));
         };
-        // Slots are fetched eight at a time, then the points they name (widths are multiples of 4).
+        // Slots are fetched eight at a time, then the points they name.
         for (int i = 0; i < lb.width; i += 8)
         {
             int j[8];
@@ -443,9 +443,9 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
         const Lists<false> lists_a = lists_at<false>(workspace, b, n, m);
         const Lists<false> lists_b = lists_at<false>(static_cast<char*>(workspace) + second, b, m, n);
         ListJob<false, int32_t> job_a, job_b;
-        int st = make_list_job<1, false, int32_t>(b, n, m, m, m, idx2, nullptr, lists_a, &job_a);
+        int st = make_list_job<1, false, int32_t>(b, n, m, m, m, 1, idx2, nullptr, lists_a, &job_a);
         if (st == TPK_OK)
-            st = make_list_job<1, false, int32_t>(b, m, n, n, n, idx1, nullptr, lists_b, &job_b);
+            st = make_list_job<1, false, int32_t>(b, m, n, n, n, 1, idx1, nullptr, lists_b, &job_b);
         if (st == TPK_OK)
             st = launch_list_jobs<1, false, int32_t>(job_a, job_b, s);
         if (st == TPK_OK)

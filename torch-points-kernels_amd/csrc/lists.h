@@ -36,7 +36,7 @@ struct ListEntry<false>
 constexpr int L_MAX_TARGETS = 15360; // targets whose bookkeeping fits in LDS (2 ints each)
 constexpr int L_BLOCK = TPK_WAVE;    // targets per block of lists: one per lane
 constexpr int L_SLACK = 576;         // entry slots a block owns beyond three per entry
-constexpr int L_WIDTH_STEP = 4;      // widths of the padded parts are multiples of this
+constexpr int L_WIDTH_STEP = 4;      // widths of the padded parts are multiples of 1, 2 or this (the walker's choice)
 
 // Layout of the lists of one cloud ("sliced": made to be walked by one lane per target).
 // Targets are taken in blocks of 64; `counts` holds the length of every target's list (0 in the
@@ -44,7 +44,7 @@ constexpr int L_WIDTH_STEP = 4;      // widths of the padded parts are multiples
 //   start_b = 3 * (entries of all earlier targets) + L_SLACK * b
 // and stores slot i of its target L at start_b + i * 64 + L for i < width_b, so that the 64
 // lanes read consecutive entries in every step.  width_b = min(longest list of the block,
-// 2 * ceil(entries of the block / 64) + 4), rounded up to a multiple of 4; shorter lists are
+// 2 * ceil(entries of the block / 64) + 4), rounded up to a multiple of at most 4; shorter lists are
 // padded with (pad_j, 0) entries.  The entries of a list beyond width_b follow the padded part,
 // list after list in target order.  Padded part <= 2 * entries + 574 slots, the rest <= entries:
 // a block never leaves its own slots, whatever the index looks like.
@@ -136,7 +136,7 @@ __device__ __forceinline__ void list_extra(int count, int width, int& extra, int
 template <bool WEIGHTED, typename IdxT>
 struct ListJob
 {
-    int m, cloud_total, parts, part_total, splits, span, pad_j, workgroups;
+    int m, cloud_total, parts, part_total, splits, span, pad_j, width_step, workgroups;
     const IdxT* idx;
     const float* weight;
     Lists<WEIGHTED> lists;
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
     const ListJob<WEIGHTED, IdxT>& job = second ? second_job : first_job;
     const int workgroup = second ? blockIdx.x - first_job.workgroups : blockIdx.x;
     const int m = job.m, cloud_total = job.cloud_total, parts = job.parts, part_total = job.part_total;
-    const int splits = job.splits, span = job.span, pad_j = job.pad_j;
+    const int splits = job.splits, span = job.span, pad_j = job.pad_j, width_step = job.width_step;
     const IdxT* __restrict__ idx = job.idx;
     const float* __restrict__ weight = job.weight;
     const Lists<WEIGHTED>& lists = job.lists;
@@ -247,8 +247,8 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
         const int before = wave_exclusive_sum(count);
         const int block_entries = __builtin_amdgcn_readlane(before + count, TPK_WAVE - 1);
         const int longest = wave_max_i32(count);
-        const int w = (min(longest, 2 * ((block_entries + L_BLOCK - 1) / L_BLOCK) + 4) + L_WIDTH_STEP - 1) &
-                      ~(L_WIDTH_STEP - 1);
+        const int w = (min(longest, 2 * ((block_entries + L_BLOCK - 1) / L_BLOCK) + 4) + width_step - 1) &
+                      ~(width_step - 1);
         const int start = 3 * first + L_SLACK * (i0 / L_BLOCK + blk);
         int extra, extra_at;
         list_extra(count, w, extra, extra_at);
@@ -308,16 +308,17 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
 
 // Describes the job of building the lists of `clouds` clouds of `m` targets and `cloud_total`
 // index entries each, in parts of `part_total` entries (`lists` sized for clouds * parts clouds
-// of part_total entries); padding entries refer to column `pad_j`.  Returns TPK_ERR_UNSUPPORTED
+// of part_total entries); padding entries refer to column `pad_j`, padded widths are multiples of
+// `width_step`.  Returns TPK_ERR_UNSUPPORTED
 // when a span of targets would not fit in LDS or entry positions would not fit an int.
 template <int K, bool WEIGHTED, typename IdxT>
-int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, int pad_j, const IdxT* idx,
-                  const float* weight, const Lists<WEIGHTED>& lists, ListJob<WEIGHTED, IdxT>* job)
+int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, int pad_j, int width_step,
+                  const IdxT* idx, const float* weight, const Lists<WEIGHTED>& lists, ListJob<WEIGHTED, IdxT>* job)
 {
     *job = ListJob<WEIGHTED, IdxT>{};
     if (clouds <= 0 || m <= 0 || cloud_total <= 0)
         return TPK_OK; // nothing to build: no workgroups
-    if (part_total <= 0 || part_total % K != 0)
+    if (part_total <= 0 || part_total % K != 0 || (width_step != 1 && width_step != 2 && width_step != L_WIDTH_STEP))
         return TPK_ERR_INVALID_ARG;
     const int64_t parts = tpk_ceil_div(cloud_total, part_total);
     if (list_capacity(m, part_total) > 0x7fffffffLL || cloud_total > 0x7fffffffLL ||
@@ -340,6 +341,7 @@ int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, in
     job->splits = splits;
     job->span = span;
     job->pad_j = pad_j;
+    job->width_step = width_step;
     job->workgroups = static_cast<int>(clouds * parts * splits);
     job->idx = idx;
     job->weight = weight;
@@ -369,7 +371,7 @@ int launch_build_lists(int clouds, int m, int64_t cloud_total, int64_t part_tota
                        const float* weight, const Lists<WEIGHTED>& lists, hipStream_t s)
 {
     ListJob<WEIGHTED, IdxT> job, none{};
-    const int st = make_list_job<K, WEIGHTED, IdxT>(clouds, m, cloud_total, part_total, pad_j, idx, weight, lists, &job);
+    const int st = make_list_job<K, WEIGHTED, IdxT>(clouds, m, cloud_total, part_total, pad_j, L_WIDTH_STEP, idx, weight, lists, &job);
     return st == TPK_OK ? launch_list_jobs<K, WEIGHTED, IdxT>(job, none, s) : st;
 }
 
