@@ -462,6 +462,27 @@ def test_three_interpolate_colliding_indices(tpk, oracle, dev):
     _assert_scatter_sum_close(_np(f.grad), want, abs_sum)  # sums of ~5000 terms each
 
 
+
+@pytest.mark.parametrize("n,m,C", [(20001, 130, 3), (16388, 64, 2), (40000, 1000, 5)])
+def test_three_interpolate_grad_long_rows(tpk, oracle, dev, n, m, C):
+    # rows of grad_out longer than one staged piece (16384 columns): lists per piece, later
+    # pieces add to earlier ones; a few targets with very long lists, some with none
+    B = 2
+    feats, idx, w, gout = _interp_case(B, C, m, n, n + m)
+    g = torch.Generator().manual_seed(n)
+    heavy = torch.rand(B, n, 3, generator=g) < 0.3
+    idx = torch.where(heavy, torch.randint(0, 3, (B, n, 3), generator=g).int(), idx)
+    idx[idx == m - 1] = 0  # the last target keeps an empty list
+    f = feats.to(dev).requires_grad_(True)
+    out = tpk.three_interpolate(f, idx.to(dev), w.to(dev))
+    np.testing.assert_array_equal(_np(out), oracle.three_interpolate(feats.numpy(), idx.numpy(), w.numpy()))
+    out.backward(gout.to(dev))
+    want = oracle.three_interpolate_grad(gout.numpy(), idx.numpy(), w.numpy(), m)
+    abs_sum = oracle.three_interpolate_grad(gout.abs().numpy(), idx.numpy(), w.numpy(), m)
+    _assert_scatter_sum_close(_np(f.grad), want, abs_sum)
+    assert (_np(f.grad)[:, :, m - 1] == 0).all()
+
+
 def test_interpolate_full_config3a(tpk, oracle, dev):
     w = W.cfg3a_interpolate()
     unknown, known = w["unknown"].to(dev), w["known"].to(dev)
@@ -487,6 +508,24 @@ def test_grouping_parity(tpk, oracle, dev, B, C, N, npoint, nsample):
     g = torch.Generator().manual_seed(N + npoint)
     feats = torch.randn(B, C, N, generator=g)
     idx = torch.randint(0, N, (B, npoint, nsample), generator=g)
+    gout = torch.randn(B, C, npoint, nsample, generator=g)
+    f = feats.to(dev).requires_grad_(True)
+    out = tpk.grouping_operation(f, idx.to(dev))
+    np.testing.assert_array_equal(_np(out), oracle.grouping_operation(feats.numpy(), idx.numpy()))
+    out.backward(gout.to(dev))
+    want = oracle.grouping_operation_grad(gout.numpy(), idx.numpy(), N)
+    _assert_scatter_sum_close(_np(f.grad), want, oracle.grouping_operation_grad(gout.abs().numpy(), idx.numpy(), N))
+
+
+
+@pytest.mark.parametrize("N,npoint,nsample,C", [(1000, 1250, 32, 3), (70, 2049, 8, 2), (5000, 333, 50, 1)])
+def test_grouping_grad_long_rows(tpk, oracle, dev, N, npoint, nsample, C):
+    # npoint * nsample above one staged piece; clustered indices give long and empty lists
+    B = 2
+    g = torch.Generator().manual_seed(N + npoint)
+    feats = torch.randn(B, C, N, generator=g)
+    idx = torch.randint(0, N, (B, npoint, nsample), generator=g)
+    idx[:, :, : nsample // 2] = idx[:, :, : nsample // 2] % 5
     gout = torch.randn(B, C, npoint, nsample, generator=g)
     f = feats.to(dev).requires_grad_(True)
     out = tpk.grouping_operation(f, idx.to(dev))
