@@ -41,7 +41,9 @@ def test_library_exports_every_declared_symbol():
     assert lib.tpk_version() >= 100
     lib.tpk_fps_workspace_bytes.restype = ctypes.c_size_t
     assert lib.tpk_fps_workspace_bytes(4, 16384) == 0
-    assert lib.tpk_fps_workspace_bytes(4, 50000) == 4 * 50000 * 4
+    # 16385..163840 points: records (16 B), boxes (160 B per cell of 64) and minima (4 B) of whole windows of 16384
+    assert lib.tpk_fps_workspace_bytes(4, 50000) == 4 * 4 * 256 * (64 * 16 + 160 + 64 * 4)
+    assert lib.tpk_fps_workspace_bytes(2, 200000) == 2 * 200000 * 4  # larger: the minima only
     # searches over curve-ordered cells: 16 bytes per point padded to cells of 64, 160 bytes per cell;
     # 0 = the shape is served by the all-pairs scan, no workspace wanted
     for name in ("tpk_three_nn_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes"):

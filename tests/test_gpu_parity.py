@@ -289,12 +289,43 @@ def test_fps_parity(tpk, oracle, dev, B, N, npoint):
     np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), npoint))
 
 
+@pytest.mark.parametrize("B,N,npoint", [(2, 20000, 150), (1, 16385, 90), (2, 50001, 300), (1, 163840, 64)])
+def test_fps_cells_in_memory_parity(tpk, oracle, dev, B, N, npoint):
+    # more points than one workgroup keeps in registers: cells of 64 points in memory
+    g = torch.Generator().manual_seed(N)
+    xyz = _clustered(g, B, N) if N % 2 else torch.rand(B, N, 3, generator=g)
+    out = tpk.furthest_point_sample(xyz.to(dev), npoint)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), npoint))
+
+
+def test_fps_cells_in_memory_ties(tpk, oracle, dev):
+    g = torch.Generator().manual_seed(11)
+    ax = torch.arange(30, dtype=torch.float32)
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3) + 1.0
+    shuffled = lattice[:, torch.randperm(lattice.shape[1], generator=g)]
+    for pts in (lattice, shuffled):
+        out = tpk.furthest_point_sample(pts.contiguous().to(dev), 300)
+        np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(pts.numpy(), 300))
+    # every point three times, some points never eligible, 2 clouds, more samples than distinct points
+    base = torch.rand(2, 7000, 3, generator=g) * 4.0 - 2.0
+    base[:, :37] *= 0.004
+    xyz = torch.cat([base, base.flip(1), base], 1)[:, torch.randperm(21000, generator=g)].contiguous()
+    out = tpk.furthest_point_sample(xyz.to(dev), 7100)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), 7100))
+    # nothing eligible; a single eligible point
+    tiny = torch.full((2, 20000, 3), 0.001)
+    assert (tpk.furthest_point_sample(tiny.to(dev), 10) == 0).all()
+    tiny[1, 18123] = 1.0
+    np.testing.assert_array_equal(_np(tpk.furthest_point_sample(tiny.to(dev), 5)),
+                                  oracle.furthest_point_sample(tiny.numpy(), 5))
+
+
 def test_fps_streaming_path_parity(tpk, oracle, dev):
-    # more points than one workgroup keeps in registers
+    # more points than the cell kernel keeps summaries for
     g = torch.Generator().manual_seed(77)
-    xyz = torch.rand(2, 20000, 3, generator=g)
-    out = tpk.furthest_point_sample(xyz.to(dev), 150)
-    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), 150))
+    xyz = torch.rand(2, 170000, 3, generator=g)
+    out = tpk.furthest_point_sample(xyz.to(dev), 40)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), 40))
 
 
 def test_fps_ties_origin_skip_and_exhaustion(tpk, oracle, dev):

@@ -2,7 +2,7 @@
 // the chosen set, pick the point whose distance is largest".
 //
 // One workgroup (one compute unit) owns a cloud for the whole call; the rounds of a cloud
-// depend on each other, so a call runs as many workgroups as there are clouds.  Three kernels
+// depend on each other, so a call runs as many workgroups as there are clouds.  Four kernels
 // by cloud size:
 //   up to 512 points     fps_resident_kernel: one point per lane in registers, every point
 //                        updated every round, one 24-byte LDS record per wavefront and one
@@ -10,6 +10,10 @@
 //   up to 16384 points   fps_pruned_kernel: up to 32 points per lane in registers, cloud
 //                        ordered along a space filling curve so that most updates can be
 //                        skipped exactly (described at the kernel);
+//   up to 163840 points  fps_cells_kernel: the cloud ordered along the curve into cells of 64
+//                        points that stay in memory (the caller's workspace); boxes, largest
+//                        distance and best point of every cell in LDS; a round touches only
+//                        the cells the new sample can change (described at the kernel);
 //   larger clouds        fps_streaming_kernel: the selection code of the first kernel over
 //                        points streamed from global memory, running minima in a workspace
 //                        provided by the caller.
@@ -24,7 +28,7 @@
 // k among its own equal maxima, and the halving tree then prefers the thread whose number
 // has the smaller bit-reversal.  Both rules together are "smallest tie key", with
 //   key(k) = bitrev(k mod BS) * ceil(n / BS) + floor(k / BS).
-#include "curve_order.h"
+#include "curve_cells.h"
 
 #include <cmath>
 
@@ -616,6 +620,183 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         out[npoint - 1] = static_cast<int>(sort_keys[pending] & 0x3FFFu);
 }
 
+constexpr int FPS_CELL_WINDOW = CURVE_MAX_POINTS;            // points ordered together
+constexpr int FPS_WINDOW_CELLS = FPS_CELL_WINDOW / NG_CELL;  // 256
+constexpr int FPS_MAX_CELLS = 2560;                          // cells whose state fits in LDS
+constexpr int FPS_CELL_POINTS = FPS_MAX_CELLS * NG_CELL;     // 163840
+constexpr int FPS_LIVE_CAPACITY = (FPS_MAX_CELLS + FPS_THREADS - 1) / FPS_THREADS * TPK_WAVE; // live cells per wavefront
+constexpr int FPS_CELL_BATCH = 4;                            // cells whose points a wavefront requests together
+
+// Clouds too large for registers.  The cloud has been cut into windows of 16384 consecutive
+// points, each ordered along the curve into 256 cells of 64 (curve_cells_kernel): records
+// (x, y, z, index inside the window) and the cells' boxes are in `sorted` / `boxes`; the running
+// minima live in `temp`, in the same order (ineligible points and padding hold -1).  LDS keeps,
+// for every cell, its box, its largest minimum, the tie key of the point holding it, and that
+// point (x, y, z, index in the cloud).
+// A minimum can only change if the new sample is closer than it, and no minimum of a cell
+// exceeds the cell's largest: a cell whose box is not closer to the sample than its largest
+// minimum is skipped (margin for rounding as in the register kernel), exactly.  Cell c belongs
+// to wavefront c mod 16 (neighbours on the curve go to different wavefronts): the wavefront
+// tests the boxes of its cells (one per lane and step), then updates the live ones - 64 points
+// per cell, a few cells' loads in flight together - and renews their LDS entries.  After a
+// Every wavefront then finds the best of its cells, the 16 results are exchanged through LDS
+// and reduced as in the other kernels.  One barrier per round.
+// dynamic LDS: 48 bytes per cell + FPS_LIVE_CAPACITY * 16 * 2.
+__global__ __launch_bounds__(FPS_THREADS) void fps_cells_kernel(
+    int n, int npoint, int log2_bs, int groups, int cells, const float* __restrict__ xyz,
+    const float4* __restrict__ sorted, const float4* __restrict__ boxes, float* __restrict__ temp,
+    int32_t* __restrict__ out)
+{
+    extern __shared__ float4 cell_best[];                                  // [cells] x, y, z, index
+    float* const box = reinterpret_cast<float*>(cell_best + cells);        // [6][cells] lo.xyz, hi.xyz
+    int* const cell_max = reinterpret_cast<int*>(box + 6 * cells);         // [cells] bits of the largest minimum
+    unsigned* const cell_tie = reinterpret_cast<unsigned*>(cell_max + cells); // [cells]
+    unsigned short* const live_all = reinterpret_cast<unsigned short*>(cell_tie + cells);
+    __shared__ WaveRecord records[2][FPS_WAVES];
+
+    xyz += static_cast<int64_t>(blockIdx.x) * n * 3;
+    sorted += static_cast<int64_t>(blockIdx.x) * cells * NG_CELL;
+    boxes += static_cast<int64_t>(blockIdx.x) * cells * NG_BOX;
+    temp += static_cast<int64_t>(blockIdx.x) * cells * NG_CELL;
+    out += static_cast<int64_t>(blockIdx.x) * npoint;
+    const int tid = threadIdx.x;
+    const int lane = tid & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
+    unsigned short* const live = live_all + wave * FPS_LIVE_CAPACITY;
+    const int steps = (cells + FPS_THREADS - 1) / FPS_THREADS; // cells per lane
+    const unsigned bs_mask = (1u << log2_bs) - 1u;
+    auto tie_key = [&](unsigned k) __attribute__((always_inline)) {
+        const unsigned rev = log2_bs ? (__brev(k & bs_mask) >> (32 - log2_bs)) : 0u;
+        return rev * static_cast<unsigned>(groups) + (k >> log2_bs);
+    };
+
+    // Set-up: minima, boxes and largest minima (best points are found by the first update).
+    for (int c = wave; c < cells; c += FPS_WAVES)
+    {
+        const float4 r = sorted[c * NG_CELL + lane];
+        const bool takes_part = __float_as_int(r.w) != 0x7FFFFFFF && eligible(r.x, r.y, r.z);
+        temp[c * NG_CELL + lane] = takes_part ? 1e10f : -1.0f;
+        const bool any = __ballot(takes_part) != 0;
+        if (lane < 6)
+        {
+            const float4 b = boxes[c * NG_BOX + lane / 3];
+            const int a = lane % 3;
+            box[lane * cells + c] = a == 0 ? b.x : a == 1 ? b.y : b.z;
+        }
+        if (lane == 6)
+        {
+            cell_max[c] = ordered_bits(any ? 1e10f : -1.0f);
+            cell_tie[c] = 0xFFFFFFFFu;
+        }
+    }
+    const float p0x = xyz[0], p0y = xyz[1], p0z = xyz[2];
+    float sx = p0x, sy = p0y, sz = p0z;
+    if (tid == 0)
+        out[0] = 0;
+    __syncthreads();
+
+    for (int j = 1; j < npoint; ++j)
+    {
+        // 1. the live cells among this wavefront's
+        int count = 0;
+        for (int step = 0; step < steps; ++step)
+        {
+            const int c = (step * TPK_WAVE + lane) * FPS_WAVES + wave;
+            bool is_live = false;
+            if (c < cells)
+            {
+                const float dx = fmaxf(fmaxf(box[0 * cells + c] - sx, sx - box[3 * cells + c]), 0.f);
+                const float dy = fmaxf(fmaxf(box[1 * cells + c] - sy, sy - box[4 * cells + c]), 0.f);
+                const float dz = fmaxf(fmaxf(box[2 * cells + c] - sz, sz - box[5 * cells + c]), 0.f);
+                const float lb = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz));
+                is_live = lb * 0.999998f < __int_as_float(cell_max[c]);
+            }
+            const unsigned long long mask = __ballot(is_live);
+            if (is_live)
+                live[count + tpk_prefix_count(mask)] = static_cast<unsigned short>(c);
+            count += __builtin_popcountll(mask);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
+        // 2. their points: new minima, and the cell's best point
+        for (int i0 = 0; i0 < count; i0 += FPS_CELL_BATCH)
+        {
+            int c[FPS_CELL_BATCH];
+            float4 r[FPS_CELL_BATCH];
+            float m[FPS_CELL_BATCH];
+#pragma unroll
+            for (int u = 0; u < FPS_CELL_BATCH; ++u)
+            {
+                c[u] = __builtin_amdgcn_readfirstlane(static_cast<int>(live[min(i0 + u, count - 1)]));
+                r[u] = sorted[c[u] * NG_CELL + lane];
+                m[u] = temp[c[u] * NG_CELL + lane];
+            }
+#pragma unroll
+            for (int u = 0; u < FPS_CELL_BATCH; ++u)
+            {
+                if (i0 + u >= count) // wave-uniform
+                    break;
+                const float d = tpk_dist2(r[u].x, r[u].y, r[u].z, sx, sy, sz);
+                const int old_bits = ordered_bits(m[u]);
+                const int new_bits = min(ordered_bits(d), old_bits); // -1 stays -1
+                if (new_bits != old_bits)
+                    temp[c[u] * NG_CELL + lane] = __int_as_float(new_bits);
+                const unsigned k = static_cast<unsigned>(c[u] / FPS_WINDOW_CELLS) * FPS_CELL_WINDOW +
+                                   static_cast<unsigned>(__float_as_int(r[u].w));
+                const unsigned tk = tie_key(k);
+                int cell_val;
+                const int wl = winning_lane(new_bits, tk, cell_val);
+                if (lane == wl)
+                {
+                    cell_max[c[u]] = cell_val;
+                    cell_tie[c[u]] = tk;
+                    cell_best[c[u]] = make_float4(r[u].x, r[u].y, r[u].z, __int_as_float(static_cast<int>(k)));
+                }
+            }
+        }
+
+        // 3. the best of this wavefront's cells (steps 1 - 3 touch no other wavefront's cells, so
+        // the records below are the only exchange: one barrier per round, records double buffered)
+        int best = INT_MIN, best_cell = 0;
+        unsigned best_tk = 0xFFFFFFFFu;
+        for (int step = 0; step < steps; ++step)
+        {
+            const int c = (step * TPK_WAVE + lane) * FPS_WAVES + wave;
+            if (c < cells)
+            {
+                const int v = cell_max[c];
+                const unsigned t = cell_tie[c];
+                const bool better = v > best || (v == best && t < best_tk);
+                best = better ? v : best;
+                best_tk = better ? t : best_tk;
+                best_cell = better ? c : best_cell;
+            }
+        }
+        int wave_val;
+        const int wl = winning_lane(best, best_tk, wave_val);
+        const int wave_cell = __builtin_amdgcn_readlane(best_cell, wl);
+        const float4 b = cell_best[wave_cell];
+        if (lane == 0)
+        {
+            WaveRecord rec;
+            rec.val = wave_val;
+            rec.tk = __builtin_amdgcn_readlane(best_tk, wl);
+            rec.k = __float_as_int(b.w);
+            rec.x = b.x;
+            rec.y = b.y;
+            rec.z = b.z;
+            records[j & 1][wave] = rec;
+        }
+        lds_barrier();
+        int k, gv_unused;
+        reduce_records<FPS_WAVES>(records[j & 1], lane, p0x, p0y, p0z, k, sx, sy, sz, gv_unused);
+        if (tid == 0)
+            out[j] = k;
+    }
+}
+
+
 // Clouds too large for registers: points and running minima stream from global memory.
 __global__ __launch_bounds__(FPS_THREADS) void fps_streaming_kernel(
     int n, int npoint, int log2_bs, int groups, const float* __restrict__ xyz,
@@ -711,7 +892,6 @@ void launch_resident(int b, int n, int npoint, int log2_bs, int groups, const fl
                        npoint, log2_bs, groups, xyz, out);
 }
 
-} // namespace
 
 template <int PPT, int THREADS, int GS>
 int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float* xyz,
@@ -730,11 +910,37 @@ int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float
     return tpk_launch_status();
 }
 
+// Workspace of the cell kernel: ordered records, boxes, minima (each 256-byte aligned).
+struct CellLayout
+{
+    int cells; // per cloud
+    size_t sorted, boxes, temp, total;
+};
+CellLayout cell_layout(int b, int n)
+{
+    auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    CellLayout l;
+    l.cells = static_cast<int>(tpk_ceil_div(n, FPS_CELL_WINDOW)) * FPS_WINDOW_CELLS;
+    const size_t all = static_cast<size_t>(b) * l.cells;
+    l.sorted = 0;
+    l.boxes = up(all * NG_CELL * sizeof(float4));
+    l.temp = up(l.boxes + all * NG_BOX * sizeof(float4));
+    l.total = up(l.temp + all * NG_CELL * sizeof(float));
+    return l;
+}
+
+size_t streaming_bytes(int b, int n)
+{
+    return static_cast<size_t>(b) * static_cast<size_t>(n) * sizeof(float);
+}
+
+} // namespace
+
 extern "C" size_t tpk_fps_workspace_bytes(int b, int n)
 {
     if (b <= 0 || n <= FPS_REGISTER_POINTS)
         return 0;
-    return static_cast<size_t>(b) * static_cast<size_t>(n) * sizeof(float);
+    return n <= FPS_CELL_POINTS ? cell_layout(b, n).total : streaming_bytes(b, n);
 }
 
 extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* workspace,
@@ -777,9 +983,29 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
         return launch_pruned<16, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_REGISTER_POINTS)
         return launch_pruned<32, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+    else if (n <= FPS_CELL_POINTS && workspace && workspace_bytes >= cell_layout(b, n).total)
+    {
+        // Cells of 64 points in memory, their summaries in LDS.
+        const CellLayout l = cell_layout(b, n);
+        char* const w = static_cast<char*>(workspace);
+        PointSet cloud{xyz, nullptr, static_cast<int64_t>(b) * n, n, FPS_CELL_WINDOW,
+                       reinterpret_cast<float4*>(w + l.sorted), reinterpret_cast<float4*>(w + l.boxes), nullptr, nullptr};
+        PointSet none{nullptr, nullptr, 0, 1, FPS_CELL_WINDOW, nullptr, nullptr, nullptr, nullptr};
+        int st = launch_curve_cells(cloud, none, nullptr, s);
+        if (st != TPK_OK)
+            return st;
+        const size_t lds = static_cast<size_t>(l.cells) * 48 + FPS_LIVE_CAPACITY * FPS_WAVES * sizeof(unsigned short);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fps_cells_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        if (e != hipSuccess)
+            return static_cast<int>(e);
+        hipLaunchKernelGGL(fps_cells_kernel, dim3(b), dim3(FPS_THREADS), lds, s, n, npoint, log2_bs, groups, l.cells,
+                           xyz, cloud.sorted, cloud.boxes, reinterpret_cast<float*>(w + l.temp), idx_out);
+    }
     else
     {
-        const size_t need = tpk_fps_workspace_bytes(b, n);
+        // (also serves callers that sized the workspace for the minima only)
+        const size_t need = streaming_bytes(b, n);
         if (!workspace || workspace_bytes < need)
             return TPK_ERR_WORKSPACE;
         hipLaunchKernelGGL(fps_streaming_kernel, dim3(b), dim3(FPS_THREADS), 0, s, n, npoint,
