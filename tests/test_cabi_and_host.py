@@ -49,9 +49,12 @@ def test_library_exports_every_declared_symbol():
     for name in ("tpk_three_nn_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_size_t
-        assert fn(2, 100, 100) == 0 and fn(2, 20000, 1000) == 0 and fn(0, 1000, 1000) == 0
+        assert fn(2, 100, 100) == 0 and fn(2, 200000, 1000) == 0 and fn(0, 1000, 1000) == 0
         want = sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((11, 1024), (15, 1024), (11, 160), (15, 160)))
         assert fn(2, 700, 900) == want
+        # clouds above 16384 points: whole windows of 16384 points (256 cells each)
+        want = sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((512, 1024), (15, 1024), (512, 160), (15, 160)))
+        assert fn(2, 20000, 900) == want
     lib.tpk_ball_query_partial_workspace_bytes.restype = ctypes.c_size_t
     lib.tpk_ball_query_partial_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
     assert lib.tpk_ball_query_partial_workspace_bytes(8191, 100, 16) == 0

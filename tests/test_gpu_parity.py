@@ -405,7 +405,8 @@ def test_three_nn_parity(tpk, oracle, dev, B, n, m):
     np.testing.assert_array_equal(_np(dist), np.sqrt(wd))
 
 
-@pytest.mark.parametrize("B,n,m", [(2, 512, 512), (3, 1000, 777), (2, 5000, 515), (1, 16384, 4096), (2, 700, 16384)])
+@pytest.mark.parametrize("B,n,m", [(2, 512, 512), (3, 1000, 777), (2, 5000, 515), (1, 16384, 4096), (2, 700, 16384),
+                                   (2, 20000, 600), (1, 3000, 40000), (1, 33000, 16385)])
 def test_three_nn_cell_search_parity(tpk, oracle, dev, B, n, m):
     # cloud sizes served by the search over curve-ordered cells (512..16384 points each side)
     native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
@@ -430,6 +431,13 @@ def test_three_nn_cell_search_ties(tpk, oracle, dev):
              (lattice + 0.5, lattice[:, torch.randperm(1000, generator=g)]),
              (lattice, lattice),
              (torch.rand(1, 520, 3, generator=g), torch.full((1, 600, 3), 0.5))]
+    # the same above 16384 points, where a cloud is ordered in several windows: equal points in
+    # different windows, a lattice of 27000 points
+    k = torch.rand(1, 7000, 3, generator=g)
+    big = torch.cat([k, k.flip(1), k], 1)[:, torch.randperm(21000, generator=g)]
+    ax = torch.arange(30, dtype=torch.float32)
+    big_lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3)
+    cases += [(torch.rand(1, 900, 3, generator=g), big), (big_lattice[:, :17000] + 0.5, big_lattice)]
     for unknown, known in cases:
         unknown, known = unknown.contiguous(), known.contiguous()
         dist2, idx = native.three_nn(unknown.to(dev), known.to(dev))
@@ -620,7 +628,8 @@ def test_chamfer_ties_take_lowest_index(tpk, oracle, dev):
     np.testing.assert_array_equal(_np(d2), w2)
 
 
-@pytest.mark.parametrize("B,n,m", [(2, 512, 512), (3, 1000, 777), (2, 4099, 513), (1, 16384, 16384), (2, 9000, 16000)])
+@pytest.mark.parametrize("B,n,m", [(2, 512, 512), (3, 1000, 777), (2, 4099, 513), (1, 16384, 16384), (2, 9000, 16000),
+                                   (2, 20000, 700), (1, 16385, 40001)])
 def test_chamfer_cell_search_parity(tpk, oracle, dev, B, n, m):
     # cloud sizes served by the search over curve-ordered cells (float32, 512..16384 points)
     from torch_points_kernels._native import native
@@ -649,6 +658,12 @@ def test_chamfer_cell_search_ties(tpk, oracle, dev):
     cases = [(lattice, shifted[:, torch.randperm(1000, generator=g)]),
              (lattice[:, torch.randperm(1000, generator=g)], lattice),
              (doubled, base[:, :640]), (doubled, doubled.flip(1)), (base, collapsed), (collapsed, collapsed)]
+    # above 16384 points (clouds ordered in several windows): every point three times, a large lattice
+    base = torch.rand(1, 6000, 3, generator=g)
+    tripled = torch.cat([base, base, base.flip(1)], 1)[:, torch.randperm(18000, generator=g)]
+    ax = torch.arange(27, dtype=torch.float32)
+    big_lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3)
+    cases += [(tripled, base[:, :5000]), (big_lattice, big_lattice[:, torch.randperm(19683, generator=g)] + 0.5)]
     for a, b in cases:
         a, b = a.contiguous(), b.contiguous()
         d1, d2, i1, i2 = native().chamfer_dist(a.to(dev), b.to(dev))

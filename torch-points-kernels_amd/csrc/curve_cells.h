@@ -15,7 +15,7 @@ constexpr int NG_BOX = 10;            // float4 per cell: box of the cell, then 
 // A set of points to be ordered: `total` points in clouds of `cloud_points` consecutive points,
 // every cloud cut into windows of `stride` consecutive points (the last window of a cloud may be
 // shorter; a packed array of unequal clouds is one "cloud" whose windows hold whatever clouds
-// lie there).  Every window gets stride / 64 (rounded up) cells of 64 records, in curve order; a record is (x, y, z, index inside the window), the
+// lie there).  Every window gets stride / 64 (rounded up) cells of 64 records, in curve order; a record is (x, y, z, index inside the cloud), the
 // padding records are infinitely far away with index 0x7FFFFFFF; a cell without points has an
 // empty box (lo = +inf, hi = -inf).
 struct PointSet
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
                 continue;
             const bool real = k[u] >= 0;
             const float inf = __builtin_inff();
-            sorted[q] = real ? make_float4(v[u][0], v[u][1], v[u][2], __int_as_float(k[u]))
+            sorted[q] = real ? make_float4(v[u][0], v[u][1], v[u][2], __int_as_float(static_cast<int>(in_cloud) + k[u]))
                              : make_float4(inf, inf, inf, __int_as_float(0x7FFFFFFF));
             if (!boxes) // uniform
                 continue;

@@ -629,7 +629,7 @@ constexpr int FPS_CELL_BATCH = 4;                            // cells whose poin
 
 // Clouds too large for registers.  The cloud has been cut into windows of 16384 consecutive
 // points, each ordered along the curve into 256 cells of 64 (curve_cells_kernel): records
-// (x, y, z, index inside the window) and the cells' boxes are in `sorted` / `boxes`; the running
+// (x, y, z, index in the cloud) and the cells' boxes are in `sorted` / `boxes`; the running
 // minima live in `temp`, in the same order (ineligible points and padding hold -1).  LDS keeps,
 // for every cell, its box, its largest minimum, the tie key of the point holding it, and that
 // point (x, y, z, index in the cloud).
@@ -742,8 +742,7 @@ __global__ __launch_bounds__(FPS_THREADS) void fps_cells_kernel(
                 const int new_bits = min(ordered_bits(d), old_bits); // -1 stays -1
                 if (new_bits != old_bits)
                     temp[c[u] * NG_CELL + lane] = __int_as_float(new_bits);
-                const unsigned k = static_cast<unsigned>(c[u] / FPS_WINDOW_CELLS) * FPS_CELL_WINDOW +
-                                   static_cast<unsigned>(__float_as_int(r[u].w));
+                const unsigned k = static_cast<unsigned>(__float_as_int(r[u].w));
                 const unsigned tk = tie_key(k);
                 int cell_val;
                 const int wl = winning_lane(new_bits, tk, cell_val);

@@ -18,15 +18,19 @@
 // an extra pass that collects the lowest index among all candidates at that distance.
 //
 // Workspace per cloud: 16 bytes per point (x, y, z, original index) padded to whole cells, and
-// 32 bytes per cell (box).  Clouds of up to 16384 points (the curve ordering works in LDS).
+// 160 bytes per cell (its box and those of its four runs of 16 points).  The curve ordering works
+// in LDS on at most 16384 points: a larger cloud (up to 163840 points) is ordered in windows of
+// 16384 consecutive points, which the search sees as more - and wider - cells of the same cloud.
 #include "curve_cells.h"
 
+#include <algorithm>
 #include <cmath>
 #include "nn_grid.h"
 
 namespace {
 
-constexpr int NG_MAX_CELLS = 256;            // candidate cells per cloud (their box distances sit in LDS)
+constexpr int NG_MAX_CELLS = 2560;           // candidate cells per cloud (their box distances sit in LDS)
+constexpr int NG_WINDOW = CURVE_MAX_POINTS;  // larger clouds are ordered in windows of this many points
 constexpr int NG_SCAN_THREADS = 256;         // 4 wavefronts, each searching on its own
 constexpr float NG_MARGIN = 0.999998f;
 constexpr int NG_CHUNK = 8;
@@ -82,17 +86,16 @@ __device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, const
 // block mapping) = cloud * (cells1 + cells2) + cell; the cells of cloud 1 query cloud 2 and
 // write dist1 / idx1, those of cloud 2 the other way round.
 __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
-    int n, int m, int clouds, const float4* __restrict__ sorted1,
+    int n, int m, int cells1, int cells2, int clouds, const float4* __restrict__ sorted1,
     const float4* __restrict__ sorted2, const float4* __restrict__ boxes1,
     const float4* __restrict__ boxes2, float* __restrict__ dist1, float* __restrict__ dist2,
     int32_t* __restrict__ idx1, int32_t* __restrict__ idx2)
 {
     __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
-    __shared__ float lows_all[NG_SCAN_THREADS / TPK_WAVE][NG_MAX_CELLS];
+    extern __shared__ float lows_all[]; // [wavefronts][largest number of candidate cells, in whole groups of 64]
 
     const int lane = threadIdx.x & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
-    const int cells1 = (n + NG_CELL - 1) / NG_CELL, cells2 = (m + NG_CELL - 1) / NG_CELL;
     const int per_cloud = cells1 + cells2;
     const int64_t task = static_cast<int64_t>(xcd_local_block(blockIdx.x, gridDim.x)) *
                              (NG_SCAN_THREADS / TPK_WAVE) + wave;
@@ -112,11 +115,13 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
     float* __restrict__ dout = (second ? dist2 : dist1) + static_cast<int64_t>(cloud) * qcount;
     int32_t* __restrict__ iout = (second ? idx2 : idx1) + static_cast<int64_t>(cloud) * qcount;
     float4* const stage = stages[wave];
-    float* const lows = lows_all[wave];
+    float* const lows = lows_all + wave * ((max(cells1, cells2) + NG_CELL - 1) / NG_CELL * NG_CELL);
 
     const float4 query = qpts[qcell * NG_CELL + lane];
     const float qx = query.x, qy = query.y, qz = query.z;
     const int qindex = __float_as_int(query.w); // 0x7FFFFFFF: padding, nothing to store
+    if (__ballot(qindex != 0x7FFFFFFF) == 0)
+        return; // a cell without points (the last window of a cloud may have some)
     const float4 qlo = qbox[qcell * NG_BOX + 0], qhi = qbox[qcell * NG_BOX + 1];
 
     // Box distances to all candidate cells, kept in the wavefront's LDS row (lane l computes
@@ -130,17 +135,17 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
         const int cc = valid ? c : 0;
         const float lb = box_box_dist2(qlo, qhi, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
         lows[c] = valid ? lb : __builtin_inff();
-        // approximately the nearest cell (the two lowest bits of the distance carry g)
-        const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~3u) | static_cast<unsigned>(g);
+        // approximately the nearest cell (the six lowest bits of the distance carry g)
+        const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~63u) | static_cast<unsigned>(g);
         seed_key = valid && key < seed_key ? key : seed_key;
     }
     Nearest s;
-    s.best = __builtin_inff();
+    s.best = qindex == 0x7FFFFFFF ? -1.f : __builtin_inff(); // (a padding lane never asks for a scan)
     s.chunk = 0;
     s.tie = false;
     {
         const unsigned lowest = wave_min_u32(seed_key);
-        int seed = static_cast<int>(lowest & 3u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
+        int seed = static_cast<int>(lowest & 63u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
         if (seed >= ccells) // no lane had a usable key (NaN boxes)
             seed = 0;
         scan_cell(cpts, cbox, seed, stage, lane, qx, qy, qz, s);
@@ -293,16 +298,15 @@ __device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, cons
 
 // One wavefront = the 64 unknown points of one cell; logical wavefront = cloud * qcells + cell.
 __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
-    int n, int m, int clouds, const float4* __restrict__ sorted_unknown,
+    int n, int m, int qcells, int ccells, int clouds, const float4* __restrict__ sorted_unknown,
     const float4* __restrict__ sorted_known, const float4* __restrict__ boxes_unknown,
     const float4* __restrict__ boxes_known, float* __restrict__ dist2, int32_t* __restrict__ idx)
 {
     __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
-    __shared__ float lows_all[NG_SCAN_THREADS / TPK_WAVE][NG_MAX_CELLS];
+    extern __shared__ float lows_all[]; // [wavefronts][candidate cells, in whole groups of 64]
 
     const int lane = threadIdx.x & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
-    const int qcells = (n + NG_CELL - 1) / NG_CELL, ccells = (m + NG_CELL - 1) / NG_CELL;
     const int64_t task = static_cast<int64_t>(xcd_local_block(blockIdx.x, gridDim.x)) *
                              (NG_SCAN_THREADS / TPK_WAVE) + wave;
     if (task >= static_cast<int64_t>(qcells) * clouds)
@@ -316,11 +320,13 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     dist2 += static_cast<int64_t>(cloud) * n * 3;
     idx += static_cast<int64_t>(cloud) * n * 3;
     float4* const stage = stages[wave];
-    float* const lows = lows_all[wave];
+    float* const lows = lows_all + wave * ((ccells + NG_CELL - 1) / NG_CELL * NG_CELL);
 
     const float4 query = qpts[qcell * NG_CELL + lane];
     const float qx = query.x, qy = query.y, qz = query.z;
     const int qindex = __float_as_int(query.w); // 0x7FFFFFFF: padding, nothing to store
+    if (__ballot(qindex != 0x7FFFFFFF) == 0)
+        return; // a cell without points (the last window of a cloud may have some)
     const float4 qlo = qbox[qcell * NG_BOX + 0], qhi = qbox[qcell * NG_BOX + 1];
 
     const int groups = (ccells + NG_CELL - 1) / NG_CELL;
@@ -332,15 +338,15 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
         const int cc = valid ? c : 0;
         const float lb = box_box_dist2(qlo, qhi, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
         lows[c] = valid ? lb : __builtin_inff();
-        const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~3u) | static_cast<unsigned>(g);
+        const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~63u) | static_cast<unsigned>(g);
         seed_key = valid && key < seed_key ? key : seed_key;
     }
     Nearest3 s;
-    s.b1 = s.b2 = s.b3 = __builtin_inff();
+    s.b1 = s.b2 = s.b3 = qindex == 0x7FFFFFFF ? -1.f : __builtin_inff(); // (a padding lane never asks for a scan)
     s.i1 = s.i2 = s.i3 = 0;
     {
         const unsigned lowest = wave_min_u32(seed_key);
-        int seed = static_cast<int>(lowest & 3u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
+        int seed = static_cast<int>(lowest & 63u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
         if (seed >= ccells)
             seed = 0;
         scan_cell3(cpts, cbox, seed, stage, lane, qx, qy, qz, s);
@@ -529,7 +535,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 const float4 p = sorted_x[has ? at_x : 0];
                 const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-                const int row = (at_x & ~(CURVE_MAX_POINTS - 1)) + __float_as_int(p.w);
+                const int row = __float_as_int(p.w);
                 const bool hit = has && d <= radius2 && row >= s0 && row < s1;
                 const unsigned long long mask = __ballot(hit);
                 if (mask == 0)
@@ -611,11 +617,23 @@ struct GridLayout
     size_t sorted_a, sorted_b, boxes_a, boxes_b, total;
 };
 
+// Cells of a cloud of n points: ordered whole up to NG_WINDOW points, else in windows of NG_WINDOW
+// consecutive points (the last one padded with cells that hold nothing).
+int grid_cells(int n)
+{
+    return n <= NG_WINDOW ? (n + NG_CELL - 1) / NG_CELL
+                          : static_cast<int>(tpk_ceil_div(n, NG_WINDOW)) * (NG_WINDOW / NG_CELL);
+}
+int grid_stride(int n)
+{
+    return n <= NG_WINDOW ? n : NG_WINDOW;
+}
+
 GridLayout grid_layout(int b, int n, int m)
 {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
-    const size_t cells_a = static_cast<size_t>((n + NG_CELL - 1) / NG_CELL);
-    const size_t cells_b = static_cast<size_t>((m + NG_CELL - 1) / NG_CELL);
+    const size_t cells_a = static_cast<size_t>(grid_cells(n));
+    const size_t cells_b = static_cast<size_t>(grid_cells(m));
     GridLayout l;
     size_t pos = 0;
     l.sorted_a = pos;
@@ -632,9 +650,9 @@ GridLayout grid_layout(int b, int n, int m)
 
 bool grid_supported(int b, int n, int m)
 {
-    // Small clouds are served as fast by the all-pairs scan; large ones do not fit the LDS sort.
-    return b > 0 && n >= 512 && m >= 512 && n <= CURVE_MAX_POINTS && m <= CURVE_MAX_POINTS &&
-           (m + NG_CELL - 1) / NG_CELL <= NG_MAX_CELLS && (n + NG_CELL - 1) / NG_CELL <= NG_MAX_CELLS;
+    // Small clouds are served as fast by the all-pairs scan; the box distances of very large ones
+    // do not fit in LDS.
+    return b > 0 && n >= 512 && m >= 512 && grid_cells(n) <= NG_MAX_CELLS && grid_cells(m) <= NG_MAX_CELLS;
 }
 
 } // namespace
@@ -654,19 +672,22 @@ int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xy
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
-    PointSet a{xyz1, nullptr, static_cast<int64_t>(b) * n, n, n, reinterpret_cast<float4*>(w + l.sorted_a),
+    PointSet a{xyz1, nullptr, static_cast<int64_t>(b) * n, n, grid_stride(n), reinterpret_cast<float4*>(w + l.sorted_a),
                reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
-    PointSet c{xyz2, nullptr, static_cast<int64_t>(b) * m, m, m, reinterpret_cast<float4*>(w + l.sorted_b),
+    PointSet c{xyz2, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted_b),
                reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
     int st = launch_curve_cells(a, c, nullptr, s);
     if (st != TPK_OK)
         return st;
-    const int64_t waves = static_cast<int64_t>((n + NG_CELL - 1) / NG_CELL + (m + NG_CELL - 1) / NG_CELL) * b;
+    const int cells1 = grid_cells(n), cells2 = grid_cells(m);
+    const int64_t waves = static_cast<int64_t>(cells1 + cells2) * b;
     const int64_t blocks = tpk_ceil_div(waves, NG_SCAN_THREADS / TPK_WAVE);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(chamfer_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, n,
-                       m, b, a.sorted, c.sorted, a.boxes, c.boxes, dist1, dist2, idx1, idx2);
+    const size_t lds = static_cast<size_t>(NG_SCAN_THREADS / TPK_WAVE) *
+                       ((std::max(cells1, cells2) + NG_CELL - 1) / NG_CELL * NG_CELL) * sizeof(float);
+    hipLaunchKernelGGL(chamfer_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
+                       m, cells1, cells2, b, a.sorted, c.sorted, a.boxes, c.boxes, dist1, dist2, idx1, idx2);
     return tpk_launch_status();
 }
 
@@ -684,19 +705,22 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
-    PointSet a{unknown, nullptr, static_cast<int64_t>(b) * n, n, n, reinterpret_cast<float4*>(w + l.sorted_a),
+    PointSet a{unknown, nullptr, static_cast<int64_t>(b) * n, n, grid_stride(n), reinterpret_cast<float4*>(w + l.sorted_a),
                reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
-    PointSet c{known, nullptr, static_cast<int64_t>(b) * m, m, m, reinterpret_cast<float4*>(w + l.sorted_b),
+    PointSet c{known, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted_b),
                reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
     int st = launch_curve_cells(a, c, nullptr, s);
     if (st != TPK_OK)
         return st;
-    const int64_t waves = static_cast<int64_t>((n + NG_CELL - 1) / NG_CELL) * b;
+    const int qcells = grid_cells(n), ccells = grid_cells(m);
+    const int64_t waves = static_cast<int64_t>(qcells) * b;
     const int64_t blocks = tpk_ceil_div(waves, NG_SCAN_THREADS / TPK_WAVE);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(three_nn_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, n,
-                       m, b, a.sorted, c.sorted, a.boxes, c.boxes, dist2, idx);
+    const size_t lds = static_cast<size_t>(NG_SCAN_THREADS / TPK_WAVE) * ((ccells + NG_CELL - 1) / NG_CELL * NG_CELL) *
+                       sizeof(float);
+    hipLaunchKernelGGL(three_nn_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
+                       m, qcells, ccells, b, a.sorted, c.sorted, a.boxes, c.boxes, dist2, idx);
     return tpk_launch_status();
 }
 
