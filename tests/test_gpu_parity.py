@@ -246,6 +246,7 @@ def test_ball_query_full_config4(tpk, oracle, dev):
         ((16384, 16384), 0.1, 0.05, 1),
         (tuple([50] * 200), 1.0, 0.3, 16),          # many tiny clouds in one window
         ((40000,), 0.3, 0.012, 32),                 # most balls hold the query point only
+        ((90000, 20000), 0.05, 0.04, 32),           # 6 windows x 27 bins: more (window, bin) pairs than lanes
     ],
 )
 def test_ball_query_partial_cell_search_parity(tpk, oracle, dev, sizes, qfrac, r, ns):

@@ -401,8 +401,9 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
 // query's cloud.  The hits (at most 64) are collected in LDS, ranked by row, and written in
 // ascending row order, then -1: the rows a serial scan in index order that stops after nsample
 // hits (cuda/src/ball_query_gpu.cu:54-95) would have produced.
-// A query whose ball touches more than 64 bins of a window, or that has more than 64 hits, is
-// answered by that serial scan itself, 64 rows per step with early exit: those are the dense
+// The (window, bin) pairs of a query are walked 64 at a time.  A query whose ball touches more
+// than 64 bins of one window or 512 in all, or that has more than 64 hits, is answered by that
+// serial scan itself, 64 rows per step with early exit: those are the dense
 // neighbourhoods, where the scan ends soon.
 // ---------------------------------------------------------------------------------------
 constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
@@ -500,16 +501,19 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
         }
         const int pairs_before = wave_exclusive_sum(nbins);
         const int pairs = __builtin_amdgcn_readlane(pairs_before + nbins, TPK_WAVE - 1);
-        serial = pairs > TPK_WAVE;
-        if (!serial)
+        // (a ball that touches more than 64 bins of one window, or 512 in all, covers so much of
+        // its cloud that the scan in index order ends early)
+        serial = __ballot(nbins > TPK_WAVE) != 0 || pairs > 8 * TPK_WAVE;
+        // 64 (window, bin) pairs at a time
+        for (int pair0 = 0; pair0 < pairs && !serial; pair0 += TPK_WAVE)
         {
-            // one descriptor per (window, bin) pair, written by the window's lane
-            for (int i = 0; i < nbins; ++i)
-                slots[pairs_before + i] = block | (i << 20);
+            // one descriptor per pair, written by the window's lane
+            for (int i = max(0, pair0 - pairs_before); i < nbins && pairs_before + i < pair0 + TPK_WAVE; ++i)
+                slots[pairs_before + i - pair0] = block | (i << 20);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            // lane p: where the points of pair p start in the ordered array, and how many
+            // lane p: where the points of pair pair0 + p start in the ordered array, and how many
             int start = 0, size = 0;
-            if (lane < pairs)
+            if (pair0 + lane < pairs)
             {
                 const int d = slots[lane];
                 const int fx = d & 15, fy = (d >> 4) & 15, fz = (d >> 8) & 15;
