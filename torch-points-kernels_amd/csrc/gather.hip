@@ -17,9 +17,9 @@
 // per-target lists (for target position i the columns j that reference it, with their
 // weights) using LDS *integer* atomics, which are fast, and an LDS prefix sum, laid out so that
 // one lane per target can walk them with coalesced reads (lists.h); the main kernel then
-// stages rows of grad_out in LDS - whole rows when up to 128 KiB of them fit, else one row in
-// pieces of 64 KiB with lists per piece - and every lane sums the listed columns of its
-// target.  No float atomics, no zero fill, each output written by one lane.  The lists cost
+// stages rows of grad_out in LDS - four rows in pieces of 8192 columns, or one longer row in
+// pieces of 16384 columns, with lists per piece - and every lane sums the listed columns of
+// its target.  No float atomics, no zero fill, each output written by one lane.  The lists cost
 // about 3 entries of 8 bytes (4 unweighted) per index entry of workspace, passed in by the
 // caller.  The order in which a target's terms are added differs from run to run only through
 // the order of its list, as with the reference's global atomics
@@ -180,8 +180,8 @@ constexpr int GB_STEPS = L_WIDTH_STEP;  // list slots per request group (widths 
 // of every row).  The few lists longer than the block's padded part are then summed by the
 // whole wavefront, 64 entries at a time.  Results leave as one contiguous store per feature
 // row; parts after the first add to what the same lane stored for the part before.
-// Two workgroups share a compute unit (64 KiB of LDS and 64 registers each): one stages while
-// the other walks its lists, and 32 wavefronts hide the latency of the entry reads.
+// With pieces of 64 KiB two workgroups share a compute unit (64 registers each): one stages
+// while the other walks its lists, and 32 wavefronts hide the latency of the entry reads.
 // dynamic LDS: R * (part_len + 4) floats.
 template <int K, bool WEIGHTED, int R>
 __global__ __launch_bounds__(G_THREADS, 2) void gather_bwd_lists_kernel(
@@ -425,11 +425,12 @@ struct BwdShape
 BwdShape bwd_shape(int64_t n)
 {
     BwdShape sh;
-    // Whole rows while up to 128 KiB of them fit (lists over whole rows have the least padding);
-    // longer rows go one at a time in pieces of 64 KiB, two workgroups to a compute unit.
-    sh.rows = n <= GB_BUFFER_FLOATS / 2 ? 4 : n <= GB_BUFFER_FLOATS ? 2 : 1;
+    // Measured on MI355X (config shapes): rows of up to 16384 floats go four at a time in pieces of
+    // 8192 columns (one workgroup per compute unit: the lists of a piece are read once per four
+    // rows); longer rows one at a time in pieces of 16384 columns, two workgroups per compute unit.
+    sh.rows = n <= GB_BUFFER_FLOATS ? 4 : 1;
     const int64_t n4 = (n + 3) & ~static_cast<int64_t>(3);
-    sh.part_len = static_cast<int>(tpk_min64(n4, GB_BUFFER_FLOATS));
+    sh.part_len = static_cast<int>(tpk_min64(n4, sh.rows == 4 ? GB_BUFFER_FLOATS / 2 : GB_BUFFER_FLOATS));
     sh.parts = static_cast<int>(tpk_min64(tpk_ceil_div(n, sh.part_len), 0x7fffffff));
     return sh;
 }
@@ -489,8 +490,6 @@ int gather_bwd(int b, int c, int m, int64_t n, const float* grad_out, const IdxT
         {
             if (sh.rows == 4)
                 return launch_bwd_lists<K, WEIGHTED, 4>(b, c, m, n, sh, grad_out, lists, grad_src, s);
-            if (sh.rows == 2)
-                return launch_bwd_lists<K, WEIGHTED, 2>(b, c, m, n, sh, grad_out, lists, grad_src, s);
             return launch_bwd_lists<K, WEIGHTED, 1>(b, c, m, n, sh, grad_out, lists, grad_src, s);
         }
         if (st != TPK_ERR_UNSUPPORTED)
