@@ -207,24 +207,26 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
     }
     __syncthreads();
 
-    // Prefix sum of the list lengths (every thread owns a run of `per` consecutive targets):
-    // where the entries of every target would start.
-    atomicAdd(&below_total, below);
+    // Prefix sum of the list lengths (every thread owns a run of `per` consecutive targets; sums
+    // inside a wavefront by DPP, across wavefronts through LDS): where the entries of every
+    // target would start.
+    {
+        const int below_before = wave_exclusive_sum(below);
+        if (lane == TPK_WAVE - 1)
+            atomicAdd(&below_total, below_before + below);
+    }
     const int per = (width + G_THREADS - 1) / G_THREADS;
     const int lo = min(tid * per, width), hi = min(lo + per, width);
     int sum = 0;
     for (int t = lo; t < hi; ++t)
         sum += counters[t];
-    scan[tid] = sum;
+    const int before_in_wave = wave_exclusive_sum(sum);
+    if (lane == TPK_WAVE - 1)
+        scan[wave] = before_in_wave + sum;
     __syncthreads();
-    for (int step = 1; step < G_THREADS; step <<= 1)
-    {
-        const int add = tid >= step ? scan[tid - step] : 0;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
-    }
-    int run = below_total + scan[tid] - sum;
+    int run = below_total + before_in_wave;
+    for (int w = 0; w < wave; ++w)
+        run += scan[w];
     for (int t = lo; t < hi; ++t)
     {
         aux[t] = run;
@@ -284,25 +286,35 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
             if constexpr (WEIGHTED)
                 wv[u] = weight[e];
         }
+        // (the cursor updates of a batch are all issued before their results are used)
+        int slot[BATCH];
 #pragma unroll
         for (int u = 0; u < BATCH; ++u)
         {
             const bool mine = iv[u] >= i0 && iv[u] < i1 && e0 + u * G_THREADS < total;
-            if (mine)
+            slot[u] = mine ? atomicAdd(&counters[static_cast<int>(iv[u]) - i0], 1) : -1;
+        }
+        // (and so are the look-ups of where the entries go)
+        int at[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+        {
+            const int t = slot[u] >= 0 ? static_cast<int>(iv[u]) - i0 : 0;
+            const int blk = t / L_BLOCK;
+            const int w = block_width[blk];
+            at[u] = block_start[blk] +
+                    (slot[u] < w ? slot[u] * L_BLOCK + (t & (L_BLOCK - 1)) : w * L_BLOCK + aux[t] + (slot[u] - w));
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+            if (slot[u] >= 0)
             {
-                const int t = static_cast<int>(iv[u]) - i0;
-                const int slot = atomicAdd(&counters[t], 1);
-                const int blk = t / L_BLOCK;
-                const int w = block_width[blk];
-                const int at = block_start[blk] +
-                               (slot < w ? slot * L_BLOCK + (t & (L_BLOCK - 1)) : w * L_BLOCK + aux[t] + (slot - w));
                 ListEntry<WEIGHTED> entry;
                 entry.j = (e0 + u * G_THREADS) / K;
                 if constexpr (WEIGHTED)
                     entry.w = wv[u];
-                entries[at] = entry;
+                entries[at[u]] = entry;
             }
-        }
     }
 }
 
