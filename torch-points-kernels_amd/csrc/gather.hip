@@ -239,10 +239,14 @@ __global__ __launch_bounds__(G_THREADS, 2) void gather_bwd_lists_kernel(
             const ListBlock next_lb = list_block(blocks, min(blk + WAVES, nblocks - 1));
             const ListEntry<WEIGHTED>* __restrict__ e = entries + lb.start + lane;
             const int tgt = blk * L_BLOCK + lane;
-            float acc[R];
+            // (what the parts before stored for these targets is requested now, needed at the end)
+            float acc[R], old[R];
 #pragma unroll
             for (int r = 0; r < R; ++r)
+            {
                 acc[r] = 0.f;
+                old[r] = part > 0 && tgt < m && r < nrows ? d[static_cast<int64_t>(r) * m + tgt] : 0.f;
+            }
             for (int i = 0; i < lb.width; i += STEPS)
             {
                 // all requests of this round, then all the sums (widths are multiples of
@@ -296,10 +300,7 @@ __global__ __launch_bounds__(G_THREADS, 2) void gather_bwd_lists_kernel(
 #pragma unroll
                 for (int r = 0; r < R; ++r)
                     if (r < nrows)
-                    {
-                        float* const out = d + static_cast<int64_t>(r) * m + tgt;
-                        *out = part == 0 ? acc[r] : *out + acc[r];
-                    }
+                        d[static_cast<int64_t>(r) * m + tgt] = old[r] + acc[r];
             }
             lb = next_lb;
         }
