@@ -504,9 +504,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
         // (a ball that touches more than 64 bins of one window, or 512 in all, covers so much of
         // its cloud that the scan in index order ends early)
         serial = __ballot(nbins > TPK_WAVE) != 0 || pairs > 8 * TPK_WAVE;
-        // 64 (window, bin) pairs at a time
-        for (int pair0 = 0; pair0 < pairs && !serial; pair0 += TPK_WAVE)
-        {
+        // 64 (window, bin) pairs at a time; nearly always there are no more than that
+        auto walk_pairs = [&](int pair0) __attribute__((always_inline)) {
             // one descriptor per pair, written by the window's lane
             for (int i = max(0, pair0 - pairs_before); i < nbins && pairs_before + i < pair0 + TPK_WAVE; ++i)
                 slots[pairs_before + i - pair0] = block | (i << 20);
@@ -553,7 +552,11 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 cnt += __builtin_popcountll(mask);
                 serial = cnt > BQB_HITS;
             }
-        }
+        };
+        if (!serial)
+            walk_pairs(0);
+        for (int pair0 = TPK_WAVE; pair0 < pairs && !serial; pair0 += TPK_WAVE)
+            walk_pairs(pair0);
     }
 
     if (!serial)
