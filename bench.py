@@ -36,10 +36,10 @@ PEAK_FP32_TFLOPS = 157.3  # published fp32 figure (vector = matrix); it counts e
 MEASURED_TRAFFIC_BYTES = {
     "fps": 4030000,                    # 3.76 MB read (the clouds; set-up passes mostly hit L2) + 0.26 MB written (the indices)
     "three_interpolate_fwd": 174130000,  # = algorithmic bytes: nothing is read twice from HBM
-    "three_interpolate_bwd": 292600000,  # list build 96 MB + list walk 196 MB (lists re-read per row pair)
+    "three_interpolate_bwd": 308500000,  # list build 57 MB + list walk 252 MB (two column pieces per four rows)
     "grouping_fwd": 352500000,         # rows staged twice (two column halves per row block)
-    "grouping_bwd": 407300000,         # list build 26 MB + walk 381 MB (two column pieces per row: outputs written twice)
-    "chamfer_bwd": 142000000,          # list build 80.6 MB (padded lists) + list walk 61.4 MB
+    "grouping_bwd": 407900000,         # list build 27 MB + walk 381 MB (two column pieces per row: outputs written twice)
+    "chamfer_bwd": 128000000,          # list build 72.4 MB (padded lists) + list walk 55.6 MB
 }
 
 
