@@ -87,24 +87,31 @@ __device__ __forceinline__ void scan_run(Tile& tile, const float* __restrict__ s
             break;
         const int tcnt = static_cast<int>(tpk_min64(BQ_TILE, s1 - base));
         const int tpad = (tcnt + TPK_WAVE - 1) & ~(TPK_WAVE - 1);
-        for (int t = tid; t < tpad; t += BQ_THREADS)
+        // (the loads of a whole tile are issued before the first LDS write: one memory latency per
+        // tile, not one per 256 points)
+        constexpr int PER_THREAD = BQ_TILE / BQ_THREADS;
+        float px[PER_THREAD], py[PER_THREAD], pz[PER_THREAD];
+#pragma unroll
+        for (int u = 0; u < PER_THREAD; ++u)
         {
-            float px, py, pz;
-            if (t < tcnt)
-            {
-                const float* src = support + (base + t) * 3;
-                px = src[0];
-                py = src[1];
-                pz = src[2];
-            }
-            else
+            const int t = min(tid + u * BQ_THREADS, tcnt - 1);
+            const float* src = support + (base + t) * 3;
+            px[u] = src[0];
+            py[u] = src[1];
+            pz[u] = src[2];
+        }
+#pragma unroll
+        for (int u = 0; u < PER_THREAD; ++u)
+        {
+            const int t = tid + u * BQ_THREADS;
+            if (t < tpad)
             {
                 // Padding: infinitely far away, fails both radius tests.
-                px = py = pz = __builtin_inff();
+                const bool real = t < tcnt;
+                tile.x[t] = real ? px[u] : __builtin_inff();
+                tile.y[t] = real ? py[u] : __builtin_inff();
+                tile.z[t] = real ? pz[u] : __builtin_inff();
             }
-            tile.x[t] = px;
-            tile.y[t] = py;
-            tile.z[t] = pz;
         }
         __syncthreads();
 
