@@ -133,11 +133,17 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
         const int c = g * NG_CELL + lane;
         const bool valid = c < ccells;
         const int cc = valid ? c : 0;
-        const float lb = box_box_dist2(qlo, qhi, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
+        const float4 clo = cbox[cc * NG_BOX + 0], chi = cbox[cc * NG_BOX + 1];
+        const float lb = box_box_dist2(qlo, qhi, clo, chi);
         lows[c] = valid ? lb : __builtin_inff();
-        // approximately the nearest cell (the six lowest bits of the distance carry g)
-        const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~63u) | static_cast<unsigned>(g);
-        seed_key = valid && key < seed_key ? key : seed_key;
+        // The first cell to scan: the one whose box centre is nearest to the centre of the queries'
+        // box (many boxes overlap it; a good first answer lets the lanes turn most of them down).
+        // The six lowest bits of the distance carry g.
+        const float ex = (clo.x + chi.x) - (qlo.x + qhi.x), ey = (clo.y + chi.y) - (qlo.y + qhi.y);
+        const float ez = (clo.z + chi.z) - (qlo.z + qhi.z);
+        const float centre = __builtin_fmaf(ex, ex, __builtin_fmaf(ey, ey, ez * ez));
+        const unsigned key = (static_cast<unsigned>(__float_as_int(centre)) & ~63u) | static_cast<unsigned>(g);
+        seed_key = valid && lb < __builtin_inff() && key < seed_key ? key : seed_key;
     }
     Nearest s;
     s.best = qindex == 0x7FFFFFFF ? -1.f : __builtin_inff(); // (a padding lane never asks for a scan)
@@ -336,10 +342,15 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
         const int c = g * NG_CELL + lane;
         const bool valid = c < ccells;
         const int cc = valid ? c : 0;
-        const float lb = box_box_dist2(qlo, qhi, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
+        const float4 clo = cbox[cc * NG_BOX + 0], chi = cbox[cc * NG_BOX + 1];
+        const float lb = box_box_dist2(qlo, qhi, clo, chi);
         lows[c] = valid ? lb : __builtin_inff();
-        const unsigned key = (static_cast<unsigned>(__float_as_int(lb)) & ~63u) | static_cast<unsigned>(g);
-        seed_key = valid && key < seed_key ? key : seed_key;
+        // the first cell to scan: nearest box centre (the six lowest bits of the distance carry g)
+        const float ex = (clo.x + chi.x) - (qlo.x + qhi.x), ey = (clo.y + chi.y) - (qlo.y + qhi.y);
+        const float ez = (clo.z + chi.z) - (qlo.z + qhi.z);
+        const float centre = __builtin_fmaf(ex, ex, __builtin_fmaf(ey, ey, ez * ez));
+        const unsigned key = (static_cast<unsigned>(__float_as_int(centre)) & ~63u) | static_cast<unsigned>(g);
+        seed_key = valid && lb < __builtin_inff() && key < seed_key ? key : seed_key;
     }
     Nearest3 s;
     s.b1 = s.b2 = s.b3 = qindex == 0x7FFFFFFF ? -1.f : __builtin_inff(); // (a padding lane never asks for a scan)
