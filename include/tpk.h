@@ -110,6 +110,23 @@ int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* kno
                      void* stream);
 
 /* ---------------------------------------------------------------------------------------
+ * k nearest neighbours, dense layout.
+ * Replaces dense_knn(support, query, k) (cpu/src/knn.cpp:43-62, bound in
+ * cpu/src/bindings.cpp; torch_points_kernels/knn.py:4-18 refuses CUDA tensors: the reference
+ * has no GPU implementation of this operator).
+ *   support (b, n_support, 3)   query (b, m_query, 3)
+ *   idx (b, m_query, k) int64   dist2 (b, m_query, k) float32 squared distances
+ * Entries ascend by (squared distance, index): equal distances keep the lower index first, the
+ * rule of three_nn (nanoflann leaves that order open).  k > n_support is TPK_ERR_INVALID_ARG
+ * (cpu/src/knn.cpp:12-14 raises).  `workspace` (tpk_knn_workspace_bytes() bytes - 0 for shapes
+ * not served that way -, 256-byte aligned): search over curve-ordered cells instead of all
+ * pairs, same results.
+ * ------------------------------------------------------------------------------------- */
+size_t tpk_knn_workspace_bytes(int b, int n_support, int m_query);
+int tpk_knn_f32(int b, int n_support, int m_query, int k, const float* support, const float* query,
+                int64_t* idx, float* dist2, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------
  * Three-point interpolation, forward and backward.
  * Replace three_interpolate_kernel_wrapper(b, c, m, n, points, idx, weight, out) and
  * three_interpolate_grad_kernel_wrapper(b, c, n, m, grad_out, idx, weight, grad_points)

@@ -141,6 +141,22 @@ def three_nn(unknown, known):
     return dist2, idx
 
 
+def knn(support, query, k):
+    """-> (idx int64 (B,m,k), dist2 f32 (B,m,k)), ascending by (distance, index)."""
+    support = _c(support, np.float32)
+    query = _c(query, np.float32)
+    b, n, _ = support.shape
+    m = query.shape[1]
+    idx = np.empty((b, m, k), np.int64)
+    dist2 = np.empty((b, m, k), np.float32)
+    lib().tpk_oracle_knn.restype = ctypes.c_int
+    rc = lib().tpk_oracle_knn(ctypes.c_int(b), ctypes.c_int(n), ctypes.c_int(m), ctypes.c_int(k),
+                              _p(support, _f32p), _p(query, _f32p), _p(idx, _i64p), _p(dist2, _f32p))
+    if rc != 0:
+        raise RuntimeError("Not enough points in support to find %d neighboors" % k)
+    return idx, dist2
+
+
 def three_interpolate(points, idx, weight):
     points = _c(points, np.float32)
     idx = _c(idx, np.int32)

@@ -235,6 +235,54 @@ int tpk_oracle_fps(int b, int n, int m, const float* xyz, int32_t* out)
 }
 
 /* ------------------------------------------------------------------------- */
+/* k nearest neighbours, dense layout: the three_nn scan above with k entries.   */
+/* The reference has this operator on the CPU only (torch_points_kernels/       */
+/* knn.py:4-18, cpu/src/knn.cpp:8-62, nanoflann's knnSearch underneath); the     */
+/* support points are visited in index order and enter the list only when        */
+/* strictly smaller than an entry, so equal distances keep the lower index       */
+/* first (nanoflann leaves the order of exactly equal distances open).           */
+/* support (b,n,3), query (b,m,3); idx (b,m,k) int64, dist2 (b,m,k) ascending.   */
+/* Returns -1 when k > n (cpu/src/knn.cpp:12-14 raises), else 0.                 */
+/* ------------------------------------------------------------------------- */
+int tpk_oracle_knn(int b, int n, int m, int k, const float* support, const float* query,
+                   int64_t* idx, float* dist2)
+{
+    if (k > n)
+        return -1;
+    for (int bi = 0; bi < b; ++bi)
+    {
+        const float* s = support + (int64_t)bi * n * 3;
+        const float* q = query + (int64_t)bi * m * 3;
+        for (int j = 0; j < m; ++j)
+        {
+            const float ux = q[j * 3 + 0], uy = q[j * 3 + 1], uz = q[j * 3 + 2];
+            float* d = dist2 + ((int64_t)bi * m + j) * k;
+            int64_t* ix = idx + ((int64_t)bi * m + j) * k;
+            int have = 0;
+            for (int p = 0; p < n; ++p)
+            {
+                const float x = s[p * 3 + 0], y = s[p * 3 + 1], z = s[p * 3 + 2];
+                const float dd = (ux - x) * (ux - x) + (uy - y) * (uy - y) + (uz - z) * (uz - z);
+                if (have == k && !(dd < d[k - 1]))
+                    continue;
+                int at = have < k ? have : k - 1;
+                while (at > 0 && dd < d[at - 1])
+                {
+                    d[at] = d[at - 1];
+                    ix[at] = ix[at - 1];
+                    --at;
+                }
+                d[at] = dd;
+                ix[at] = p;
+                if (have < k)
+                    ++have;
+            }
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
 /* three nearest neighbours.  cuda/src/interpolate_gpu.cu:9-65; outputs        */
 /* zero-initialised (cuda/src/interpolate.cpp:22-25).  unknown (b,n,3), known  */
 /* (b,m,3); dist2 (b,n,3) squared distances ascending, idx (b,n,3) int32.      */

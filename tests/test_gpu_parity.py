@@ -590,6 +590,54 @@ def test_grouping_full_config3b(tpk, oracle, dev):
     _assert_scatter_sum_close(_np(f.grad), want, abs_sum)
 
 
+# ------------------------------------------------------------------ knn (general k)
+
+
+@pytest.mark.parametrize("B,n,m,k", [(1, 3, 1, 3), (2, 40, 70, 5), (2, 300, 515, 16), (1, 1000, 100, 33), (2, 70, 9, 70),
+                                     (2, 512, 512, 1), (3, 1000, 777, 8), (1, 4096, 2500, 16), (2, 600, 700, 40),
+                                     (1, 20000, 900, 12), (1, 3000, 17000, 4)])
+def test_knn_parity(tpk, oracle, dev, B, n, m, k):
+    # n support points, m queries; below 512 points all pairs are tested, above the search goes over cells
+    g = torch.Generator().manual_seed(n + m + k)
+    for support, query in ((torch.rand(B, n, 3, generator=g), torch.rand(B, m, 3, generator=g)),
+                           (_clustered(g, B, n), _clustered(g, B, m))):
+        idx, dist2 = tpk.knn(support.to(dev), query.to(dev), k)
+        wi, wd = oracle.knn(support.numpy(), query.numpy(), k)
+        assert idx.dtype == torch.int64 and idx.shape == (B, m, k)
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist2), wd)
+
+
+def test_knn_ties_and_errors(tpk, oracle, dev):
+    # reference test/test_knn.py:14-23
+    support = torch.tensor([[[0, 0, 0], [1, 0, 0], [2, 0, 0]]]).float().to(dev)
+    query = torch.tensor([[[0, 0, 0]]]).float().to(dev)
+    idx, dist = tpk.knn(support, query, 3)
+    assert idx.tolist() == [[[0, 1, 2]]] and dist.tolist() == [[[0.0, 1.0, 4.0]]]
+    assert tpk.knn(support, query, 2)[0].tolist() == [[[0, 1]]]
+    with pytest.raises(RuntimeError):
+        tpk.knn(support, query, 5)
+    with pytest.raises(NotImplementedError):
+        tpk.knn(support.cpu(), query.cpu(), 2)
+    # equal distances everywhere: tripled points, lattices, a collapsed cloud; small and large clouds
+    g = torch.Generator().manual_seed(8)
+    base = torch.rand(1, 400, 3, generator=g)
+    tripled = torch.cat([base, base.flip(1), base], 1)[:, torch.randperm(1200, generator=g)]
+    ax = torch.arange(10, dtype=torch.float32)
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3)
+    big = torch.rand(1, 6000, 3, generator=g)
+    big3 = torch.cat([big, big.flip(1), big], 1)[:, torch.randperm(18000, generator=g)]
+    cases = [(tripled, torch.rand(1, 600, 3, generator=g), 7), (lattice, lattice + 0.5, 9), (lattice, lattice, 27),
+             (torch.full((1, 600, 3), 0.5), torch.rand(1, 520, 3, generator=g), 40),
+             (tripled[:, :300], base[:, :50], 10), (big3, big[:, :700], 5)]
+    for support, query, k in cases:
+        support, query = support.contiguous(), query.contiguous()
+        idx, dist2 = tpk.knn(support.to(dev), query.to(dev), k)
+        wi, wd = oracle.knn(support.numpy(), query.numpy(), k)
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist2), wd)
+
+
 # ------------------------------------------------------------------ chamfer
 
 

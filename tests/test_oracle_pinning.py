@@ -267,6 +267,61 @@ def test_three_nn_vs_reference_cpu_module(oracle, ref_cpu):
     np.testing.assert_array_equal(idx, idx_r.numpy())
 
 
+# ----------------------------------------------------------------------------- knn (general k)
+
+
+def test_knn_reference_kat(oracle):
+    # reference test/test_knn.py:14-23
+    support = np.array([[[0, 0, 0], [1, 0, 0], [2, 0, 0]]], np.float32)
+    query = np.array([[[0, 0, 0]]], np.float32)
+    idx, dist2 = oracle.knn(support, query, 3)
+    np.testing.assert_array_equal(idx, [[[0, 1, 2]]])
+    np.testing.assert_array_equal(dist2, [[[0.0, 1.0, 4.0]]])
+    idx, _ = oracle.knn(support, query, 2)
+    np.testing.assert_array_equal(idx, [[[0, 1]]])
+    with pytest.raises(RuntimeError):
+        oracle.knn(support, query, 5)
+
+
+def test_knn_is_a_stable_sort_of_the_distances(oracle):
+    # ascending (distance, index) = a stable argsort of the fp32 distances; duplicated points and a
+    # quantised cloud give many exactly equal distances
+    rng = np.random.default_rng(5)
+    base = rng.random((2, 60, 3)).astype(np.float32)
+    support = np.concatenate([base, base[:, ::-1], np.round(rng.random((2, 50, 3)) * 4).astype(np.float32) / 4], 1)
+    query = np.concatenate([base[:, :20], rng.random((2, 30, 3)).astype(np.float32)], 1)
+    for k in (1, 7, 33, support.shape[1]):
+        idx, dist2 = oracle.knn(support, query, k)
+        dx, dy, dz = (query[:, :, None, a] - support[:, None, :, a] for a in range(3))
+        full = (dx * dx + dy * dy) + dz * dz  # fp32, unfused, the oracle's order of operations
+        order = np.argsort(full, axis=2, kind="stable")[:, :, :k]
+        np.testing.assert_array_equal(idx, order)
+        np.testing.assert_array_equal(dist2, np.take_along_axis(full, order, 2))
+
+
+def test_knn_with_three_neighbours_is_three_nn(oracle):
+    rng = np.random.default_rng(6)
+    known = np.round(rng.random((3, 90, 3)) * 6).astype(np.float32) / 3  # ties included
+    unknown = rng.random((3, 70, 3)).astype(np.float32) * 2
+    idx, dist2 = oracle.knn(known, unknown, 3)
+    d3, i3 = oracle.three_nn(unknown, known)
+    np.testing.assert_array_equal(idx, i3)
+    np.testing.assert_array_equal(dist2, d3)
+
+
+def test_knn_vs_reference_cpu_module(oracle, ref_cpu):
+    # tie-free data: nanoflann's order is then fixed by the distances alone
+    _need_ref(ref_cpu)
+    g = torch.Generator().manual_seed(17)
+    support = torch.randn(3, 400, 3, generator=g)
+    query = torch.randn(3, 150, 3, generator=g)
+    for k in (1, 5, 16, 40):
+        idx_r, dist2_r = ref_cpu.dense_knn(support, query, k)
+        idx, dist2 = oracle.knn(support.numpy(), query.numpy(), k)
+        np.testing.assert_array_equal(dist2, dist2_r.numpy())
+        np.testing.assert_array_equal(idx, idx_r.numpy())
+
+
 # ----------------------------------------------------------------------------- interpolate
 
 

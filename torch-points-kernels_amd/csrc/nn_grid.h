@@ -19,6 +19,12 @@ size_t tpk_grid_three_nn_workspace_bytes(int b, int n, int m);
 int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2,
                       int32_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+// k nearest neighbours, float32 (n queries, m support points per cloud; idx int64, both outputs
+// (b, n, k), ascending by (squared distance, index)): same conventions.
+size_t tpk_grid_knn_workspace_bytes(int b, int n, int m);
+int tpk_grid_knn(int b, int n, int m, int k, const float* query, const float* support, float* dist2,
+                 int64_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);
+
 // Ball query, packed layout (a hit has squared distance <= radius2 = radius * radius as the caller
 // rounds it): same conventions.  Queries with dense neighbourhoods are answered by a scan in
 // index order inside the same kernel.

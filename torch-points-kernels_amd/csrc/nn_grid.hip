@@ -26,6 +26,7 @@
 #include <algorithm>
 #include <cmath>
 #include "nn_grid.h"
+#include "topk.h"
 
 namespace {
 
@@ -400,6 +401,155 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// k nearest neighbours over cells: three_nn's search with a list of up to 32 entries per lane
+// (topk.h).  A larger k is served in rounds: round r finds the entries 32 r .. 32 r + 31, which
+// are the smallest pairs after the last one of the round before.  A cell is skipped when its box
+// is further away than the last kept entry of every lane.
+// ---------------------------------------------------------------------------------------
+template <int K>
+__device__ __forceinline__ void scan_cell_k(const float4* __restrict__ cand, const float4* __restrict__ boxes,
+                                            int cell, float4* stage, int lane, float qx, float qy, float qz,
+                                            NearestK<K>& s)
+{
+    stage[lane] = cand[cell * NG_CELL + lane];
+    const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
+    {
+        // a run of 16 candidates whose box no lane's last entry reaches is passed over
+        if ((ch & 1) == 0)
+        {
+            const float lb = point_box_dist2(qx, qy, qz, quarter[ch], quarter[ch + 1]);
+            if (__ballot(lb * NG_MARGIN <= s.d[K - 1]) == 0)
+            {
+                ++ch;
+                continue;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NG_CHUNK; ++c)
+        {
+            const float4 p = stage[ch * NG_CHUNK + c];
+            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            const int ci = __float_as_int(p.w);
+            const bool in = s.admits(d, ci);
+            if (__ballot(in) == 0)
+                continue;
+            if (in)
+                s.insert(d, ci);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One wavefront = the 64 queries of one cell; logical wavefront = cloud * qcells + cell.
+// first: number of entries found by earlier rounds; count: entries this round finds (<= K).
+template <int K>
+__global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
+    int n, int k, int first, int count, int qcells, int ccells, int clouds,
+    const float4* __restrict__ sorted_query, const float4* __restrict__ sorted_support,
+    const float4* __restrict__ boxes_query, const float4* __restrict__ boxes_support,
+    float* __restrict__ dist2, int64_t* __restrict__ idx)
+{
+    __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
+    extern __shared__ float lows_all[]; // [wavefronts][candidate cells, in whole groups of 64]
+
+    const int lane = threadIdx.x & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
+    const int64_t task = static_cast<int64_t>(xcd_local_block(blockIdx.x, gridDim.x)) *
+                             (NG_SCAN_THREADS / TPK_WAVE) + wave;
+    if (task >= static_cast<int64_t>(qcells) * clouds)
+        return; // (no workgroup barrier anywhere in this kernel)
+    const int cloud = static_cast<int>(task / qcells);
+    const int qcell = static_cast<int>(task - static_cast<int64_t>(cloud) * qcells);
+    const float4* __restrict__ qpts = sorted_query + static_cast<int64_t>(cloud) * qcells * NG_CELL;
+    const float4* __restrict__ qbox = boxes_query + static_cast<int64_t>(cloud) * qcells * NG_BOX;
+    const float4* __restrict__ cpts = sorted_support + static_cast<int64_t>(cloud) * ccells * NG_CELL;
+    const float4* __restrict__ cbox = boxes_support + static_cast<int64_t>(cloud) * ccells * NG_BOX;
+    dist2 += static_cast<int64_t>(cloud) * n * k;
+    idx += static_cast<int64_t>(cloud) * n * k;
+    float4* const stage = stages[wave];
+    float* const lows = lows_all + wave * ((ccells + NG_CELL - 1) / NG_CELL * NG_CELL);
+
+    const float4 query = qpts[qcell * NG_CELL + lane];
+    const float qx = query.x, qy = query.y, qz = query.z;
+    const int qindex = __float_as_int(query.w); // 0x7FFFFFFF: padding, nothing to store
+    if (__ballot(qindex != 0x7FFFFFFF) == 0)
+        return; // a cell without points (the last window of a cloud may have some)
+    const bool real = qindex != 0x7FFFFFFF;
+    const float4 qlo = qbox[qcell * NG_BOX + 0], qhi = qbox[qcell * NG_BOX + 1];
+
+    NearestK<K> s;
+    {
+        // the last pair of the round before (rounds of one call run one after the other)
+        const int64_t at = static_cast<int64_t>(real ? qindex : 0) * k + first - 1;
+        const bool later = first > 0 && real;
+        s.reset(later ? dist2[at] : -1.f, later ? static_cast<int>(idx[at]) : -1, !real);
+    }
+
+    const int groups = (ccells + NG_CELL - 1) / NG_CELL;
+    unsigned seed_key = 0xFFFFFFFFu;
+    for (int g = 0; g < groups; ++g)
+    {
+        const int c = g * NG_CELL + lane;
+        const bool valid = c < ccells;
+        const int cc = valid ? c : 0;
+        const float4 clo = cbox[cc * NG_BOX + 0], chi = cbox[cc * NG_BOX + 1];
+        const float lb = box_box_dist2(qlo, qhi, clo, chi);
+        lows[c] = valid ? lb : __builtin_inff();
+        // the first cell to scan: nearest box centre (the six lowest bits of the distance carry g)
+        const float ex = (clo.x + chi.x) - (qlo.x + qhi.x), ey = (clo.y + chi.y) - (qlo.y + qhi.y);
+        const float ez = (clo.z + chi.z) - (qlo.z + qhi.z);
+        const float centre = __builtin_fmaf(ex, ex, __builtin_fmaf(ey, ey, ez * ez));
+        const unsigned key = (static_cast<unsigned>(__float_as_int(centre)) & ~63u) | static_cast<unsigned>(g);
+        seed_key = valid && lb < __builtin_inff() && key < seed_key ? key : seed_key;
+    }
+    {
+        const unsigned lowest = wave_min_u32(seed_key);
+        int seed = static_cast<int>(lowest & 63u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
+        if (seed >= ccells)
+            seed = 0;
+        scan_cell_k<K>(cpts, cbox, seed, stage, lane, qx, qy, qz, s);
+        if (lane == (seed & (NG_CELL - 1)))
+            lows[seed] = __builtin_inff();
+    }
+    for (int phase = 0; phase < 2; ++phase)
+        for (int g = 0; g < groups; ++g)
+        {
+            const float lw = lows[g * NG_CELL + lane];
+            float bound = __int_as_float(wave_max_i32(__float_as_int(s.d[K - 1])));
+            unsigned long long live =
+                __ballot(lw < __builtin_inff() && (phase == 0 ? lw == 0.f : lw * NG_MARGIN <= bound));
+            while (live != 0)
+            {
+                const int bit = __builtin_ctzll(live);
+                const int c = g * NG_CELL + bit;
+                live &= live - 1;
+                const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
+                if (__ballot(lb * NG_MARGIN <= s.d[K - 1]) != 0)
+                    scan_cell_k<K>(cpts, cbox, c, stage, lane, qx, qy, qz, s);
+                if (lane == bit)
+                    lows[c] = __builtin_inff(); // scanned, or useless now and ever after
+                if (phase)
+                {
+                    bound = __int_as_float(wave_max_i32(__float_as_int(s.d[K - 1])));
+                    live &= __ballot(lw * NG_MARGIN <= bound);
+                }
+            }
+        }
+    if (real)
+    {
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+            if (j < count)
+            {
+                dist2[static_cast<int64_t>(qindex) * k + first + j] = s.d[j];
+                idx[static_cast<int64_t>(qindex) * k + first + j] = s.i[j];
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Ball query over bins, packed layout (several clouds back to back, sorted cloud id per point).
 //
 // The support array is cut into windows of CURVE_MAX_POINTS consecutive rows, each ordered on its
@@ -740,6 +890,64 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
     hipLaunchKernelGGL(three_nn_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
                        m, qcells, ccells, b, a.sorted, c.sorted, a.boxes, c.boxes, dist2, idx);
     return tpk_launch_status();
+}
+
+size_t tpk_grid_knn_workspace_bytes(int b, int n, int m)
+{
+    return grid_supported(b, n, m) ? grid_layout(b, n, m).total : 0;
+}
+
+namespace {
+
+template <int K>
+int launch_knn_grid(int b, int n, int k, int qcells, int ccells, const PointSet& a, const PointSet& c,
+                    float* dist2, int64_t* idx, hipStream_t s)
+{
+    const int64_t waves = static_cast<int64_t>(qcells) * b;
+    const int64_t blocks = tpk_ceil_div(waves, NG_SCAN_THREADS / TPK_WAVE);
+    if (blocks > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    const size_t lds = static_cast<size_t>(NG_SCAN_THREADS / TPK_WAVE) * ((ccells + NG_CELL - 1) / NG_CELL * NG_CELL) *
+                       sizeof(float);
+    for (int first = 0; first < k; first += K)
+    {
+        hipLaunchKernelGGL(knn_grid_kernel<K>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
+                           k, first, k - first < K ? k - first : K, qcells, ccells, b, a.sorted, c.sorted, a.boxes,
+                           c.boxes, dist2, idx);
+        const int st = tpk_launch_status();
+        if (st != TPK_OK)
+            return st;
+    }
+    return TPK_OK;
+}
+
+} // namespace
+
+// n queries and m support points per cloud.
+int tpk_grid_knn(int b, int n, int m, int k, const float* query, const float* support, float* dist2,
+                 int64_t* idx, void* workspace, size_t workspace_bytes, hipStream_t s)
+{
+    if (!grid_supported(b, n, m) || static_cast<int64_t>(b) * 2 > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    const GridLayout l = grid_layout(b, n, m);
+    if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return TPK_ERR_WORKSPACE;
+    char* w = static_cast<char*>(workspace);
+    PointSet a{query, nullptr, static_cast<int64_t>(b) * n, n, grid_stride(n), reinterpret_cast<float4*>(w + l.sorted_a),
+               reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
+    PointSet c{support, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted_b),
+               reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
+    int st = launch_curve_cells(a, c, nullptr, s);
+    if (st != TPK_OK)
+        return st;
+    const int qcells = grid_cells(n), ccells = grid_cells(m);
+    if (k <= 4)
+        return launch_knn_grid<4>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
+    if (k <= 8)
+        return launch_knn_grid<8>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
+    if (k <= 16)
+        return launch_knn_grid<16>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
+    return launch_knn_grid<KNN_MAX_K>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
 }
 
 namespace {

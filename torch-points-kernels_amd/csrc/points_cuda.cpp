@@ -120,6 +120,42 @@ std::vector<at::Tensor> three_nn(at::Tensor unknowns, at::Tensor knows)
     return {dist2, idx};
 }
 
+// cpu/src/knn.cpp:43-62 (dense_knn; the reference has it for CPU tensors only)
+std::pair<at::Tensor, at::Tensor> dense_knn(at::Tensor support, at::Tensor query, int64_t k)
+{
+    check_contiguous(support, "support");
+    check_contiguous(query, "query");
+    check_f32(support, "support");
+    check_f32(query, "query");
+    check_gpu(support, "support");
+    check_gpu(query, "query");
+    check_same_device(support, query, "support and query");
+    check_points(support, 3, "support");
+    check_points(query, 3, "query");
+    TORCH_CHECK(support.size(0) == query.size(0), "support and query differ in batch size");
+    TORCH_CHECK(k >= 0, "k must not be negative");
+    // cpu/src/knn.cpp:12-14
+    TORCH_CHECK(support.size(1) >= k, "Not enough points in support to find " + std::to_string(k) + " neighboors");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(support.device());
+
+    at::Tensor idx = torch::empty({query.size(0), query.size(1), k},
+                                  at::device(query.device()).dtype(at::ScalarType::Long));
+    at::Tensor dist2 = torch::empty({query.size(0), query.size(1), k},
+                                    at::device(query.device()).dtype(at::ScalarType::Float));
+    const int b = as_int(query.size(0), "batch size");
+    const int n = as_int(support.size(1), "number of support points");
+    const int m = as_int(query.size(1), "number of query points");
+    const size_t ws_bytes = tpk_knn_workspace_bytes(b, n, m);
+    at::Tensor ws;
+    if (ws_bytes)
+        ws = torch::empty({static_cast<int64_t>(ws_bytes)}, query.options().dtype(torch::kUInt8));
+    check_status(tpk_knn_f32(b, n, m, as_int(k, "k"), support.data_ptr<float>(), query.data_ptr<float>(),
+                             idx.data_ptr<int64_t>(), dist2.data_ptr<float>(),
+                             ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, current_stream(query)),
+                 "dense_knn");
+    return std::make_pair(idx, dist2);
+}
+
 // cuda/src/interpolate.cpp:34-54
 at::Tensor three_interpolate(at::Tensor points, at::Tensor idx, at::Tensor weight)
 {
@@ -440,6 +476,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     m.def("furthest_point_sampling", &furthest_point_sampling);
     m.def("three_nn", &three_nn);
+    m.def("dense_knn", &dense_knn);
     m.def("three_interpolate", &three_interpolate);
     m.def("three_interpolate_grad", &three_interpolate_grad);
     m.def("ball_query_dense", &ball_query_dense);

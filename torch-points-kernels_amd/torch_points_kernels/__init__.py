@@ -1,6 +1,6 @@
 """torch_points_kernels for AMD MI355X: the spatial-search operators of
 torch-points3d/torch-points-kernels (furthest point sampling, ball query, three_nn /
-three_interpolate, grouping, Chamfer distance) on hand-written HIP kernels.
+three_interpolate, grouping, Chamfer distance, dense knn) on hand-written HIP kernels.
 
 Same names and call signatures as the reference package (torch_points_kernels/__init__.py);
 GPU tensors only.
@@ -16,6 +16,7 @@ from .torchpoints import (
     three_interpolate,
     three_nn,
 )
+from .knn import knn
 from .chamfer_dist import ChamferFunction
 from . import chamfer_dist  # the reference exports the submodule under this name
 
@@ -25,6 +26,7 @@ __all__ = [
     "grouping_operation",
     "three_interpolate",
     "three_nn",
+    "knn",
     "chamfer_dist",
     "ChamferFunction",
 ]
