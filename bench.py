@@ -198,6 +198,21 @@ def bench_others(dev, steps, warmup, with_cpu):
                              "sample": "%d of 16 clouds, reference cpu/src/knn.cpp (nanoflann k=3), 1 thread" % sub}
     out["three_nn"] = e
 
+    # beyond the BASELINE configurations: dense knn (k = 16) on the clouds of configs[2]a; the reference
+    # has this operator on the CPU only
+    knn_k = 16
+    wall, ev = _time_gpu(lambda: nat.dense_knn(known, unknown, knn_k), steps, warmup)
+    e = {"workload": "dense knn k=16, queries (16,16384,3), support (16,4096,3) (clouds of configs[2]a; not a BASELINE configuration)",
+         "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
+         "roofline": _roof_flops(pairs, 8, ev), "pairs": pairs}
+    e["roofline"]["note"] += PRUNED_NOTE
+    if ref is not None:
+        sub = 4  # clouds
+        secs = _cpu_time(lambda: ref.dense_knn(w["known"][:sub], w["unknown"][:sub], knn_k))
+        e["cpu_baseline"] = {"value": (nq * sub / 16) / secs, "unit": "queries/s", "cores": 1, "kind": "reference",
+                             "sample": "%d of 16 clouds, reference cpu/src/knn.cpp (nanoflann k=16), 1 thread" % sub}
+    out["knn_k16"] = e
+
     dist, idx = tpk.three_nn(unknown, known)
     weight = W.inverse_distance_weights(dist).contiguous()
     feats = w["features"].to(dev)

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(KNN_THREADS) void knn_kernel(
     {
         // the last pair of the round before (rounds of one call run one after the other)
         const int64_t at = static_cast<int64_t>(jj) * k + first - 1;
-        s.reset(first > 0 ? dist2[at] : -1.f, first > 0 ? static_cast<int>(idx[at]) : -1, !real);
+        s.reset(first > 0, first > 0 ? dist2[at] : 0.f, first > 0 ? static_cast<int>(idx[at]) : 0, !real);
     }
 
     for (int base = 0; base < m; base += KNN_TILE)
@@ -71,9 +71,9 @@ __global__ __launch_bounds__(KNN_THREADS) void knn_kernel(
         for (int c = 0; c < cnt; ++c)
         {
             const float4 p = tile[c];
-            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-            if (s.admits(d, base + c))
-                s.insert(d, base + c);
+            const unsigned long long cand = knn_key(tpk_dist2(qx, qy, qz, p.x, p.y, p.z), base + c);
+            if (s.admits(cand))
+                s.insert(cand);
         }
     }
 
@@ -83,8 +83,8 @@ __global__ __launch_bounds__(KNN_THREADS) void knn_kernel(
         for (int e = 0; e < K; ++e)
             if (e < count)
             {
-                dist2[static_cast<int64_t>(j) * k + first + e] = s.d[e];
-                idx[static_cast<int64_t>(j) * k + first + e] = s.i[e];
+                dist2[static_cast<int64_t>(j) * k + first + e] = s.dist(e);
+                idx[static_cast<int64_t>(j) * k + first + e] = s.index(e);
             }
     }
 }

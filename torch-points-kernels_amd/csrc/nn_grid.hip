@@ -413,6 +413,7 @@ __device__ __forceinline__ void scan_cell_k(const float4* __restrict__ cand, con
 {
     stage[lane] = cand[cell * NG_CELL + lane];
     const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
+    float worst = s.worst(); // distance of the lane's last entry
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
     {
@@ -420,24 +421,35 @@ __device__ __forceinline__ void scan_cell_k(const float4* __restrict__ cand, con
         if ((ch & 1) == 0)
         {
             const float lb = point_box_dist2(qx, qy, qz, quarter[ch], quarter[ch + 1]);
-            if (__ballot(lb * NG_MARGIN <= s.d[K - 1]) == 0)
+            if (__ballot(lb * NG_MARGIN <= worst) == 0)
             {
                 ++ch;
                 continue;
             }
         }
+        float mn = 0.f;
 #pragma unroll
         for (int c = 0; c < NG_CHUNK; ++c)
         {
             const float4 p = stage[ch * NG_CHUNK + c];
             const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-            const int ci = __float_as_int(p.w);
-            const bool in = s.admits(d, ci);
+            mn = c == 0 ? d : fminf(mn, d);
+        }
+        if (__ballot(mn <= worst) == 0)
+            continue; // no candidate of this group enters any lane's list
+#pragma unroll
+        for (int c = 0; c < NG_CHUNK; ++c)
+        {
+            const float4 p = stage[ch * NG_CHUNK + c];
+            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            const unsigned long long cand = knn_key(d, __float_as_int(p.w));
+            const bool in = s.admits(cand);
             if (__ballot(in) == 0)
                 continue;
             if (in)
-                s.insert(d, ci);
+                s.insert(cand);
         }
+        worst = s.worst();
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
@@ -484,7 +496,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
         // the last pair of the round before (rounds of one call run one after the other)
         const int64_t at = static_cast<int64_t>(real ? qindex : 0) * k + first - 1;
         const bool later = first > 0 && real;
-        s.reset(later ? dist2[at] : -1.f, later ? static_cast<int>(idx[at]) : -1, !real);
+        s.reset(first > 0, later ? dist2[at] : 0.f, later ? static_cast<int>(idx[at]) : 0, !real);
     }
 
     const int groups = (ccells + NG_CELL - 1) / NG_CELL;
@@ -517,7 +529,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
         for (int g = 0; g < groups; ++g)
         {
             const float lw = lows[g * NG_CELL + lane];
-            float bound = __int_as_float(wave_max_i32(__float_as_int(s.d[K - 1])));
+            float bound = __int_as_float(wave_max_i32(__float_as_int(s.worst())));
             unsigned long long live =
                 __ballot(lw < __builtin_inff() && (phase == 0 ? lw == 0.f : lw * NG_MARGIN <= bound));
             while (live != 0)
@@ -526,13 +538,13 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
                 const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
-                if (__ballot(lb * NG_MARGIN <= s.d[K - 1]) != 0)
+                if (__ballot(lb * NG_MARGIN <= s.worst()) != 0)
                     scan_cell_k<K>(cpts, cbox, c, stage, lane, qx, qy, qz, s);
                 if (lane == bit)
                     lows[c] = __builtin_inff(); // scanned, or useless now and ever after
                 if (phase)
                 {
-                    bound = __int_as_float(wave_max_i32(__float_as_int(s.d[K - 1])));
+                    bound = __int_as_float(wave_max_i32(__float_as_int(s.worst())));
                     live &= __ballot(lw * NG_MARGIN <= bound);
                 }
             }
@@ -543,8 +555,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
         for (int j = 0; j < K; ++j)
             if (j < count)
             {
-                dist2[static_cast<int64_t>(qindex) * k + first + j] = s.d[j];
-                idx[static_cast<int64_t>(qindex) * k + first + j] = s.i[j];
+                dist2[static_cast<int64_t>(qindex) * k + first + j] = s.dist(j);
+                idx[static_cast<int64_t>(qindex) * k + first + j] = s.index(j);
             }
     }
 }

@@ -11,51 +11,62 @@ namespace {
 
 constexpr int KNN_MAX_K = 32; // entries a lane keeps; larger k is served in rounds of this many
 
-__device__ __forceinline__ bool knn_pair_less(float d, int ci, float b, int i)
+// A (squared distance, index) pair as one integer: distances are >= 0, so their bit patterns
+// order like unsigned integers, and one 64-bit comparison orders by distance, then index.
+__device__ __forceinline__ unsigned long long knn_key(float d, int i)
 {
-    return d < b || (d == b && ci < i);
+    return (static_cast<unsigned long long>(static_cast<unsigned>(__float_as_int(d))) << 32) |
+           static_cast<unsigned>(i);
 }
 
 template <int K>
 struct NearestK
 {
-    float d[K];
-    int i[K];
-    // Entries must come after this pair (the last one found by the round before; (-1, -1) in the
-    // first round: every distance is >= 0).
-    float after_d;
-    int after_i;
+    unsigned long long key[K]; // ascending
+    // Entries must come after this pair (the last one found by the round before; 0 with
+    // `from_start` in the first round).
+    unsigned long long after;
+    bool from_start;
 
-    __device__ __forceinline__ void reset(float from_d, int from_i, bool inert)
+    // An inert lane (no query) never admits a candidate.
+    __device__ __forceinline__ void reset(bool later_round, float last_d, int last_i, bool inert)
     {
 #pragma unroll
         for (int j = 0; j < K; ++j)
-        {
-            d[j] = inert ? -1.f : __builtin_inff(); // (an inert lane never admits a candidate)
-            i[j] = inert ? -1 : 0x7FFFFFFF;
-        }
-        after_d = from_d;
-        after_i = from_i;
+            key[j] = inert ? 0ull : knn_key(__builtin_inff(), 0x7FFFFFFF);
+        after = later_round ? knn_key(last_d, last_i) : 0ull;
+        from_start = !later_round;
     }
-    // True when (dist, ci) belongs into the list.
-    __device__ __forceinline__ bool admits(float dist, int ci) const
+    // Squared distance of the last entry (+inf while the list is not full; -1 for an inert lane).
+    __device__ __forceinline__ float worst() const
     {
-        return knn_pair_less(dist, ci, d[K - 1], i[K - 1]) && knn_pair_less(after_d, after_i, dist, ci);
+        return key[K - 1] == 0ull ? -1.f : __int_as_float(static_cast<int>(key[K - 1] >> 32));
+    }
+    // True when the pair belongs into the list.
+    __device__ __forceinline__ bool admits(unsigned long long cand) const
+    {
+        return cand < key[K - 1] && (from_start || cand > after);
     }
     // Inserts a pair that admits() accepted.
-    __device__ __forceinline__ void insert(float dist, int ci)
+    __device__ __forceinline__ void insert(unsigned long long cand)
     {
+        bool before_this = true; // cand < key[K - 1]
 #pragma unroll
         for (int j = K - 1; j > 0; --j)
         {
-            const bool before_prev = knn_pair_less(dist, ci, d[j - 1], i[j - 1]);
-            const bool before_this = knn_pair_less(dist, ci, d[j], i[j]);
-            d[j] = before_prev ? d[j - 1] : (before_this ? dist : d[j]);
-            i[j] = before_prev ? i[j - 1] : (before_this ? ci : i[j]);
+            const bool before_prev = cand < key[j - 1];
+            key[j] = before_prev ? key[j - 1] : (before_this ? cand : key[j]);
+            before_this = before_prev;
         }
-        const bool first = knn_pair_less(dist, ci, d[0], i[0]);
-        d[0] = first ? dist : d[0];
-        i[0] = first ? ci : i[0];
+        key[0] = before_this ? cand : key[0];
+    }
+    __device__ __forceinline__ float dist(int j) const
+    {
+        return __int_as_float(static_cast<int>(key[j] >> 32));
+    }
+    __device__ __forceinline__ int index(int j) const
+    {
+        return static_cast<int>(key[j] & 0xFFFFFFFFull);
     }
 };
 
