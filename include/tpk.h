@@ -4,7 +4,8 @@
  *
  * Every entry point takes plain device pointers and sizes, launches on the HIP stream
  * passed as `stream` (a hipStream_t cast to void*; NULL = the null stream), never
- * allocates, never synchronises the host and keeps no state between calls.  The caller
+ * allocates, never synchronises the host (tpk_grow_proximity, whose output sizes depend on
+ * the data, is the one exception) and keeps no state between calls.  The caller
  * owns all memory.  All arrays are dense row-major ("contiguous").  Outputs need not be
  * initialised: every element of every output array is written by the call.
  *
@@ -199,6 +200,36 @@ int tpk_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, const double* x
                         const int32_t* idx1, const int32_t* idx2, const double* grad_dist1,
                         const double* grad_dist2, double* grad_xyz1, double* grad_xyz2,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Clusters grown over a neighbour matrix (PointGroup's region growing).
+ * Replaces _grow_proximity_core(neighbours, min_cluster_size), the numba routine that
+ * grow_proximity() runs on the host after copying the matrix there
+ * (torch_points_kernels/cluster.py:9-37, called at :40-45 and from region_grow() at :48-109);
+ * the reference has no device code for it.
+ *   neighbours (n, nsample) int64: row i lists neighbours of point i and ends at its first -1
+ *     (what ball_query_partial_dense returns for a self query); entries in [-1, n), a row
+ *     repeats no index.
+ *   members (n) int64: the clusters with at least min_cluster_size members, one after the
+ *     other, ordered by their first (smallest) point as the reference orders them;
+ *     starts (n + 1) int64: their offsets into `members`, then the total.
+ *   found (2, HOST memory): number of clusters, number of members written.  Only that many
+ *     entries of starts (+1) and members are defined.
+ *   member_order: TPK_MEMBERS_AS_REFERENCE - inside a cluster, the order of the reference's
+ *     lists (the order its stack walk appends points; a serial walk per cluster, clusters in
+ *     parallel); TPK_MEMBERS_BY_INDEX - ascending index (all steps data-parallel; same
+ *     clusters, same cluster order).
+ * `workspace`: tpk_grow_proximity_workspace_bytes(n) bytes (0 when n is 0, beyond 2^30, or
+ * no device is present to size the sort's temporary storage), 256-byte aligned, required.
+ * This entry point waits for the stream (several times): the number of label sweeps and the
+ * output sizes depend on the data.
+ * ------------------------------------------------------------------------------------- */
+#define TPK_MEMBERS_AS_REFERENCE 0
+#define TPK_MEMBERS_BY_INDEX 1
+size_t tpk_grow_proximity_workspace_bytes(int64_t n);
+int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbours, int64_t min_cluster_size,
+                       int member_order, int64_t* members, int64_t* starts, int64_t* found,
+                       void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

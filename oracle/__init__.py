@@ -157,6 +157,46 @@ def knn(support, query, k):
     return idx, dist2
 
 
+def grow_proximity_core(neighbours, min_cluster_size):
+    """Clusters over a neighbour matrix (n, nsample) int64 -> list of lists, as the numba routine of the
+    reference (torch_points_kernels/cluster.py:9-37) returns them."""
+    neighbours = _c(neighbours, np.int64)
+    n, nsample = neighbours.shape
+    members = np.empty(max(n, 1), np.int64)
+    starts = np.empty(n + 1, np.int64)
+    fn = lib().tpk_oracle_grow_proximity
+    fn.restype = ctypes.c_int64
+    count = fn(ctypes.c_int64(n), ctypes.c_int(nsample), _p(neighbours, _i64p), ctypes.c_int64(min_cluster_size),
+               _p(members, _i64p), _p(starts, _i64p))
+    return [members[starts[c]:starts[c + 1]].tolist() for c in range(count)]
+
+
+def grow_proximity(pos, batch, nsample=16, radius=0.02, min_cluster_size=32):
+    """torch_points_kernels/cluster.py:40-45 for tensors on the GPU: neighbours by the packed ball query
+    (self query), then the growth above."""
+    idx, _ = ball_query_partial_dense(radius, nsample, pos, pos, batch, batch)
+    return grow_proximity_core(idx, min_cluster_size)
+
+
+def region_grow(pos, labels, batch, ignore_labels=(), nsample=16, radius=0.02, min_cluster_size=32):
+    """torch_points_kernels/cluster.py:48-109: grow_proximity per label value (ascending), clouds renumbered
+    to consecutive values, clusters given as arrays of indices into pos."""
+    pos = np.asarray(pos)
+    labels = np.asarray(labels)
+    batch = np.asarray(batch)
+    clusters = []
+    ind = np.arange(pos.shape[0])
+    for l in np.unique(labels):
+        if l in ignore_labels:
+            continue
+        mask = labels == l
+        local = ind[mask]
+        _, remapped = np.unique(batch[mask], return_inverse=True)
+        for cluster in grow_proximity(pos[mask], remapped.astype(np.int64), nsample, radius, min_cluster_size):
+            clusters.append(local[np.asarray(cluster, np.int64)])
+    return clusters
+
+
 def three_interpolate(points, idx, weight):
     points = _c(points, np.float32)
     idx = _c(idx, np.int32)

@@ -552,3 +552,58 @@ void tpk_oracle_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, const d
     chamfer_grad_dir_f64(b, n, xyz1, m, xyz2, grad_dist1, idx1, grad_xyz1, grad_xyz2);
     chamfer_grad_dir_f64(b, m, xyz2, n, xyz1, grad_dist2, idx2, grad_xyz2, grad_xyz1);
 }
+
+/* ------------------------------------------------------------------------- */
+/* Clusters grown over a neighbour matrix (torch_points_kernels/cluster.py:9-37, */
+/* the numba routine behind grow_proximity).  neighbours (n, nsample) int64,     */
+/* each row ends at its first -1.  Points are taken in index order; an unseen    */
+/* point starts a cluster and a stack; the last entry of the stack is taken off  */
+/* and its row read left to right, every unseen neighbour being marked, put on   */
+/* the stack and appended to the cluster at once.  Clusters with at least        */
+/* min_cluster_size members are kept, in the order of their first point.         */
+/* members (n) receives the kept clusters one after the other, starts            */
+/* (up to n + 1) their offsets; returns the number of kept clusters.             */
+/* ------------------------------------------------------------------------- */
+int64_t tpk_oracle_grow_proximity(int64_t n, int nsample, const int64_t* neighbours,
+                                  int64_t min_cluster_size, int64_t* members, int64_t* starts)
+{
+    unsigned char* seen = (unsigned char*)calloc((size_t)(n > 0 ? n : 1), 1);
+    int64_t* stack = (int64_t*)malloc(sizeof(int64_t) * (size_t)(n > 0 ? n : 1));
+    int64_t clusters = 0, filled = 0;
+    starts[0] = 0;
+    for (int64_t i = 0; i < n; ++i)
+    {
+        if (seen[i])
+            continue;
+        int64_t* cluster = members + filled;
+        int64_t size = 0, top = 0;
+        seen[i] = 1;
+        stack[top++] = i;
+        cluster[size++] = i;
+        while (top > 0)
+        {
+            const int64_t k = stack[--top];
+            const int64_t* row = neighbours + k * nsample;
+            for (int j = 0; j < nsample; ++j)
+            {
+                const int64_t nei = row[j];
+                if (nei == -1)
+                    break;
+                if (!seen[nei])
+                {
+                    seen[nei] = 1;
+                    stack[top++] = nei;
+                    cluster[size++] = nei;
+                }
+            }
+        }
+        if (size >= min_cluster_size)
+        {
+            filled += size;
+            starts[++clusters] = filled;
+        }
+    }
+    free(stack);
+    free(seen);
+    return clusters;
+}

@@ -638,6 +638,107 @@ def test_knn_ties_and_errors(tpk, oracle, dev):
         np.testing.assert_array_equal(_np(dist2), wd)
 
 
+# ------------------------------------------------------------------ region growing
+
+
+def _blobs(g, clouds, n, spread):
+    """Packed clouds of blobs of different density plus scattered points, so that rows of the
+    neighbour matrix are cut at nsample in places and clusters of all sizes appear."""
+    pos, batch = [], []
+    for c in range(clouds):
+        centres = torch.rand(12, 3, generator=g)
+        which = torch.randint(0, 12, (n,), generator=g)
+        scale = spread * (0.3 + torch.rand(12, generator=g))[which].unsqueeze(-1)
+        pts = centres[which] + scale * torch.randn(n, 3, generator=g)
+        pts[: n // 8] = torch.rand(n // 8, 3, generator=g)
+        pos.append(pts[torch.randperm(n, generator=g)])
+        batch.append(torch.full((n,), c, dtype=torch.long))
+    return torch.cat(pos).contiguous(), torch.cat(batch)
+
+
+def test_kat_region_grow(tpk, dev):
+    # reference test/test_cluster.py:14-44 (positions as floats)
+    pos = torch.tensor([[0, 0, 0], [1, 0, 0], [2, 0, 0], [10, 0, 0]] * 2).float().to(dev)
+    batch = torch.tensor([0, 0, 0, 0, 1, 1, 1, 1]).to(dev)
+    labels = torch.tensor([0, 0, 1, 1, 0, 1, 1, 10]).to(dev)
+    from torch_points_kernels.cluster import grow_proximity, region_grow
+
+    for order in ("reference", "index"):
+        assert grow_proximity(pos, batch, radius=2, min_cluster_size=1, member_order=order) == [[0, 1, 2], [3], [4, 5, 6], [7]]
+        assert grow_proximity(pos, batch, radius=2, min_cluster_size=3, member_order=order) == [[0, 1, 2], [4, 5, 6]]
+        assert grow_proximity(pos, batch, radius=2, min_cluster_size=5, member_order=order) == []
+        clusters = region_grow(pos, labels, batch, radius=2, min_cluster_size=1, member_order=order)
+        assert [c.tolist() for c in clusters] == [[0, 1], [4], [2], [3], [5, 6], [7]]
+        assert all(c.is_cuda and c.dtype == torch.int64 for c in clusters)
+        clusters = region_grow(pos, labels, batch, ignore_labels=[1, 10], radius=2, min_cluster_size=1, member_order=order)
+        assert [c.tolist() for c in clusters] == [[0, 1], [4]]
+    with pytest.raises(NotImplementedError):
+        grow_proximity(pos.cpu(), batch.cpu(), radius=2)
+    with pytest.raises(ValueError):
+        grow_proximity(pos, batch, radius=2, member_order="sorted")
+
+
+@pytest.mark.parametrize("clouds,n,spread,radius,nsample,min_size",
+                         [(1, 300, 0.05, 0.05, 16, 1), (2, 2000, 0.03, 0.02, 16, 32), (3, 9000, 0.03, 0.03, 4, 8),
+                          (1, 30000, 0.05, 0.02, 16, 32), (2, 12000, 0.02, 0.05, 70, 2), (1, 5000, 0.1, 0.004, 16, 1),
+                          (1, 20000, 0.5, 0.03, 2, 3)])
+def test_grow_proximity_parity(tpk, oracle, dev, clouds, n, spread, radius, nsample, min_size):
+    from torch_points_kernels.cluster import grow_proximity
+
+    g = torch.Generator().manual_seed(n + nsample)
+    pos, batch = _blobs(g, clouds, n, spread)
+    want = oracle.grow_proximity(pos.numpy(), batch.numpy(), nsample, radius, min_size)
+    assert len(want) > 0
+    got = grow_proximity(pos.to(dev), batch.to(dev), nsample, radius, min_size)
+    assert got == want  # the reference's lists, member for member
+    got = grow_proximity(pos.to(dev), batch.to(dev), nsample, radius, min_size, member_order="index")
+    assert got == [sorted(c) for c in want]
+
+
+def test_region_grow_parity(tpk, oracle, dev):
+    from torch_points_kernels.cluster import region_grow
+
+    g = torch.Generator().manual_seed(77)
+    pos, batch = _blobs(g, 3, 6000, 0.03)
+    labels = torch.randint(0, 4, (pos.shape[0] // 50,), generator=g).repeat_interleave(50) * 3 - 1  # runs of one label
+    want = oracle.region_grow(pos.numpy(), labels.numpy(), batch.numpy(), ignore_labels=[2], radius=0.04, min_cluster_size=10)
+    got = region_grow(pos.to(dev), labels.to(dev), batch.to(dev), ignore_labels=[2], radius=0.04, min_cluster_size=10)
+    assert len(got) == len(want) > 0
+    for a, b in zip(got, want):
+        np.testing.assert_array_equal(_np(a), b)
+
+
+def test_grow_proximity_any_matrix(tpk, oracle, dev):
+    """Matrices that no ball query produces: rows ending early, entries after a -1 (ignored, the row has ended), chains
+    in both directions, points nobody lists, no columns at all."""
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    g = torch.Generator().manual_seed(5)
+    cases = []
+    for n, ns in ((1, 1), (50, 3), (700, 5), (4000, 2), (3000, 80)):
+        rows = torch.stack([torch.randperm(n, generator=g)[: min(ns, n)] for _ in range(n)])  # no repeats in a row
+        if rows.shape[1] < ns:
+            rows = torch.cat([rows, torch.full((n, ns - rows.shape[1]), -1)], 1)
+        cut = torch.randint(0, ns + 1, (n,), generator=g)
+        rows[torch.arange(ns).unsqueeze(0) == cut.unsqueeze(1)] = -1  # a -1 somewhere: the row ends there
+        rows[torch.rand(n, generator=g) < 0.5, 0] = -1  # empty rows
+        cases.append(rows)
+    n = 5000
+    up = torch.arange(1, n + 1).unsqueeze(1)
+    up[-1] = -1
+    cases.append(up)  # 0 -> 1 -> 2 ...: one cluster
+    cases.append((torch.arange(n) - 1).unsqueeze(1))  # 1 -> 0, 2 -> 1, ...: nobody reaches a later point
+    cases.append(torch.zeros(9, 0, dtype=torch.long))
+    for rows in cases:
+        rows = rows.contiguous()
+        for min_size in (1, 2, 40):
+            want = oracle.grow_proximity_core(rows.numpy(), min_size)
+            for reference_order in (True, False):
+                members, starts = native.grow_proximity(rows.to(dev), min_size, reference_order)
+                members, starts = members.tolist(), starts.tolist()
+                got = [members[a:b] for a, b in zip(starts[:-1], starts[1:])]
+                assert got == (want if reference_order else [sorted(c) for c in want])
+
+
 # ------------------------------------------------------------------ chamfer
 
 

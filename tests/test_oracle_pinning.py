@@ -456,3 +456,51 @@ def test_chamfer_backward_closed_form(oracle):
         g1.numpy().astype(np.float32), g2.numpy().astype(np.float32))
     np.testing.assert_allclose(ga32, a.grad.numpy(), rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(gb32, b.grad.numpy(), rtol=1e-4, atol=1e-5)
+
+
+# ------------------------------------------------------------------ region growing
+
+
+def test_grow_proximity_reference_vectors(oracle):
+    # reference test/test_cluster.py:14-44
+    pos = np.array([[0, 0, 0], [1, 0, 0], [2, 0, 0], [10, 0, 0]] * 2, np.float32)
+    batch = np.array([0, 0, 0, 0, 1, 1, 1, 1])
+    labels = np.array([0, 0, 1, 1, 0, 1, 1, 10])
+    assert oracle.grow_proximity(pos, batch, radius=2, min_cluster_size=1) == [[0, 1, 2], [3], [4, 5, 6], [7]]
+    assert oracle.grow_proximity(pos, batch, radius=2, min_cluster_size=3) == [[0, 1, 2], [4, 5, 6]]
+    clusters = oracle.region_grow(pos, labels, batch, radius=2, min_cluster_size=1)
+    assert [c.tolist() for c in clusters] == [[0, 1], [4], [2], [3], [5, 6], [7]]
+
+
+def test_grow_proximity_walk_order_by_hand(oracle):
+    # 0 lists 3 then 1; the last pushed (1) is expanded first and brings 2, then 3 brings 4.
+    rows = np.array([[3, 1, -1], [2, 0, -1], [-1, 4, 4], [4, -1, 0], [-1, -1, -1], [5, -1, -1]], np.int64)
+    assert oracle.grow_proximity_core(rows, 1) == [[0, 3, 1, 2, 4], [5]]
+    assert oracle.grow_proximity_core(rows, 2) == [[0, 3, 1, 2, 4]]
+    # one-directional rows: 2 lists 0, nobody lists 2 -> 2 stays alone although it "touches" the first cluster
+    rows = np.array([[1, -1], [0, -1], [0, 1]], np.int64)
+    assert oracle.grow_proximity_core(rows, 1) == [[0, 1], [2]]
+
+
+def test_grow_proximity_clusters_are_classes_of_the_smallest_reaching_point(oracle):
+    """Independent statement of what the walk computes: v belongs to the cluster started by the smallest point
+    that reaches v along rows (transitive closure by repeated squaring of the boolean matrix)."""
+    rng = np.random.default_rng(3)
+    for n, ns, fill in ((12, 2, 0.6), (40, 3, 0.5), (90, 2, 0.8), (64, 4, 0.3)):
+        rows = np.full((n, ns), -1, np.int64)
+        for i in range(n):
+            take = rng.permutation(n)[: rng.binomial(ns, fill)]
+            rows[i, : len(take)] = take
+        reach = np.eye(n, dtype=bool)
+        for i in range(n):
+            for j in rows[i]:
+                if j < 0:
+                    break
+                reach[i, j] = True
+        for _ in range(8):
+            reach = reach | ((reach.astype(np.int32) @ reach.astype(np.int32)) > 0)
+        first = reach.argmax(axis=0)  # smallest i with reach[i, v]
+        want = [sorted(np.nonzero(first == s)[0].tolist()) for s in sorted(set(first.tolist()))]
+        got = oracle.grow_proximity_core(rows, 1)
+        assert [sorted(c) for c in got] == want
+        assert [c[0] for c in got] == [c[0] for c in want]  # a cluster starts with its smallest point

@@ -156,6 +156,38 @@ std::pair<at::Tensor, at::Tensor> dense_knn(at::Tensor support, at::Tensor query
     return std::make_pair(idx, dist2);
 }
 
+// torch_points_kernels/cluster.py:9-37 (_grow_proximity_core; host code in the reference)
+// -> (members, starts): clusters one after the other and their offsets (one more than clusters).
+std::pair<at::Tensor, at::Tensor> grow_proximity(at::Tensor neighbours, int64_t min_cluster_size,
+                                                 bool reference_order)
+{
+    check_contiguous(neighbours, "neighbours");
+    check_dtype(neighbours, at::kLong, "neighbours");
+    check_gpu(neighbours, "neighbours");
+    TORCH_CHECK(neighbours.dim() == 2, "neighbours must have shape (N, nsample)");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(neighbours.device());
+    const int64_t n = neighbours.size(0);
+    auto options = at::device(neighbours.device()).dtype(at::ScalarType::Long);
+    at::Tensor members = torch::empty({n}, options);
+    at::Tensor starts = torch::empty({n + 1}, options);
+    int64_t found[2] = {0, 0};
+    if (n > 0)
+    {
+        const size_t ws_bytes = tpk_grow_proximity_workspace_bytes(n);
+        TORCH_CHECK(ws_bytes > 0, "grow_proximity: too many points");
+        at::Tensor ws = torch::empty({static_cast<int64_t>(ws_bytes)}, options.dtype(torch::kUInt8));
+        check_status(tpk_grow_proximity(n, as_int(neighbours.size(1), "nsample"), neighbours.data_ptr<int64_t>(),
+                                        min_cluster_size,
+                                        reference_order ? TPK_MEMBERS_AS_REFERENCE : TPK_MEMBERS_BY_INDEX,
+                                        members.data_ptr<int64_t>(), starts.data_ptr<int64_t>(), found,
+                                        ws.data_ptr(), ws_bytes, current_stream(neighbours)),
+                     "grow_proximity");
+    }
+    if (found[0] == 0)
+        return std::make_pair(members.narrow(0, 0, 0), torch::zeros({1}, options));
+    return std::make_pair(members.narrow(0, 0, found[1]), starts.narrow(0, 0, found[0] + 1));
+}
+
 // cuda/src/interpolate.cpp:34-54
 at::Tensor three_interpolate(at::Tensor points, at::Tensor idx, at::Tensor weight)
 {
@@ -477,6 +509,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("furthest_point_sampling", &furthest_point_sampling);
     m.def("three_nn", &three_nn);
     m.def("dense_knn", &dense_knn);
+    m.def("grow_proximity", &grow_proximity);
     m.def("three_interpolate", &three_interpolate);
     m.def("three_interpolate_grad", &three_interpolate_grad);
     m.def("ball_query_dense", &ball_query_dense);

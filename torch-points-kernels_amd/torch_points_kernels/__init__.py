@@ -1,6 +1,6 @@
 """torch_points_kernels for AMD MI355X: the spatial-search operators of
 torch-points3d/torch-points-kernels (furthest point sampling, ball query, three_nn /
-three_interpolate, grouping, Chamfer distance, dense knn) on hand-written HIP kernels.
+three_interpolate, grouping, Chamfer distance, dense knn, region growing) on hand-written HIP kernels.
 
 Same names and call signatures as the reference package (torch_points_kernels/__init__.py);
 GPU tensors only.
@@ -17,6 +17,7 @@ from .torchpoints import (
     three_nn,
 )
 from .knn import knn
+from .cluster import grow_proximity, region_grow
 from .chamfer_dist import ChamferFunction
 from . import chamfer_dist  # the reference exports the submodule under this name
 
@@ -27,6 +28,7 @@ __all__ = [
     "three_interpolate",
     "three_nn",
     "knn",
+    "region_grow",
     "chamfer_dist",
     "ChamferFunction",
 ]

@@ -1,0 +1,87 @@
+"""Region growing over ball-query neighbourhoods (reference: torch_points_kernels/cluster.py).
+
+The reference searches the neighbours on the device, copies the matrix to the host and grows the
+clusters there with a numba routine; here both steps run on the device.
+"""
+from typing import List
+
+import torch
+
+from ._native import native, require_gpu
+from .torchpoints import ball_query_partial_dense
+
+
+def _grow(pos, batch, nsample, radius, min_cluster_size, member_order):
+    if member_order not in ("reference", "index"):
+        raise ValueError("member_order must be 'reference' or 'index'")
+    assert pos.shape[0] == batch.shape[0]
+    require_gpu(pos, "grow_proximity")
+    require_gpu(batch, "grow_proximity")
+    neighbours = ball_query_partial_dense(radius, nsample, pos, pos, batch, batch)[0]
+    members, starts = native().grow_proximity(neighbours, int(min_cluster_size), member_order == "reference")
+    return members, starts
+
+
+def grow_proximity(pos, batch, nsample=16, radius=0.02, min_cluster_size=32, member_order="reference"):
+    """Grow based on proximity only (reference cluster.py:40-45).
+
+    Returns the clusters as a list of lists of point indices, ordered by their first point.
+    member_order: "reference" lists the members of a cluster in the order the reference does (the
+    order in which its walk over the neighbour matrix meets them); "index" lists them in ascending
+    order, which is faster for large clusters.  The clusters themselves are the same.
+    """
+    members, starts = _grow(pos, batch, nsample, radius, min_cluster_size, member_order)
+    members = members.tolist()
+    starts = starts.tolist()
+    return [members[a:b] for a, b in zip(starts[:-1], starts[1:])]
+
+
+def region_grow(
+    pos, labels, batch, ignore_labels=[], nsample=16, radius=0.02, min_cluster_size=32, member_order="reference"
+) -> List[torch.Tensor]:
+    """Region growing clustering algorithm proposed in
+    PointGroup: Dual-Set Point Grouping for 3D Instance Segmentation
+    https://arxiv.org/pdf/2004.01658.pdf
+    for instance segmentation (reference cluster.py:48-109)
+
+    Parameters
+    ----------
+    pos: torch.Tensor [N, 3]
+        Location of the points
+    labels: torch.Tensor [N,]
+        labels of each point
+    ignore_labels:
+        Labels that should be ignored, no region growing will be performed on those
+    nsample:
+        maximum number of neighbours to consider
+    radius:
+        radius for the neighbour search
+    min_cluster_size:
+        Number of points above which a cluster is considered valid
+    member_order:
+        see grow_proximity
+    """
+    assert labels.dim() == 1
+    assert pos.dim() == 2
+    assert pos.shape[0] == labels.shape[0]
+
+    clusters = []
+    ind = torch.arange(0, pos.shape[0], device=pos.device)
+    for l in torch.unique(labels).tolist():
+        if l in ignore_labels:
+            continue
+
+        # points of this label only, their clouds renumbered to 0, 1, 2, ...
+        label_mask = labels == l
+        local_ind = ind[label_mask]
+        remaped_batch = torch.unique(batch[label_mask], return_inverse=True)[1]
+
+        members, starts = _grow(
+            pos[label_mask, :].contiguous(), remaped_batch, nsample, radius, min_cluster_size, member_order
+        )
+        members = local_ind[members]
+        starts = starts.tolist()
+        for a, b in zip(starts[:-1], starts[1:]):
+            clusters.append(members[a:b])
+
+    return clusters
