@@ -213,6 +213,42 @@ def bench_others(dev, steps, warmup, with_cpu):
                              "sample": "%d of 16 clouds, reference cpu/src/knn.cpp (nanoflann k=16), 1 thread" % sub}
     out["knn_k16"] = e
 
+    # beyond the BASELINE configurations: region growing on the workload of the reference's
+    # benchmark/region_cluster.py; the reference grows the clusters on the host (numba) after copying the
+    # neighbour matrix there
+    rc = W.region_cluster()
+    pos, batch = rc["pos"].to(dev), rc["batch"].to(dev)
+    neighbours = tpk.ball_query_partial_dense(rc["radius"], rc["nsample"], pos, pos, batch, batch)[0]
+    npts = pos.shape[0]
+    nbytes = neighbours.numel() * 8
+    grow = {}
+    for order, name in ((False, "index"), (True, "reference")):
+        wall, ev = _time_gpu(lambda: nat.grow_proximity(neighbours, rc["min_cluster_size"], order), max(3, steps // 4), 1)
+        grow[name] = (wall, ev)
+    members, starts = nat.grow_proximity(neighbours, rc["min_cluster_size"], False)
+    wall, ev = grow["index"]
+    e = {"workload": "grow_proximity over the neighbour matrix (300000, 16) of benchmark/region_cluster.py (3 x 100000 uniform "
+                     "points, r=0.02, nsample=16, min_cluster_size=32; not a BASELINE configuration); members by index",
+         "metric": "points/s", "value": npts / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
+         "members_in_reference_order_wall_ms": grow["reference"][0],
+         "clusters": int(starts.numel() - 1), "members": int(members.numel()),
+         "largest_cluster": int((starts[1:] - starts[:-1]).max()) if starts.numel() > 1 else 0,
+         "roofline": _roof_bytes(nbytes + members.numel() * 8, ev, "grow_proximity"),
+         "algorithmic_bytes": nbytes + members.numel() * 8}
+    e["roofline"]["note"] = ("algorithmic bytes = the matrix read once + the members written; the call is about 45 short "
+                             "kernels and three waits for the stream (data-dependent sweep count and output size), so launch "
+                             "and wait time, not bandwidth, decides; kernel_ms is the time between events around the whole call. "
+                             "Members in the reference's order need a serial walk per cluster (largest cluster decides)")
+    if with_cpu:
+        import oracle
+
+        matrix = neighbours.cpu().numpy()
+        secs = _cpu_time(lambda: oracle.grow_proximity_core(matrix, rc["min_cluster_size"]))
+        e["cpu_baseline"] = {"value": npts / secs, "unit": "points/s", "cores": 1, "kind": "port",
+                             "sample": "the whole matrix; C restatement of the reference's numba routine (cluster.py:9-37); the "
+                                       "reference also copies the matrix (38 MB) to the host first, not timed here"}
+    out["grow_proximity"] = e
+
     dist, idx = tpk.three_nn(unknown, known)
     weight = W.inverse_distance_weights(dist).contiguous()
     feats = w["features"].to(dev)

@@ -219,14 +219,14 @@ int tpk_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, const double* x
  *     lists (the order its stack walk appends points; a serial walk per cluster, clusters in
  *     parallel); TPK_MEMBERS_BY_INDEX - ascending index (all steps data-parallel; same
  *     clusters, same cluster order).
- * `workspace`: tpk_grow_proximity_workspace_bytes(n) bytes (0 when n is 0, beyond 2^30, or
+ * `workspace`: tpk_grow_proximity_workspace_bytes(n, nsample) bytes (0 when n is 0, beyond 2^30, or
  * no device is present to size the sort's temporary storage), 256-byte aligned, required.
  * This entry point waits for the stream (several times): the number of label sweeps and the
  * output sizes depend on the data.
  * ------------------------------------------------------------------------------------- */
 #define TPK_MEMBERS_AS_REFERENCE 0
 #define TPK_MEMBERS_BY_INDEX 1
-size_t tpk_grow_proximity_workspace_bytes(int64_t n);
+size_t tpk_grow_proximity_workspace_bytes(int64_t n, int nsample);
 int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbours, int64_t min_cluster_size,
                        int member_order, int64_t* members, int64_t* starts, int64_t* found,
                        void* workspace, size_t workspace_bytes, void* stream);

@@ -25,7 +25,7 @@ def test_header_declares_the_expected_entry_points():
         "tpk_fps_f32", "tpk_fps_workspace_bytes", "tpk_ball_query_dense_f32", "tpk_ball_query_partial_workspace_bytes", "tpk_ball_query_partial_f32",
         "tpk_three_nn_workspace_bytes", "tpk_three_nn_f32", "tpk_knn_workspace_bytes", "tpk_knn_f32", "tpk_three_interpolate_f32", "tpk_three_interpolate_grad_f32", "tpk_group_f32",
         "tpk_group_grad_f32", "tpk_chamfer_fwd_workspace_bytes", "tpk_chamfer_fwd_f32", "tpk_chamfer_fwd_f64", "tpk_chamfer_bwd_f32",
-        "tpk_chamfer_bwd_f64", "tpk_status_string", "tpk_version",
+        "tpk_chamfer_bwd_f64", "tpk_grow_proximity_workspace_bytes", "tpk_grow_proximity", "tpk_status_string", "tpk_version",
     ):
         assert want in names
 
@@ -86,6 +86,15 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.tpk_fps_f32(1, 4, 2, null, null, ctypes.c_size_t(0), null, null) == -1
     # empty problems succeed trivially
     assert lib.tpk_three_nn_f32(0, 4, 4, null, null, null, null, null) == 0
+    found = (ctypes.c_int64 * 2)(5, 5)
+    grow = lib.tpk_grow_proximity
+    grow.argtypes = [ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int] + [ctypes.c_void_p] * 4 + [
+        ctypes.c_size_t, ctypes.c_void_p]
+    assert grow(0, 16, None, 1, 0, None, None, found, None, 0, None) == 0 and list(found) == [0, 0]
+    assert grow(-1, 16, None, 1, 0, None, None, found, None, 0, None) == -1
+    assert grow(5, 16, None, 1, 0, None, None, found, None, 0, None) == -1  # no arrays
+    assert grow(0, 16, None, 1, 7, None, None, found, None, 0, None) == -1  # unknown member order
+    assert grow(0, 16, None, 1, 0, None, None, None, None, 0, None) == -1  # nowhere to report the counts
     assert lib.tpk_group_f32(0, 1, 1, 1, 1, null, null, null, null) == 0
 
 

@@ -151,3 +151,14 @@ def bytes_grouping(B=16, C=128, N=4096, npoint=1024, nsample=32):
 
 def bytes_chamfer_bwd(B=32, N=16384):
     return 2 * (2 * B * N * 3 * 4) + 2 * B * N * 4 + 2 * B * N * 4
+
+
+def region_cluster(num_points=100000):
+    """The workload of the reference's benchmark/region_cluster.py: three unit cubes of uniform points, offset by 2,
+    as one cloud; neighbours within 0.02, at most 16 (the defaults of grow_proximity)."""
+    import torch
+
+    g = torch.Generator().manual_seed(0)
+    pos = torch.cat([torch.rand(num_points, 3, generator=g) + 2.0 * i for i in range(3)]).contiguous()
+    batch = torch.ones(3 * num_points, dtype=torch.long)
+    return {"pos": pos, "batch": batch, "radius": 0.02, "nsample": 16, "min_cluster_size": 32}

@@ -10,9 +10,12 @@
 // reached by no smaller one, so it is unseen at its turn and starts a cluster, and every other
 // point that reaches v comes later.  The labels are therefore the fixed point of
 //     label[v] = min(v, label[u] for every row u that lists v),
-// which is found here by repeated sweeps with atomicMin, shortened by following label[label[..]]
-// (valid because reaching is transitive).  Clusters are numbered by their first point, as in the
-// reference, and those below min_cluster_size are dropped.
+// which is found here in two steps.  Points that list each other (all of them, where no row was
+// cut) are first merged into groups by union-find: they reach and are reached by the same points.
+// Then repeated sweeps hand labels from group to group with atomicMin, shortened by following
+// the label of a label (valid because reaching is transitive).  Without the merging a label
+// would cross a cluster one row per sweep.  Clusters are numbered by their first point, as in
+// the reference, and those below min_cluster_size are dropped.
 //
 // Members inside a cluster, two orders:
 //   TPK_MEMBERS_AS_REFERENCE  the order in which the reference's stack walk appends them.  The walk
@@ -42,14 +45,18 @@ constexpr int64_t CL_MAX_POINTS = (int64_t)1 << 30;
 
 using u64 = unsigned long long;
 
-__global__ void __launch_bounds__(CL_THREADS) cluster_init_kernel(int n, int* label, int* size, int* mark, int* changed)
+__global__ void __launch_bounds__(CL_THREADS)
+    cluster_init_kernel(int n, int words, int* parent, int* label, int* size, int* handed, unsigned* mutual, int* changed)
 {
     const int v = blockIdx.x * CL_THREADS + threadIdx.x;
     if (v < n)
     {
+        parent[v] = v;
         label[v] = v;
         size[v] = 0;
-        mark[v] = 0;
+        handed[v] = n; // nothing handed over yet
+        for (int w = 0; w < words; ++w)
+            mutual[(int64_t)v * words + w] = 0;
     }
     if (v < CL_SWEEPS)
         changed[v] = 0;
@@ -61,50 +68,181 @@ __global__ void __launch_bounds__(CL_THREADS) cluster_clear_kernel(int* changed)
         changed[threadIdx.x] = 0;
 }
 
-// One sweep: every point hands the smallest label it can find by following its own label to the
-// points its row lists.  Sweep `sweep` of a batch does nothing when the one before changed
-// nothing, so a batch can be enqueued without looking at the flags in between.
+// The part of a row that counts: lanes of a group of CL_ROW_LANES hold consecutive entries (-1
+// beyond the row's width); returns how many of them come before the row's end and whether the
+// row ends in this chunk.
+__device__ __forceinline__ int entries_before_end(int64_t nei, int shift, bool* row_ends)
+{
+    const unsigned ends = (unsigned)(__ballot(nei == -1) >> shift) & 0xffffu;
+    *row_ends = ends != 0;
+    return ends ? __builtin_ctz(ends) : CL_ROW_LANES;
+}
+
+// Bit j of a point's mask: entry j of its row is a point whose own row lists this point back.
 __global__ void __launch_bounds__(CL_THREADS)
-    cluster_sweep_kernel(int n, int nsample, const int64_t* __restrict__ neighbours, int* label, int* changed, int sweep)
+    cluster_mutual_kernel(int n, int nsample, int words, const int64_t* __restrict__ neighbours, unsigned* mutual)
+{
+    const int64_t t = (int64_t)blockIdx.x * CL_THREADS + threadIdx.x;
+    const int64_t point = t / CL_ROW_LANES;
+    const int g = (int)(t % CL_ROW_LANES);
+    if (point >= n)
+        return; // the whole group of lanes leaves together
+    const int u = (int)point;
+    const int shift = (int)(tpk_lane_id() & (TPK_WAVE - CL_ROW_LANES)); // first lane of this row's group
+    for (int first = 0; first < nsample; first += CL_ROW_LANES)
+    {
+        const int j = first + g;
+        const int64_t nei = j < nsample ? neighbours[(int64_t)u * nsample + j] : -1;
+        bool row_ends;
+        const int valid = entries_before_end(nei, shift, &row_ends);
+        bool back = false;
+        if (g < valid && nei >= 0 && nei < n && nei != u)
+        {
+            const int64_t* other = neighbours + nei * nsample;
+            for (int i = 0; i < nsample; ++i)
+            {
+                const int64_t e = other[i];
+                if (e == -1)
+                    break;
+                if (e == u)
+                {
+                    back = true;
+                    break;
+                }
+            }
+        }
+        const unsigned bits = (unsigned)(__ballot(back) >> shift) & 0xffffu;
+        if (g == 0 && bits)
+            atomicOr(&mutual[(int64_t)u * words + (first >> 5)], bits << (first & 31));
+        if (row_ends)
+            break;
+    }
+}
+
+__device__ __forceinline__ int find_root(const int* parent, int v)
+{
+    for (int up = parent[v]; up < v; up = parent[v])
+        v = up;
+    return v;
+}
+
+// Points that list each other reach the same points and are reached by the same points, so they
+// can be merged outright: union-find over the mutual entries (the tree of the larger root is hung
+// under the smaller root), repeated until no tree is hung any more.  Each mutual pair is handled
+// from its smaller point.
+__global__ void __launch_bounds__(CL_THREADS)
+    cluster_merge_kernel(int n, int nsample, int words, const int64_t* __restrict__ neighbours,
+                         const unsigned* __restrict__ mutual, int* parent, int* changed, int sweep)
 {
     if (sweep > 0 && changed[sweep - 1] == 0)
         return;
     const int64_t t = (int64_t)blockIdx.x * CL_THREADS + threadIdx.x;
     const int64_t point = t / CL_ROW_LANES;
     const int g = (int)(t % CL_ROW_LANES);
-    const bool real = point < n;
-    const int u = real ? (int)point : n - 1;
+    if (point >= n)
+        return;
+    const int u = (int)point;
+    const int mine = find_root(parent, u);
+    bool hung = false;
+    for (int j = g; j < nsample; j += CL_ROW_LANES)
+    {
+        if (((mutual[(int64_t)u * words + (j >> 5)] >> (j & 31)) & 1u) == 0)
+            continue;
+        const int nei = (int)neighbours[(int64_t)u * nsample + j];
+        if (nei < u)
+            continue;
+        const int theirs = find_root(parent, nei);
+        if (theirs != mine)
+        {
+            const int low = min(mine, theirs), high = max(mine, theirs);
+            hung |= atomicMin(&parent[high], low) > low;
+        }
+    }
+    if (g == 0 && mine < parent[u])
+        atomicMin(&parent[u], mine);
+    if (hung)
+        changed[sweep] = 1;
+}
+
+// parent[v] becomes the smallest point of v's merged group.
+__global__ void __launch_bounds__(CL_THREADS) cluster_flatten_kernel(int n, int* parent)
+{
+    const int v = blockIdx.x * CL_THREADS + threadIdx.x;
+    if (v < n)
+    {
+        const int root = find_root(parent, v);
+        if (root < parent[v])
+            atomicMin(&parent[v], root);
+    }
+}
+
+// One sweep over all entries.  Labels live at the first point of every merged group (`group`):
+// label[group[v]] is a point that reaches v.  Every point hands the smallest label it can find by
+// following its own (label of the group of the label ...) to the groups of the points its row
+// lists - unless that is what it handed over last time (`handed`): labels only fall, so those
+// groups still hold it or less.  Sweep `sweep` of a batch does nothing when the one before
+// changed nothing, so a batch can be enqueued without looking at the flags in between.
+__global__ void __launch_bounds__(CL_THREADS)
+    cluster_sweep_kernel(int n, int nsample, const int64_t* __restrict__ neighbours, const int* __restrict__ group,
+                         int* label, int* handed, int* changed, int sweep)
+{
+    if (sweep > 0 && changed[sweep - 1] == 0)
+        return;
+    const int64_t t = (int64_t)blockIdx.x * CL_THREADS + threadIdx.x;
+    const int64_t point = t / CL_ROW_LANES;
+    const int g = (int)(t % CL_ROW_LANES);
+    if (point >= n)
+        return; // the whole group of lanes leaves together
+    const int u = (int)point;
     const int shift = (int)(tpk_lane_id() & (TPK_WAVE - CL_ROW_LANES)); // first lane of this row's group
-    const int mine = label[u];
-    // A few steps along label[label[..]]: any point found this way reaches u, and storing it in
-    // label[u] makes the next sweep's steps that much longer, so chains shorten geometrically.
+    const int home = group[u];
+    const int mine = label[home];
+    const int before = handed[u];
+    // A few steps upstream: any point found this way reaches u, and storing it makes the next
+    // sweep's steps that much longer, so chains shorten geometrically.
     int root = mine;
     for (int step = 0; step < CL_FOLLOW; ++step)
     {
-        const int up = label[root];
+        const int up = label[group[root]];
         if (up >= root)
             break;
         root = up;
     }
+    if (root == before)
+        return;
     bool lowered = false;
-    if (real && g == 0 && root < mine)
+    if (g == 0)
     {
-        atomicMin(&label[u], root);
-        lowered = true;
+        handed[u] = root;
+        if (root < mine)
+            lowered = atomicMin(&label[home], root) > root;
     }
     for (int first = 0; first < nsample; first += CL_ROW_LANES)
     {
         const int j = first + g;
         const int64_t nei = j < nsample ? neighbours[(int64_t)u * nsample + j] : -1;
-        const unsigned ends = (unsigned)(__ballot(nei == -1) >> shift) & 0xffffu;
-        const int valid = ends ? __builtin_ctz(ends) : CL_ROW_LANES;
-        if (real && g < valid && nei >= 0 && nei < n && label[nei] > root)
-            lowered |= atomicMin(&label[nei], root) > root;
-        if (ends)
+        bool row_ends;
+        const int valid = entries_before_end(nei, shift, &row_ends);
+        if (g < valid && nei >= 0 && nei < n)
+        {
+            const int there = group[nei];
+            if (there != home && label[there] > root)
+                lowered |= atomicMin(&label[there], root) > root;
+        }
+        if (row_ends)
             break;
     }
     if (lowered)
         changed[sweep] = 1;
+}
+
+// Every point takes the label of its group.  Labels of other points than the first of a group
+// are read by nobody, so this can be done in place.
+__global__ void __launch_bounds__(CL_THREADS) cluster_spread_kernel(int n, const int* __restrict__ group, int* label)
+{
+    const int v = blockIdx.x * CL_THREADS + threadIdx.x;
+    if (v < n && group[v] != v)
+        label[v] = label[group[v]];
 }
 
 // Members per cluster, counted at the cluster's first point.  Lanes with the same label add once.
@@ -186,13 +324,14 @@ __global__ void __launch_bounds__(CL_THREADS) cluster_widen_kernel(int count, co
 
 // The reference's walk (cluster.py:15-33), one wavefront per kept cluster: the point taken off
 // the stack has its row read by the lanes; the unseen members of the cluster among the entries
-// are marked, and appended to the stack and to the cluster in row order.  `mark` decides with an
-// atomic exchange, so a point enters once even if a row repeats it.  The stack of a cluster
-// occupies the cluster's own range of `stack` (it never holds more than the cluster has members).
+// are marked, and appended to the stack and to the cluster in row order.  A member is unseen
+// while its label still is the cluster's first point; one compare-and-swap tests and marks it
+// (the label becomes the complement), so a point enters once even if a row repeats it, and the
+// labels are used up by this kernel.  The stack of a cluster occupies the cluster's own range of
+// `stack` (it never holds more than the cluster has members).
 __global__ void __launch_bounds__(CL_THREADS)
-    cluster_walk_kernel(int n, int nsample, int clusters, const int64_t* __restrict__ neighbours,
-                        const int* __restrict__ label, const int* __restrict__ seeds, const int64_t* __restrict__ starts,
-                        int* mark, int* stack, int64_t* members)
+    cluster_walk_kernel(int n, int nsample, int clusters, const int64_t* __restrict__ neighbours, int* label,
+                        const int* __restrict__ seeds, const int64_t* __restrict__ starts, int* stack, int64_t* members)
 {
     const int c = blockIdx.x * (CL_THREADS / TPK_WAVE) + threadIdx.x / TPK_WAVE;
     if (c >= clusters)
@@ -205,7 +344,7 @@ __global__ void __launch_bounds__(CL_THREADS)
     int64_t* mine = members + base;
     if (lane == 0)
     {
-        mark[seed] = 1;
+        label[seed] = ~seed;
         mine[0] = seed;
     }
     int filled = 1, top = 0;
@@ -219,9 +358,9 @@ __global__ void __launch_bounds__(CL_THREADS)
             const int64_t nei = j < nsample ? neighbours[(int64_t)k * nsample + j] : -1;
             const u64 ends = __ballot(nei == -1);
             const int valid = ends ? __builtin_ctzll(ends) : TPK_WAVE;
-            bool take = lane < valid && nei >= 0 && nei < n && label[nei] == seed;
-            if (take)
-                take = atomicExch(&mark[nei], 1) == 0;
+            bool take = false;
+            if (lane < valid && nei >= 0 && nei < n)
+                take = atomicCAS(&label[nei], seed, ~seed) == seed;
             const u64 taken = __ballot(take);
             const int count = __builtin_popcountll(taken);
             if (count > 0 && filled + count <= capacity)
@@ -254,9 +393,15 @@ __global__ void __launch_bounds__(CL_THREADS)
 
 struct Layout
 {
-    size_t label, size, mark, number, seeds, stack, keys_in, keys_out, values_in, values_out, packed, scanned, changed,
+    size_t parent, mutual, label, size, number, seeds, stack, keys_in, keys_out, values_in, values_out, packed, scanned, changed,
         temp, temp_bytes, total;
 };
+
+// 32-bit words of a point's mask of mutual entries.
+int mask_words(int nsample)
+{
+    return nsample > 0 ? (nsample + 31) / 32 : 1;
+}
 
 size_t aligned(size_t v)
 {
@@ -278,7 +423,7 @@ bool temp_bytes(int64_t n, size_t* bytes)
     return true;
 }
 
-bool layout(int64_t n, Layout* l)
+bool layout(int64_t n, int nsample, Layout* l)
 {
     size_t temp = 0;
     if (!temp_bytes(n, &temp))
@@ -290,9 +435,10 @@ bool layout(int64_t n, Layout* l)
         return here;
     };
     const size_t ints = (size_t)n * 4;
+    l->parent = take(ints);
+    l->mutual = take(ints * (size_t)mask_words(nsample));
     l->label = take(ints);
     l->size = take(ints);
-    l->mark = take(ints);
     l->number = take(ints);
     l->seeds = take(ints);
     l->stack = take(ints);
@@ -311,10 +457,10 @@ bool layout(int64_t n, Layout* l)
 
 } // namespace
 
-extern "C" size_t tpk_grow_proximity_workspace_bytes(int64_t n)
+extern "C" size_t tpk_grow_proximity_workspace_bytes(int64_t n, int nsample)
 {
     Layout l;
-    if (n <= 0 || n > CL_MAX_POINTS || !layout(n, &l))
+    if (n <= 0 || n > CL_MAX_POINTS || nsample < 0 || !layout(n, nsample, &l))
         return 0;
     return l.total;
 }
@@ -333,15 +479,16 @@ extern "C" int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbo
     if (n > CL_MAX_POINTS)
         return TPK_ERR_UNSUPPORTED;
     Layout l;
-    if (!layout(n, &l))
+    if (!layout(n, nsample, &l))
         return TPK_ERR_UNSUPPORTED;
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
         return TPK_ERR_WORKSPACE;
     hipStream_t s = tpk_stream(stream);
     char* ws = static_cast<char*>(workspace);
+    int* parent = reinterpret_cast<int*>(ws + l.parent);
+    unsigned* mutual = reinterpret_cast<unsigned*>(ws + l.mutual);
     int* label = reinterpret_cast<int*>(ws + l.label);
     int* size = reinterpret_cast<int*>(ws + l.size);
-    int* mark = reinterpret_cast<int*>(ws + l.mark);
     int* number = reinterpret_cast<int*>(ws + l.number);
     int* seeds = reinterpret_cast<int*>(ws + l.seeds);
     int* stack = reinterpret_cast<int*>(ws + l.stack);
@@ -361,23 +508,39 @@ extern "C" int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbo
     const unsigned sweep_blocks = (unsigned)tpk_ceil_div(n * CL_ROW_LANES, CL_THREADS);
     const int min_size = (int)(min_cluster_size > n ? n + 1 : (min_cluster_size < 0 ? 0 : min_cluster_size));
 
-    cluster_init_kernel<<<blocks > 1 ? blocks : 1, CL_THREADS, 0, s>>>(ni, label, size, mark, changed);
+    const int words = mask_words(nsample);
+    // `stack` serves the sweeps as `handed` first
+    cluster_init_kernel<<<blocks, CL_THREADS, 0, s>>>(ni, words, parent, label, size, stack, mutual, changed);
     if (nsample > 0)
     {
-        while (true)
-        {
-            for (int sweep = 0; sweep < CL_SWEEPS; ++sweep)
-                cluster_sweep_kernel<<<sweep_blocks, CL_THREADS, 0, s>>>(ni, nsample, neighbours, label, changed, sweep);
-            int last = 0;
-            hipError_t e = hipMemcpyAsync(&last, changed + CL_SWEEPS - 1, sizeof(int), hipMemcpyDeviceToHost, s);
-            if (e == hipSuccess)
-                e = hipStreamSynchronize(s);
-            if (e != hipSuccess)
-                return (int)e;
-            if (last == 0)
-                break;
-            cluster_clear_kernel<<<1, CL_THREADS, 0, s>>>(changed);
-        }
+        // Enqueues batches of sweeps until the last sweep of a batch reports no change.
+        auto until_stable = [&](auto&& launch) -> hipError_t {
+            while (true)
+            {
+                for (int sweep = 0; sweep < CL_SWEEPS; ++sweep)
+                    launch(sweep);
+                int last = 0;
+                hipError_t e = hipMemcpyAsync(&last, changed + CL_SWEEPS - 1, sizeof(int), hipMemcpyDeviceToHost, s);
+                if (e == hipSuccess)
+                    e = hipStreamSynchronize(s);
+                cluster_clear_kernel<<<1, CL_THREADS, 0, s>>>(changed);
+                if (e != hipSuccess || last == 0)
+                    return e;
+            }
+        };
+        cluster_mutual_kernel<<<sweep_blocks, CL_THREADS, 0, s>>>(ni, nsample, words, neighbours, mutual);
+        hipError_t e = until_stable([&](int sweep) {
+            cluster_merge_kernel<<<sweep_blocks, CL_THREADS, 0, s>>>(ni, nsample, words, neighbours, mutual, parent, changed, sweep);
+        });
+        if (e != hipSuccess)
+            return (int)e;
+        cluster_flatten_kernel<<<blocks, CL_THREADS, 0, s>>>(ni, parent);
+        e = until_stable([&](int sweep) {
+            cluster_sweep_kernel<<<sweep_blocks, CL_THREADS, 0, s>>>(ni, nsample, neighbours, parent, label, stack, changed, sweep);
+        });
+        if (e != hipSuccess)
+            return (int)e;
+        cluster_spread_kernel<<<blocks, CL_THREADS, 0, s>>>(ni, parent, label);
     }
     cluster_count_kernel<<<blocks, CL_THREADS, 0, s>>>(ni, label, size);
     cluster_kept_kernel<<<blocks1, CL_THREADS, 0, s>>>(ni, min_size, label, size, packed);
@@ -411,7 +574,7 @@ extern "C" int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbo
     {
         const int per_block = CL_THREADS / TPK_WAVE;
         cluster_walk_kernel<<<(unsigned)tpk_ceil_div(clusters, per_block), CL_THREADS, 0, s>>>(
-            ni, nsample, clusters, neighbours, label, seeds, starts, mark, stack, members);
+            ni, nsample, clusters, neighbours, label, seeds, starts, stack, members);
     }
     return tpk_launch_status();
 }

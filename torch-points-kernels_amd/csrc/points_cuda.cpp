@@ -173,7 +173,7 @@ std::pair<at::Tensor, at::Tensor> grow_proximity(at::Tensor neighbours, int64_t 
     int64_t found[2] = {0, 0};
     if (n > 0)
     {
-        const size_t ws_bytes = tpk_grow_proximity_workspace_bytes(n);
+        const size_t ws_bytes = tpk_grow_proximity_workspace_bytes(n, as_int(neighbours.size(1), "nsample"));
         TORCH_CHECK(ws_bytes > 0, "grow_proximity: too many points");
         at::Tensor ws = torch::empty({static_cast<int64_t>(ws_bytes)}, options.dtype(torch::kUInt8));
         check_status(tpk_grow_proximity(n, as_int(neighbours.size(1), "nsample"), neighbours.data_ptr<int64_t>(),
