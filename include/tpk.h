@@ -93,6 +93,28 @@ int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int
                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Ball query with sorted neighbours, dense and packed layouts: the `nsample` nearest support
+ * points with d2 < radius*radius, nearest first (equal distances: lower index first).
+ * The reference computes this for CPU tensors only, with sort=True: nanoflann_neighbors() /
+ * batch_nanoflann_neighbors() (cpu/src/neighbors.cpp:8-136, :139-310, reached through
+ * dense_ball_query / batch_ball_query, cpu/src/ball_query.cpp:127-146, :65-124); for CUDA
+ * tensors torch_points_kernels/torchpoints.py:152-153 and :163-164 raise.
+ * Shapes and dtypes as for tpk_ball_query_dense_f32 / tpk_ball_query_partial_f32.  Unused
+ * slots: dense - idx repeats the nearest neighbour (0 when there is none), dist -1; packed -
+ * both -1.  Dense layout: with a `workspace` (tpk_ball_query_sorted_dense_workspace_bytes()
+ * bytes - 0 for shapes not served that way -, 256-byte aligned) the search goes over
+ * curve-ordered cells within the radius instead of all pairs, same results.  The packed
+ * layout tests all pairs of a query with its cloud.
+ * ------------------------------------------------------------------------------------- */
+size_t tpk_ball_query_sorted_dense_workspace_bytes(int b, int n, int m);
+int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius, int nsample,
+                                    const float* new_xyz, const float* xyz, int64_t* idx, float* dist,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y, float radius, int nsample,
+                                      const float* x, const float* y, const int64_t* batch_x,
+                                      const int64_t* batch_y, int64_t* idx, float* dist, void* stream);
+
+/* ---------------------------------------------------------------------------------------
  * Three nearest neighbours.
  * Replaces three_nn_kernel_wrapper(b, n, m, unknown, known, dist2, idx)
  * (cuda/src/interpolate_gpu.cu:67-76, declared cuda/src/interpolate.cpp:5-6).

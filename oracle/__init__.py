@@ -116,6 +116,35 @@ def ball_query_partial_dense(radius, nsample, x, y, batch_x, batch_y, return_pai
     return idx, dist
 
 
+def ball_query_sorted_dense(radius, nsample, xyz, new_xyz):
+    """sort=True, dense layout: xyz (B,n,3) support, new_xyz (B,m,3) queries -> idx int64 (B,m,ns), dist."""
+    xyz = _c(xyz, np.float32)
+    new_xyz = _c(new_xyz, np.float32)
+    b, n, _ = xyz.shape
+    m = new_xyz.shape[1]
+    idx = np.empty((b, m, nsample), np.int64)
+    dist = np.empty((b, m, nsample), np.float32)
+    lib().tpk_oracle_ball_query_sorted_dense(ctypes.c_int(b), ctypes.c_int(n), ctypes.c_int(m), ctypes.c_float(radius),
+                                             ctypes.c_int(nsample), _p(new_xyz, _f32p), _p(xyz, _f32p),
+                                             _p(idx, _i64p), _p(dist, _f32p))
+    return idx, dist
+
+
+def ball_query_sorted_partial(radius, nsample, x, y, batch_x, batch_y):
+    """sort=True, packed layout: x (Nx,3) support, y (Ny,3) queries, sorted int64 batch vectors."""
+    x = _c(x, np.float32)
+    y = _c(y, np.float32)
+    batch_x = _c(batch_x, np.int64)
+    batch_y = _c(batch_y, np.int64)
+    ny = y.shape[0]
+    idx = np.empty((ny, nsample), np.int64)
+    dist = np.empty((ny, nsample), np.float32)
+    lib().tpk_oracle_ball_query_sorted_partial(ctypes.c_int64(x.shape[0]), ctypes.c_int64(ny), ctypes.c_float(radius),
+                                               ctypes.c_int(nsample), _p(x, _f32p), _p(y, _f32p), _p(batch_x, _i64p),
+                                               _p(batch_y, _i64p), _p(idx, _i64p), _p(dist, _f32p))
+    return idx, dist
+
+
 def furthest_point_sample(xyz, npoint):
     xyz = _c(xyz, np.float32)
     b, n, _ = xyz.shape

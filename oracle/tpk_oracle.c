@@ -607,3 +607,96 @@ int64_t tpk_oracle_grow_proximity(int64_t n, int nsample, const int64_t* neighbo
     free(seen);
     return clusters;
 }
+
+/* ------------------------------------------------------------------------- */
+/* Ball query with sorted neighbours: what the reference computes for CPU      */
+/* tensors with sort=True (and refuses for CUDA tensors,                       */
+/* torch_points_kernels/torchpoints.py:152-153, :163-164).                      */
+/* cpu/src/neighbors.cpp:8-136 (dense, per cloud) and :139-310 (packed):       */
+/* nanoflann's radiusSearch keeps a support point when its squared distance,   */
+/* accumulated as ((dx*dx) + dy*dy) + dz*dz in the points' type, is            */
+/* < radius*radius (a float product, :19 and :153), sorts the matches by       */
+/* distance, and the first max_num = nsample are written.  nanoflann sorts by  */
+/* distance only; here equal distances keep the lower index first.             */
+/* Unused slots: dense - index of the first (nearest) match, distance -1, and  */
+/* index 0 when there is no match (:60-61, :88-105); packed - index -1,        */
+/* distance -1 (:248-275).  In the packed layout a query searches the support  */
+/* points that carry its own cloud id (the reference walks both batch vectors  */
+/* in step, which is the same thing when every cloud has queries).             */
+/* first/last (per query) delimit the support range searched.                  */
+/* ------------------------------------------------------------------------- */
+static void sorted_hits(const float* q, const float* support, int64_t first, int64_t last,
+                        float radius2, int nsample, int64_t* idx, float* dist, int* found)
+{
+    int have = 0;
+    for (int64_t p = first; p < last; ++p)
+    {
+        float d = 0;
+        for (int t = 0; t < 3; ++t)
+            d += (q[t] - support[p * 3 + t]) * (q[t] - support[p * 3 + t]);
+        if (!(d < radius2))
+            continue;
+        if (have == nsample && !(d < dist[nsample - 1]))
+            continue;
+        int at = have < nsample ? have : nsample - 1;
+        while (at > 0 && d < dist[at - 1])
+        {
+            dist[at] = dist[at - 1];
+            idx[at] = idx[at - 1];
+            --at;
+        }
+        dist[at] = d;
+        idx[at] = p;
+        if (have < nsample)
+            ++have;
+    }
+    *found = have;
+}
+
+void tpk_oracle_ball_query_sorted_dense(int b, int n, int m, float radius, int nsample,
+                                        const float* new_xyz, const float* xyz, int64_t* idx, float* dist)
+{
+    const float radius2 = radius * radius;
+    if (nsample <= 0)
+        return;
+    for (int bi = 0; bi < b; ++bi)
+        for (int j = 0; j < m; ++j)
+        {
+            int64_t* io = idx + ((int64_t)bi * m + j) * nsample;
+            float* dout = dist + ((int64_t)bi * m + j) * nsample;
+            int found = 0;
+            sorted_hits(new_xyz + ((int64_t)bi * m + j) * 3, xyz + (int64_t)bi * n * 3, 0, n, radius2, nsample,
+                        io, dout, &found);
+            const int64_t token = found > 0 ? io[0] : 0;
+            for (int s = found; s < nsample; ++s)
+            {
+                io[s] = token;
+                dout[s] = -1.0f;
+            }
+        }
+}
+
+void tpk_oracle_ball_query_sorted_partial(int64_t size_x, int64_t size_y, float radius, int nsample,
+                                          const float* x, const float* y, const int64_t* batch_x,
+                                          const int64_t* batch_y, int64_t* idx, float* dist)
+{
+    const float radius2 = radius * radius;
+    if (nsample <= 0)
+        return;
+    for (int64_t j = 0; j < size_y; ++j)
+    {
+        int64_t first = 0, last;
+        while (first < size_x && batch_x[first] < batch_y[j])
+            ++first;
+        last = first;
+        while (last < size_x && batch_x[last] == batch_y[j])
+            ++last;
+        int found = 0;
+        sorted_hits(y + j * 3, x, first, last, radius2, nsample, idx + j * nsample, dist + j * nsample, &found);
+        for (int s = found; s < nsample; ++s)
+        {
+            idx[j * nsample + s] = -1;
+            dist[j * nsample + s] = -1.0f;
+        }
+    }
+}

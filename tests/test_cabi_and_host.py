@@ -25,7 +25,8 @@ def test_header_declares_the_expected_entry_points():
         "tpk_fps_f32", "tpk_fps_workspace_bytes", "tpk_ball_query_dense_f32", "tpk_ball_query_partial_workspace_bytes", "tpk_ball_query_partial_f32",
         "tpk_three_nn_workspace_bytes", "tpk_three_nn_f32", "tpk_knn_workspace_bytes", "tpk_knn_f32", "tpk_three_interpolate_f32", "tpk_three_interpolate_grad_f32", "tpk_group_f32",
         "tpk_group_grad_f32", "tpk_chamfer_fwd_workspace_bytes", "tpk_chamfer_fwd_f32", "tpk_chamfer_fwd_f64", "tpk_chamfer_bwd_f32",
-        "tpk_chamfer_bwd_f64", "tpk_grow_proximity_workspace_bytes", "tpk_grow_proximity", "tpk_status_string", "tpk_version",
+        "tpk_chamfer_bwd_f64", "tpk_grow_proximity_workspace_bytes", "tpk_grow_proximity", "tpk_ball_query_sorted_dense_workspace_bytes",
+        "tpk_ball_query_sorted_dense_f32", "tpk_ball_query_sorted_partial_f32", "tpk_status_string", "tpk_version",
     ):
         assert want in names
 
@@ -46,7 +47,8 @@ def test_library_exports_every_declared_symbol():
     assert lib.tpk_fps_workspace_bytes(2, 200000) == 2 * 200000 * 4  # larger: the minima only
     # searches over curve-ordered cells: 16 bytes per point padded to cells of 64, 160 bytes per cell;
     # 0 = the shape is served by the all-pairs scan, no workspace wanted
-    for name in ("tpk_three_nn_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes", "tpk_knn_workspace_bytes"):
+    for name in ("tpk_three_nn_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes", "tpk_knn_workspace_bytes",
+                 "tpk_ball_query_sorted_dense_workspace_bytes"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_size_t
         assert fn(2, 100, 100) == 0 and fn(2, 200000, 1000) == 0 and fn(0, 1000, 1000) == 0

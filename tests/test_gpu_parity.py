@@ -59,8 +59,13 @@ def test_kat_ball_query_dense(tpk, dev):
     assert idx.dtype == torch.int64 and dist.dtype == torch.float32
     np.testing.assert_array_equal(_np(idx), [[[0, 1]], [[2, 2]]])
     np.testing.assert_array_equal(_np(dist), np.array([[[0, 1]], [[1, -1]]], np.float32))
-    with pytest.raises(NotImplementedError):
-        tpk.ball_query(1.01, 2, a, b, sort=True)  # reference torchpoints.py:152-153
+    # sort=True: reference test/test_ballquerry.py:25-34 (CPU tensors there; its CUDA path raises)
+    idx, dist = tpk.ball_query(1.01, 2, a, b, sort=True)
+    np.testing.assert_array_equal(_np(idx), [[[0, 1]], [[2, 2]]])
+    np.testing.assert_array_equal(_np(dist), np.array([[[0, 1]], [[1, -1]]], np.float32))
+    c = torch.tensor([[[0, 0, 0], [1, 0, 0], [1, 1, 0]]]).float().to(dev)
+    idx, dist = tpk.ball_query(1.01, 3, c, c, sort=True)
+    np.testing.assert_array_equal(_np(idx), [[[0, 1, 0], [1, 0, 2], [2, 1, 2]]])
 
 
 def test_kat_ball_query_partial(tpk, dev):
@@ -273,6 +278,68 @@ def test_ball_query_partial_cell_search_edges(tpk, oracle, dev):
         wi, wd = oracle.ball_query_partial_dense(r, ns, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
         np.testing.assert_array_equal(_np(idx), wi)
         np.testing.assert_array_equal(_np(dist), wd)
+
+
+# ------------------------------------------------------------------ ball query, sort=True
+
+
+@pytest.mark.parametrize("B,n,m,r,ns", [(2, 40, 30, 0.5, 5), (2, 300, 515, 0.2, 16), (1, 1000, 100, 0.15, 33), (3, 777, 600, 0.1, 8),
+                                        (1, 4096, 2500, 0.08, 32), (2, 600, 700, 0.3, 70), (1, 20000, 900, 0.05, 12),
+                                        (2, 70, 9, 2.0, 100), (1, 3000, 17000, 0.04, 4), (2, 0, 5, 0.5, 3)])
+def test_ball_query_sorted_dense_parity(tpk, oracle, dev, B, n, m, r, ns):
+    # n support points, m queries; from 512 points on the search goes over cells, nsample above 32 in rounds
+    g = torch.Generator().manual_seed(n + m + ns)
+    cases = [(torch.rand(B, n, 3, generator=g), torch.rand(B, m, 3, generator=g))]
+    if n >= 10:
+        cases.append((_clustered(g, B, n) * 0.3, _clustered(g, B, m) * 0.3))
+    for support, query in cases:
+        idx, dist = tpk.ball_query(r, ns, support.to(dev), query.to(dev), sort=True)
+        wi, wd = oracle.ball_query_sorted_dense(r, ns, support.numpy(), query.numpy())
+        assert idx.dtype == torch.int64 and idx.shape == (B, m, ns)
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist), wd)
+
+
+def test_ball_query_sorted_ties_and_boundary(tpk, oracle, dev):
+    # lattice: many equal distances, and points exactly at the radius (d2 == r2 does not count: strict <)
+    ax = torch.arange(9, dtype=torch.float32) * 0.25
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3).contiguous()
+    g = torch.Generator().manual_seed(2)
+    base = torch.rand(1, 300, 3, generator=g)
+    tripled = torch.cat([base, base.flip(1), base], 1)[:, torch.randperm(900, generator=g)].contiguous()
+    for support, query, r, ns in ((lattice, lattice, 0.25, 7), (lattice, lattice, 0.5, 40), (lattice, lattice + 0.125, 0.3, 9),
+                                  (tripled, base, 0.2, 10), (tripled, base, 0.05, 3)):
+        idx, dist = tpk.ball_query(r, ns, support.to(dev), query.contiguous().to(dev), sort=True)
+        wi, wd = oracle.ball_query_sorted_dense(r, ns, support.numpy(), query.numpy())
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist), wd)
+    idx, dist = tpk.ball_query(0.25, 7, lattice.to(dev), lattice.to(dev), sort=True)
+    assert (_np(dist)[0, :, 0] == 0).all() and (_np(dist)[0, :, 1:] == -1).all()  # only the point itself is inside
+
+
+@pytest.mark.parametrize("sizes,qfrac,r,ns", [((50, 70, 10), 0.5, 0.3, 8), ((3000, 1, 2100, 4500), 0.25, 0.1, 16),
+                                               ((2048, 2049), 0.1, 0.2, 64), ((700,), 1.0, 0.5, 100),
+                                               ((20000, 300), 0.05, 0.05, 12)])
+def test_ball_query_sorted_partial_parity(tpk, oracle, dev, sizes, qfrac, r, ns):
+    x, y, bx, by = _packed_case(17 + len(sizes), sizes, qfrac, 0.01)
+    idx, dist = tpk.ball_query(r, ns, x.to(dev), y.to(dev), mode="partial_dense", batch_x=bx.to(dev), batch_y=by.to(dev), sort=True)
+    wi, wd = oracle.ball_query_sorted_partial(r, ns, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), wd)
+
+
+def test_ball_query_sorted_partial_missing_clouds(tpk, oracle, dev):
+    # cloud ids with a gap (0, 2), queries whose cloud has no support points (1, 3), a cloud without queries
+    g = torch.Generator().manual_seed(6)
+    x = torch.rand(500, 3, generator=g)
+    bx = torch.cat([torch.zeros(100), torch.full((200,), 2), torch.full((200,), 5)]).long()
+    y = torch.rand(90, 3, generator=g)
+    by = torch.cat([torch.zeros(30), torch.ones(20), torch.full((30,), 2), torch.full((10,), 3)]).long()
+    idx, dist = tpk.ball_query(0.4, 12, x.to(dev), y.to(dev), mode="partial_dense", batch_x=bx.to(dev), batch_y=by.to(dev), sort=True)
+    wi, wd = oracle.ball_query_sorted_partial(0.4, 12, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), wd)
+    assert (_np(idx)[30:50] == -1).all() and (_np(idx)[80:] == -1).all()
 
 
 # ------------------------------------------------------------------ FPS

@@ -504,3 +504,69 @@ def test_grow_proximity_clusters_are_classes_of_the_smallest_reaching_point(orac
         got = oracle.grow_proximity_core(rows, 1)
         assert [sorted(c) for c in got] == want
         assert [c[0] for c in got] == [c[0] for c in want]  # a cluster starts with its smallest point
+
+
+# ------------------------------------------------------------------ ball query, sort=True
+
+
+def test_ball_query_sorted_reference_vectors(oracle):
+    # reference test/test_ballquerry.py:25-34
+    a = np.array([[[0, 0, 0], [1, 0, 0], [2, 0, 0]], [[0, 0, 0], [1, 0, 0], [2, 0, 0]]], np.float32)
+    b = np.array([[[0, 0, 0]], [[3, 0, 0]]], np.float32)
+    idx, dist = oracle.ball_query_sorted_dense(1.01, 2, a, b)
+    np.testing.assert_array_equal(idx, [[[0, 1]], [[2, 2]]])
+    np.testing.assert_array_equal(dist, np.array([[[0, 1]], [[1, -1]]], np.float32))
+    a = np.array([[[0, 0, 0], [1, 0, 0], [1, 1, 0]]], np.float32)
+    idx, _ = oracle.ball_query_sorted_dense(1.01, 3, a, a)
+    np.testing.assert_array_equal(idx, [[[0, 1, 0], [1, 0, 2], [2, 1, 2]]])
+    # reference test/test_ballquerry.py:81-96 (one hit, so the order plays no part)
+    x = np.array([[10, 0, 0], [0.1, 0, 0], [10, 0, 0], [10.1, 0, 0]], np.float32)
+    idx, dist = oracle.ball_query_sorted_partial(1.0, 2, x, np.zeros((1, 3), np.float32), np.zeros(4, np.int64), np.zeros(1, np.int64))
+    np.testing.assert_array_equal(idx, [[1, -1]])
+    np.testing.assert_allclose(dist, [[0.01, -1]], rtol=1e-6)
+
+
+def test_ball_query_sorted_is_a_stable_sort_of_the_hits(oracle):
+    """Independent statement: hits = d2 < r2 (float32, strict), order = stable argsort of their distances; duplicated
+    points and a lattice give equal distances, lattice spacing = radius gives points exactly on the sphere."""
+    rng = np.random.default_rng(11)
+    base = rng.random((2, 150, 3), dtype=np.float32)
+    ax = np.arange(6, dtype=np.float32) * 0.25
+    lattice = np.stack(np.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3)
+    for support, query, r, ns in ((np.concatenate([base, base[:, ::-1]], 1), base[:, :40], 0.3, 12), (lattice, lattice, 0.25, 5),
+                                  (lattice, lattice, 0.5, 30), (base, base[:, :10], 0.01, 4)):
+        idx, dist = oracle.ball_query_sorted_dense(r, ns, support, query)
+        d = ((query[:, :, None, :] - support[:, None, :, :]) ** 2)
+        d = (d[..., 0] + d[..., 1]) + d[..., 2]
+        r2 = np.float32(r) * np.float32(r)
+        for b in range(support.shape[0]):
+            for j in range(query.shape[1]):
+                hits = np.nonzero(d[b, j] < r2)[0]
+                order = hits[np.argsort(d[b, j][hits], kind="stable")][:ns]
+                k = len(order)
+                np.testing.assert_array_equal(idx[b, j, :k], order)
+                np.testing.assert_array_equal(dist[b, j, :k], d[b, j][order])
+                assert (dist[b, j, k:] == -1).all() and (idx[b, j, k:] == (order[0] if k else 0)).all()
+
+
+def test_ball_query_sorted_against_reference_cpu_module(oracle, ref_cpu):
+    # the reference's own sort=True path (cpu/src/ball_query.cpp, nanoflann) on data without equal distances: bit-exact
+    if ref_cpu is None:
+        pytest.skip("oracle/_ref not built")
+    import torch
+
+    g = torch.Generator().manual_seed(4)
+    for n, m, r, ns in ((500, 200, 0.6, 12), (64, 300, 1.0, 70), (2000, 100, 0.2, 5), (30, 20, 0.01, 4)):
+        support, query = torch.randn(3, n, 3, generator=g), torch.randn(3, m, 3, generator=g)
+        ri, rd = ref_cpu.dense_ball_query(query, support, r, ns, 0, True)
+        oi, od = oracle.ball_query_sorted_dense(r, ns, support.numpy(), query.numpy())
+        np.testing.assert_array_equal(oi, ri.numpy())
+        np.testing.assert_array_equal(od, rd.numpy())
+    x, y = torch.randn(900, 3, generator=g), torch.randn(300, 3, generator=g)
+    bx = torch.sort(torch.randint(0, 3, (900,), generator=g))[0]
+    by = torch.sort(torch.randint(0, 3, (300,), generator=g))[0]
+    for r, ns in ((0.5, 9), (1.5, 40), (0.05, 3)):
+        ri, rd = ref_cpu.batch_ball_query(x, y, bx, by, r, ns, 0, True)
+        oi, od = oracle.ball_query_sorted_partial(r, ns, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+        np.testing.assert_array_equal(oi, ri.numpy())
+        np.testing.assert_array_equal(od, rd.numpy())

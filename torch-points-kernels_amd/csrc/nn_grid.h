@@ -20,9 +20,10 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
                       int32_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 // k nearest neighbours, float32 (n queries, m support points per cloud; idx int64, both outputs
-// (b, n, k), ascending by (squared distance, index)): same conventions.
+// (b, n, k), ascending by (squared distance, index)): same conventions.  Only support points with
+// squared distance < limit count (+inf: all); entries that stay empty are written as (limit, 0).
 size_t tpk_grid_knn_workspace_bytes(int b, int n, int m);
-int tpk_grid_knn(int b, int n, int m, int k, const float* query, const float* support, float* dist2,
+int tpk_grid_knn(int b, int n, int m, int k, float limit, const float* query, const float* support, float* dist2,
                  int64_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 // Ball query, packed layout (a hit has squared distance <= radius2 = radius * radius as the caller

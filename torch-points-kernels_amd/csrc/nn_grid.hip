@@ -458,7 +458,7 @@ __device__ __forceinline__ void scan_cell_k(const float4* __restrict__ cand, con
 // first: number of entries found by earlier rounds; count: entries this round finds (<= K).
 template <int K>
 __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
-    int n, int k, int first, int count, int qcells, int ccells, int clouds,
+    int n, int k, int first, int count, float limit, int qcells, int ccells, int clouds,
     const float4* __restrict__ sorted_query, const float4* __restrict__ sorted_support,
     const float4* __restrict__ boxes_query, const float4* __restrict__ boxes_support,
     float* __restrict__ dist2, int64_t* __restrict__ idx)
@@ -496,7 +496,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
         // the last pair of the round before (rounds of one call run one after the other)
         const int64_t at = static_cast<int64_t>(real ? qindex : 0) * k + first - 1;
         const bool later = first > 0 && real;
-        s.reset(first > 0, later ? dist2[at] : 0.f, later ? static_cast<int>(idx[at]) : 0, !real);
+        s.reset(first > 0, later ? dist2[at] : 0.f, later ? static_cast<int>(idx[at]) : 0, !real, limit);
     }
 
     const int groups = (ccells + NG_CELL - 1) / NG_CELL;
@@ -912,7 +912,7 @@ size_t tpk_grid_knn_workspace_bytes(int b, int n, int m)
 namespace {
 
 template <int K>
-int launch_knn_grid(int b, int n, int k, int qcells, int ccells, const PointSet& a, const PointSet& c,
+int launch_knn_grid(int b, int n, int k, float limit, int qcells, int ccells, const PointSet& a, const PointSet& c,
                     float* dist2, int64_t* idx, hipStream_t s)
 {
     const int64_t waves = static_cast<int64_t>(qcells) * b;
@@ -924,7 +924,7 @@ int launch_knn_grid(int b, int n, int k, int qcells, int ccells, const PointSet&
     for (int first = 0; first < k; first += K)
     {
         hipLaunchKernelGGL(knn_grid_kernel<K>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
-                           k, first, k - first < K ? k - first : K, qcells, ccells, b, a.sorted, c.sorted, a.boxes,
+                           k, first, k - first < K ? k - first : K, limit, qcells, ccells, b, a.sorted, c.sorted, a.boxes,
                            c.boxes, dist2, idx);
         const int st = tpk_launch_status();
         if (st != TPK_OK)
@@ -936,7 +936,7 @@ int launch_knn_grid(int b, int n, int k, int qcells, int ccells, const PointSet&
 } // namespace
 
 // n queries and m support points per cloud.
-int tpk_grid_knn(int b, int n, int m, int k, const float* query, const float* support, float* dist2,
+int tpk_grid_knn(int b, int n, int m, int k, float limit, const float* query, const float* support, float* dist2,
                  int64_t* idx, void* workspace, size_t workspace_bytes, hipStream_t s)
 {
     if (!grid_supported(b, n, m) || static_cast<int64_t>(b) * 2 > 0x7fffffffLL)
@@ -954,12 +954,12 @@ int tpk_grid_knn(int b, int n, int m, int k, const float* query, const float* su
         return st;
     const int qcells = grid_cells(n), ccells = grid_cells(m);
     if (k <= 4)
-        return launch_knn_grid<4>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
+        return launch_knn_grid<4>(b, n, k, limit, qcells, ccells, a, c, dist2, idx, s);
     if (k <= 8)
-        return launch_knn_grid<8>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
+        return launch_knn_grid<8>(b, n, k, limit, qcells, ccells, a, c, dist2, idx, s);
     if (k <= 16)
-        return launch_knn_grid<16>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
-    return launch_knn_grid<KNN_MAX_K>(b, n, k, qcells, ccells, a, c, dist2, idx, s);
+        return launch_knn_grid<16>(b, n, k, limit, qcells, ccells, a, c, dist2, idx, s);
+    return launch_knn_grid<KNN_MAX_K>(b, n, k, limit, qcells, ccells, a, c, dist2, idx, s);
 }
 
 namespace {

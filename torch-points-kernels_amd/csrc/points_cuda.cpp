@@ -258,8 +258,10 @@ at::Tensor three_interpolate_grad(at::Tensor grad_out, at::Tensor idx, at::Tenso
 }
 
 // cuda/src/ball_query.cpp:15-36.  Query centres first, as in the reference.
+// sorted: the nsample nearest neighbours within the radius, nearest first (what the reference
+// computes for CPU tensors with sort=True, cpu/src/ball_query.cpp:127-146).
 std::pair<at::Tensor, at::Tensor> ball_query_dense(at::Tensor new_xyz, at::Tensor xyz,
-                                                   const float radius, const int nsample)
+                                                   const float radius, const int nsample, const bool sorted)
 {
     check_contiguous(new_xyz, "new_xyz");
     check_contiguous(xyz, "xyz");
@@ -278,6 +280,21 @@ std::pair<at::Tensor, at::Tensor> ball_query_dense(at::Tensor new_xyz, at::Tenso
                                   at::device(new_xyz.device()).dtype(at::ScalarType::Long));
     at::Tensor dist = torch::empty({new_xyz.size(0), new_xyz.size(1), nsample},
                                    at::device(new_xyz.device()).dtype(at::ScalarType::Float));
+    if (sorted)
+    {
+        const int b = as_int(xyz.size(0), "batch size"), n = as_int(xyz.size(1), "support points");
+        const int m = as_int(new_xyz.size(1), "query points");
+        const size_t ws_bytes = tpk_ball_query_sorted_dense_workspace_bytes(b, n, m);
+        at::Tensor ws;
+        if (ws_bytes)
+            ws = torch::empty({static_cast<int64_t>(ws_bytes)}, new_xyz.options().dtype(torch::kUInt8));
+        check_status(tpk_ball_query_sorted_dense_f32(b, n, m, radius, nsample, new_xyz.data_ptr<float>(),
+                                                     xyz.data_ptr<float>(), idx.data_ptr<int64_t>(),
+                                                     dist.data_ptr<float>(), ws_bytes ? ws.data_ptr() : nullptr,
+                                                     ws_bytes, current_stream(new_xyz)),
+                     "ball_query_dense (sorted)");
+        return std::make_pair(idx, dist);
+    }
     check_status(tpk_ball_query_dense_f32(
                      as_int(xyz.size(0), "batch size"), as_int(xyz.size(1), "support points"),
                      as_int(new_xyz.size(1), "query points"), radius, nsample,
@@ -291,7 +308,7 @@ std::pair<at::Tensor, at::Tensor> ball_query_dense(at::Tensor new_xyz, at::Tenso
 // are found on the device from the sorted batch vectors; nothing is copied to the host.
 std::pair<at::Tensor, at::Tensor> ball_query_partial_dense(at::Tensor x, at::Tensor y,
                                                            at::Tensor batch_x, at::Tensor batch_y,
-                                                           const float radius, const int nsample)
+                                                           const float radius, const int nsample, const bool sorted)
 {
     check_contiguous(x, "x");
     check_contiguous(y, "y");
@@ -321,6 +338,16 @@ std::pair<at::Tensor, at::Tensor> ball_query_partial_dense(at::Tensor x, at::Ten
         torch::empty({y.size(0), nsample}, at::device(y.device()).dtype(at::ScalarType::Long));
     at::Tensor dist =
         torch::empty({y.size(0), nsample}, at::device(y.device()).dtype(at::ScalarType::Float));
+    if (sorted)
+    {
+        // cpu/src/ball_query.cpp:65-124 with sorted = true
+        check_status(tpk_ball_query_sorted_partial_f32(x.size(0), y.size(0), radius, nsample, x.data_ptr<float>(),
+                                                       y.data_ptr<float>(), batch_x.data_ptr<int64_t>(),
+                                                       batch_y.data_ptr<int64_t>(), idx.data_ptr<int64_t>(),
+                                                       dist.data_ptr<float>(), current_stream(x)),
+                     "ball_query_partial_dense (sorted)");
+        return std::make_pair(idx, dist);
+    }
     const size_t ws_bytes = tpk_ball_query_partial_workspace_bytes(x.size(0), y.size(0), nsample);
     at::Tensor ws;
     if (ws_bytes)
@@ -512,8 +539,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("grow_proximity", &grow_proximity);
     m.def("three_interpolate", &three_interpolate);
     m.def("three_interpolate_grad", &three_interpolate_grad);
-    m.def("ball_query_dense", &ball_query_dense);
-    m.def("ball_query_partial_dense", &ball_query_partial_dense);
+    m.def("ball_query_dense", &ball_query_dense, pybind11::arg("new_xyz"), pybind11::arg("xyz"), pybind11::arg("radius"),
+          pybind11::arg("nsample"), pybind11::arg("sorted") = false);
+    m.def("ball_query_partial_dense", &ball_query_partial_dense, pybind11::arg("x"), pybind11::arg("y"),
+          pybind11::arg("batch_x"), pybind11::arg("batch_y"), pybind11::arg("radius"), pybind11::arg("nsample"),
+          pybind11::arg("sorted") = false);
     m.def("grouping_operation", &grouping_operation);
     m.def("grouping_operation_grad", &grouping_operation_grad);
     m.def("chamfer_dist", &chamfer_dist);

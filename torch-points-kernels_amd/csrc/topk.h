@@ -28,16 +28,19 @@ struct NearestK
     unsigned long long after;
     bool from_start;
 
-    // An inert lane (no query) never admits a candidate.
-    __device__ __forceinline__ void reset(bool later_round, float last_d, int last_i, bool inert)
+    // An inert lane (no query) never admits a candidate.  Only candidates closer than `limit`
+    // (squared; +inf for a plain k-nearest search) are admitted; entries that stay empty read
+    // (limit, 0), which no candidate equals.
+    __device__ __forceinline__ void reset(bool later_round, float last_d, int last_i, bool inert, float limit)
     {
+        const unsigned long long empty = knn_key(limit, limit == __builtin_inff() ? 0x7FFFFFFF : 0);
 #pragma unroll
         for (int j = 0; j < K; ++j)
-            key[j] = inert ? 0ull : knn_key(__builtin_inff(), 0x7FFFFFFF);
+            key[j] = inert ? 0ull : empty;
         after = later_round ? knn_key(last_d, last_i) : 0ull;
         from_start = !later_round;
     }
-    // Squared distance of the last entry (+inf while the list is not full; -1 for an inert lane).
+    // Squared distance of the last entry (the limit while the list is not full; -1 for an inert lane).
     __device__ __forceinline__ float worst() const
     {
         return key[K - 1] == 0ull ? -1.f : __int_as_float(static_cast<int>(key[K - 1] >> 32));

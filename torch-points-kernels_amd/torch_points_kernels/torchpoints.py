@@ -83,18 +83,17 @@ def grouping_operation(features, idx):
 def ball_query_dense(radius, nsample, xyz, new_xyz, batch_xyz=None, batch_new_xyz=None, sort=False):
     """Reference: torchpoints.py:149-157.  Returns (idx int64 (B, M, nsample), dist2 float32)."""
     require_gpu(new_xyz, "ball_query_dense")
-    if sort:
-        raise NotImplementedError("CUDA version does not sort the neighbors")
-    ind, dist = native().ball_query_dense(new_xyz, xyz, radius, nsample)
+    # sort=True: the nsample nearest neighbours within the radius, nearest first - what the reference
+    # computes for CPU tensors (torchpoints.py:154-155); its CUDA path raises NotImplementedError.
+    ind, dist = native().ball_query_dense(new_xyz, xyz, radius, nsample, bool(sort))
     return ind, dist
 
 
 def ball_query_partial_dense(radius, nsample, x, y, batch_x, batch_y, sort=False):
     """Reference: torchpoints.py:160-168.  Returns (idx int64 (|y|, nsample), dist2 float32)."""
     require_gpu(x, "ball_query_partial_dense")
-    if sort:
-        raise NotImplementedError("CUDA version does not sort the neighbors")
-    ind, dist = native().ball_query_partial_dense(x, y, batch_x, batch_y, radius, nsample)
+    # sort=True: as for the dense layout (reference, CPU tensors only: torchpoints.py:165-166)
+    ind, dist = native().ball_query_partial_dense(x, y, batch_x, batch_y, radius, nsample, bool(sort))
     return ind, dist
 
 
