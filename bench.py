@@ -161,6 +161,19 @@ def bench_others(dev, steps, warmup, with_cpu):
                              "sample": "whole configuration, reference cpu/src (nanoflann kd-tree), 1 thread"}
     out["ball_query_dense"] = e
 
+    # beyond the BASELINE configurations: the same query with sort=True (nearest nsample first), which the
+    # reference computes for CPU tensors only
+    wall, ev = _time_gpu(lambda: tpk.ball_query(w["radius"], w["nsample"], xyz, new_xyz, mode="dense", sort=True), steps, warmup)
+    e = {"workload": "ball_query dense sort=True on configs[0] (B=8 N=4096 M=1024 r=0.1 nsample=32; the reference has this "
+                     "mode for CPU tensors only)", "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev,
+         "wall_ms": wall, "roofline": _roof_flops(pairs, 8, ev), "pairs": pairs}
+    e["roofline"]["note"] += PRUNED_NOTE
+    if ref is not None:
+        secs = _cpu_time(lambda: ref.dense_ball_query(w["new_xyz"], w["xyz"], w["radius"], w["nsample"], 0, True))
+        e["cpu_baseline"] = {"value": nq / secs, "unit": "queries/s", "cores": 1, "kind": "reference",
+                             "sample": "whole configuration, reference cpu/src (nanoflann radius search, sorted), 1 thread"}
+    out["ball_query_dense_sorted"] = e
+
     # configs[3]: partial dense ball query
     w = W.cfg4_ball_query_partial()
     x, y, bx, by = (w[k].to(dev) for k in ("x", "y", "batch_x", "batch_y"))
@@ -180,6 +193,18 @@ def bench_others(dev, steps, warmup, with_cpu):
         e["cpu_baseline"] = {"value": nq / secs, "unit": "queries/s", "cores": 1, "kind": "reference",
                              "sample": "whole configuration, reference cpu/src (nanoflann kd-tree per cloud), 1 thread"}
     out["ball_query_partial_dense"] = e
+    wall, ev = _time_gpu(lambda: tpk.ball_query(w["radius"], w["nsample"], x, y, mode="partial_dense", batch_x=bx, batch_y=by,
+                                                sort=True), max(3, steps // 4), 1)
+    e = {"workload": "ball_query partial_dense sort=True on configs[3] (the reference has this mode for CPU tensors only)",
+         "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
+         "roofline": _roof_flops(pairs, 8, ev), "pairs": pairs}
+    e["roofline"]["note"] += "; every pair of a query with its cloud is tested (no cell search for this mode yet)"
+    if ref is not None:
+        secs = _cpu_time(lambda: ref.batch_ball_query(w["x"], w["y"], w["batch_x"], w["batch_y"], w["radius"],
+                                                      w["nsample"], 0, True))
+        e["cpu_baseline"] = {"value": nq / secs, "unit": "queries/s", "cores": 1, "kind": "reference",
+                             "sample": "whole configuration, reference cpu/src (nanoflann radius search per cloud, sorted), 1 thread"}
+    out["ball_query_partial_dense_sorted"] = e
 
     # configs[2](a): three_nn + three_interpolate fwd/bwd
     w = W.cfg3a_interpolate()

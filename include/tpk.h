@@ -4,8 +4,8 @@
  *
  * Every entry point takes plain device pointers and sizes, launches on the HIP stream
  * passed as `stream` (a hipStream_t cast to void*; NULL = the null stream), never
- * allocates, never synchronises the host (tpk_grow_proximity, whose output sizes depend on
- * the data, is the one exception) and keeps no state between calls.  The caller
+ * allocates, never synchronises the host (exceptions, documented below: tpk_grow_proximity and
+ * tpk_ball_query_sorted_partial_f32 with a workspace) and keeps no state between calls.  The caller
  * owns all memory.  All arrays are dense row-major ("contiguous").  Outputs need not be
  * initialised: every element of every output array is written by the call.
  *
@@ -101,18 +101,21 @@ int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int
  * tensors torch_points_kernels/torchpoints.py:152-153 and :163-164 raise.
  * Shapes and dtypes as for tpk_ball_query_dense_f32 / tpk_ball_query_partial_f32.  Unused
  * slots: dense - idx repeats the nearest neighbour (0 when there is none), dist -1; packed -
- * both -1.  Dense layout: with a `workspace` (tpk_ball_query_sorted_dense_workspace_bytes()
- * bytes - 0 for shapes not served that way -, 256-byte aligned) the search goes over
- * curve-ordered cells within the radius instead of all pairs, same results.  The packed
- * layout tests all pairs of a query with its cloud.
+ * both -1.  With a `workspace` (tpk_ball_query_sorted_*_workspace_bytes() bytes - 0 for
+ * shapes not served that way -, 256-byte aligned) the search goes over curve-ordered cells
+ * within the radius instead of all pairs, same results.  In the packed layout this is done
+ * cloud by cloud (clouds of 512..163840 points and queries, cloud ids below 1024; others by
+ * all pairs), and the call then waits for the stream once, to read where the clouds start.
  * ------------------------------------------------------------------------------------- */
 size_t tpk_ball_query_sorted_dense_workspace_bytes(int b, int n, int m);
 int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius, int nsample,
                                     const float* new_xyz, const float* xyz, int64_t* idx, float* dist,
                                     void* workspace, size_t workspace_bytes, void* stream);
+size_t tpk_ball_query_sorted_partial_workspace_bytes(int64_t size_x, int64_t size_y);
 int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y, float radius, int nsample,
                                       const float* x, const float* y, const int64_t* batch_x,
-                                      const int64_t* batch_y, int64_t* idx, float* dist, void* stream);
+                                      const int64_t* batch_y, int64_t* idx, float* dist,
+                                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Three nearest neighbours.

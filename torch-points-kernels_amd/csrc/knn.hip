@@ -20,6 +20,49 @@ namespace {
 constexpr int KNN_THREADS = 256;
 constexpr int KNN_TILE = 1024; // support points per LDS tile (16 KiB)
 
+constexpr int KNN_GROUP = 8;   // candidates whose distances are formed together
+
+// The `cnt` candidates of an LDS tile (indices base, base + 1, ...) offered to the lane's list.
+// Distances are formed KNN_GROUP at a time, so that the LDS reads overlap; the list is only
+// touched when the nearest of a group can enter it.
+template <int K>
+__device__ __forceinline__ void scan_tile(const float4* tile, int cnt, int base, float qx, float qy, float qz,
+                                          NearestK<K>& s)
+{
+    float worst = s.worst();
+    int c = 0;
+    for (; c + KNN_GROUP <= cnt; c += KNN_GROUP)
+    {
+        float d[KNN_GROUP];
+        float nearest = 0.f;
+#pragma unroll
+        for (int i = 0; i < KNN_GROUP; ++i)
+        {
+            const float4 p = tile[c + i];
+            d[i] = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            nearest = i == 0 ? d[i] : fminf(nearest, d[i]);
+        }
+        if (nearest <= worst)
+        {
+#pragma unroll
+            for (int i = 0; i < KNN_GROUP; ++i)
+            {
+                const unsigned long long cand = knn_key(d[i], base + c + i);
+                if (s.admits(cand))
+                    s.insert(cand);
+            }
+            worst = s.worst();
+        }
+    }
+    for (; c < cnt; ++c)
+    {
+        const float4 p = tile[c];
+        const unsigned long long cand = knn_key(tpk_dist2(qx, qy, qz, p.x, p.y, p.z), base + c);
+        if (s.admits(cand))
+            s.insert(cand);
+    }
+}
+
 // first: number of entries found by earlier rounds; count: entries this round finds (<= K).
 template <int K>
 __global__ __launch_bounds__(KNN_THREADS) void knn_kernel(
@@ -68,13 +111,7 @@ __global__ __launch_bounds__(KNN_THREADS) void knn_kernel(
         }
         __syncthreads();
 
-        for (int c = 0; c < cnt; ++c)
-        {
-            const float4 p = tile[c];
-            const unsigned long long cand = knn_key(tpk_dist2(qx, qy, qz, p.x, p.y, p.z), base + c);
-            if (s.admits(cand))
-                s.insert(cand);
-        }
+        scan_tile<K>(tile, cnt, base, qx, qy, qz, s);
     }
 
     if (real)
@@ -166,15 +203,22 @@ extern "C" int tpk_knn_f32(int b, int n_support, int m_query, int k, const float
 namespace {
 
 // Slots the search left empty read (limit, 0); they become the padding of the layout.
+// Indices of found neighbours are raised by `add` (packed layout searched cloud by cloud: the
+// position of the cloud's first support point).
 __global__ __launch_bounds__(KNN_THREADS) void pad_sorted_kernel(int64_t slots, int nsample, float limit, bool packed,
-                                                                 int64_t* __restrict__ idx, float* __restrict__ dist)
+                                                                 int64_t add, int64_t* __restrict__ idx,
+                                                                 float* __restrict__ dist)
 {
     const int64_t o = static_cast<int64_t>(blockIdx.x) * KNN_THREADS + threadIdx.x;
     if (o >= slots)
         return;
     const float d = dist[o];
     if (d < limit)
+    {
+        if (add != 0)
+            idx[o] += add;
         return;
+    }
     // The first slot of the row: the nearest neighbour, or the empty entry's 0 (also after this
     // kernel has padded it, in the dense layout).
     const int64_t token = packed ? -1 : idx[o - o % nsample];
@@ -183,14 +227,15 @@ __global__ __launch_bounds__(KNN_THREADS) void pad_sorted_kernel(int64_t slots, 
     dist[o] = -1.0f;
 }
 
-int pad_sorted(int64_t rows, int nsample, float limit, bool packed, int64_t* idx, float* dist, hipStream_t s)
+int pad_sorted(int64_t rows, int nsample, float limit, bool packed, int64_t add, int64_t* idx, float* dist,
+               hipStream_t s)
 {
     const int64_t slots = rows * nsample;
     const int64_t blocks = tpk_ceil_div(slots, KNN_THREADS);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(pad_sorted_kernel, dim3(static_cast<unsigned>(blocks)), dim3(KNN_THREADS), 0, s, slots, nsample,
-                       limit, packed, idx, dist);
+                       limit, packed, add, idx, dist);
     return tpk_launch_status();
 }
 
@@ -252,14 +297,7 @@ __global__ __launch_bounds__(KNN_THREADS) void nearest_packed_kernel(
             }
             __syncthreads();
             if (in_run)
-                for (int p = 0; p < cnt; ++p)
-                {
-                    const float4 v = tile[p];
-                    const unsigned long long cand =
-                        knn_key(tpk_dist2(qx, qy, qz, v.x, v.y, v.z), static_cast<int>(base + p));
-                    if (s.admits(cand))
-                        s.insert(cand);
-                }
+                scan_tile<K>(tile, cnt, static_cast<int>(base), qx, qy, qz, s);
         }
         run_start = run_end > run_start ? run_end : run_start + 1;
     }
@@ -319,12 +357,60 @@ extern "C" int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius
     const int st = nearest_within(b, n, m, nsample, limit, xyz, new_xyz, idx, dist, workspace, workspace_bytes, s);
     if (st != TPK_OK)
         return st;
-    return pad_sorted(static_cast<int64_t>(b) * m, nsample, limit, false, idx, dist, s);
+    return pad_sorted(static_cast<int64_t>(b) * m, nsample, limit, false, 0, idx, dist, s);
+}
+
+namespace {
+
+constexpr int NP_MAX_CLOUDS = 1024; // cloud ids served cloud by cloud; larger ids: all pairs in one launch
+
+// ranges[c] / ranges[NP_MAX_CLOUDS + 1 + c]: position of the first support point / query with
+// cloud id >= c, for c = 0 .. NP_MAX_CLOUDS.
+__global__ __launch_bounds__(KNN_THREADS) void cloud_ranges_kernel(int64_t size_x, int64_t size_y,
+                                                                   const int64_t* __restrict__ batch_x,
+                                                                   const int64_t* __restrict__ batch_y,
+                                                                   int64_t* __restrict__ ranges)
+{
+    const int c = blockIdx.x * KNN_THREADS + threadIdx.x;
+    if (c > NP_MAX_CLOUDS)
+        return;
+    ranges[c] = first_not_below(batch_x, size_x, c);
+    ranges[NP_MAX_CLOUDS + 1 + c] = first_not_below(batch_y, size_y, c);
+}
+
+int nearest_packed(int64_t size_x, int64_t size_y, int nsample, float limit, const float* x, const float* y,
+                   const int64_t* batch_x, const int64_t* batch_y, int64_t* idx, float* dist, hipStream_t s)
+{
+    if (nsample <= 4)
+        return launch_nearest_packed<4>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
+    if (nsample <= 8)
+        return launch_nearest_packed<8>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
+    if (nsample <= 16)
+        return launch_nearest_packed<16>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
+    return launch_nearest_packed<KNN_MAX_K>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
+}
+
+constexpr size_t NP_RANGES_BYTES = (2 * (NP_MAX_CLOUDS + 1) * sizeof(int64_t) + 255) / 256 * 256;
+constexpr int64_t NP_GRID_POINTS = 163840; // largest cloud the search over cells takes
+
+} // namespace
+
+// The workspace lets clouds of 512..163840 points (support and queries) be searched over
+// curve-ordered cells, one cloud after the other; the call then waits for the stream once, to
+// read the clouds' ranges.
+extern "C" size_t tpk_ball_query_sorted_partial_workspace_bytes(int64_t size_x, int64_t size_y)
+{
+    if (size_x < 512 || size_y < 512)
+        return 0;
+    const size_t grid = tpk_grid_knn_workspace_bytes(1, static_cast<int>(tpk_min64(size_y, NP_GRID_POINTS)),
+                                                     static_cast<int>(tpk_min64(size_x, NP_GRID_POINTS)));
+    return grid ? NP_RANGES_BYTES + grid : 0;
 }
 
 extern "C" int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y, float radius, int nsample,
                                                  const float* x, const float* y, const int64_t* batch_x,
-                                                 const int64_t* batch_y, int64_t* idx, float* dist, void* stream)
+                                                 const int64_t* batch_y, int64_t* idx, float* dist, void* workspace,
+                                                 size_t workspace_bytes, void* stream)
 {
     if (size_x < 0 || size_y < 0 || nsample < 0)
         return TPK_ERR_INVALID_ARG;
@@ -336,16 +422,58 @@ extern "C" int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y,
         return TPK_ERR_UNSUPPORTED;
     hipStream_t s = tpk_stream(stream);
     const float limit = radius * radius; // fp32 product (cpu/src/neighbors.cpp:153)
-    int st;
-    if (nsample <= 4)
-        st = launch_nearest_packed<4>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
-    else if (nsample <= 8)
-        st = launch_nearest_packed<8>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
-    else if (nsample <= 16)
-        st = launch_nearest_packed<16>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
-    else
-        st = launch_nearest_packed<KNN_MAX_K>(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
-    if (st != TPK_OK)
-        return st;
-    return pad_sorted(size_y, nsample, limit, true, idx, dist, s);
+    const size_t wanted = tpk_ball_query_sorted_partial_workspace_bytes(size_x, size_y);
+    if (!workspace || wanted == 0)
+    {
+        const int st = nearest_packed(size_x, size_y, nsample, limit, x, y, batch_x, batch_y, idx, dist, s);
+        return st != TPK_OK ? st : pad_sorted(size_y, nsample, limit, true, 0, idx, dist, s);
+    }
+    if (workspace_bytes < wanted || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return TPK_ERR_WORKSPACE;
+
+    // Where every cloud starts in both arrays.
+    static_assert(NP_MAX_CLOUDS + 1 <= 5 * KNN_THREADS, "one thread per cloud id");
+    int64_t* ranges_dev = static_cast<int64_t*>(workspace);
+    hipLaunchKernelGGL(cloud_ranges_kernel, dim3(5), dim3(KNN_THREADS), 0, s, size_x, size_y, batch_x, batch_y, ranges_dev);
+    int64_t ranges[2 * (NP_MAX_CLOUDS + 1)];
+    hipError_t e = hipMemcpyAsync(ranges, ranges_dev, sizeof(ranges), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(s);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    const int64_t* rx = ranges;
+    const int64_t* ry = ranges + NP_MAX_CLOUDS + 1;
+    void* grid_ws = static_cast<char*>(workspace) + NP_RANGES_BYTES;
+    const size_t grid_bytes = workspace_bytes - NP_RANGES_BYTES;
+
+    // Queries q0..q1 (one cloud when `points` >= 0: its support points are s0 .. s0 + points).
+    auto segment = [&](int64_t q0, int64_t q1, int64_t s0, int64_t points) -> int {
+        if (q1 <= q0)
+            return TPK_OK;
+        const int64_t queries = q1 - q0;
+        int64_t* idx_c = idx + q0 * nsample;
+        float* dist_c = dist + q0 * nsample;
+        int st = TPK_ERR_UNSUPPORTED;
+        int64_t add = 0;
+        if (points >= 0 && queries <= NP_GRID_POINTS && points <= NP_GRID_POINTS &&
+            tpk_grid_knn_workspace_bytes(1, static_cast<int>(queries), static_cast<int>(points)) != 0)
+        {
+            // search over cells; it numbers the support points from the cloud's first one
+            st = tpk_grid_knn(1, static_cast<int>(queries), static_cast<int>(points), nsample, limit, y + q0 * 3,
+                              x + s0 * 3, dist_c, idx_c, grid_ws, grid_bytes, s);
+            add = s0;
+        }
+        if (st == TPK_ERR_UNSUPPORTED)
+        {
+            st = nearest_packed(size_x, queries, nsample, limit, x, y + q0 * 3, batch_x, batch_y + q0, idx_c, dist_c, s);
+            add = 0;
+        }
+        return st != TPK_OK ? st : pad_sorted(queries, nsample, limit, true, add, idx_c, dist_c, s);
+    };
+    int st = segment(0, ry[0], 0, -1); // negative cloud ids, if any: all pairs
+    for (int c = 0; c < NP_MAX_CLOUDS && st == TPK_OK; ++c)
+        st = segment(ry[c], ry[c + 1], rx[c], rx[c + 1] - rx[c]);
+    if (st == TPK_OK)
+        st = segment(ry[NP_MAX_CLOUDS], size_y, 0, -1); // cloud ids of NP_MAX_CLOUDS and more: all pairs
+    return st;
 }

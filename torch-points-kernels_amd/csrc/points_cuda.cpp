@@ -341,10 +341,16 @@ std::pair<at::Tensor, at::Tensor> ball_query_partial_dense(at::Tensor x, at::Ten
     if (sorted)
     {
         // cpu/src/ball_query.cpp:65-124 with sorted = true
+        const size_t sorted_ws_bytes = tpk_ball_query_sorted_partial_workspace_bytes(x.size(0), y.size(0));
+        at::Tensor sorted_ws;
+        if (sorted_ws_bytes)
+            sorted_ws = torch::empty({static_cast<int64_t>(sorted_ws_bytes)}, x.options().dtype(torch::kUInt8));
         check_status(tpk_ball_query_sorted_partial_f32(x.size(0), y.size(0), radius, nsample, x.data_ptr<float>(),
                                                        y.data_ptr<float>(), batch_x.data_ptr<int64_t>(),
                                                        batch_y.data_ptr<int64_t>(), idx.data_ptr<int64_t>(),
-                                                       dist.data_ptr<float>(), current_stream(x)),
+                                                       dist.data_ptr<float>(),
+                                                       sorted_ws_bytes ? sorted_ws.data_ptr() : nullptr, sorted_ws_bytes,
+                                                       current_stream(x)),
                      "ball_query_partial_dense (sorted)");
         return std::make_pair(idx, dist);
     }
