@@ -256,6 +256,28 @@ int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbours, int64_
                        int member_order, int64_t* members, int64_t* starts, int64_t* found,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * IoU between proposed instances and ground-truth instances.
+ * Replaces instance_iou_kernel_wrapper(total_gt_instances, max_gt_instances, nInstance,
+ * nProposal, proposals_idx, proposals_offset, instance_labels, offset_num_gt_instances, batch,
+ * instance_pointnum, proposals_iou) (cuda/src/metrics_gpu.cu:50-61, declared
+ * cuda/src/metrics.cpp:5-10; max_gt_instances only sized the reference's blocks).
+ *   proposals_idx (sum of proposal sizes) int64: point indices, proposal after proposal
+ *   proposals_offset (n_proposals + 1) int64     instance_labels (n_points) int64: k + 1 for
+ *   ground-truth instance k of the point's sample, 0 or negative for none
+ *   batch (n_points) int64: sample of a point     num_gt_instances, offset_num_gt_instances
+ *   (n_samples, n_samples + 1) int64: instances per sample and their first output column
+ *   instance_pointnum (total_gt_instances) int64: points per ground-truth instance
+ *   proposals_iou (n_proposals, total_gt_instances) float32: intersection / (union + 1e-5)
+ *   with the instances of the sample of the proposal's first point, 0 elsewhere.
+ * n_points and n_samples bound what the kernel reads; indices outside are ignored.
+ * ------------------------------------------------------------------------------------- */
+int tpk_instance_iou(int64_t total_gt_instances, int64_t n_proposals, int64_t n_points, int64_t n_samples,
+                     const int64_t* num_gt_instances, const int64_t* proposals_idx,
+                     const int64_t* proposals_offset, const int64_t* instance_labels,
+                     const int64_t* offset_num_gt_instances, const int64_t* batch,
+                     const int64_t* instance_pointnum, float* proposals_iou, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -314,3 +314,29 @@ def chamfer_bwd(xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2):
         _p(idx1, _i32p), _p(idx2, _i32p), _p(grad_dist1, pt), _p(grad_dist2, pt), _p(g1, pt),
         _p(g2, pt))
     return g1, g2
+
+
+def instance_iou(instance_idx, gt_instances, batch=None):
+    """torch_points_kernels/metrics.py:37-104 (front end) + cuda/src/metrics_gpu.cu:9-43: instance_idx is a list of
+    index arrays (the proposals), gt_instances the label of every point (0: none), batch the sample of every point.
+    -> float32 (proposals, ground-truth instances of all samples)."""
+    gt = _c(gt_instances, np.int64)
+    batch = np.zeros_like(gt) if batch is None else _c(batch, np.int64)
+    sizes, counts = [], []
+    for s in range(int(batch[-1]) + 1):
+        sample = gt[batch == s]
+        count = int(sample.max())
+        counts.append(count)
+        for k in range(1, count + 1):
+            sizes.append(int((sample == k).sum()))
+    counts = np.asarray(counts, np.int64)
+    sizes = np.asarray(sizes, np.int64)
+    offsets = np.concatenate([[0], np.cumsum([len(i) for i in instance_idx])]).astype(np.int64)
+    idx = _c(np.concatenate([np.asarray(i, np.int64) for i in instance_idx]), np.int64)
+    first = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    total = int(counts.sum())
+    out = np.empty((len(instance_idx), total), np.float32)
+    lib().tpk_oracle_instance_iou(ctypes.c_int64(total), ctypes.c_int64(len(instance_idx)), _p(counts, _i64p),
+                                  _p(idx, _i64p), _p(offsets, _i64p), _p(gt, _i64p), _p(first, _i64p),
+                                  _p(batch, _i64p), _p(sizes, _i64p), _p(out, _f32p))
+    return out

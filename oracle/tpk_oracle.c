@@ -700,3 +700,46 @@ void tpk_oracle_ball_query_sorted_partial(int64_t size_x, int64_t size_y, float 
         }
     }
 }
+
+/* ------------------------------------------------------------------------- */
+/* IoU between proposed instances and ground-truth instances.                  */
+/* cuda/src/metrics_gpu.cu:9-43 (kernel), cuda/src/metrics.cpp:37-39 (output   */
+/* pre-zeroed).  proposals_idx: the proposals' point indices one after the     */
+/* other, proposals_offset (n_proposals + 1) their boundaries; labels (per     */
+/* point; ground-truth instance k of a sample carries label k + 1, 0 and       */
+/* negative values mean "none"); batch (per point) the sample of a point;      */
+/* n_instances / instance_offset (per sample) count and first column of the    */
+/* sample's instances; instance_pointnum (per column) their sizes.  A          */
+/* proposal is compared with the instances of the sample of its first point.   */
+/* The quotient is formed as the kernel's expression types dictate: float      */
+/* operands, the 1e-5 a double, the result stored as float.                    */
+/* iou (n_proposals, total_instances).                                         */
+/* ------------------------------------------------------------------------- */
+void tpk_oracle_instance_iou(int64_t total_instances, int64_t n_proposals, const int64_t* n_instances,
+                             const int64_t* proposals_idx, const int64_t* proposals_offset,
+                             const int64_t* labels, const int64_t* instance_offset, const int64_t* batch,
+                             const int64_t* instance_pointnum, float* iou)
+{
+    for (int64_t t = 0; t < n_proposals * total_instances; ++t)
+        iou[t] = 0.0f;
+    for (int64_t p = 0; p < n_proposals; ++p)
+    {
+        const int start = (int)proposals_offset[p], end = (int)proposals_offset[p + 1];
+        if (end <= start)
+            continue; /* the kernel would read past the proposal; every quotient is 0 anyway */
+        const int sample = (int)batch[proposals_idx[start]];
+        const int count = (int)n_instances[sample];
+        const int first = (int)instance_offset[sample];
+        const int proposal_total = end - start;
+        for (int k = 0; k < count; ++k)
+        {
+            const int instance_total = (int)instance_pointnum[first + k];
+            int intersection = 0;
+            for (int i = start; i < end; ++i)
+                if ((int)labels[proposals_idx[i]] == k + 1)
+                    ++intersection;
+            iou[first + k + p * total_instances] =
+                (float)((float)intersection / ((float)(proposal_total + instance_total - intersection) + 1e-5));
+        }
+    }
+}

@@ -806,6 +806,50 @@ def test_grow_proximity_any_matrix(tpk, oracle, dev):
                 assert got == (want if reference_order else [sorted(c) for c in want])
 
 
+# ------------------------------------------------------------------ instance IoU
+
+
+def test_kat_instance_iou(tpk, dev):
+    # reference test/test_metrics.py:16-55
+    from torch_points_kernels.metrics import instance_iou
+
+    gt = torch.tensor([1, 2, 1, 2, 2, 3, 0]).to(dev)
+    ious = instance_iou([torch.tensor([0, 2]).to(dev), torch.tensor([1, 4]).to(dev), torch.tensor([3, 5]).to(dev)], gt)
+    torch.testing.assert_close(ious.cpu(), torch.tensor([[1, 0, 0], [0, 2 / 3.0, 0], [0, 1.0 / 4.0, 1.0 / 2.0]]), rtol=1e-4, atol=1e-5)
+    batch = torch.tensor([0, 0, 1, 1, 1, 1, 1]).to(dev)
+    ious = instance_iou([torch.tensor([0, 1]).to(dev), torch.tensor([3, 4]).to(dev), torch.tensor([5]).to(dev)], gt, batch=batch)
+    want = torch.tensor([[0.5, 0.5, 0, 0, 0], [0, 0, 0, 1, 0], [0, 0, 0, 0, 1.0]])
+    torch.testing.assert_close(ious.cpu(), want, rtol=1e-4, atol=1e-5)
+    with pytest.raises(NotImplementedError):
+        instance_iou([torch.tensor([0, 2])], gt.cpu())
+
+
+@pytest.mark.parametrize("samples,points,instances,proposals,longest", [(1, 1000, 9, 20, 50), (3, 5000, 40, 300, 700),
+                                                                         (2, 30000, 300, 64, 9000), (1, 20000, 9000, 5, 4000)])
+def test_instance_iou_parity(tpk, oracle, dev, samples, points, instances, proposals, longest):
+    # the last case has more instances in a sample than the kernel counts in LDS
+    from torch_points_kernels.metrics import instance_iou
+
+    g = torch.Generator().manual_seed(points + proposals)
+    batch = torch.sort(torch.randint(0, samples, (points,), generator=g))[0]
+    batch[0], batch[-1] = 0, samples - 1
+    gt = torch.randint(0, instances + 1, (points,), generator=g)
+    gt[torch.rand(points, generator=g) < 0.1] = -100  # the ignore label of the segmentation data sets
+    for s in range(samples):
+        gt[(batch == s).nonzero()[0]] = instances  # every sample has its last instance
+    props = []
+    for p in range(proposals):
+        size = int(torch.randint(1, longest + 1, (1,), generator=g))
+        sample = int(torch.randint(0, samples, (1,), generator=g))
+        members = (batch == sample).nonzero().flatten()
+        props.append(members[torch.randint(0, members.numel(), (size,), generator=g)])  # repeats allowed
+    got = instance_iou([p.to(dev) for p in props], gt.to(dev), batch.to(dev))
+    want = oracle.instance_iou([p.numpy() for p in props], gt.numpy(), batch.numpy())
+    assert got.dtype == torch.float32 and got.shape == want.shape
+    np.testing.assert_array_equal(_np(got), want)  # integer counts and one correctly rounded quotient: bit-exact
+    assert (want > 0).any()
+
+
 # ------------------------------------------------------------------ chamfer
 
 

@@ -570,3 +570,37 @@ def test_ball_query_sorted_against_reference_cpu_module(oracle, ref_cpu):
         oi, od = oracle.ball_query_sorted_partial(r, ns, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
         np.testing.assert_array_equal(oi, ri.numpy())
         np.testing.assert_array_equal(od, rd.numpy())
+
+
+# ------------------------------------------------------------------ instance IoU
+
+
+def test_instance_iou_reference_vectors(oracle):
+    # reference test/test_metrics.py:16-55 (its own tolerance: assert_allclose defaults)
+    gt = np.array([1, 2, 1, 2, 2, 3, 0])
+    ious = oracle.instance_iou([[0, 2], [1, 4], [3, 5]], gt)
+    np.testing.assert_allclose(ious, [[1, 0, 0], [0, 2 / 3.0, 0], [0, 1.0 / 4.0, 1.0 / 2.0]], rtol=1e-4, atol=1e-5)
+    ious = oracle.instance_iou([[0, 1], [3, 4], [5]], gt, np.array([0, 0, 1, 1, 1, 1, 1]))
+    np.testing.assert_allclose(ious, [[0.5, 0.5, 0, 0, 0], [0, 0, 0, 1, 0], [0, 0, 0, 0, 1]], rtol=1e-4, atol=1e-5)
+
+
+def test_instance_iou_is_intersection_over_union_of_sets(oracle):
+    rng = np.random.default_rng(9)
+    n = 400
+    batch = np.sort(rng.integers(0, 3, n))
+    batch[0], batch[-1] = 0, 2
+    gt = rng.integers(0, 7, n)
+    for s in range(3):
+        gt[np.nonzero(batch == s)[0][0]] = 6
+    props = [rng.choice(np.nonzero(batch == s)[0], size=rng.integers(1, 60), replace=False) for s in (0, 1, 2, 1, 0)]
+    ious = oracle.instance_iou(props, gt, batch)
+    assert ious.shape == (5, 18)
+    for p, prop in enumerate(props):
+        s = batch[prop[0]]
+        for k in range(6):
+            inst = set(np.nonzero((batch == s) & (gt == k + 1))[0].tolist())
+            want = len(inst & set(prop.tolist())) / (len(inst | set(prop.tolist())) + 1e-5)
+            assert abs(ious[p, s * 6 + k] - want) < 1e-6
+        other = np.ones(18, bool)
+        other[s * 6 : s * 6 + 6] = False
+        assert (ious[p, other] == 0).all()

@@ -368,6 +368,40 @@ std::pair<at::Tensor, at::Tensor> ball_query_partial_dense(at::Tensor x, at::Ten
     return std::make_pair(idx, dist);
 }
 
+// cuda/src/metrics.cpp:12-52
+at::Tensor instance_iou_cuda(at::Tensor instance_idx, at::Tensor instance_offsets, at::Tensor gt_instances,
+                             at::Tensor gt_instance_sizes, at::Tensor num_gt_instances, at::Tensor batch)
+{
+    const at::Tensor* all[] = {&instance_idx, &instance_offsets, &gt_instances, &gt_instance_sizes, &num_gt_instances, &batch};
+    const char* names[] = {"instance_idx", "instance_offsets", "gt_instances", "gt_instance_sizes", "num_gt_instances", "batch"};
+    for (int i = 0; i < 6; ++i)
+    {
+        check_contiguous(*all[i], names[i]);
+        check_gpu(*all[i], names[i]);
+        check_dtype(*all[i], at::kLong, names[i]);
+        check_same_device(*all[i], gt_instances, names[i]);
+        TORCH_CHECK(all[i]->dim() == 1, names[i], " must have one dimension");
+    }
+    TORCH_CHECK(instance_offsets.size(0) >= 1, "instance_offsets must hold at least one entry");
+    TORCH_CHECK(batch.size(0) == gt_instances.size(0), "batch and gt_instances differ in length");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(gt_instances.device());
+    const int64_t num_proposed_instances = instance_offsets.size(0) - 1;
+    // as the reference: the total is read back to size the output
+    const int64_t total_gt_instances = num_gt_instances.numel() ? num_gt_instances.sum().item<int64_t>() : 0;
+    TORCH_CHECK(gt_instance_sizes.size(0) == total_gt_instances, "gt_instance_sizes must hold one entry per ground-truth instance");
+    at::Tensor output = torch::empty({num_proposed_instances, total_gt_instances},
+                                     at::device(gt_instances.device()).dtype(at::ScalarType::Float));
+    at::Tensor offset_num_gt_instances = at::cat({at::zeros(1, num_gt_instances.options()), num_gt_instances.cumsum(0)}, 0);
+    check_status(tpk_instance_iou(total_gt_instances, num_proposed_instances, gt_instances.size(0), num_gt_instances.size(0),
+                                  num_gt_instances.data_ptr<int64_t>(), instance_idx.data_ptr<int64_t>(),
+                                  instance_offsets.data_ptr<int64_t>(), gt_instances.data_ptr<int64_t>(),
+                                  offset_num_gt_instances.data_ptr<int64_t>(), batch.data_ptr<int64_t>(),
+                                  gt_instance_sizes.data_ptr<int64_t>(), output.data_ptr<float>(),
+                                  current_stream(gt_instances)),
+                 "instance_iou_cuda");
+    return output;
+}
+
 // No counterpart in the reference's native module: its grouping_operation is
 // torch.gather on a repeated index (torch_points_kernels/torchpoints.py:129-146).
 at::Tensor grouping_operation(at::Tensor features, at::Tensor idx)
@@ -543,6 +577,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("three_nn", &three_nn);
     m.def("dense_knn", &dense_knn);
     m.def("grow_proximity", &grow_proximity);
+    m.def("instance_iou_cuda", &instance_iou_cuda);
     m.def("three_interpolate", &three_interpolate);
     m.def("three_interpolate_grad", &three_interpolate_grad);
     m.def("ball_query_dense", &ball_query_dense, pybind11::arg("new_xyz"), pybind11::arg("xyz"), pybind11::arg("radius"),

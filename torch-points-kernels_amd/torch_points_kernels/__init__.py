@@ -1,6 +1,6 @@
 """torch_points_kernels for AMD MI355X: the spatial-search operators of
 torch-points3d/torch-points-kernels (furthest point sampling, ball query, three_nn /
-three_interpolate, grouping, Chamfer distance, dense knn, region growing) on hand-written HIP kernels.
+three_interpolate, grouping, Chamfer distance, dense knn, region growing, instance IoU) on hand-written HIP kernels.
 
 Same names and call signatures as the reference package (torch_points_kernels/__init__.py);
 GPU tensors only.
@@ -18,6 +18,7 @@ from .torchpoints import (
 )
 from .knn import knn
 from .cluster import grow_proximity, region_grow
+from .metrics import instance_iou
 from .chamfer_dist import ChamferFunction
 from . import chamfer_dist  # the reference exports the submodule under this name
 
@@ -29,6 +30,7 @@ __all__ = [
     "three_nn",
     "knn",
     "region_grow",
+    "instance_iou",
     "chamfer_dist",
     "ChamferFunction",
 ]

@@ -1,0 +1,67 @@
+"""IoU between proposed and ground-truth instances (reference: torch_points_kernels/metrics.py)."""
+from typing import List, Optional
+
+import torch
+
+from ._native import native, require_gpu
+
+
+def instance_iou(
+    instance_idx: List[torch.Tensor],
+    gt_instances: torch.Tensor,
+    batch: Optional[torch.Tensor] = None,
+):
+    """Computes the IoU between each proposed instance in instance_idx and ground truth instances. Returns a
+    tensor of shape [instance_idx.shape[0], num_instances] that contains the iou between the proposed instances and all gt instances
+    Instance label 0 is reserved for non instance points
+
+    Parameters
+    ----------
+    instance_idx : List[torch.Tensor]
+        List of instances. Each tensor in this list is a proposed and contains the index of the points
+        that belong to that particular instance
+    gt_instances : torch.Tensor
+        Ground truth instances, contains the index of the instance for each point
+
+    Returns
+    -------
+    ious: torch.Tensor[nb_proposals, nb_groundtruth]
+
+    Reference: metrics.py:37-104; GPU tensors only here.
+    """
+    require_gpu(gt_instances, "instance_iou")
+    if batch is None:
+        batch = torch.zeros_like(gt_instances)
+
+    # Number of ground-truth instances per sample and their sizes (one bincount per sample in place of the
+    # reference's loop over instance ids)
+    gt_instance_sizes = []
+    num_gt_instances = []
+    batch_size = int(batch[-1]) + 1
+    for s in range(batch_size):
+        sample_gt_instances = gt_instances[batch == s]
+        sample_num_gt_instances = int(torch.max(sample_gt_instances).item())
+        num_gt_instances.append(sample_num_gt_instances)
+        if sample_num_gt_instances > 0:
+            counts = torch.bincount(sample_gt_instances[sample_gt_instances > 0], minlength=sample_num_gt_instances + 1)
+            gt_instance_sizes.append(counts[1 : sample_num_gt_instances + 1])
+    device = gt_instances.device
+    gt_instance_sizes = torch.cat(gt_instance_sizes) if gt_instance_sizes else torch.zeros(0, dtype=torch.long, device=device)
+    num_gt_instances = torch.tensor(num_gt_instances, dtype=torch.long, device=device)
+
+    # Instance offset when flatten
+    instance_offsets = [0]
+    cum_offset = 0
+    for instance in instance_idx:
+        cum_offset += instance.shape[0]
+        instance_offsets.append(cum_offset)
+
+    instance_idx = torch.cat(instance_idx) if len(instance_idx) else torch.zeros(0, dtype=torch.long, device=device)
+    return native().instance_iou_cuda(
+        instance_idx.to(device).long().contiguous(),
+        torch.tensor(instance_offsets, dtype=torch.long, device=device),
+        gt_instances.long().contiguous(),
+        gt_instance_sizes.long().contiguous(),
+        num_gt_instances,
+        batch.long().contiguous(),
+    )
