@@ -274,6 +274,30 @@ def bench_others(dev, steps, warmup, with_cpu):
                                        "reference also copies the matrix (38 MB) to the host first, not timed here"}
     out["grow_proximity"] = e
 
+    # beyond the BASELINE configurations: instance IoU of 500 proposals of 2000 points against 4 x 50 ground-truth
+    # instances (the native call only: the Python front end's per-sample statistics are prepared once)
+    ip = W.instance_proposals()
+    prop_idx = torch.cat(ip["proposals"]).to(dev)
+    prop_off = torch.tensor([0] + [int(p.numel()) for p in ip["proposals"]]).cumsum(0).to(dev)
+    gt_dev, batch_dev = ip["gt"].to(dev), ip["batch"].to(dev)
+    counts = torch.tensor([int(ip["gt"][ip["batch"] == s_].max()) for s_ in range(4)], device=dev)
+    sizes = torch.cat([torch.bincount(ip["gt"][ip["batch"] == s_], minlength=51)[1:51] for s_ in range(4)]).to(dev)
+    wall, ev = _time_gpu(lambda: nat.instance_iou_cuda(prop_idx, prop_off, gt_dev, sizes, counts, batch_dev), steps, warmup)
+    nbytes = prop_idx.numel() * 16 + 500 * 200 * 4  # an index and a label per proposal point, the output once
+    e = {"workload": "instance_iou: 500 proposals x 2000 points, 4 samples x 50 ground-truth instances, 300000 points "
+                     "(not a BASELINE configuration)", "metric": "proposals/s", "value": 500 / (wall * 1e-3),
+         "kernel_ms": ev, "wall_ms": wall, "roofline": _roof_bytes(nbytes, ev, "instance_iou"), "algorithmic_bytes": nbytes}
+    e["roofline"]["note"] = "kernel_ms includes the column sums PyTorch forms to size the output (two small kernels and a read-back)"
+    if with_cpu:
+        import oracle
+
+        props_np = [p.numpy() for p in ip["proposals"]]
+        secs = _cpu_time(lambda: oracle.instance_iou(props_np, ip["gt"].numpy(), ip["batch"].numpy()))
+        e["cpu_baseline"] = {"value": 500 / secs, "unit": "proposals/s", "cores": 1, "kind": "port",
+                             "sample": "the whole workload; C restatement of the reference's CUDA kernel loops (the reference's "
+                                       "CPU path is a numba routine of the same shape)"}
+    out["instance_iou"] = e
+
     dist, idx = tpk.three_nn(unknown, known)
     weight = W.inverse_distance_weights(dist).contiguous()
     feats = w["features"].to(dev)

@@ -162,3 +162,19 @@ def region_cluster(num_points=100000):
     pos = torch.cat([torch.rand(num_points, 3, generator=g) + 2.0 * i for i in range(3)]).contiguous()
     batch = torch.ones(3 * num_points, dtype=torch.long)
     return {"pos": pos, "batch": batch, "radius": 0.02, "nsample": 16, "min_cluster_size": 32}
+
+
+def instance_proposals(samples=4, points_per_sample=75000, instances=50, proposals=500, proposal_points=2000):
+    """A PointGroup-like scoring step: proposals (index tensors) against the ground-truth instances of their sample."""
+    import torch
+
+    g = torch.Generator().manual_seed(7)
+    n = samples * points_per_sample
+    batch = torch.arange(samples).repeat_interleave(points_per_sample)
+    gt = torch.randint(0, instances + 1, (n,), generator=g)
+    gt[::points_per_sample] = instances
+    props = []
+    for p in range(proposals):
+        s = p % samples
+        props.append(torch.randint(s * points_per_sample, (s + 1) * points_per_sample, (proposal_points,), generator=g))
+    return {"gt": gt, "batch": batch, "proposals": props}
