@@ -79,8 +79,11 @@ __device__ __forceinline__ int entries_before_end(int64_t nei, int shift, bool* 
 }
 
 // Bit j of a point's mask: entry j of its row is a point whose own row lists this point back.
+// The smallest such point below u becomes u's first parent (a plain store: only u's lanes
+// write parent[u] in this kernel), which leaves far fewer trees for the merge sweeps to hang.
 __global__ void __launch_bounds__(CL_THREADS)
-    cluster_mutual_kernel(int n, int nsample, int words, const int64_t* __restrict__ neighbours, unsigned* mutual)
+    cluster_mutual_kernel(int n, int nsample, int words, const int64_t* __restrict__ neighbours, unsigned* mutual,
+                          int* parent)
 {
     const int64_t t = (int64_t)blockIdx.x * CL_THREADS + threadIdx.x;
     const int64_t point = t / CL_ROW_LANES;
@@ -89,6 +92,7 @@ __global__ void __launch_bounds__(CL_THREADS)
         return; // the whole group of lanes leaves together
     const int u = (int)point;
     const int shift = (int)(tpk_lane_id() & (TPK_WAVE - CL_ROW_LANES)); // first lane of this row's group
+    int lowest = u;
     for (int first = 0; first < nsample; first += CL_ROW_LANES)
     {
         const int j = first + g;
@@ -114,9 +118,16 @@ __global__ void __launch_bounds__(CL_THREADS)
         const unsigned bits = (unsigned)(__ballot(back) >> shift) & 0xffffu;
         if (g == 0 && bits)
             atomicOr(&mutual[(int64_t)u * words + (first >> 5)], bits << (first & 31));
+        if (back && (int)nei < lowest)
+            lowest = (int)nei;
         if (row_ends)
             break;
     }
+    // minimum over the group's lanes (the lanes of a group are together again here)
+    for (int step = 1; step < CL_ROW_LANES; step <<= 1)
+        lowest = min(lowest, __shfl_xor(lowest, step, CL_ROW_LANES));
+    if (g == 0 && lowest < u)
+        parent[u] = lowest;
 }
 
 __device__ __forceinline__ int find_root(const int* parent, int v)
@@ -154,14 +165,42 @@ __global__ void __launch_bounds__(CL_THREADS)
         const int theirs = find_root(parent, nei);
         if (theirs != mine)
         {
+            // Many entries join the same two trees; only while the higher root still is a root
+            // is it worth an atomic on that one address.  Otherwise another entry has hung it
+            // meanwhile and this pair is looked at again in the next sweep.
             const int low = min(mine, theirs), high = max(mine, theirs);
-            hung |= atomicMin(&parent[high], low) > low;
+            if (__hip_atomic_load(&parent[high], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == high)
+                hung |= atomicMin(&parent[high], low) > low;
+            else
+                hung = true;
         }
     }
     if (g == 0 && mine < parent[u])
         atomicMin(&parent[u], mine);
     if (hung)
         changed[sweep] = 1;
+}
+
+// Shortens the trees before a merge sweep: every point moves its parent a few steps up (only
+// the point's own thread writes its entry in this kernel).
+__global__ void __launch_bounds__(CL_THREADS) cluster_jump_kernel(int n, int* parent, const int* changed, int sweep)
+{
+    if (sweep > 0 && changed[sweep - 1] == 0)
+        return;
+    const int v = blockIdx.x * CL_THREADS + threadIdx.x;
+    if (v >= n)
+        return;
+    const int first = parent[v];
+    int p = first;
+    for (int step = 0; step < CL_FOLLOW; ++step)
+    {
+        const int up = parent[p];
+        if (up >= p)
+            break;
+        p = up;
+    }
+    if (p < first)
+        parent[v] = p;
 }
 
 // parent[v] becomes the smallest point of v's merged group.
@@ -528,8 +567,9 @@ extern "C" int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbo
                     return e;
             }
         };
-        cluster_mutual_kernel<<<sweep_blocks, CL_THREADS, 0, s>>>(ni, nsample, words, neighbours, mutual);
+        cluster_mutual_kernel<<<sweep_blocks, CL_THREADS, 0, s>>>(ni, nsample, words, neighbours, mutual, parent);
         hipError_t e = until_stable([&](int sweep) {
+            cluster_jump_kernel<<<blocks, CL_THREADS, 0, s>>>(ni, parent, changed, sweep);
             cluster_merge_kernel<<<sweep_blocks, CL_THREADS, 0, s>>>(ni, nsample, words, neighbours, mutual, parent, changed, sweep);
         });
         if (e != hipSuccess)
