@@ -278,6 +278,60 @@ int tpk_instance_iou(int64_t total_gt_instances, int64_t n_proposals, int64_t n_
                      const int64_t* offset_num_gt_instances, const int64_t* batch,
                      const int64_t* instance_pointnum, float* proposals_iou, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Gridding (GRNet): point clouds to occupancy grids by trilinear weights, and the gradient.
+ * Replaces gridding_kernel_warpper(min_x, max_x, min_y, max_y, min_z, max_z, ptcloud, stream)
+ * and gridding_grad_kernel_warpper(grid_pt_weights, grid_pt_indexes, grad_grid, stream)
+ * (cuda/src/gridding_gpu.cu:193-218, :307-331; host functions cuda/src/gridding.cpp:4-26).
+ *   ptcloud (b, n_pts, 3) in grid units; the grid spans [min, max] per axis, len = max-min+1
+ *   grid_weights (b, len_x*len_y*len_z): sum over points of wx*wy*wz at the 8 vertices around
+ *   a point, w = 1 - |coordinate - vertex|; grid_pt_weights (b, n_pts, 8, 3) the three factors,
+ *   grid_pt_indexes (b, n_pts, 8) int32 the vertices (order LLL, LLU, LUL, LUU, ULL, ULU, UUL,
+ *   UUU; -1 for a vertex outside the grid, where the reference computes an index regardless).
+ *   grad_grid (b, n_grid_vertices) -> grad_ptcloud (b, n_pts, 3).
+ * float32 and float64 (the reference dispatches on both).  Sums into the grid are atomic, in
+ * no fixed order; the gradient is summed in the reference's order.
+ * ------------------------------------------------------------------------------------- */
+int tpk_gridding_f32(int b, int n_pts, float min_x, float max_x, float min_y, float max_y, float min_z,
+                     float max_z, const float* ptcloud, float* grid_weights, float* grid_pt_weights,
+                     int32_t* grid_pt_indexes, void* stream);
+int tpk_gridding_f64(int b, int n_pts, float min_x, float max_x, float min_y, float max_y, float min_z,
+                     float max_z, const double* ptcloud, double* grid_weights, double* grid_pt_weights,
+                     int32_t* grid_pt_indexes, void* stream);
+int tpk_gridding_grad_f32(int b, int n_pts, int n_grid_vertices, const float* grid_pt_weights,
+                          const int32_t* grid_pt_indexes, const float* grad_grid, float* grad_ptcloud,
+                          void* stream);
+int tpk_gridding_grad_f64(int b, int n_pts, int n_grid_vertices, const double* grid_pt_weights,
+                          const int32_t* grid_pt_indexes, const double* grad_grid, double* grad_ptcloud,
+                          void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Cubic feature sampling (GRNet): the features of the grid vertices around every point.
+ * Replaces cubic_feature_sampling_kernel_wrapper(scale, neighborhood_size, ptcloud,
+ * cubic_features, stream) and cubic_feature_sampling_grad_kernel_wrapper(scale,
+ * neighborhood_size, grad_point_features, grid_pt_indexes, stream)
+ * (cuda/src/cubic_feature_sampling_gpu.cu:107-136, :177-210; host functions
+ * cuda/src/cubic_feature_sampling.cpp:4-30).
+ *   ptcloud (b, n_pts, 3) in grid units   cubic_features (b, channels, scale, scale, scale)
+ *   point_features (b, n_pts, n_vertices, channels), n_vertices = (2*neighborhood_size)^3:
+ *   the features at the vertices floor-(ns-1) .. ceil+(ns-1) per axis, x slowest; 0 where the
+ *   vertex lies outside the grid; grid_pt_indexes (b, n_pts, n_vertices) int32, -1 outside.
+ *   Gradient: grad_cubic_features (b, channels, scale^3) = scatter-add of grad_point_features;
+ *   grad_ptcloud (b, n_pts, 3) = 0 (the coordinates only choose vertices).
+ * ------------------------------------------------------------------------------------- */
+int tpk_cubic_feature_sampling_f32(int b, int n_pts, int channels, int scale, int neighborhood_size,
+                                   const float* ptcloud, const float* cubic_features, float* point_features,
+                                   int32_t* grid_pt_indexes, void* stream);
+int tpk_cubic_feature_sampling_f64(int b, int n_pts, int channels, int scale, int neighborhood_size,
+                                   const double* ptcloud, const double* cubic_features, double* point_features,
+                                   int32_t* grid_pt_indexes, void* stream);
+int tpk_cubic_feature_sampling_grad_f32(int b, int n_pts, int channels, int scale, int neighborhood_size,
+                                        const float* grad_point_features, const int32_t* grid_pt_indexes,
+                                        float* grad_ptcloud, float* grad_cubic_features, void* stream);
+int tpk_cubic_feature_sampling_grad_f64(int b, int n_pts, int channels, int scale, int neighborhood_size,
+                                        const double* grad_point_features, const int32_t* grid_pt_indexes,
+                                        double* grad_ptcloud, double* grad_cubic_features, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

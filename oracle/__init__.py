@@ -340,3 +340,70 @@ def instance_iou(instance_idx, gt_instances, batch=None):
                                   _p(idx, _i64p), _p(offsets, _i64p), _p(gt, _i64p), _p(first, _i64p),
                                   _p(batch, _i64p), _p(sizes, _i64p), _p(out, _f32p))
     return out
+
+
+def _grid_types(a):
+    a = np.asarray(a)
+    if a.dtype == np.float64:
+        return np.float64, ctypes.POINTER(ctypes.c_double), "f64"
+    return np.float32, _f32p, "f32"
+
+
+def gridding(ptcloud, scale):
+    """GriddingFunction.forward (torch_points_kernels/gridding.py:9-22): ptcloud (B,n,3) in grid units ->
+    (grid (B,(2*scale)^3), grid_pt_weights (B,n,8,3), grid_pt_indexes (B,n,8) int32)."""
+    dt, ptr, suf = _grid_types(ptcloud)
+    p = _c(ptcloud, dt)
+    b, n, _ = p.shape
+    side = 2 * scale
+    grid = np.empty((b, side ** 3), dt)
+    weights = np.empty((b, n, 8, 3), dt)
+    indexes = np.empty((b, n, 8), np.int32)
+    f = ctypes.c_float
+    getattr(lib(), "tpk_oracle_gridding_" + suf)(ctypes.c_int(b), ctypes.c_int(n), f(-scale), f(scale - 1), f(-scale),
+                                                  f(scale - 1), f(-scale), f(scale - 1), _p(p, ptr), _p(grid, ptr),
+                                                  _p(weights, ptr), _p(indexes, _i32p))
+    return grid, weights, indexes
+
+
+def gridding_grad(grid_pt_weights, grid_pt_indexes, grad_grid):
+    dt, ptr, suf = _grid_types(grid_pt_weights)
+    w = _c(grid_pt_weights, dt)
+    ix = _c(grid_pt_indexes, np.int32)
+    g = _c(grad_grid, dt)
+    b, n = ix.shape[:2]
+    out = np.empty((b, n, 3), dt)
+    getattr(lib(), "tpk_oracle_gridding_grad_" + suf)(ctypes.c_int(b), ctypes.c_int(n), ctypes.c_int(g.shape[1]),
+                                                       _p(w, ptr), _p(ix, _i32p), _p(g, ptr), _p(out, ptr))
+    return out
+
+
+def cubic_feature_sampling(ptcloud, cubic_features, neighborhood_size=1):
+    """CubicFeatureSamplingFunction.forward (cubic_feature_sampling.py:9-19): ptcloud (B,n,3) in grid units,
+    cubic_features (B,c,m,m,m) -> (point_features (B,n,(2*ns)^3,c), grid_pt_indexes int32)."""
+    dt, ptr, suf = _grid_types(ptcloud)
+    p = _c(ptcloud, dt)
+    feats = _c(cubic_features, dt)
+    b, n, _ = p.shape
+    c, scale = feats.shape[1], feats.shape[2]
+    nv = (2 * neighborhood_size) ** 3
+    out = np.empty((b, n, nv, c), dt)
+    indexes = np.empty((b, n, nv), np.int32)
+    getattr(lib(), "tpk_oracle_cubic_feature_sampling_" + suf)(ctypes.c_int(b), ctypes.c_int(n), ctypes.c_int(c),
+                                                                ctypes.c_int(scale), ctypes.c_int(neighborhood_size),
+                                                                _p(p, ptr), _p(feats, ptr), _p(out, ptr), _p(indexes, _i32p))
+    return out, indexes
+
+
+def cubic_feature_sampling_grad(scale, neighborhood_size, grad_point_features, grid_pt_indexes):
+    dt, ptr, suf = _grid_types(grad_point_features)
+    g = _c(grad_point_features, dt)
+    ix = _c(grid_pt_indexes, np.int32)
+    b, n, nv, c = g.shape
+    grad_pt = np.empty((b, n, 3), dt)
+    grad_feats = np.empty((b, c, scale, scale, scale), dt)
+    getattr(lib(), "tpk_oracle_cubic_feature_sampling_grad_" + suf)(ctypes.c_int(b), ctypes.c_int(n), ctypes.c_int(c),
+                                                                     ctypes.c_int(scale), ctypes.c_int(neighborhood_size),
+                                                                     _p(g, ptr), _p(ix, _i32p), _p(grad_pt, ptr),
+                                                                     _p(grad_feats, ptr))
+    return grad_pt, grad_feats

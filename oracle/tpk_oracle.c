@@ -743,3 +743,140 @@ void tpk_oracle_instance_iou(int64_t total_instances, int64_t n_proposals, const
         }
     }
 }
+
+/* ------------------------------------------------------------------------- */
+/* Gridding and cubic feature sampling (GRNet).  cuda/src/gridding_gpu.cu:    */
+/* 29-191 (forward), :205-305 (gradient); cuda/src/cubic_feature_sampling_    */
+/* gpu.cu:23-105 (forward), :138-175 (gradient).  Both exist for float and     */
+/* double (AT_DISPATCH_FLOATING_TYPES).  Sums are formed in point order here;  */
+/* the kernels add atomically in no fixed order.  Vertices outside the grid    */
+/* (where the reference forms an index regardless and writes out of bounds or  */
+/* into a neighbouring row) get index -1 and take no part.                     */
+/* ------------------------------------------------------------------------- */
+#define TPK_GRID_OPS(T, SUFFIX, FLOOR, CEIL, FABS)                                                          \
+    static void planes_##SUFFIX(T v, int* lower, int* upper)                                                \
+    {                                                                                                       \
+        *lower = (int)FLOOR(v);                                                                             \
+        *upper = (int)CEIL(v);                                                                              \
+        if (*lower == *upper)                                                                               \
+            *upper += 1;                                                                                    \
+    }                                                                                                       \
+    void tpk_oracle_gridding_##SUFFIX(int b, int n_pts, float min_x, float max_x, float min_y, float max_y, \
+                                      float min_z, float max_z, const T* ptcloud, T* grid_weights,          \
+                                      T* grid_pt_weights, int32_t* grid_pt_indexes)                         \
+    {                                                                                                       \
+        const int len_x = (int)(max_x - min_x + 1), len_y = (int)(max_y - min_y + 1);                       \
+        const int len_z = (int)(max_z - min_z + 1);                                                         \
+        const int64_t vertices = (int64_t)len_x * len_y * len_z;                                            \
+        for (int64_t t = 0; t < b * vertices; ++t)                                                          \
+            grid_weights[t] = 0;                                                                            \
+        for (int64_t j = 0; j < (int64_t)b * n_pts; ++j)                                                    \
+        {                                                                                                   \
+            T* grid = grid_weights + (j / n_pts) * vertices;                                                \
+            const T p[3] = {ptcloud[j * 3 + 0], ptcloud[j * 3 + 1], ptcloud[j * 3 + 2]};                    \
+            const float lo[3] = {min_x, min_y, min_z};                                                      \
+            const int len[3] = {len_x, len_y, len_z};                                                       \
+            int plane[3][2], off[3][2];                                                                     \
+            T w[3][2];                                                                                      \
+            for (int a = 0; a < 3; ++a)                                                                     \
+            {                                                                                               \
+                planes_##SUFFIX(p[a], &plane[a][0], &plane[a][1]);                                          \
+                for (int s = 0; s < 2; ++s)                                                                 \
+                {                                                                                           \
+                    off[a][s] = (int)(plane[a][s] - lo[a]);                                                 \
+                    w[a][s] = 1 - FABS(p[a] - (T)plane[a][s]);                                              \
+                }                                                                                           \
+            }                                                                                               \
+            for (int v = 0; v < 8; ++v)                                                                     \
+            {                                                                                               \
+                const int s[3] = {v >> 2, (v >> 1) & 1, v & 1};                                             \
+                int inside = 1;                                                                             \
+                for (int a = 0; a < 3; ++a)                                                                 \
+                    inside = inside && off[a][s[a]] >= 0 && off[a][s[a]] < len[a];                          \
+                const int index = inside ? off[0][s[0]] * len_y * len_z + off[1][s[1]] * len_z + off[2][s[2]] : -1; \
+                grid_pt_indexes[j * 8 + v] = index;                                                         \
+                for (int a = 0; a < 3; ++a)                                                                 \
+                    grid_pt_weights[j * 24 + v * 3 + a] = w[a][s[a]];                                       \
+                if (inside)                                                                                 \
+                    grid[index] += w[0][s[0]] * w[1][s[1]] * w[2][s[2]];                                    \
+            }                                                                                               \
+        }                                                                                                   \
+    }                                                                                                       \
+    void tpk_oracle_gridding_grad_##SUFFIX(int b, int n_pts, int n_grid_vertices, const T* grid_pt_weights, \
+                                           const int32_t* grid_pt_indexes, const T* grad_grid,             \
+                                           T* grad_ptcloud)                                                 \
+    {                                                                                                       \
+        for (int64_t j = 0; j < (int64_t)b * n_pts; ++j)                                                    \
+        {                                                                                                   \
+            const T* grad = grad_grid + (j / n_pts) * n_grid_vertices;                                      \
+            T gx = 0, gy = 0, gz = 0;                                                                       \
+            for (int v = 0; v < 8; ++v)                                                                     \
+            {                                                                                               \
+                const int index = grid_pt_indexes[j * 8 + v];                                               \
+                const T g = index >= 0 && index < n_grid_vertices ? grad[index] : 0;                        \
+                const T wx = grid_pt_weights[j * 24 + v * 3 + 0], wy = grid_pt_weights[j * 24 + v * 3 + 1]; \
+                const T wz = grid_pt_weights[j * 24 + v * 3 + 2];                                           \
+                /* upper side +, lower side - (gridding_gpu.cu:228-303) */                                  \
+                gx += ((v >> 2) ? g : -g) * wy * wz;                                                        \
+                gy += (((v >> 1) & 1) ? g : -g) * wx * wz;                                                  \
+                gz += ((v & 1) ? g : -g) * wx * wy;                                                         \
+            }                                                                                               \
+            grad_ptcloud[j * 3 + 0] = gx;                                                                   \
+            grad_ptcloud[j * 3 + 1] = gy;                                                                   \
+            grad_ptcloud[j * 3 + 2] = gz;                                                                   \
+        }                                                                                                   \
+    }                                                                                                       \
+    void tpk_oracle_cubic_feature_sampling_##SUFFIX(int b, int n_pts, int channels, int scale,              \
+                                                    int neighborhood_size, const T* ptcloud,                \
+                                                    const T* cubic_features, T* point_features,             \
+                                                    int32_t* grid_pt_indexes)                               \
+    {                                                                                                       \
+        const int side = 2 * neighborhood_size, nv = side * side * side, ns = neighborhood_size - 1;        \
+        const int64_t cub = (int64_t)scale * scale * scale;                                                 \
+        for (int64_t i = 0; i < (int64_t)b * n_pts; ++i)                                                    \
+        {                                                                                                   \
+            const T* feats = cubic_features + (i / n_pts) * channels * cub;                                 \
+            int lx, ux, ly, uy, lz, uz, at = 0;                                                             \
+            planes_##SUFFIX(ptcloud[i * 3 + 0], &lx, &ux);                                                  \
+            planes_##SUFFIX(ptcloud[i * 3 + 1], &ly, &uy);                                                  \
+            planes_##SUFFIX(ptcloud[i * 3 + 2], &lz, &uz);                                                  \
+            for (int j = lx - ns; j <= ux + ns; ++j)                                                        \
+                for (int k = ly - ns; k <= uy + ns; ++k)                                                    \
+                    for (int m = lz - ns; m <= uz + ns; ++m)                                                \
+                    {                                                                                       \
+                        const int out = j < 0 || j >= scale || k < 0 || k >= scale || m < 0 || m >= scale;  \
+                        grid_pt_indexes[i * nv + at++] = out ? -1 : j * scale * scale + k * scale + m;      \
+                    }                                                                                       \
+            for (int j = 0; j < nv; ++j)                                                                    \
+                for (int k = 0; k < channels; ++k)                                                          \
+                {                                                                                           \
+                    const int vertex = grid_pt_indexes[i * nv + j];                                         \
+                    point_features[(i * nv + j) * channels + k] = vertex == -1 ? 0 : feats[k * cub + vertex]; \
+                }                                                                                           \
+        }                                                                                                   \
+    }                                                                                                       \
+    void tpk_oracle_cubic_feature_sampling_grad_##SUFFIX(int b, int n_pts, int channels, int scale,         \
+                                                         int neighborhood_size, const T* grad_point_features, \
+                                                         const int32_t* grid_pt_indexes, T* grad_ptcloud,   \
+                                                         T* grad_cubic_features)                            \
+    {                                                                                                       \
+        const int side = 2 * neighborhood_size, nv = side * side * side;                                    \
+        const int64_t cub = (int64_t)scale * scale * scale;                                                 \
+        for (int64_t t = 0; t < (int64_t)b * n_pts * 3; ++t)                                                \
+            grad_ptcloud[t] = 0;                                                                            \
+        for (int64_t t = 0; t < b * channels * cub; ++t)                                                    \
+            grad_cubic_features[t] = 0;                                                                     \
+        for (int64_t i = 0; i < (int64_t)b * n_pts; ++i)                                                    \
+            for (int j = 0; j < nv; ++j)                                                                    \
+            {                                                                                               \
+                const int vertex = grid_pt_indexes[i * nv + j];                                             \
+                if (vertex == -1)                                                                           \
+                    continue;                                                                               \
+                for (int k = 0; k < channels; ++k)                                                          \
+                    grad_cubic_features[((i / n_pts) * channels + k) * cub + vertex] +=                     \
+                        grad_point_features[(i * nv + j) * channels + k];                                   \
+            }                                                                                               \
+    }
+
+TPK_GRID_OPS(float, f32, floorf, ceilf, fabsf)
+TPK_GRID_OPS(double, f64, floor, ceil, fabs)

@@ -850,6 +850,88 @@ def test_instance_iou_parity(tpk, oracle, dev, samples, points, instances, propo
     assert (want > 0).any()
 
 
+# ------------------------------------------------------------------ gridding, cubic feature sampling
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("B,n,scale", [(1, 32, 4), (2, 2048, 32), (3, 700, 8), (1, 1, 2)])
+def test_gridding_parity(tpk, oracle, dev, dtype, B, n, scale):
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    g = torch.Generator().manual_seed(n + scale)
+    p = ((torch.rand(B, n, 3, generator=g, dtype=torch.float64) * 2 - 1) * scale).to(dtype)  # the last cell's outer vertices fall outside
+    p[0, 0] = torch.tensor([1.0, -2.0, 0.0], dtype=dtype)  # integral coordinates
+    grid, weights, indexes = native.gridding(-scale, scale - 1, -scale, scale - 1, -scale, scale - 1, p.to(dev))
+    wg, ww, wi = oracle.gridding(p.numpy(), scale)
+    assert grid.dtype == dtype and indexes.dtype == torch.int32
+    np.testing.assert_array_equal(_np(indexes), wi)
+    np.testing.assert_array_equal(_np(weights), ww)
+    # the grid is a sum in no fixed order (atomics, as in the reference)
+    np.testing.assert_allclose(_np(grid), wg, rtol=1e-5 if dtype == torch.float32 else 1e-12, atol=1e-5 if dtype == torch.float32 else 1e-12)
+    r = torch.randn(B, (2 * scale) ** 3, generator=g, dtype=torch.float64).to(dtype)
+    grad = native.gridding_grad(weights, indexes, r.to(dev))
+    np.testing.assert_array_equal(_np(grad), oracle.gridding_grad(ww, wi, r.numpy()))  # one thread's sum in the reference's order
+
+
+def test_gridding_front_end_and_gradcheck(tpk, oracle, dev):
+    from torch_points_kernels.gridding import GriddingFunction, gridding
+
+    # reference test/test_gridding.py:19-29
+    for n, scale in ((32, 4), (64, 8)):
+        x = torch.rand(1, n, 3, dtype=torch.float64, device=dev, requires_grad=True)
+        assert torch.autograd.gradcheck(GriddingFunction.apply, [x, scale])
+    # the front end (gridding.py:34-60): scaled by `scale`, points whose coordinates sum to zero dropped per cloud
+    g = torch.Generator().manual_seed(3)
+    p = torch.rand(2, 100, 3, generator=g) * 1.8 - 0.9
+    p[1, 10:30] = 0
+    got = gridding(p.to(dev), 8)
+    assert got.shape == (2, 16 ** 3)
+    for b in range(2):
+        kept = (p[b] * 8)[(p[b] * 8).sum(1) != 0].unsqueeze(0)
+        np.testing.assert_allclose(_np(got[b : b + 1]), oracle.gridding(kept.numpy(), 8)[0], rtol=1e-5, atol=1e-5)
+    with pytest.raises(ValueError):
+        gridding(p[0].to(dev), 8)
+    with pytest.raises(NotImplementedError):
+        gridding(p, 8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("B,n,c,scale,ns", [(2, 64, 4, 8, 1), (2, 32, 2, 8, 2), (1, 32, 2, 16, 3), (2, 2048, 64, 16, 1), (1, 300, 7, 4, 2)])
+def test_cubic_feature_sampling_parity(tpk, oracle, dev, dtype, B, n, c, scale, ns):
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    g = torch.Generator().manual_seed(n + c + ns)
+    p = (torch.rand(B, n, 3, generator=g, dtype=torch.float64) * (scale + 2) - 1).to(dtype)  # some points outside the grid
+    p[0, 0] = torch.tensor([2.0, 3.0, 0.0], dtype=dtype)
+    feats = torch.rand(B, c, scale, scale, scale, generator=g, dtype=torch.float64).to(dtype)
+    out, indexes = native.cubic_feature_sampling(scale, ns, p.to(dev), feats.to(dev))
+    wo, wi = oracle.cubic_feature_sampling(p.numpy(), feats.numpy(), ns)
+    np.testing.assert_array_equal(_np(indexes), wi)
+    np.testing.assert_array_equal(_np(out), wo)
+    go = torch.randn(out.shape, generator=g, dtype=torch.float64).to(dtype)
+    grad_p, grad_f = native.cubic_feature_sampling_grad(scale, ns, go.to(dev), indexes)
+    wp, wf = oracle.cubic_feature_sampling_grad(scale, ns, go.numpy(), wi)
+    assert (_np(grad_p) == 0).all() and grad_f.shape == feats.shape
+    tol = 1e-4 if dtype == torch.float32 else 1e-11  # sums of up to n * n_vertices terms in no fixed order
+    np.testing.assert_allclose(_np(grad_f), wf, rtol=tol, atol=tol)
+
+
+def test_cubic_feature_sampling_front_end_and_gradcheck(tpk, oracle, dev):
+    from torch_points_kernels.cubic_feature_sampling import CubicFeatureSamplingFunction, cubic_feature_sampling
+
+    # reference test/test_cubic_feature_sampling.py:20-56
+    for B, n, c, scale, ns in ((2, 64, 4, 8, 1), (2, 32, 2, 8, 2), (1, 32, 2, 16, 3)):
+        p = (torch.rand(B, n, 3, dtype=torch.float64, device=dev) * 2 - 1).requires_grad_()
+        feats = torch.rand(B, c, scale, scale, scale, dtype=torch.float64, device=dev, requires_grad=True)
+        assert torch.autograd.gradcheck(CubicFeatureSamplingFunction.apply, [p, feats, ns])
+    # front end (cubic_feature_sampling.py:34-59): coordinates in [-1, 1) mapped to grid units
+    g = torch.Generator().manual_seed(4)
+    p = torch.rand(2, 50, 3, generator=g) * 2 - 1
+    feats = torch.rand(2, 3, 8, 8, 8, generator=g)
+    got = cubic_feature_sampling(p.to(dev), feats.to(dev), 2)
+    np.testing.assert_array_equal(_np(got), oracle.cubic_feature_sampling((p * 4.0 + 4.0).numpy(), feats.numpy(), 2)[0])
+    with pytest.raises(ValueError):
+        cubic_feature_sampling(p[0].to(dev), feats.to(dev))
+
+
 # ------------------------------------------------------------------ chamfer
 
 

@@ -604,3 +604,94 @@ def test_instance_iou_is_intersection_over_union_of_sets(oracle):
         other = np.ones(18, bool)
         other[s * 6 : s * 6 + 6] = False
         assert (ious[p, other] == 0).all()
+
+
+# ------------------------------------------------------------------ gridding, cubic feature sampling
+
+
+def _trilinear_grid(p, scale):
+    """Independent float64 statement of gridding: cell = floor, fractions t, vertex weights (1 - t) / t per axis."""
+    side = 2 * scale
+    grid = np.zeros((p.shape[0], side, side, side))
+    for b in range(p.shape[0]):
+        for x, y, z in p[b]:
+            cell = np.floor([x, y, z]).astype(int)
+            t = np.array([x, y, z]) - cell
+            for dx in (0, 1):
+                for dy in (0, 1):
+                    for dz in (0, 1):
+                        w = (t[0] if dx else 1 - t[0]) * (t[1] if dy else 1 - t[1]) * (t[2] if dz else 1 - t[2])
+                        i, j, k = cell + scale + (dx, dy, dz)
+                        if 0 <= i < side and 0 <= j < side and 0 <= k < side:
+                            grid[b, i, j, k] += w
+    return grid.reshape(p.shape[0], -1)
+
+
+def test_gridding_matches_trilinear_closed_form(oracle):
+    rng = np.random.default_rng(1)
+    scale = 4
+    p = (rng.random((2, 60, 3)) * 2 - 1) * scale  # some points fall into the last cell: their outer vertices are dropped
+    p[0, 0] = [1.0, -2.0, 0.0]  # on a vertex: all weight there
+    p[0, 1] = [-4.0, -4.0, -4.0]  # the grid's first vertex
+    for dtype, tol in ((np.float64, 1e-12), (np.float32, 1e-5)):
+        grid, weights, indexes = oracle.gridding(p.astype(dtype), scale)
+        np.testing.assert_allclose(grid, _trilinear_grid(p.astype(dtype).astype(np.float64), scale), rtol=tol, atol=tol)
+        assert grid.dtype == dtype and indexes.dtype == np.int32
+        # vertex order LLL .. UUU and the weights stored per axis
+        prod = weights.prod(axis=3)
+        inside = indexes >= 0
+        np.testing.assert_allclose(np.where(inside, prod, 0).sum(), grid.sum(), rtol=1e-5)
+        assert indexes[0, 0, 0] == (1 + 4) * 64 + (-2 + 4) * 8 + 4 and prod[0, 0, 0] == 1 and (prod[0, 0, 1:] == 0).all()
+        assert indexes[0, 1, 0] == 0
+    inner = (rng.random((1, 40, 3)) * 2 - 1) * (scale - 1)  # all 8 vertices inside: every point deposits exactly 1
+    np.testing.assert_allclose(oracle.gridding(inner, scale)[0].sum(), 40, rtol=1e-12)
+
+
+def test_gridding_grad_matches_finite_differences(oracle):
+    rng = np.random.default_rng(2)
+    scale = 3
+    p = (rng.random((2, 12, 3)) * 2 - 1) * (scale - 1)
+    r = rng.standard_normal((2, (2 * scale) ** 3))
+    grid, weights, indexes = oracle.gridding(p, scale)
+    grad = oracle.gridding_grad(weights, indexes, r)
+    eps = 1e-6
+    for b, j, a in ((0, 0, 0), (0, 5, 1), (1, 3, 2), (1, 11, 0), (0, 7, 2)):
+        hi, lo = p.copy(), p.copy()
+        hi[b, j, a] += eps
+        lo[b, j, a] -= eps
+        fd = ((oracle.gridding(hi, scale)[0] - oracle.gridding(lo, scale)[0]) * r).sum() / (2 * eps)
+        assert abs(fd - grad[b, j, a]) < 1e-6 * max(1.0, abs(fd))
+
+
+def test_cubic_feature_sampling_is_a_gather(oracle):
+    rng = np.random.default_rng(3)
+    for ns, scale in ((1, 8), (2, 8), (3, 6)):
+        p = rng.random((2, 30, 3)) * (scale + 2) - 1  # some points outside the grid
+        p[0, 0] = [2.0, 3.0, 0.0]
+        feats = rng.random((2, 5, scale, scale, scale))
+        out, indexes = oracle.cubic_feature_sampling(p, feats, ns)
+        nv = (2 * ns) ** 3
+        assert out.shape == (2, 30, nv, 5) and indexes.shape == (2, 30, nv)
+        for b in range(2):
+            for i in range(30):
+                lo = np.floor(p[b, i]).astype(int)
+                hi = np.where(np.ceil(p[b, i]) == lo, lo + 1, np.ceil(p[b, i])).astype(int)
+                at = 0
+                for x in range(lo[0] - ns + 1, hi[0] + ns):
+                    for y in range(lo[1] - ns + 1, hi[1] + ns):
+                        for z in range(lo[2] - ns + 1, hi[2] + ns):
+                            ok = 0 <= x < scale and 0 <= y < scale and 0 <= z < scale
+                            assert indexes[b, i, at] == ((x * scale + y) * scale + z if ok else -1)
+                            np.testing.assert_array_equal(out[b, i, at], feats[b, :, x, y, z] if ok else np.zeros(5))
+                            at += 1
+                assert at == nv
+        g = rng.standard_normal(out.shape)
+        grad_p, grad_f = oracle.cubic_feature_sampling_grad(scale, ns, g, indexes)
+        want = np.zeros((2, 5, scale ** 3))
+        for b in range(2):
+            for i in range(30):
+                for v in range(nv):
+                    if indexes[b, i, v] >= 0:
+                        want[b, :, indexes[b, i, v]] += g[b, i, v]
+        np.testing.assert_allclose(grad_f.reshape(2, 5, -1), want, rtol=1e-12, atol=1e-12)
+        assert (grad_p == 0).all()

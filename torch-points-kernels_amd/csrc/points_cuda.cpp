@@ -402,6 +402,146 @@ at::Tensor instance_iou_cuda(at::Tensor instance_idx, at::Tensor instance_offset
     return output;
 }
 
+// cuda/src/gridding.cpp:4-12 -> {grid_weights, grid_pt_weights, grid_pt_indexes}
+std::vector<at::Tensor> gridding(float min_x, float max_x, float min_y, float max_y, float min_z, float max_z,
+                                 at::Tensor ptcloud)
+{
+    check_gpu(ptcloud, "ptcloud");
+    check_contiguous(ptcloud, "ptcloud");
+    TORCH_CHECK(ptcloud.scalar_type() == at::kFloat || ptcloud.scalar_type() == at::kDouble,
+                "ptcloud must be float32 or float64");
+    TORCH_CHECK(ptcloud.dim() == 3 && ptcloud.size(2) == 3, "ptcloud must have shape (B, n_pts, 3)");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(ptcloud.device());
+    const int b = as_int(ptcloud.size(0), "batch size"), n = as_int(ptcloud.size(1), "number of points");
+    const int64_t len_x = static_cast<int>(max_x - min_x + 1), len_y = static_cast<int>(max_y - min_y + 1);
+    const int64_t len_z = static_cast<int>(max_z - min_z + 1);
+    TORCH_CHECK(len_x > 0 && len_y > 0 && len_z > 0, "gridding: empty grid");
+    at::Tensor grid = torch::empty({b, len_x * len_y * len_z}, ptcloud.options());
+    at::Tensor weights = torch::empty({b, n, 8, 3}, ptcloud.options());
+    at::Tensor indexes = torch::empty({b, n, 8}, ptcloud.options().dtype(at::kInt));
+    if (ptcloud.scalar_type() == at::kFloat)
+        check_status(tpk_gridding_f32(b, n, min_x, max_x, min_y, max_y, min_z, max_z, ptcloud.data_ptr<float>(),
+                                      grid.data_ptr<float>(), weights.data_ptr<float>(), indexes.data_ptr<int32_t>(),
+                                      current_stream(ptcloud)),
+                     "gridding");
+    else
+        check_status(tpk_gridding_f64(b, n, min_x, max_x, min_y, max_y, min_z, max_z, ptcloud.data_ptr<double>(),
+                                      grid.data_ptr<double>(), weights.data_ptr<double>(), indexes.data_ptr<int32_t>(),
+                                      current_stream(ptcloud)),
+                     "gridding");
+    return {grid, weights, indexes};
+}
+
+// cuda/src/gridding.cpp:14-26
+at::Tensor gridding_grad(at::Tensor grid_pt_weights, at::Tensor grid_pt_indexes, at::Tensor grad_grid)
+{
+    check_gpu(grid_pt_weights, "grid_pt_weights");
+    check_gpu(grid_pt_indexes, "grid_pt_indexes");
+    check_gpu(grad_grid, "grad_grid");
+    check_contiguous(grid_pt_weights, "grid_pt_weights");
+    check_contiguous(grid_pt_indexes, "grid_pt_indexes");
+    check_contiguous(grad_grid, "grad_grid");
+    check_dtype(grid_pt_indexes, at::kInt, "grid_pt_indexes");
+    TORCH_CHECK(grid_pt_weights.scalar_type() == at::kFloat || grid_pt_weights.scalar_type() == at::kDouble,
+                "grid_pt_weights must be float32 or float64");
+    TORCH_CHECK(grad_grid.scalar_type() == grid_pt_weights.scalar_type(), "grad_grid and grid_pt_weights differ in dtype");
+    TORCH_CHECK(grid_pt_indexes.dim() == 3 && grid_pt_indexes.size(2) == 8, "grid_pt_indexes must have shape (B, n_pts, 8)");
+    TORCH_CHECK(grid_pt_weights.dim() == 4 && grid_pt_weights.size(0) == grid_pt_indexes.size(0) &&
+                    grid_pt_weights.size(1) == grid_pt_indexes.size(1) && grid_pt_weights.size(2) == 8 &&
+                    grid_pt_weights.size(3) == 3,
+                "grid_pt_weights must have shape (B, n_pts, 8, 3)");
+    TORCH_CHECK(grad_grid.dim() == 2 && grad_grid.size(0) == grid_pt_indexes.size(0), "grad_grid must have shape (B, n_grid_vertices)");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_grid.device());
+    const int b = as_int(grad_grid.size(0), "batch size"), n = as_int(grid_pt_indexes.size(1), "number of points");
+    const int vertices = as_int(grad_grid.size(1), "grid vertices");
+    at::Tensor grad = torch::empty({b, n, 3}, grid_pt_weights.options());
+    if (grid_pt_weights.scalar_type() == at::kFloat)
+        check_status(tpk_gridding_grad_f32(b, n, vertices, grid_pt_weights.data_ptr<float>(),
+                                           grid_pt_indexes.data_ptr<int32_t>(), grad_grid.data_ptr<float>(),
+                                           grad.data_ptr<float>(), current_stream(grad_grid)),
+                     "gridding_grad");
+    else
+        check_status(tpk_gridding_grad_f64(b, n, vertices, grid_pt_weights.data_ptr<double>(),
+                                           grid_pt_indexes.data_ptr<int32_t>(), grad_grid.data_ptr<double>(),
+                                           grad.data_ptr<double>(), current_stream(grad_grid)),
+                     "gridding_grad");
+    return grad;
+}
+
+// cuda/src/cubic_feature_sampling.cpp:4-16 -> {point_features, grid_pt_indexes}
+std::vector<at::Tensor> cubic_feature_sampling(int scale, int neighborhood_size, at::Tensor ptcloud,
+                                               at::Tensor cubic_features)
+{
+    check_gpu(ptcloud, "ptcloud");
+    check_gpu(cubic_features, "cubic_features");
+    check_contiguous(ptcloud, "ptcloud");
+    check_contiguous(cubic_features, "cubic_features");
+    check_same_device(ptcloud, cubic_features, "ptcloud and cubic_features");
+    TORCH_CHECK(ptcloud.scalar_type() == at::kFloat || ptcloud.scalar_type() == at::kDouble,
+                "ptcloud must be float32 or float64");
+    TORCH_CHECK(cubic_features.scalar_type() == ptcloud.scalar_type(), "ptcloud and cubic_features differ in dtype");
+    TORCH_CHECK(ptcloud.dim() == 3 && ptcloud.size(2) == 3, "ptcloud must have shape (B, n_pts, 3)");
+    TORCH_CHECK(cubic_features.dim() == 5 && cubic_features.size(0) == ptcloud.size(0) && cubic_features.size(2) == scale &&
+                    cubic_features.size(3) == scale && cubic_features.size(4) == scale,
+                "cubic_features must have shape (B, c, scale, scale, scale)");
+    TORCH_CHECK(neighborhood_size >= 1 && neighborhood_size <= 64, "neighborhood_size out of range");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(ptcloud.device());
+    const int b = as_int(ptcloud.size(0), "batch size"), n = as_int(ptcloud.size(1), "number of points");
+    const int channels = as_int(cubic_features.size(1), "channels");
+    const int64_t side = 2 * static_cast<int64_t>(neighborhood_size), vertices = side * side * side;
+    at::Tensor features = torch::empty({b, n, vertices, channels}, ptcloud.options());
+    at::Tensor indexes = torch::empty({b, n, vertices}, ptcloud.options().dtype(at::kInt));
+    if (ptcloud.scalar_type() == at::kFloat)
+        check_status(tpk_cubic_feature_sampling_f32(b, n, channels, scale, neighborhood_size, ptcloud.data_ptr<float>(),
+                                                    cubic_features.data_ptr<float>(), features.data_ptr<float>(),
+                                                    indexes.data_ptr<int32_t>(), current_stream(ptcloud)),
+                     "cubic_feature_sampling");
+    else
+        check_status(tpk_cubic_feature_sampling_f64(b, n, channels, scale, neighborhood_size, ptcloud.data_ptr<double>(),
+                                                    cubic_features.data_ptr<double>(), features.data_ptr<double>(),
+                                                    indexes.data_ptr<int32_t>(), current_stream(ptcloud)),
+                     "cubic_feature_sampling");
+    return {features, indexes};
+}
+
+// cuda/src/cubic_feature_sampling.cpp:18-30 -> {grad_ptcloud, grad_cubic_features}
+std::vector<at::Tensor> cubic_feature_sampling_grad(int scale, int neighborhood_size, at::Tensor grad_point_features,
+                                                    at::Tensor grid_pt_indexes)
+{
+    check_gpu(grad_point_features, "grad_point_features");
+    check_gpu(grid_pt_indexes, "grid_pt_indexes");
+    check_contiguous(grad_point_features, "grad_point_features");
+    check_contiguous(grid_pt_indexes, "grid_pt_indexes");
+    check_dtype(grid_pt_indexes, at::kInt, "grid_pt_indexes");
+    TORCH_CHECK(grad_point_features.scalar_type() == at::kFloat || grad_point_features.scalar_type() == at::kDouble,
+                "grad_point_features must be float32 or float64");
+    TORCH_CHECK(neighborhood_size >= 1 && neighborhood_size <= 64, "neighborhood_size out of range");
+    TORCH_CHECK(scale > 0, "scale must be positive");
+    const int64_t side = 2 * static_cast<int64_t>(neighborhood_size), vertices = side * side * side;
+    TORCH_CHECK(grid_pt_indexes.dim() == 3 && grid_pt_indexes.size(2) == vertices, "grid_pt_indexes must have shape (B, n_pts, n_vertices)");
+    TORCH_CHECK(grad_point_features.dim() == 4 && grad_point_features.size(0) == grid_pt_indexes.size(0) &&
+                    grad_point_features.size(1) == grid_pt_indexes.size(1) && grad_point_features.size(2) == vertices,
+                "grad_point_features must have shape (B, n_pts, n_vertices, c)");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_point_features.device());
+    const int b = as_int(grad_point_features.size(0), "batch size"), n = as_int(grid_pt_indexes.size(1), "number of points");
+    const int channels = as_int(grad_point_features.size(3), "channels");
+    at::Tensor grad_ptcloud = torch::empty({b, n, 3}, grad_point_features.options());
+    at::Tensor grad_cubic = torch::empty({b, channels, scale, scale, scale}, grad_point_features.options());
+    if (grad_point_features.scalar_type() == at::kFloat)
+        check_status(tpk_cubic_feature_sampling_grad_f32(b, n, channels, scale, neighborhood_size,
+                                                         grad_point_features.data_ptr<float>(),
+                                                         grid_pt_indexes.data_ptr<int32_t>(), grad_ptcloud.data_ptr<float>(),
+                                                         grad_cubic.data_ptr<float>(), current_stream(grad_point_features)),
+                     "cubic_feature_sampling_grad");
+    else
+        check_status(tpk_cubic_feature_sampling_grad_f64(b, n, channels, scale, neighborhood_size,
+                                                         grad_point_features.data_ptr<double>(),
+                                                         grid_pt_indexes.data_ptr<int32_t>(), grad_ptcloud.data_ptr<double>(),
+                                                         grad_cubic.data_ptr<double>(), current_stream(grad_point_features)),
+                     "cubic_feature_sampling_grad");
+    return {grad_ptcloud, grad_cubic};
+}
+
 // No counterpart in the reference's native module: its grouping_operation is
 // torch.gather on a repeated index (torch_points_kernels/torchpoints.py:129-146).
 at::Tensor grouping_operation(at::Tensor features, at::Tensor idx)
@@ -578,6 +718,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("dense_knn", &dense_knn);
     m.def("grow_proximity", &grow_proximity);
     m.def("instance_iou_cuda", &instance_iou_cuda);
+    m.def("gridding", &gridding);
+    m.def("gridding_grad", &gridding_grad);
+    m.def("cubic_feature_sampling", &cubic_feature_sampling);
+    m.def("cubic_feature_sampling_grad", &cubic_feature_sampling_grad);
     m.def("three_interpolate", &three_interpolate);
     m.def("three_interpolate_grad", &three_interpolate_grad);
     m.def("ball_query_dense", &ball_query_dense, pybind11::arg("new_xyz"), pybind11::arg("xyz"), pybind11::arg("radius"),

@@ -1,6 +1,6 @@
 """torch_points_kernels for AMD MI355X: the spatial-search operators of
 torch-points3d/torch-points-kernels (furthest point sampling, ball query, three_nn /
-three_interpolate, grouping, Chamfer distance, dense knn, region growing, instance IoU) on hand-written HIP kernels.
+three_interpolate, grouping, Chamfer distance, dense knn, region growing, instance IoU, GRNet's gridding and cubic feature sampling) on hand-written HIP kernels.
 
 Same names and call signatures as the reference package (torch_points_kernels/__init__.py);
 GPU tensors only.
@@ -19,6 +19,8 @@ from .torchpoints import (
 from .knn import knn
 from .cluster import grow_proximity, region_grow
 from .metrics import instance_iou
+from .cubic_feature_sampling import cubic_feature_sampling
+from .gridding import gridding
 from .chamfer_dist import ChamferFunction
 from . import chamfer_dist  # the reference exports the submodule under this name
 
@@ -31,6 +33,8 @@ __all__ = [
     "knn",
     "region_grow",
     "instance_iou",
+    "cubic_feature_sampling",
+    "gridding",
     "chamfer_dist",
     "ChamferFunction",
 ]
