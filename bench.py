@@ -298,6 +298,53 @@ def bench_others(dev, steps, warmup, with_cpu):
                                        "CPU path is a numba routine of the same shape)"}
     out["instance_iou"] = e
 
+    # beyond the BASELINE configurations: GRNet's grid operators at its sizes (32 clouds of 2048 points; 64^3 grid;
+    # feature map 64 channels x 16^3)
+    gg = torch.Generator().manual_seed(11)
+    cloud = ((torch.rand(32, 2048, 3, generator=gg) * 2 - 1) * 31.0).to(dev)
+    wall, ev = _time_gpu(lambda: nat.gridding(-32.0, 31.0, -32.0, 31.0, -32.0, 31.0, cloud), steps, warmup)
+    grid, gw, gi = nat.gridding(-32.0, 31.0, -32.0, 31.0, -32.0, 31.0, cloud)
+    npts = 32 * 2048
+    nbytes = npts * (12 + 96 + 32) + grid.numel() * 4  # points in; weights and indexes out; the grid written once
+    e = {"workload": "gridding forward: 32 clouds x 2048 points into 64^3 grids (not a BASELINE configuration)", "metric": "points/s",
+         "value": npts / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall, "roofline": _roof_bytes(nbytes, ev, "gridding_fwd"),
+         "algorithmic_bytes": nbytes}
+    if with_cpu:
+        import oracle
+
+        sub = cloud[:4].cpu().numpy()
+        secs = _cpu_time(lambda: oracle.gridding(sub, 32))
+        e["cpu_baseline"] = {"value": 4 * 2048 / secs, "unit": "points/s", "cores": 1, "kind": "port",
+                             "sample": "4 of 32 clouds; C restatement of the reference's CUDA kernel (the reference has no CPU path)"}
+    out["gridding_fwd"] = e
+    ggrad = torch.randn(grid.shape, generator=gg).to(dev)
+    wall, ev = _time_gpu(lambda: nat.gridding_grad(gw, gi, ggrad), steps, warmup)
+    nbytes = npts * (96 + 32 + 32 + 12)  # weights, indexes, 8 gathered gradients per point; 12 bytes out
+    out["gridding_bwd"] = {"workload": "gridding backward, same sizes", "metric": "points/s", "value": npts / (wall * 1e-3),
+                           "kernel_ms": ev, "wall_ms": wall, "roofline": _roof_bytes(nbytes, ev, "gridding_bwd"),
+                           "algorithmic_bytes": nbytes}
+    feats = torch.rand(32, 64, 16, 16, 16, generator=gg).to(dev)
+    pts16 = (torch.rand(32, 2048, 3, generator=gg) * 15.0).to(dev)
+    wall, ev = _time_gpu(lambda: nat.cubic_feature_sampling(16, 1, pts16, feats), steps, warmup)
+    pf, pi = nat.cubic_feature_sampling(16, 1, pts16, feats)
+    nbytes = pf.numel() * 8 + pi.numel() * 4 + npts * 12  # every sampled feature read and written once
+    e = {"workload": "cubic_feature_sampling forward: 32 clouds x 2048 points, 64 channels x 16^3, neighborhood 1 (not a BASELINE "
+                     "configuration)", "metric": "GB/s", "value": nbytes / (wall * 1e-3) / 1e9, "kernel_ms": ev, "wall_ms": wall,
+         "roofline": _roof_bytes(nbytes, ev, "cubic_fwd"), "algorithmic_bytes": nbytes}
+    if with_cpu:
+        import oracle
+
+        secs = _cpu_time(lambda: oracle.cubic_feature_sampling(pts16[:4].cpu().numpy(), feats[:4].cpu().numpy(), 1))
+        e["cpu_baseline"] = {"value": nbytes / 8 / secs / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                             "sample": "4 of 32 clouds; C restatement of the reference's CUDA kernel (the reference has no CPU path)"}
+    out["cubic_feature_sampling_fwd"] = e
+    gpf = torch.randn(pf.shape, generator=gg).to(dev)
+    wall, ev = _time_gpu(lambda: nat.cubic_feature_sampling_grad(16, 1, gpf, pi), steps, warmup)
+    nbytes = pf.numel() * 4 + pi.numel() * 4 + feats.numel() * 4 + npts * 12
+    out["cubic_feature_sampling_bwd"] = {"workload": "cubic_feature_sampling backward, same sizes", "metric": "GB/s",
+                                         "value": nbytes / (wall * 1e-3) / 1e9, "kernel_ms": ev, "wall_ms": wall,
+                                         "roofline": _roof_bytes(nbytes, ev, "cubic_bwd"), "algorithmic_bytes": nbytes}
+
     dist, idx = tpk.three_nn(unknown, known)
     weight = W.inverse_distance_weights(dist).contiguous()
     feats = w["features"].to(dev)

@@ -188,6 +188,43 @@ __global__ __launch_bounds__(GR_THREADS) void cubic_scatter_kernel(
         atomicAdd(&grad_cubic_features[(cloud * channels + k) * cub_scale + vertex], grad_point_features[e]);
 }
 
+// The same sum with the destination in LDS: a workgroup owns `group` channels of one cloud's
+// feature map (group * scale^3 accumulators), walks all (point, vertex) entries of the cloud
+// and adds its channels' gradients with LDS atomics, then writes the map out in order.  One
+// global atomic per term (a cache line each, at device scope) is what makes the kernel above slow.
+template <typename T>
+__global__ __launch_bounds__(GR_THREADS) void cubic_scatter_lds_kernel(
+    int n_pts, int n_vertices, int channels, int group, int64_t cub_scale, const T* __restrict__ grad_point_features,
+    const int* __restrict__ grid_pt_indexes, T* __restrict__ grad_cubic_features)
+{
+    extern __shared__ __align__(16) unsigned char cubic_lds[];
+    T* sums = reinterpret_cast<T*>(cubic_lds);
+    const int groups = (channels + group - 1) / group;
+    const int cloud = blockIdx.x / groups;
+    const int k0 = (blockIdx.x - cloud * groups) * group;
+    const int width = min(group, channels - k0);
+    const int64_t cells = static_cast<int64_t>(width) * cub_scale;
+    for (int64_t t = threadIdx.x; t < cells; t += GR_THREADS)
+        sums[t] = T(0);
+    __syncthreads();
+    const int64_t entries = static_cast<int64_t>(n_pts) * n_vertices;
+    const int* indexes = grid_pt_indexes + cloud * entries;
+    const T* grads = grad_point_features + cloud * entries * channels;
+    // consecutive threads take the channels of one entry, then the next entry
+    for (int64_t t = threadIdx.x; t < entries * width; t += GR_THREADS)
+    {
+        const int64_t entry = t / width;
+        const int k = static_cast<int>(t - entry * width);
+        const int vertex = indexes[entry];
+        if (vertex >= 0 && vertex < cub_scale)
+            atomicAdd(&sums[k * cub_scale + vertex], grads[entry * channels + k0 + k]);
+    }
+    __syncthreads();
+    T* out = grad_cubic_features + (static_cast<int64_t>(cloud) * channels + k0) * cub_scale;
+    for (int64_t t = threadIdx.x; t < cells; t += GR_THREADS)
+        out[t] = sums[t];
+}
+
 template <typename T>
 int gridding_fwd(int b, int n_pts, float min_x, float max_x, float min_y, float max_y, float min_z, float max_z,
                  const T* ptcloud, T* grid_weights, T* grid_pt_weights, int32_t* grid_pt_indexes, hipStream_t s)
@@ -289,13 +326,35 @@ int cubic_bwd(int b, int n_pts, int channels, int scale, int neighborhood_size, 
     // the coordinates only choose the vertices (floor and ceil): their gradient is zero
     // (cuda/src/cubic_feature_sampling_gpu.cu:165-170)
     int st = fill_zero<T>(static_cast<int64_t>(b) * n_pts * 3, grad_ptcloud, s);
-    if (st == TPK_OK)
-        st = fill_zero<T>(static_cast<int64_t>(b) * channels * cub, grad_cubic_features, s);
+    if (st != TPK_OK)
+        return st;
     const int64_t total = static_cast<int64_t>(b) * n_pts * nv * channels;
+    if (total > 0 && (!grad_point_features || !grid_pt_indexes))
+        return TPK_ERR_INVALID_ARG;
+    // Feature maps that fit in LDS (at least one channel of scale^3 sums in 128 KiB) are summed there.
+    const int64_t fit = (128 * 1024) / (cub * static_cast<int64_t>(sizeof(T)));
+    if (fit >= 1 && channels > 0 && nv <= 0x7fffffffLL)
+    {
+        // as many channels per workgroup as fit, but enough workgroups to fill the chip
+        int64_t group = fit < channels ? fit : channels;
+        while (group > 1 && static_cast<int64_t>(b) * tpk_ceil_div(channels, group) < 512)
+            group = (group + 1) / 2;
+        const int64_t blocks = static_cast<int64_t>(b) * tpk_ceil_div(channels, group);
+        if (blocks <= 0x7fffffffLL)
+        {
+            const size_t lds = static_cast<size_t>(group * cub) * sizeof(T);
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(cubic_scatter_lds_kernel<T>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            if (e != hipSuccess)
+                return static_cast<int>(e);
+            hipLaunchKernelGGL(cubic_scatter_lds_kernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(GR_THREADS), lds, s, n_pts, static_cast<int>(nv), channels,
+                               static_cast<int>(group), cub, grad_point_features, grid_pt_indexes, grad_cubic_features);
+            return tpk_launch_status();
+        }
+    }
+    st = fill_zero<T>(static_cast<int64_t>(b) * channels * cub, grad_cubic_features, s);
     if (st != TPK_OK || total == 0)
         return st;
-    if (!grad_point_features || !grid_pt_indexes)
-        return TPK_ERR_INVALID_ARG;
     const int64_t blocks = tpk_ceil_div(total, GR_THREADS);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
