@@ -192,26 +192,31 @@ __global__ __launch_bounds__(GR_THREADS) void cubic_scatter_kernel(
 // feature map (group * scale^3 accumulators), walks all (point, vertex) entries of the cloud
 // and adds its channels' gradients with LDS atomics, then writes the map out in order.  One
 // global atomic per term (a cache line each, at device scope) is what makes the kernel above slow.
+constexpr int CS_THREADS = 1024; // LDS atomics are slow: many wavefronts keep the unit busy
+
 template <typename T>
-__global__ __launch_bounds__(GR_THREADS) void cubic_scatter_lds_kernel(
+__global__ __launch_bounds__(CS_THREADS) void cubic_scatter_lds_kernel(
     int n_pts, int n_vertices, int channels, int group, int64_t cub_scale, const T* __restrict__ grad_point_features,
     const int* __restrict__ grid_pt_indexes, T* __restrict__ grad_cubic_features)
 {
     extern __shared__ __align__(16) unsigned char cubic_lds[];
     T* sums = reinterpret_cast<T*>(cubic_lds);
+    // the workgroups of one cloud read the same lines of the gradient (each its own channels): they
+    // are kept on one die, so that one L2 serves them
     const int groups = (channels + group - 1) / group;
-    const int cloud = blockIdx.x / groups;
-    const int k0 = (blockIdx.x - cloud * groups) * group;
+    const int block = static_cast<int>(xcd_local_block(blockIdx.x, gridDim.x));
+    const int cloud = block / groups;
+    const int k0 = (block - cloud * groups) * group;
     const int width = min(group, channels - k0);
     const int64_t cells = static_cast<int64_t>(width) * cub_scale;
-    for (int64_t t = threadIdx.x; t < cells; t += GR_THREADS)
+    for (int64_t t = threadIdx.x; t < cells; t += CS_THREADS)
         sums[t] = T(0);
     __syncthreads();
     const int64_t entries = static_cast<int64_t>(n_pts) * n_vertices;
     const int* indexes = grid_pt_indexes + cloud * entries;
     const T* grads = grad_point_features + cloud * entries * channels;
     // consecutive threads take the channels of one entry, then the next entry
-    for (int64_t t = threadIdx.x; t < entries * width; t += GR_THREADS)
+    for (int64_t t = threadIdx.x; t < entries * width; t += CS_THREADS)
     {
         const int64_t entry = t / width;
         const int k = static_cast<int>(t - entry * width);
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(GR_THREADS) void cubic_scatter_lds_kernel(
     }
     __syncthreads();
     T* out = grad_cubic_features + (static_cast<int64_t>(cloud) * channels + k0) * cub_scale;
-    for (int64_t t = threadIdx.x; t < cells; t += GR_THREADS)
+    for (int64_t t = threadIdx.x; t < cells; t += CS_THREADS)
         out[t] = sums[t];
 }
 
@@ -335,9 +340,10 @@ int cubic_bwd(int b, int n_pts, int channels, int scale, int neighborhood_size, 
     const int64_t fit = (128 * 1024) / (cub * static_cast<int64_t>(sizeof(T)));
     if (fit >= 1 && channels > 0 && nv <= 0x7fffffffLL)
     {
-        // as many channels per workgroup as fit, but enough workgroups to fill the chip
+        // as many channels per workgroup as fit (the fewer workgroups share a line of the gradient, the
+        // less often it is read), but a workgroup for every compute unit
         int64_t group = fit < channels ? fit : channels;
-        while (group > 1 && static_cast<int64_t>(b) * tpk_ceil_div(channels, group) < 512)
+        while (group > 1 && static_cast<int64_t>(b) * tpk_ceil_div(channels, group) < 256)
             group = (group + 1) / 2;
         const int64_t blocks = static_cast<int64_t>(b) * tpk_ceil_div(channels, group);
         if (blocks <= 0x7fffffffLL)
@@ -347,7 +353,7 @@ int cubic_bwd(int b, int n_pts, int channels, int scale, int neighborhood_size, 
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
             if (e != hipSuccess)
                 return static_cast<int>(e);
-            hipLaunchKernelGGL(cubic_scatter_lds_kernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(GR_THREADS), lds, s, n_pts, static_cast<int>(nv), channels,
+            hipLaunchKernelGGL(cubic_scatter_lds_kernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(CS_THREADS), lds, s, n_pts, static_cast<int>(nv), channels,
                                static_cast<int>(group), cub, grad_point_features, grid_pt_indexes, grad_cubic_features);
             return tpk_launch_status();
         }
