@@ -160,7 +160,8 @@ __global__ __launch_bounds__(GR_THREADS) void cubic_gather_kernel(
     int64_t total, int n_pts, int n_vertices, int channels, int64_t cub_scale, const T* __restrict__ cubic_features,
     const int* __restrict__ grid_pt_indexes, T* __restrict__ point_features)
 {
-    const int64_t e = static_cast<int64_t>(blockIdx.x) * GR_THREADS + threadIdx.x;
+    // consecutive logical blocks (one cloud's) run on one die, whose L2 then holds that cloud's feature map
+    const int64_t e = static_cast<int64_t>(xcd_local_block(blockIdx.x, gridDim.x)) * GR_THREADS + threadIdx.x;
     if (e >= total)
         return;
     const int k = static_cast<int>(e % channels);
