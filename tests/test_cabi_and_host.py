@@ -147,6 +147,39 @@ def test_cpu_tensors_raise_instead_of_falling_back(tpk):
         tpk.grouping_operation(torch.rand(1, 2, 16), torch.zeros(1, 4, 2, dtype=torch.long))
 
 
+def test_added_operators_raise_for_cpu_tensors_and_bad_shapes(tpk):
+    from torch_points_kernels.cluster import grow_proximity, region_grow
+    from torch_points_kernels.cubic_feature_sampling import cubic_feature_sampling
+    from torch_points_kernels.gridding import gridding
+    from torch_points_kernels.metrics import instance_iou
+
+    pos = torch.rand(20, 3)
+    batch = torch.zeros(20, dtype=torch.long)
+    with pytest.raises(NotImplementedError):
+        tpk.knn(pos.unsqueeze(0), pos.unsqueeze(0), 3)
+    with pytest.raises(NotImplementedError):
+        tpk.ball_query(0.5, 4, pos.unsqueeze(0), pos.unsqueeze(0), sort=True)
+    with pytest.raises(NotImplementedError):
+        grow_proximity(pos, batch)
+    with pytest.raises(NotImplementedError):
+        region_grow(pos, torch.zeros(20, dtype=torch.long), batch)
+    with pytest.raises(AssertionError):
+        region_grow(pos, torch.zeros(20, 1, dtype=torch.long), batch)  # reference cluster.py:71
+    with pytest.raises(ValueError):
+        grow_proximity(pos, batch, member_order="sorted")
+    with pytest.raises(NotImplementedError):
+        instance_iou([torch.tensor([0, 1])], torch.tensor([1, 1, 0]))
+    # reference gridding.py:50-51, cubic_feature_sampling.py:53-54
+    with pytest.raises(ValueError):
+        gridding(torch.rand(10, 3), 4)
+    with pytest.raises(ValueError):
+        cubic_feature_sampling(torch.rand(10, 3), torch.rand(1, 2, 4, 4, 4))
+    with pytest.raises(NotImplementedError):
+        gridding(torch.rand(1, 10, 3), 4)
+    with pytest.raises(NotImplementedError):
+        cubic_feature_sampling(torch.rand(1, 10, 3), torch.rand(1, 2, 4, 4, 4))
+
+
 def test_product_package_does_not_reference_the_oracle():
     pkg = os.path.join(ROOT, "torch-points-kernels_amd")
     for dirpath, _, files in os.walk(pkg):
