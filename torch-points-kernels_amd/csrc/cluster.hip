@@ -39,7 +39,7 @@ namespace
 
 constexpr int CL_THREADS = 256;
 constexpr int CL_ROW_LANES = 16; // lanes that share one row of the matrix in a sweep
-constexpr int CL_SWEEPS = 16;    // sweeps enqueued between two looks at the `changed` flags
+constexpr int CL_SWEEPS = 8;     // sweeps enqueued between two looks at the `changed` flags
 constexpr int CL_FOLLOW = 16;    // labels followed per point and sweep
 constexpr int64_t CL_MAX_POINTS = (int64_t)1 << 30;
 
