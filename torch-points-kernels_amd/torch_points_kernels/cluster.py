@@ -39,27 +39,15 @@ def grow_proximity(pos, batch, nsample=16, radius=0.02, min_cluster_size=32, mem
 def region_grow(
     pos, labels, batch, ignore_labels=[], nsample=16, radius=0.02, min_cluster_size=32, member_order="reference"
 ) -> List[torch.Tensor]:
-    """Region growing clustering algorithm proposed in
-    PointGroup: Dual-Set Point Grouping for 3D Instance Segmentation
-    https://arxiv.org/pdf/2004.01658.pdf
-    for instance segmentation (reference cluster.py:48-109)
+    """PointGroup's region growing (https://arxiv.org/pdf/2004.01658.pdf): clusters of points of equal label
+    that are chained by neighbourhoods of the given radius, label by label.
 
-    Parameters
-    ----------
-    pos: torch.Tensor [N, 3]
-        Location of the points
-    labels: torch.Tensor [N,]
-        labels of each point
-    ignore_labels:
-        Labels that should be ignored, no region growing will be performed on those
-    nsample:
-        maximum number of neighbours to consider
-    radius:
-        radius for the neighbour search
-    min_cluster_size:
-        Number of points above which a cluster is considered valid
-    member_order:
-        see grow_proximity
+    pos (N, 3), labels (N,), batch (N,) sorted sample ids; labels in ignore_labels are skipped; a row of the
+    neighbour search holds at most nsample points; clusters below min_cluster_size are dropped.
+    Returns a list of index tensors into pos (on pos.device), label after label, ordered by first point
+    inside a label.  member_order: see grow_proximity.
+
+    Reference: cluster.py:48-109.
     """
     assert labels.dim() == 1
     assert pos.dim() == 2

@@ -1,58 +1,42 @@
-"""Gridding of point clouds (GRNet; reference: torch_points_kernels/gridding.py)."""
+"""GRNet's gridding operator: point clouds to occupancy grids (API of the reference's
+torch_points_kernels/gridding.py: GriddingFunction, gridding)."""
 import torch
 
 from ._native import native, require_gpu
 
 
 class GriddingFunction(torch.autograd.Function):
-    """Reference gridding.py:7-31."""
+    """Trilinear deposit of points given in grid units into a grid spanning [-scale, scale - 1] on
+    every axis; returns the grid flattened to (B, (2 * scale) ** 3).  Differentiable in the points
+    (reference gridding.py:7-31)."""
 
     @staticmethod
     def forward(ctx, ptcloud, scale):
         require_gpu(ptcloud, "gridding")
-        grid, grid_pt_weights, grid_pt_indexes = native().gridding(
-            -scale, scale - 1, -scale, scale - 1, -scale, scale - 1, ptcloud.contiguous()
-        )
-        # grid (batch_size, n_grid_vertices), grid_pt_weights (batch_size, n_pts, 8, 3),
-        # grid_pt_indexes (batch_size, n_pts, 8)
-        ctx.save_for_backward(grid_pt_weights, grid_pt_indexes)
+        lo, hi = -scale, scale - 1
+        grid, weights, vertices = native().gridding(lo, hi, lo, hi, lo, hi, ptcloud.contiguous())
+        ctx.save_for_backward(weights, vertices)  # (B, n, 8, 3) factors and (B, n, 8) vertex numbers per point
         return grid
 
     @staticmethod
     def backward(ctx, grad_grid):
-        grid_pt_weights, grid_pt_indexes = ctx.saved_tensors
-        grad_ptcloud = native().gridding_grad(grid_pt_weights, grid_pt_indexes, grad_grid.contiguous())
-        return grad_ptcloud, None
+        weights, vertices = ctx.saved_tensors
+        return native().gridding_grad(weights, vertices, grad_grid.contiguous()), None
 
 
 def gridding(ptcloud, scale):
-    r"""
-    Converts the input point clouds into 3D grids by trilinear interpolcation.
-    Please refer to https://arxiv.org/pdf/2006.03761 for more information
+    """Grids of resolution 2 * scale per axis from clouds with coordinates in [-1, 1).
 
-    Parameters
-    ----------
-    ptcloud : torch.Tensor (dtype=torch.float32)
-        (B, n_pts, 3) B point clouds containing n_pts points
-    scale : Int
-        the resolution of the 3D grid
-
-    Returns
-    -------
-    grid: torch.Tensor
-        (B, scale, scale, scale): the grid of the resolution of scale * scale * scale
-
-    Reference: gridding.py:34-60 (points whose coordinates sum to zero are dropped, cloud by cloud).
+    ptcloud: (B, n_pts, 3) floating point tensor on the GPU; scale: int.
+    Returns (B, (2 * scale) ** 3).  As in the reference (gridding.py:34-60) the coordinates are
+    multiplied by `scale`, and each cloud is gridded on its own after dropping the points whose
+    three coordinates sum to zero (padding).
     """
-    if len(ptcloud.shape) != 3 or ptcloud.size(2) != 3:
+    if ptcloud.dim() != 3 or ptcloud.size(2) != 3:
         raise ValueError("The input point cloud should be of size (B, n_pts, 3)")
-
-    ptcloud = ptcloud * scale
-    _ptcloud = torch.split(ptcloud, 1, dim=0)
+    scaled = ptcloud * scale
     grids = []
-    for p in _ptcloud:
-        non_zeros = torch.sum(p, dim=2).ne(0)
-        p = p[non_zeros].unsqueeze(dim=0)
-        grids.append(GriddingFunction.apply(p, scale))
-
+    for cloud in scaled.unbind(0):
+        kept = cloud[cloud.sum(dim=1) != 0]
+        grids.append(GriddingFunction.apply(kept.unsqueeze(0), scale))
     return torch.cat(grids, dim=0).contiguous()

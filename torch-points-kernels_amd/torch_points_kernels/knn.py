@@ -1,21 +1,16 @@
-"""Dense k nearest neighbours (reference: torch_points_kernels/knn.py:4-18)."""
+"""Dense k nearest neighbours (API of the reference's torch_points_kernels/knn.py)."""
 from ._native import native, require_gpu
 
 
 def knn(pos_support, pos, k):
-    """Dense knn search
+    """For every query point the k nearest support points of the same cloud.
 
-    Arguments:
-        pos_support - [B,N,3] support points
-        pos - [B,M,3] centre of queries
-        k - number of neighbours, needs to be <= N
+    pos_support (B, N, 3): points searched; pos (B, M, 3): query points; k <= N.
+    Returns (idx (B, M, k) int64, dist2 (B, M, k) squared distances), nearest first; equal distances
+    keep the lower index first.
 
-    Returns:
-        idx - [B,M,k]
-        dist2 - [B,M,k] squared distances
-
-    The reference serves CPU tensors only and raises for CUDA tensors; this build serves GPU
-    tensors only.  Neighbours ascend by (squared distance, index).
+    The reference (knn.py:4-18) serves CPU tensors only and raises for CUDA tensors; this build serves
+    GPU tensors only.
     """
     assert pos_support.dim() == 3 and pos.dim() == 3
     require_gpu(pos_support, "knn")

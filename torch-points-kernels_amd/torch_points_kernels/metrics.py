@@ -11,21 +11,13 @@ def instance_iou(
     gt_instances: torch.Tensor,
     batch: Optional[torch.Tensor] = None,
 ):
-    """Computes the IoU between each proposed instance in instance_idx and ground truth instances. Returns a
-    tensor of shape [instance_idx.shape[0], num_instances] that contains the iou between the proposed instances and all gt instances
-    Instance label 0 is reserved for non instance points
+    """IoU of every proposed instance with every ground-truth instance.
 
-    Parameters
-    ----------
-    instance_idx : List[torch.Tensor]
-        List of instances. Each tensor in this list is a proposed and contains the index of the points
-        that belong to that particular instance
-    gt_instances : torch.Tensor
-        Ground truth instances, contains the index of the instance for each point
-
-    Returns
-    -------
-    ious: torch.Tensor[nb_proposals, nb_groundtruth]
+    instance_idx: list of index tensors, one per proposal (the points it holds);
+    gt_instances: (N,) ground-truth instance of every point, numbered from 1 inside each sample, 0 (or a
+    negative value) for points of no instance; batch: (N,) sample of every point, sorted (default: one sample).
+    Returns float32 (number of proposals, ground-truth instances of all samples); a proposal is compared
+    with the instances of the sample its first point belongs to, the other columns are 0.
 
     Reference: metrics.py:37-104; GPU tensors only here.
     """
