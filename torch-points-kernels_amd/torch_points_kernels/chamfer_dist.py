@@ -23,8 +23,9 @@ class ChamferFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_dist1, grad_dist2):
         xyz1, xyz2, nearest1, nearest2 = ctx.saved_tensors
-        return native().chamfer_dist_grad(xyz1, xyz2, nearest1, nearest2, grad_dist1.contiguous(),
-                                          grad_dist2.contiguous())
+        grad_xyz1, grad_xyz2 = native().chamfer_dist_grad(xyz1, xyz2, nearest1, nearest2, grad_dist1.contiguous(),
+                                                          grad_dist2.contiguous())
+        return grad_xyz1, grad_xyz2
 
 
 def chamfer_dist(xyz1, xyz2, ignore_zeros=False):
