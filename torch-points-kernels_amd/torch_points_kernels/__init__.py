@@ -24,17 +24,8 @@ from .gridding import gridding
 from .chamfer_dist import ChamferFunction
 from . import chamfer_dist  # the reference exports the submodule under this name
 
-__all__ = [
-    "ball_query",
-    "furthest_point_sample",
-    "grouping_operation",
-    "three_interpolate",
-    "three_nn",
-    "knn",
-    "region_grow",
-    "instance_iou",
-    "cubic_feature_sampling",
-    "gridding",
-    "chamfer_dist",
-    "ChamferFunction",
-]
+# the names the reference package exports (torch_points_kernels/__init__.py), plus ChamferFunction
+__all__ = (
+    "ball_query furthest_point_sample grouping_operation three_interpolate three_nn knn region_grow "
+    "instance_iou chamfer_dist cubic_feature_sampling gridding ChamferFunction"
+).split()
