@@ -49,8 +49,7 @@ def test_library_exports_every_declared_symbol():
     assert lib.tpk_fps_workspace_bytes(2, 200000) == 2 * 200000 * 4  # larger: the minima only
     # searches over curve-ordered cells: 16 bytes per point padded to cells of 64, 160 bytes per cell;
     # 0 = the shape is served by the all-pairs scan, no workspace wanted
-    for name in ("tpk_three_nn_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes", "tpk_knn_workspace_bytes",
-                 "tpk_ball_query_sorted_dense_workspace_bytes"):
+    for name in ("tpk_three_nn_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes", "tpk_knn_workspace_bytes"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_size_t
         assert fn(2, 100, 100) == 0 and fn(2, 200000, 1000) == 0 and fn(0, 1000, 1000) == 0
@@ -59,9 +58,19 @@ def test_library_exports_every_declared_symbol():
         # clouds above 16384 points: whole windows of 16384 points (256 cells each)
         want = sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((512, 1024), (15, 1024), (512, 160), (15, 160)))
         assert fn(2, 20000, 900) == want
+    up = lambda v: -(-v // 256) * 256
+    # sorted ball query (b, support points, queries): only the support points are ordered when one wavefront serves a
+    # query (up to 64 neighbours); the size also covers the k-nearest lists that serve more neighbours
+    fn = lib.tpk_ball_query_sorted_dense_workspace_bytes
+    fn.restype = ctypes.c_size_t
+    cells = lambda n: -(-n // 64) if n <= 16384 else -(-n // 16384) * 256
+    support_only = lambda b, n: up(b * cells(n) * 1024) + up(b * cells(n) * 160)
+    assert fn(2, 100, 5000) == 0 and fn(0, 1000, 1000) == 0
+    assert fn(2, 4096, 100) == support_only(2, 4096)
+    assert fn(2, 200000, 1000) == support_only(2, 200000)
+    assert fn(2, 700, 900) == sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((11, 1024), (15, 1024), (11, 160), (15, 160)))
     # list-based backward passes: counts (4 B per target, blocks of 64), block descriptions (8 B per block),
     # entry slots (3 per index entry + 576 per block of 64 targets; 8 B weighted, 4 B plain), per column piece
-    up = lambda v: -(-v // 256) * 256
     lib.tpk_three_interpolate_grad_workspace_bytes.restype = ctypes.c_size_t
     assert lib.tpk_three_interpolate_grad_workspace_bytes(2, 1000, 100) == up(2 * 128 * 4) + up(2 * 2 * 8) + up(2 * (3 * 3000 + 576 * 2) * 8)
     # 20000 columns: one row at a time in pieces of 16384 columns -> 2 pieces per cloud

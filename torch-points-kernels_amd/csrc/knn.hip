@@ -337,7 +337,10 @@ int launch_nearest_packed(int64_t size_x, int64_t size_y, int nsample, float lim
 
 extern "C" size_t tpk_ball_query_sorted_dense_workspace_bytes(int b, int n, int m)
 {
-    return tpk_grid_knn_workspace_bytes(b, m, n);
+    // up to 64 neighbours: one wavefront per query over the ordered support points; more: the lists
+    // of the k-nearest search, which orders both sets
+    const size_t waves = tpk_grid_ball_sorted_workspace_bytes(b, n), lists = tpk_grid_knn_workspace_bytes(b, m, n);
+    return waves > lists ? waves : lists;
 }
 
 extern "C" int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius, int nsample, const float* new_xyz,
@@ -354,6 +357,13 @@ extern "C" int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius
         return TPK_ERR_UNSUPPORTED;
     hipStream_t s = tpk_stream(stream);
     const float limit = radius * radius; // fp32 product (cpu/src/neighbors.cpp:19)
+    if (workspace)
+    {
+        const int direct = tpk_grid_ball_sorted(b, m, n, nsample, limit, false, 0, new_xyz, xyz, dist, idx, workspace,
+                                                workspace_bytes, s);
+        if (direct != TPK_ERR_UNSUPPORTED)
+            return direct; // (padding included)
+    }
     const int st = nearest_within(b, n, m, nsample, limit, xyz, new_xyz, idx, dist, workspace, workspace_bytes, s);
     if (st != TPK_OK)
         return st;
@@ -395,15 +405,18 @@ constexpr int64_t NP_GRID_POINTS = 163840; // largest cloud the search over cell
 
 } // namespace
 
-// The workspace lets clouds of 512..163840 points (support and queries) be searched over
-// curve-ordered cells, one cloud after the other; the call then waits for the stream once, to
-// read the clouds' ranges.
+// The workspace lets clouds of 512..163840 support points be searched over curve-ordered cells, one
+// cloud after the other (up to 64 neighbours: one wavefront per query; more: the k-nearest lists,
+// which also want 512 queries or more); the call then waits for the stream once, to read the
+// clouds' ranges.
 extern "C" size_t tpk_ball_query_sorted_partial_workspace_bytes(int64_t size_x, int64_t size_y)
 {
-    if (size_x < 512 || size_y < 512)
+    if (size_x < 512 || size_y < 1)
         return 0;
-    const size_t grid = tpk_grid_knn_workspace_bytes(1, static_cast<int>(tpk_min64(size_y, NP_GRID_POINTS)),
-                                                     static_cast<int>(tpk_min64(size_x, NP_GRID_POINTS)));
+    const int most_x = static_cast<int>(tpk_min64(size_x, NP_GRID_POINTS));
+    const size_t lists = tpk_grid_knn_workspace_bytes(1, static_cast<int>(tpk_min64(size_y, NP_GRID_POINTS)), most_x);
+    const size_t waves = tpk_grid_ball_sorted_workspace_bytes(1, most_x);
+    const size_t grid = waves > lists ? waves : lists;
     return grid ? NP_RANGES_BYTES + grid : 0;
 }
 
@@ -455,6 +468,14 @@ extern "C" int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y,
         float* dist_c = dist + q0 * nsample;
         int st = TPK_ERR_UNSUPPORTED;
         int64_t add = 0;
+        if (points >= 0 && points <= NP_GRID_POINTS && queries <= 0x7fffffffLL)
+        {
+            // up to 64 neighbours: one wavefront per query over the cloud's ordered support points
+            st = tpk_grid_ball_sorted(1, static_cast<int>(queries), static_cast<int>(points), nsample, limit, true, s0,
+                                      y + q0 * 3, x + s0 * 3, dist_c, idx_c, grid_ws, grid_bytes, s);
+            if (st != TPK_ERR_UNSUPPORTED)
+                return st; // (padding included)
+        }
         if (points >= 0 && queries <= NP_GRID_POINTS && points <= NP_GRID_POINTS &&
             tpk_grid_knn_workspace_bytes(1, static_cast<int>(queries), static_cast<int>(points)) != 0)
         {

@@ -26,6 +26,15 @@ size_t tpk_grid_knn_workspace_bytes(int b, int n, int m);
 int tpk_grid_knn(int b, int n, int m, int k, float limit, const float* query, const float* support, float* dist2,
                  int64_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+// Ball query with sorted neighbours, float32, one wavefront per query: the nsample (<= 64) nearest of the
+// m support points of the query's cloud with squared distance < limit, nearest first; only the support
+// points are ordered (workspace for b clouds of m points).  Writes every slot: unused ones are -1 / -1
+// when `packed`, else (index of the nearest, or 0) / -1; indices are raised by index_add.
+size_t tpk_grid_ball_sorted_workspace_bytes(int b, int m);
+int tpk_grid_ball_sorted(int b, int n, int m, int nsample, float limit, bool packed, int64_t index_add,
+                         const float* query, const float* support, float* dist, int64_t* idx, void* workspace,
+                         size_t workspace_bytes, hipStream_t stream);
+
 // Ball query, packed layout (a hit has squared distance <= radius2 = radius * radius as the caller
 // rounds it): same conventions.  Queries with dense neighbourhoods are answered by a scan in
 // index order inside the same kernel.

@@ -904,6 +904,165 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
     return tpk_launch_status();
 }
 
+namespace {
+
+using u64 = unsigned long long;
+
+// The 64 keys of a wavefront sorted across its lanes (bitonic network; lane i ends with the i-th
+// smallest, or the i-th largest when `descending`).
+__device__ __forceinline__ u64 wave_sort_keys(u64 key, int lane, bool descending)
+{
+#pragma unroll
+    for (int k = 2; k <= TPK_WAVE; k <<= 1)
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1)
+        {
+            const u64 other = __shfl_xor(key, j, TPK_WAVE);
+            const bool up = ((lane & k) == 0) != descending;
+            const bool keep_min = ((lane & j) == 0) == up;
+            key = (keep_min == (key < other)) ? key : other;
+        }
+    return key;
+}
+
+// A bitonic sequence across the lanes put into ascending order.
+__device__ __forceinline__ u64 wave_merge_ascending(u64 key, int lane)
+{
+#pragma unroll
+    for (int j = TPK_WAVE / 2; j > 0; j >>= 1)
+    {
+        const u64 other = __shfl_xor(key, j, TPK_WAVE);
+        key = (((lane & j) == 0) == (key < other)) ? key : other;
+    }
+    return key;
+}
+
+__device__ __forceinline__ u64 read_lane_key(u64 key, int from)
+{
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<int>(key & 0xFFFFFFFFu), from);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<int>(key >> 32), from);
+    return (static_cast<u64>(hi) << 32) | lo;
+}
+
+// Ball query with sorted neighbours, one wavefront per query: the nsample (<= 64) nearest support
+// points with squared distance < limit.  The support points lie in curve-ordered cells of 64; a
+// cell whose box is out of reach is skipped; the others are tested one point per lane.  The
+// wavefront keeps its 64 best (distance, index) keys sorted across the lanes: the candidates of a
+// cell that beat the current nsample-th key are sorted the other way round and merged in (minimum
+// per lane, then one bitonic merge).  Dense neighbourhoods - hundreds of points inside the radius -
+// cost a few such merges, not an insertion per point.
+// Unused slots: packed layout -1 / -1; dense layout the nearest neighbour's index (0 without any)
+// and -1.  Indices are raised by index_add.
+__global__ __launch_bounds__(NG_SCAN_THREADS) void ball_sorted_wave_kernel(
+    int64_t queries, int n, int ccells, int nsample, float limit, bool packed, int64_t index_add,
+    const float* __restrict__ query, const float4* __restrict__ sorted_support,
+    const float4* __restrict__ boxes_support, float* __restrict__ dist, int64_t* __restrict__ idx)
+{
+    const int lane = threadIdx.x & (TPK_WAVE - 1);
+    const int64_t q = static_cast<int64_t>(blockIdx.x) * (NG_SCAN_THREADS / TPK_WAVE) + threadIdx.x / TPK_WAVE;
+    if (q >= queries)
+        return; // (no workgroup barrier anywhere in this kernel)
+    const int64_t cloud = q / n;
+    const float4* __restrict__ cpts = sorted_support + cloud * ccells * NG_CELL;
+    const float4* __restrict__ cbox = boxes_support + cloud * ccells * NG_BOX;
+    const float qx = query[q * 3 + 0], qy = query[q * 3 + 1], qz = query[q * 3 + 2];
+
+    constexpr u64 NONE = ~0ull;
+    u64 best = NONE;      // lane i: the i-th smallest key so far
+    u64 admit = NONE;     // the nsample-th smallest: a candidate must beat it
+    float reach = limit;  // squared distance beyond which a cell cannot help
+    for (int first = 0; first < ccells; first += NG_CELL)
+    {
+        const int c = first + lane;
+        const bool valid = c < ccells;
+        const int cc = valid ? c : 0;
+        const float lb = point_box_dist2(qx, qy, qz, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
+        u64 live = __ballot(valid && lb * NG_MARGIN <= limit);
+        while (live != 0)
+        {
+            const int bit = __builtin_ctzll(live);
+            live &= live - 1;
+            if (tpk_read_lane(lb, bit) * NG_MARGIN > reach)
+                continue; // the list has filled up with nearer points meanwhile
+            const float4 p = cpts[static_cast<int64_t>(first + bit) * NG_CELL + lane];
+            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            u64 cand = d < limit ? knn_key(d, __float_as_int(p.w)) : NONE;
+            cand = cand < admit ? cand : NONE;
+            if (__ballot(cand != NONE) == 0)
+                continue;
+            cand = wave_sort_keys(cand, lane, true);
+            best = wave_merge_ascending(best < cand ? best : cand, lane);
+            admit = read_lane_key(best, nsample - 1);
+            if (admit != NONE)
+                reach = __int_as_float(static_cast<int>(admit >> 32));
+        }
+    }
+    if (lane < nsample)
+    {
+        const u64 nearest = read_lane_key(best, 0);
+        const bool found = best != NONE;
+        const int64_t o = q * nsample + lane;
+        const int64_t pad = packed ? -1 : (nearest != NONE ? static_cast<int64_t>(nearest & 0xFFFFFFFFu) + index_add : 0);
+        idx[o] = found ? static_cast<int64_t>(best & 0xFFFFFFFFu) + index_add : pad;
+        dist[o] = found ? __int_as_float(static_cast<int>(best >> 32)) : -1.0f;
+    }
+}
+
+struct SupportLayout
+{
+    size_t sorted, boxes, total;
+};
+
+SupportLayout support_layout(int b, int m)
+{
+    auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    const size_t cells = static_cast<size_t>(grid_cells(m));
+    SupportLayout l;
+    l.sorted = 0;
+    l.boxes = up(static_cast<size_t>(b) * cells * NG_CELL * sizeof(float4));
+    l.total = l.boxes + up(static_cast<size_t>(b) * cells * NG_BOX * sizeof(float4));
+    return l;
+}
+
+// Worth ordering the support points from this many on; below, all pairs are as fast.
+bool ball_sorted_supported(int b, int m, int nsample)
+{
+    return b > 0 && m >= 512 && nsample >= 1 && nsample <= TPK_WAVE;
+}
+
+} // namespace
+
+size_t tpk_grid_ball_sorted_workspace_bytes(int b, int m)
+{
+    return ball_sorted_supported(b, m, 1) ? support_layout(b, m).total : 0;
+}
+
+// n queries and m support points per cloud; outputs complete (padding included).
+int tpk_grid_ball_sorted(int b, int n, int m, int nsample, float limit, bool packed, int64_t index_add,
+                         const float* query, const float* support, float* dist, int64_t* idx, void* workspace,
+                         size_t workspace_bytes, hipStream_t s)
+{
+    if (!ball_sorted_supported(b, m, nsample) || n < 1 || !(limit < __builtin_inff()))
+        return TPK_ERR_UNSUPPORTED;
+    const SupportLayout l = support_layout(b, m);
+    if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return TPK_ERR_WORKSPACE;
+    char* w = static_cast<char*>(workspace);
+    PointSet none{nullptr, nullptr, 0, 1, 0, nullptr, nullptr, nullptr, nullptr};
+    PointSet c{support, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted),
+               reinterpret_cast<float4*>(w + l.boxes), nullptr, nullptr};
+    int st = launch_curve_cells(none, c, nullptr, s);
+    if (st != TPK_OK)
+        return st;
+    const int64_t queries = static_cast<int64_t>(b) * n;
+    const int64_t blocks = tpk_ceil_div(queries, NG_SCAN_THREADS / TPK_WAVE);
+    if (blocks > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(ball_sorted_wave_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, queries,
+                       n, grid_cells(m), nsample, limit, packed, index_add, query, c.sorted, c.boxes, dist, idx);
+    return tpk_launch_status();
+}
+
 size_t tpk_grid_knn_workspace_bytes(int b, int n, int m)
 {
     return grid_supported(b, n, m) ? grid_layout(b, n, m).total : 0;
