@@ -203,7 +203,7 @@ def bench_others(dev, steps, warmup, with_cpu):
     e = {"workload": "ball_query partial_dense sort=True on configs[3] (the reference has this mode for CPU tensors only)",
          "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
          "roofline": _roof_flops(pairs, 8, ev), "pairs": pairs}
-    e["roofline"]["note"] += "; every pair of a query with its cloud is tested (no cell search for this mode yet)"
+    e["roofline"]["note"] += PRUNED_NOTE + "; the clouds are searched one after the other, after one wait for the stream"
     if ref is not None:
         secs = _cpu_time(lambda: ref.batch_ball_query(w["x"], w["y"], w["batch_x"], w["batch_y"], w["radius"],
                                                       w["nsample"], 0, True))
