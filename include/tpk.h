@@ -102,10 +102,12 @@ int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int
  * Shapes and dtypes as for tpk_ball_query_dense_f32 / tpk_ball_query_partial_f32.  Unused
  * slots: dense - idx repeats the nearest neighbour (0 when there is none), dist -1; packed -
  * both -1.  With a `workspace` (tpk_ball_query_sorted_*_workspace_bytes() bytes - 0 for
- * shapes not served that way -, 256-byte aligned) the search goes over curve-ordered cells
- * within the radius instead of all pairs, same results.  In the packed layout this is done
- * cloud by cloud (clouds of 512..163840 points and queries, cloud ids below 1024; others by
- * all pairs), and the call then waits for the stream once, to read where the clouds start.
+ * shapes not served that way -, 256-byte aligned) the support points are ordered along a
+ * space filling curve and a query only visits cells within its radius (clouds of 512 support
+ * points or more; up to 64 neighbours one wavefront serves a query), same results as the all
+ * pairs scan used otherwise.  In the packed layout this is done cloud by cloud (clouds of up
+ * to 163840 points, cloud ids below 1024; others by all pairs), and the call then waits for
+ * the stream once, to read where the clouds start.
  * ------------------------------------------------------------------------------------- */
 size_t tpk_ball_query_sorted_dense_workspace_bytes(int b, int n, int m);
 int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius, int nsample,
