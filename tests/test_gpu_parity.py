@@ -932,6 +932,35 @@ def test_cubic_feature_sampling_front_end_and_gradcheck(tpk, oracle, dev):
         cubic_feature_sampling(p[0].to(dev), feats.to(dev))
 
 
+# ------------------------------------------------------------------ committed reference vectors
+
+
+def test_hip_path_against_committed_reference_vectors(tpk, dev):
+    """The reference's own CPU module computed these outputs (tests/golden/make_vectors.py); the HIP path must
+    reproduce them bit for bit - no oracle in between."""
+    import os
+
+    v = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_cpu_vectors.npz"))
+    t = lambda name: torch.from_numpy(v[name]).to(dev)
+    idx, dist2 = tpk.knn(t("knn_support"), t("knn_query"), 9)
+    np.testing.assert_array_equal(_np(idx), v["knn_idx"])
+    np.testing.assert_array_equal(_np(dist2), v["knn_dist2"])
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    dist3, idx3 = native.three_nn(t("knn_query"), t("knn_support"))  # squared distances (the Python layer returns their roots)
+    np.testing.assert_array_equal(_np(idx3), v["three_nn_idx"])
+    np.testing.assert_array_equal(_np(dist3), v["three_nn_dist2"])
+    idx, dist = tpk.ball_query(float(v["ball_sorted_radius"]), 12, t("knn_support"), t("knn_query"), sort=True)
+    np.testing.assert_array_equal(_np(idx), v["ball_sorted_idx"])
+    np.testing.assert_array_equal(_np(dist), v["ball_sorted_dist"])
+    idx, dist = tpk.ball_query(float(v["packed_radius"]), 10, t("packed_x"), t("packed_y"), mode="partial_dense",
+                               batch_x=t("packed_batch_x"), batch_y=t("packed_batch_y"), sort=True)
+    np.testing.assert_array_equal(_np(idx), v["packed_sorted_idx"])
+    np.testing.assert_array_equal(_np(dist), v["packed_sorted_dist"])
+    np.testing.assert_array_equal(_np(tpk.furthest_point_sample(t("fps_xyz"), 64)), v["fps_idx"])
+    out = tpk.three_interpolate(t("interp_features"), t("interp_idx").int(), t("interp_weight"))
+    np.testing.assert_array_equal(_np(out), v["interp_out"])
+
+
 # ------------------------------------------------------------------ chamfer
 
 

@@ -695,3 +695,35 @@ def test_cubic_feature_sampling_is_a_gather(oracle):
                         want[b, :, indexes[b, i, v]] += g[b, i, v]
         np.testing.assert_allclose(grad_f.reshape(2, 5, -1), want, rtol=1e-12, atol=1e-12)
         assert (grad_p == 0).all()
+
+
+# ------------------------------------------------------------------ committed reference vectors
+
+
+def _golden():
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_cpu_vectors.npz")
+    return np.load(path)  # arrays only (allow_pickle stays off)
+
+
+def test_oracle_against_committed_reference_vectors(oracle):
+    """tests/golden/reference_cpu_vectors.npz holds what the reference's CPU module returned for these inputs
+    (tests/golden/make_vectors.py); it travels to machines without the reference checkout."""
+    v = _golden()
+    idx, dist2 = oracle.knn(v["knn_support"], v["knn_query"], 9)
+    np.testing.assert_array_equal(idx, v["knn_idx"])
+    np.testing.assert_array_equal(dist2, v["knn_dist2"])
+    dist3, idx3 = oracle.three_nn(v["knn_query"], v["knn_support"])
+    np.testing.assert_array_equal(idx3, v["three_nn_idx"])
+    np.testing.assert_array_equal(dist3, v["three_nn_dist2"])
+    idx, dist = oracle.ball_query_sorted_dense(float(v["ball_sorted_radius"]), 12, v["knn_support"], v["knn_query"])
+    np.testing.assert_array_equal(idx, v["ball_sorted_idx"])
+    np.testing.assert_array_equal(dist, v["ball_sorted_dist"])
+    idx, dist = oracle.ball_query_sorted_partial(float(v["packed_radius"]), 10, v["packed_x"], v["packed_y"],
+                                                 v["packed_batch_x"], v["packed_batch_y"])
+    np.testing.assert_array_equal(idx, v["packed_sorted_idx"])
+    np.testing.assert_array_equal(dist, v["packed_sorted_dist"])
+    np.testing.assert_array_equal(oracle.furthest_point_sample(v["fps_xyz"], 64), v["fps_idx"])
+    np.testing.assert_array_equal(oracle.three_interpolate(v["interp_features"], v["interp_idx"].astype(np.int32), v["interp_weight"]),
+                                  v["interp_out"])
