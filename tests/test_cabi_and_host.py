@@ -64,7 +64,8 @@ def test_library_exports_every_declared_symbol():
     fn = lib.tpk_ball_query_sorted_dense_workspace_bytes
     fn.restype = ctypes.c_size_t
     cells = lambda n: -(-n // 64) if n <= 16384 else -(-n // 16384) * 256
-    support_only = lambda b, n: up(b * cells(n) * 1024) + up(b * cells(n) * 160)
+    # records (1024 B per cell of 64), cell boxes (160 B), boxes of runs of 16 cells (32 B)
+    support_only = lambda b, n: up(b * cells(n) * 1024) + up(b * cells(n) * 160) + up(b * -(-cells(n) // 16) * 32)
     assert fn(2, 100, 5000) == 0 and fn(0, 1000, 1000) == 0
     assert fn(2, 4096, 100) == support_only(2, 4096)
     assert fn(2, 200000, 1000) == support_only(2, 200000)

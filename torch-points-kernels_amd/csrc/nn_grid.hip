@@ -907,6 +907,7 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
 namespace {
 
 using u64 = unsigned long long;
+constexpr int NG_RUN = 16; // consecutive cells that share a second-level box in the wavefront-per-query search
 
 // The 64 keys of a wavefront sorted across its lanes (bitonic network; lane i ends with the i-th
 // smallest, or the i-th largest when `descending`).
@@ -956,7 +957,8 @@ __device__ __forceinline__ u64 read_lane_key(u64 key, int from)
 __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_sorted_wave_kernel(
     int64_t queries, int n, int ccells, int nsample, float limit, bool packed, int64_t index_add,
     const float* __restrict__ query, const float4* __restrict__ sorted_support,
-    const float4* __restrict__ boxes_support, float* __restrict__ dist, int64_t* __restrict__ idx)
+    const float4* __restrict__ boxes_support, const float4* __restrict__ run_boxes, float* __restrict__ dist,
+    int64_t* __restrict__ idx)
 {
     const int lane = threadIdx.x & (TPK_WAVE - 1);
     const int64_t q = static_cast<int64_t>(blockIdx.x) * (NG_SCAN_THREADS / TPK_WAVE) + threadIdx.x / TPK_WAVE;
@@ -971,30 +973,76 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_sorted_wave_kernel(
     u64 best = NONE;      // lane i: the i-th smallest key so far
     u64 admit = NONE;     // the nsample-th smallest: a candidate must beat it
     float reach = limit;  // squared distance beyond which a cell cannot help
-    for (int first = 0; first < ccells; first += NG_CELL)
+    // One cell offered to the list, one point per lane.
+    auto offer = [&](int cell) __attribute__((always_inline)) {
+        const float4 p = cpts[static_cast<int64_t>(cell) * NG_CELL + lane];
+        const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+        u64 cand = d < limit ? knn_key(d, __float_as_int(p.w)) : NONE;
+        cand = cand < admit ? cand : NONE;
+        if (__ballot(cand != NONE) == 0)
+            return;
+        cand = wave_sort_keys(cand, lane, true);
+        best = wave_merge_ascending(best < cand ? best : cand, lane);
+        admit = read_lane_key(best, nsample - 1);
+        if (admit != NONE)
+            reach = __int_as_float(static_cast<int>(admit >> 32));
+    };
+    if (run_boxes == nullptr)
     {
-        const int c = first + lane;
-        const bool valid = c < ccells;
-        const int cc = valid ? c : 0;
-        const float lb = point_box_dist2(qx, qy, qz, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
-        u64 live = __ballot(valid && lb * NG_MARGIN <= limit);
-        while (live != 0)
+        // few cells: the box of every cell is tested, one cell per lane
+        for (int first = 0; first < ccells; first += NG_CELL)
         {
-            const int bit = __builtin_ctzll(live);
-            live &= live - 1;
-            if (tpk_read_lane(lb, bit) * NG_MARGIN > reach)
-                continue; // the list has filled up with nearer points meanwhile
-            const float4 p = cpts[static_cast<int64_t>(first + bit) * NG_CELL + lane];
-            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-            u64 cand = d < limit ? knn_key(d, __float_as_int(p.w)) : NONE;
-            cand = cand < admit ? cand : NONE;
-            if (__ballot(cand != NONE) == 0)
-                continue;
-            cand = wave_sort_keys(cand, lane, true);
-            best = wave_merge_ascending(best < cand ? best : cand, lane);
-            admit = read_lane_key(best, nsample - 1);
-            if (admit != NONE)
-                reach = __int_as_float(static_cast<int>(admit >> 32));
+            const int c = first + lane;
+            const bool valid = c < ccells;
+            const int cc = valid ? c : 0;
+            const float lb = point_box_dist2(qx, qy, qz, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
+            u64 live = __ballot(valid && lb * NG_MARGIN <= reach);
+            while (live != 0)
+            {
+                const int bit = __builtin_ctzll(live);
+                live &= live - 1;
+                if (tpk_read_lane(lb, bit) * NG_MARGIN <= reach) // (the list may have filled up with nearer points)
+                    offer(first + bit);
+            }
+        }
+    }
+    else
+    {
+        // Two levels: the boxes of runs of 16 consecutive cells (neighbours on the curve, so compact), one run
+        // per lane; then the cells of up to four runs in reach, one cell per lane.
+        const int runs = (ccells + NG_RUN - 1) / NG_RUN;
+        const float4* __restrict__ rbox = run_boxes + cloud * runs * 2;
+        for (int first_run = 0; first_run < runs; first_run += NG_CELL)
+        {
+            const int r = first_run + lane;
+            const int rr = r < runs ? r : 0;
+            const float run_lb = point_box_dist2(qx, qy, qz, rbox[rr * 2 + 0], rbox[rr * 2 + 1]);
+            u64 live_runs = __ballot(r < runs && run_lb * NG_MARGIN <= reach);
+            while (live_runs != 0)
+            {
+                // the next four runs in reach: lanes 16 j .. 16 j + 15 take the cells of the j-th
+                int mine = -1;
+#pragma unroll
+                for (int j = 0; j < TPK_WAVE / NG_RUN; ++j)
+                {
+                    const int bit = live_runs != 0 ? __builtin_ctzll(live_runs) : -1;
+                    live_runs &= live_runs - 1; // (0 stays 0)
+                    mine = (lane / NG_RUN) == j ? bit : mine;
+                }
+                const int c = mine < 0 ? ccells : (first_run + mine) * NG_RUN + (lane % NG_RUN);
+                const bool valid = c < ccells;
+                const int cc = valid ? c : 0;
+                const float lb = point_box_dist2(qx, qy, qz, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
+                u64 live = __ballot(valid && lb * NG_MARGIN <= reach);
+                while (live != 0)
+                {
+                    const int bit = __builtin_ctzll(live);
+                    live &= live - 1;
+                    if (tpk_read_lane(lb, bit) * NG_MARGIN > reach)
+                        continue; // the list has filled up with nearer points meanwhile
+                    offer(__builtin_amdgcn_readlane(c, bit));
+                }
+            }
         }
     }
     if (lane < nsample)
@@ -1008,9 +1056,32 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_sorted_wave_kernel(
     }
 }
 
+// Box of every run of NG_RUN consecutive cells of a cloud: (lo, hi) as two float4.
+__global__ __launch_bounds__(NG_SCAN_THREADS) void run_boxes_kernel(int64_t total_runs, int runs, int ccells,
+                                                                    const float4* __restrict__ boxes,
+                                                                    float4* __restrict__ run_boxes)
+{
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * NG_SCAN_THREADS + threadIdx.x;
+    if (t >= total_runs)
+        return;
+    const int64_t cloud = t / runs;
+    const int r = static_cast<int>(t - cloud * runs);
+    const float4* __restrict__ cbox = boxes + cloud * ccells * NG_BOX;
+    const float inf = __builtin_inff();
+    float4 lo = make_float4(inf, inf, inf, 0.f), hi = make_float4(-inf, -inf, -inf, 0.f);
+    for (int c = r * NG_RUN; c < ccells && c < (r + 1) * NG_RUN; ++c)
+    {
+        const float4 a = cbox[c * NG_BOX + 0], b = cbox[c * NG_BOX + 1]; // (an empty cell: lo = +inf, hi = -inf)
+        lo = make_float4(fminf(lo.x, a.x), fminf(lo.y, a.y), fminf(lo.z, a.z), 0.f);
+        hi = make_float4(fmaxf(hi.x, b.x), fmaxf(hi.y, b.y), fmaxf(hi.z, b.z), 0.f);
+    }
+    run_boxes[t * 2 + 0] = lo;
+    run_boxes[t * 2 + 1] = hi;
+}
+
 struct SupportLayout
 {
-    size_t sorted, boxes, total;
+    size_t sorted, boxes, runs, total;
 };
 
 SupportLayout support_layout(int b, int m)
@@ -1020,7 +1091,8 @@ SupportLayout support_layout(int b, int m)
     SupportLayout l;
     l.sorted = 0;
     l.boxes = up(static_cast<size_t>(b) * cells * NG_CELL * sizeof(float4));
-    l.total = l.boxes + up(static_cast<size_t>(b) * cells * NG_BOX * sizeof(float4));
+    l.runs = l.boxes + up(static_cast<size_t>(b) * cells * NG_BOX * sizeof(float4));
+    l.total = l.runs + up(static_cast<size_t>(b) * ((cells + NG_RUN - 1) / NG_RUN) * 2 * sizeof(float4));
     return l;
 }
 
@@ -1054,12 +1126,24 @@ int tpk_grid_ball_sorted(int b, int n, int m, int nsample, float limit, bool pac
     int st = launch_curve_cells(none, c, nullptr, s);
     if (st != TPK_OK)
         return st;
+    const int ccells = grid_cells(m), runs = (ccells + NG_RUN - 1) / NG_RUN;
+    // second-level boxes pay from a few groups of 64 cells on
+    float4* run_boxes = ccells > 4 * NG_CELL ? reinterpret_cast<float4*>(w + l.runs) : nullptr;
+    if (run_boxes)
+    {
+        const int64_t total_runs = static_cast<int64_t>(b) * runs;
+        hipLaunchKernelGGL(run_boxes_kernel, dim3(static_cast<unsigned>(tpk_ceil_div(total_runs, NG_SCAN_THREADS))),
+                           dim3(NG_SCAN_THREADS), 0, s, total_runs, runs, ccells, c.boxes, run_boxes);
+        st = tpk_launch_status();
+        if (st != TPK_OK)
+            return st;
+    }
     const int64_t queries = static_cast<int64_t>(b) * n;
     const int64_t blocks = tpk_ceil_div(queries, NG_SCAN_THREADS / TPK_WAVE);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(ball_sorted_wave_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, queries,
-                       n, grid_cells(m), nsample, limit, packed, index_add, query, c.sorted, c.boxes, dist, idx);
+                       n, ccells, nsample, limit, packed, index_add, query, c.sorted, c.boxes, run_boxes, dist, idx);
     return tpk_launch_status();
 }
 
