@@ -31,6 +31,7 @@ extern "C" {
 #define TPK_ERR_INVALID_ARG (-1) /* negative size, NULL pointer with non-empty data, ... */
 #define TPK_ERR_UNSUPPORTED (-2) /* valid request outside what the kernels cover */
 #define TPK_ERR_WORKSPACE (-3)   /* workspace missing or too small */
+#define TPK_ERR_TOO_LARGE (-4)   /* problem needs more scratch memory than the library's fixed array holds */
 
 /* Library version, major*10000 + minor*100 + patch. */
 int tpk_version(void);
@@ -136,6 +137,24 @@ size_t tpk_three_nn_workspace_bytes(int b, int n, int m);
 int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* known,
                      float* dist2, int32_t* idx, void* workspace, size_t workspace_bytes,
                      void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Three nearest neighbours without any allocation.
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory (not
+ * even a workspace to pass in): code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  Same arguments and results as tpk_three_nn_f32 with a workspace, but
+ * the curve-ordered copies of both clouds live in an array of
+ * TPK_THREE_NN_STATIC_SCRATCH_BYTES bytes of device memory that is part of the library (every GPU
+ * the library runs on holds one until the process ends).  The call allocates and frees nothing.
+ * Shapes whose workspace (tpk_three_nn_workspace_bytes()) exceeds the array are rejected with
+ * TPK_ERR_TOO_LARGE before anything is launched; shapes that need no workspace run the all
+ * pairs scan.  All calls on one GPU share that GPU's array: calls that overlap there (different
+ * streams or host threads) race; calls on one stream are safe.
+ * ------------------------------------------------------------------------------------- */
+#define TPK_THREE_NN_STATIC_SCRATCH_BYTES (8u << 20)
+size_t tpk_three_nn_static_scratch_bytes(void);
+int tpk_three_nn_static_f32(int b, int n, int m, const float* unknown, const float* known,
+                            float* dist2, int32_t* idx, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * k nearest neighbours, dense layout.

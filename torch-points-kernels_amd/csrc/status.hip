@@ -18,6 +18,8 @@ extern "C" const char* tpk_status_string(int status)
         return "size outside the supported range";
     case TPK_ERR_WORKSPACE:
         return "workspace missing or too small";
+    case TPK_ERR_TOO_LARGE:
+        return "problem needs more scratch memory than the library's fixed array holds";
     default:
         break;
     }

@@ -14,6 +14,8 @@
 // to +inf select identically and store identical values.
 #include "nn_grid.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int NN_THREADS = 256;
@@ -162,4 +164,72 @@ extern "C" int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const
     if (queries >= 2LL * NN_THREADS * 2048)
         return launch_three_nn<2>(b, n, m, unknown, known, dist2, idx, s);
     return launch_three_nn<1>(b, n, m, unknown, known, dist2, idx, s);
+}
+
+// ---------------------------------------------------------------------------------------------
+// three_nn for callers that may not allocate device memory (code under graph capture, serving
+// loops, harnesses that forbid it).  The curve-ordered copy of both clouds and the cell boxes,
+// which tpk_three_nn_f32 takes as a caller-provided workspace, live in a fixed array in device
+// memory instead.  Every GPU the library runs on holds its own copy of the array at its own
+// address until the process ends; that address is looked up once per device, with that device
+// current, and host code uses the looked-up pointer only (the array's name is not a device
+// address on the host).  The search overwrites whatever an earlier call left there (nothing has
+// to start at zero), so calls that overlap on one GPU - on different streams or from different
+// threads - race on it.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+constexpr size_t THREE_NN_STATIC_BYTES = TPK_THREE_NN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[THREE_NN_STATIC_BYTES];
+
+constexpr int SCRATCH_MAX_DEVICES = 64;
+std::mutex scratch_lock;
+void* scratch_address[SCRATCH_MAX_DEVICES]; // per device, filled at the first call on that device
+
+// Device address of `scratch` on the current device (looked up once per device).
+int static_scratch(void** out)
+{
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    if (device < 0 || device >= SCRATCH_MAX_DEVICES)
+        return TPK_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_address[device])
+    {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess)
+            return static_cast<int>(e);
+        if (!p || (reinterpret_cast<uintptr_t>(p) & 255u))
+            return TPK_ERR_WORKSPACE;
+        scratch_address[device] = p;
+    }
+    *out = scratch_address[device];
+    return TPK_OK;
+}
+
+} // namespace
+
+extern "C" size_t tpk_three_nn_static_scratch_bytes(void)
+{
+    return THREE_NN_STATIC_BYTES;
+}
+
+extern "C" int tpk_three_nn_static_f32(int b, int n, int m, const float* unknown, const float* known,
+                                       float* dist2, int32_t* idx, void* stream)
+{
+    if (b < 0 || n < 0 || m < 0)
+        return TPK_ERR_INVALID_ARG;
+    const size_t need = tpk_grid_three_nn_workspace_bytes(b, n, m);
+    if (need > THREE_NN_STATIC_BYTES)
+        return TPK_ERR_TOO_LARGE;
+    if (need == 0) // shapes the cell search does not serve use no scratch memory at all
+        return tpk_three_nn_f32(b, n, m, unknown, known, dist2, idx, nullptr, 0, stream);
+    void* ptr = nullptr;
+    const int st = static_scratch(&ptr);
+    if (st != TPK_OK)
+        return st;
+    return tpk_three_nn_f32(b, n, m, unknown, known, dist2, idx, ptr, THREE_NN_STATIC_BYTES, stream);
 }
