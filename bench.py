@@ -30,22 +30,88 @@ for _p in (ROOT, os.path.join(ROOT, "torch-points-kernels_amd")):
 PEAK_HBM_GBS = 8000.0
 PEAK_FP32_TFLOPS = 157.3  # published fp32 figure (vector = matrix); it counts every lane-op as an FMA (2 flop)
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE run + WRITE_SIZE run, each
-# scaled by the same counter's reading for a 256 MiB device copy); see profiles/*pmc*.txt.
-# None = not measured yet.
-MEASURED_TRAFFIC_BYTES = {
-    "fps": 4030000,                    # 3.76 MB read (the clouds; set-up passes mostly hit L2) + 0.26 MB written (the indices)
-    "three_interpolate_fwd": 174130000,  # = algorithmic bytes: nothing is read twice from HBM
-    "three_interpolate_bwd": 308500000,  # list build 57 MB + list walk 252 MB (two column pieces per four rows)
-    "grouping_fwd": 352500000,         # rows staged twice (two column halves per row block)
-    "grouping_bwd": 407900000,         # list build 27 MB + walk 381 MB (two column pieces per row: outputs written twice)
-    "chamfer_bwd": 128000000,          # list build 72.4 MB (padded lists) + list walk 55.6 MB
-    "gridding_fwd": 60400000,          # 1.6 MB read + 25.3 MB written + the grid's zero fill 33.5 MB
-    "gridding_bwd": 41500000,          # the eight gathered gradients of a point lie in eight lines
-    "cubic_fwd": 172800000,            # index kernel 2.9 MB + gather 35.7 MB read (the feature maps once) + 134.2 MB written
-    "cubic_bwd": 170800000,            # 136.4 MB read + 33.6 MB written + the zero fill of the points' gradient
-    "instance_iou": 13400000,
+PROFILES = os.path.join(ROOT, "profiles")
+TRAFFIC_FILE = os.path.join(PROFILES, "all_ops_baseline_configs_hbm_traffic.txt")
+VALU_FILE = os.path.join(PROFILES, "distance_scans_valu_utilisation.txt")
+
+# Kernels whose HBM traffic adds up to one launch of an operator (names as rocprofv3 prints them).
+TRAFFIC_KERNELS = {
+    "fps": ["fps_pruned_kernel<32, 512, 4>"],
+    "three_interpolate_fwd": ["gather_fwd_lds_kernel<3, true, int, true>"],
+    "three_interpolate_bwd": ["build_lists_kernel<3, true, int>", "gather_bwd_lists_kernel<3, true, 4>"],
+    "grouping_fwd": ["gather_fwd_lds_kernel<1, false, long, false>"],
+    "grouping_bwd": ["build_lists_kernel<1, false, long>", "gather_bwd_lists_kernel<1, false, 1>"],
+    "chamfer_bwd": ["build_lists_kernel<1, false, int>", "chamfer_bwd_lists_kernel<float>"],
 }
+# Kernels whose VALU counters describe a distance scan.
+VALU_KERNELS = {
+    "fps": "fps_pruned_kernel<32, 512, 4>",
+    "ball_query_dense": "ball_query_dense_kernel",
+    "ball_query_partial_dense": "ball_query_bins_kernel",
+    "three_nn": "three_nn_grid_kernel",
+    "chamfer_fwd": "chamfer_grid_kernel",
+}
+
+
+def _profile_table(path, columns):
+    """Rows 'kernel name  n= k  COUNTER value ...' of a summary under profiles/ -> {kernel: {COUNTER: value}},
+    plus the commit the summary says it was measured at."""
+    import re
+
+    table, commit = {}, None
+    if not os.path.exists(path):
+        return table, commit
+    for line in open(path):
+        m = re.match(r"Measured at commit\s+(\S+)", line)
+        if m:
+            commit = m.group(1)
+        m = re.match(r"(\S.*?)\s+n=\s*(\d+)\s+(.*)$", line)
+        if not m:
+            continue
+        vals = {}
+        for name in columns:
+            v = re.search(r"\b%s\s+([0-9.eE+-]+)" % re.escape(name), m.group(3))
+            if v:
+                vals[name] = float(v.group(1))
+        if vals:
+            table[m.group(1).strip()] = vals
+    return table, commit
+
+
+_TRAFFIC_TABLE = None
+
+
+def _measured_traffic(key):
+    """HBM bytes per launch of operator `key`: 2 x FETCH_SIZE + WRITE_SIZE (KiB, factors from the copy
+    kernel of known size in the same runs) summed over the operator's kernels, read from the tracked
+    rocprofv3 summary, with the commit it was measured at.  (None, None) when the summary lacks a kernel:
+    a renamed or re-shaped kernel thus drops its figure instead of keeping a stale one."""
+    global _TRAFFIC_TABLE
+    if _TRAFFIC_TABLE is None:
+        _TRAFFIC_TABLE = _profile_table(TRAFFIC_FILE, ("FETCH_SIZE", "WRITE_SIZE"))
+    table, commit = _TRAFFIC_TABLE
+    total = 0.0
+    for kernel in TRAFFIC_KERNELS.get(key, []):
+        row = table.get(kernel)
+        if row is None or "FETCH_SIZE" not in row or "WRITE_SIZE" not in row:
+            return None, commit
+        total += (2.0 * row["FETCH_SIZE"] + row["WRITE_SIZE"]) * 1024.0
+    return (total if key in TRAFFIC_KERNELS else None), commit
+
+
+_VALU_TABLE = None
+
+
+def _measured_valu(key):
+    global _VALU_TABLE
+    if _VALU_TABLE is None:
+        _VALU_TABLE = _profile_table(VALU_FILE, ("VALUBusy", "VALUUtilization", "SQ_INSTS_VALU"))
+    table, commit = _VALU_TABLE
+    row = table.get(VALU_KERNELS.get(key, ""))
+    if row is None:
+        return None
+    return {"valu_busy_pct": row.get("VALUBusy"), "valu_lane_utilisation_pct": row.get("VALUUtilization"),
+            "source": "profiles/" + os.path.basename(VALU_FILE), "measured_at_commit": commit}
 
 
 def _time_gpu(fn, steps, warmup):
@@ -68,24 +134,134 @@ def _time_gpu(fn, steps, warmup):
     return wall, ev
 
 
-def _roof_flops(pairs_or_updates, flops_each, ms):
-    achieved = pairs_or_updates * flops_each / (ms * 1e-3) / 1e12
-    return {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / PEAK_FP32_TFLOPS, "traffic": None,
-            "note": "fp32 VALU kernel (inner dimension 3, unfused arithmetic: no MFMA, no FMA, no packed "
-                    "fp32); peak is the published fp32 figure, which assumes FMA: without FMA the ceiling is 0.5"}
+def _roof_flops(executed, algorithmic, flops_each, ms, key=None):
+    """Roofline object of a distance scan.  `executed` = pair evaluations (or point updates) the kernels
+    performed, counted by the counting build of the library in a run outside the timed region;
+    `algorithmic` = what a brute-force scan - the reference - performs.  achieved / frac use EXECUTED work,
+    so frac <= 1; the algorithmic rate is reported beside it."""
+    achieved = executed * flops_each / (ms * 1e-3) / 1e12
+    algorithmic_rate = algorithmic * flops_each / (ms * 1e-3) / 1e12
+    r = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+         "frac": achieved / PEAK_FP32_TFLOPS, "traffic": None,
+         "executed_pairs": executed, "algorithmic_pairs": algorithmic,
+         "algorithmic_rate": algorithmic_rate, "algorithmic_speedup": algorithmic / max(executed, 1),
+         "note": "fp32 VALU kernel (inner dimension 3, unfused arithmetic: no MFMA, no FMA, no packed fp32); peak is the "
+                 "published fp32 figure, which assumes FMA: without FMA the ceiling is 0.5. achieved = executed pair "
+                 "evaluations (counted on device by libtpk_hip_counting.so, one count per lane and distance, padding "
+                 "lanes included) x %d flop / kernel time; algorithmic_rate = the pairs a brute-force scan tests "
+                 "(what the reference evaluates) x %d flop / the same time; algorithmic_speedup = their ratio" %
+                 (flops_each, flops_each)}
+    valu = _measured_valu(key) if key else None
+    if valu:
+        r["valu"] = valu
+    return r
 
 
-PRUNED_NOTE = ("; algorithmic work = all pairs (8 flop each), which is what the reference evaluates; the kernel "
-               "orders both clouds along a space filling curve and skips cells that provably hold no answer, so "
-               "the achieved figure is a rate of algorithmic, not executed, flops and may exceed the peak; "
-               "kernel_ms covers the ordering kernel and the search kernel")
+PRUNED_NOTE = ("; the kernel orders the clouds along a space filling curve and skips cells that provably hold no "
+               "answer; kernel_ms covers the ordering kernel and the search kernel")
 
 
 def _roof_bytes(nbytes, ms, key):
     achieved = nbytes / (ms * 1e-3) / 1e9
-    return {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(key)}
+    traffic, commit = _measured_traffic(key)
+    r = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+         "frac": achieved / PEAK_HBM_GBS, "traffic": traffic}
+    if traffic is not None:
+        r["traffic_source"] = "profiles/" + os.path.basename(TRAFFIC_FILE)
+        r["traffic_measured_at_commit"] = commit
+    return r
+
+
+# ---- executed work: the same call made once through the counting build of the library (ctypes on the
+# C ABI, PyTorch's current stream), outside every timed region
+_COUNTING = None
+
+
+def _counting_lib():
+    global _COUNTING
+    if _COUNTING is None:
+        import ctypes
+
+        path = os.path.join(ROOT, "torch-points-kernels_amd", "torch_points_kernels", "libtpk_hip_counting.so")
+        if not os.path.exists(path):
+            sys.exit("bench.py: %s is not built (run torch-points-kernels_amd/build.py)" % path)
+        lib = ctypes.CDLL(path)
+        for name in ("tpk_fps_workspace_bytes", "tpk_ball_query_partial_workspace_bytes", "tpk_three_nn_workspace_bytes",
+                     "tpk_chamfer_fwd_workspace_bytes", "tpk_knn_workspace_bytes",
+                     "tpk_ball_query_sorted_dense_workspace_bytes", "tpk_ball_query_sorted_partial_workspace_bytes"):
+            getattr(lib, name).restype = ctypes.c_size_t
+        _COUNTING = lib
+    return _COUNTING
+
+
+_SHIPPING = None
+
+
+def _shipping_lib():
+    """The shipping library through ctypes: for calls the extension never makes (workspace == NULL, which
+    selects the brute-force scans)."""
+    global _SHIPPING
+    if _SHIPPING is None:
+        import ctypes
+
+        _SHIPPING = ctypes.CDLL(os.path.join(ROOT, "torch-points-kernels_amd", "torch_points_kernels", "libtpk_hip.so"))
+    return _SHIPPING
+
+
+def _all_pairs_entry(call, pairs, steps, warmup, valu_kernel):
+    """Times call(lib, stream) made without workspace (brute-force scan) and counts its executed pairs."""
+    import ctypes
+
+    import torch
+
+    lib = _shipping_lib()
+
+    def run():
+        st = call(lib, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert st == 0
+
+    wall, ev = _time_gpu(run, steps, warmup)
+    executed = _executed(call)
+    roof = _roof_flops(executed, pairs, 8, ev)
+    table, commit = _profile_table(VALU_FILE, ("VALUBusy", "VALUUtilization"))
+    if valu_kernel in table:
+        roof["valu"] = {"valu_busy_pct": table[valu_kernel].get("VALUBusy"),
+                        "valu_lane_utilisation_pct": table[valu_kernel].get("VALUUtilization"),
+                        "source": "profiles/" + os.path.basename(VALU_FILE), "measured_at_commit": commit}
+    return {"what": "the same configuration through the C ABI with workspace == NULL: every query scans its whole cloud "
+                    "(the kernel the north star describes); same results", "kernel_ms": ev, "wall_ms": wall, "roofline": roof}
+
+
+COUNT_WORK = True  # --no-count: leave the counting build out (profiler runs: its kernels carry the same names)
+
+
+def _executed(call):
+    """Pair evaluations executed by call(lib, stream) -> status."""
+    import ctypes
+
+    import torch
+
+    if not COUNT_WORK:
+        return 0
+    lib = _counting_lib()
+    n = ctypes.c_ulonglong(0)
+    assert lib.tpk_work_read_reset(ctypes.byref(n)) == 0
+    st = call(lib, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0, "counting call failed with status %d" % st
+    assert lib.tpk_work_read_reset(ctypes.byref(n)) == 0
+    return int(n.value)
+
+
+def _p(t):
+    import ctypes
+
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _ws(nbytes, dev):
+    import torch
+
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=dev)
 
 
 def _cpu_time(fn, repeat=1):
@@ -99,6 +275,8 @@ def _cpu_time(fn, repeat=1):
 
 
 def bench_fps(dev, steps, warmup, with_cpu):
+    import ctypes
+
     import torch
 
     import torch_points_kernels as tpk
@@ -109,13 +287,19 @@ def bench_fps(dev, steps, warmup, with_cpu):
     npoint = w["npoint"]
     wall, ev = _time_gpu(lambda: tpk.furthest_point_sample(xyz, npoint), steps, warmup)
     updates = W.fps_point_updates()
-    roof = _roof_flops(updates, 10, ev)
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get("fps")
-    roof["note"] += "; algorithmic work = every point updated in every round (10 flop each), as the reference " \
-                    "does; the kernel skips updates it proves to be no-ops, so the achieved figure is a rate of " \
-                    "algorithmic, not executed, flops; the rounds of a cloud are sequential and one workgroup " \
-                    "owns a cloud: 16 of 256 compute units are occupied by design, fraction of those 16 CUs' " \
-                    "peak = %.4f" % (roof["frac"] * 256 / 16)
+    out_idx = torch.empty(xyz.shape[0], npoint, dtype=torch.int32, device=dev)
+    executed = _executed(lambda lib, st: lib.tpk_fps_f32(xyz.shape[0], xyz.shape[1], npoint, _p(xyz), None,
+                                                         ctypes.c_size_t(0), _p(out_idx), st))
+    roof = _roof_flops(executed, updates, 10, ev, "fps")
+    roof["traffic"], commit = _measured_traffic("fps")
+    if roof["traffic"] is not None:
+        roof["traffic_source"] = "profiles/" + os.path.basename(TRAFFIC_FILE)
+        roof["traffic_measured_at_commit"] = commit
+    roof["note"] += "; here a pair = one running minimum updated (10 flop: 8 for the distance, min, max); algorithmic " \
+                    "work = every point updated in every round, as the reference does; the kernel skips updates it " \
+                    "proves to be no-ops; the rounds of a cloud are sequential and one workgroup owns a cloud: 16 of 256 " \
+                    "compute units are occupied by design, executed fraction of those 16 CUs' peak = %.4f, " \
+                    "algorithmic %.4f" % (roof["frac"] * 256 / 16, roof["algorithmic_rate"] / PEAK_FP32_TFLOPS * 256 / 16)
     res = {"wall_ms": wall, "kernel_ms": ev, "roofline": roof, "point_updates": updates}
     if with_cpu:
         import oracle
@@ -137,6 +321,8 @@ def bench_fps(dev, steps, warmup, with_cpu):
 
 
 def bench_others(dev, steps, warmup, with_cpu):
+    import ctypes
+
     import torch
 
     import torch_points_kernels as tpk
@@ -157,9 +343,14 @@ def bench_others(dev, steps, warmup, with_cpu):
     wall, ev = _time_gpu(lambda: tpk.ball_query(w["radius"], w["nsample"], xyz, new_xyz, mode="dense"), steps, warmup)
     nq = new_xyz.shape[0] * new_xyz.shape[1]
     pairs = nq * xyz.shape[1]
+    bq_idx = torch.empty(new_xyz.shape[0], new_xyz.shape[1], w["nsample"], dtype=torch.int64, device=dev)
+    bq_dist = torch.empty(new_xyz.shape[0], new_xyz.shape[1], w["nsample"], device=dev)
+    executed = _executed(lambda lib, st: lib.tpk_ball_query_dense_f32(
+        xyz.shape[0], xyz.shape[1], new_xyz.shape[1], ctypes.c_float(w["radius"]), w["nsample"], _p(new_xyz), _p(xyz),
+        _p(bq_idx), _p(bq_dist), st))
     e = {"workload": "configs[0]: ball_query dense B=8 N=4096 M=1024 r=0.1 nsample=32", "metric": "queries/s",
          "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
-         "roofline": _roof_flops(pairs, 8, ev), "pairs_upper_bound": pairs}
+         "roofline": _roof_flops(executed, pairs, 8, ev, "ball_query_dense"), "pairs_upper_bound": pairs}
     if ref is not None:
         secs = _cpu_time(lambda: ref.dense_ball_query(w["new_xyz"], w["xyz"], w["radius"], w["nsample"], 0, False))
         e["cpu_baseline"] = {"value": nq / secs, "unit": "queries/s", "cores": 1, "kind": "reference",
@@ -171,8 +362,7 @@ def bench_others(dev, steps, warmup, with_cpu):
     wall, ev = _time_gpu(lambda: tpk.ball_query(w["radius"], w["nsample"], xyz, new_xyz, mode="dense", sort=True), steps, warmup)
     e = {"workload": "ball_query dense sort=True on configs[0] (B=8 N=4096 M=1024 r=0.1 nsample=32; the reference has this "
                      "mode for CPU tensors only)", "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev,
-         "wall_ms": wall, "roofline": _roof_flops(pairs, 8, ev), "pairs": pairs}
-    e["roofline"]["note"] += PRUNED_NOTE
+         "wall_ms": wall, "pairs": pairs, "algorithmic_rate_tflops": pairs * 8 / (ev * 1e-3) / 1e12}
     if ref is not None:
         secs = _cpu_time(lambda: ref.dense_ball_query(w["new_xyz"], w["xyz"], w["radius"], w["nsample"], 0, True))
         e["cpu_baseline"] = {"value": nq / secs, "unit": "queries/s", "cores": 1, "kind": "reference",
@@ -188,10 +378,21 @@ def bench_others(dev, steps, warmup, with_cpu):
     sizes = torch.bincount(w["batch_x"]).tolist()
     qsizes = torch.bincount(w["batch_y"]).tolist()
     pairs = sum(a * b for a, b in zip(sizes, qsizes))
+    bq_idx = torch.empty(nq, w["nsample"], dtype=torch.int64, device=dev)
+    bq_dist = torch.empty(nq, w["nsample"], device=dev)
+    ws_bytes = _counting_lib().tpk_ball_query_partial_workspace_bytes(ctypes.c_int64(x.shape[0]), ctypes.c_int64(nq),
+                                                                      w["nsample"])
+    ws = _ws(ws_bytes, dev)
+    executed = _executed(lambda lib, st: lib.tpk_ball_query_partial_f32(
+        ctypes.c_int64(x.shape[0]), ctypes.c_int64(nq), ctypes.c_float(w["radius"]), w["nsample"], _p(x), _p(y), _p(bx),
+        _p(by), _p(bq_idx), _p(bq_dist), _p(ws) if ws_bytes else None, ctypes.c_size_t(ws_bytes), st))
     e = {"workload": "configs[3]: ball_query partial_dense clouds 20k/45k/70k/100k, 25% queries, r=0.05 nsample=64",
          "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
-         "roofline": _roof_flops(pairs, 8, ev), "pairs_upper_bound": pairs}
+         "roofline": _roof_flops(executed, pairs, 8, ev, "ball_query_partial_dense"), "pairs_upper_bound": pairs}
     e["roofline"]["note"] += PRUNED_NOTE
+    e["all_pairs_kernel"] = _all_pairs_entry(lambda lib, st: lib.tpk_ball_query_partial_f32(
+        ctypes.c_int64(x.shape[0]), ctypes.c_int64(nq), ctypes.c_float(w["radius"]), w["nsample"], _p(x), _p(y), _p(bx),
+        _p(by), _p(bq_idx), _p(bq_dist), None, ctypes.c_size_t(0), st), pairs, max(3, steps // 4), 1, "ball_query_partial_kernel")
     if ref is not None:
         secs = _cpu_time(lambda: ref.batch_ball_query(w["x"], w["y"], w["batch_x"], w["batch_y"], w["radius"],
                                                       w["nsample"], 0, False))
@@ -202,8 +403,8 @@ def bench_others(dev, steps, warmup, with_cpu):
                                                 sort=True), max(3, steps // 4), 1)
     e = {"workload": "ball_query partial_dense sort=True on configs[3] (the reference has this mode for CPU tensors only)",
          "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
-         "roofline": _roof_flops(pairs, 8, ev), "pairs": pairs}
-    e["roofline"]["note"] += PRUNED_NOTE + "; the clouds are searched one after the other, after one wait for the stream"
+         "pairs": pairs, "algorithmic_rate_tflops": pairs * 8 / (ev * 1e-3) / 1e12,
+         "note": "the clouds are searched one after the other, after one wait for the stream"}
     if ref is not None:
         secs = _cpu_time(lambda: ref.batch_ball_query(w["x"], w["y"], w["batch_x"], w["batch_y"], w["radius"],
                                                       w["nsample"], 0, True))
@@ -217,10 +418,20 @@ def bench_others(dev, steps, warmup, with_cpu):
     wall, ev = _time_gpu(lambda: nat.three_nn(unknown, known), steps, warmup)
     nq = unknown.shape[0] * unknown.shape[1]
     pairs = W.pairs_three_nn()
+    nn_d = torch.empty(unknown.shape[0], unknown.shape[1], 3, device=dev)
+    nn_i = torch.empty(unknown.shape[0], unknown.shape[1], 3, dtype=torch.int32, device=dev)
+    ws_bytes = _counting_lib().tpk_three_nn_workspace_bytes(unknown.shape[0], unknown.shape[1], known.shape[1])
+    ws = _ws(ws_bytes, dev)
+    executed = _executed(lambda lib, st: lib.tpk_three_nn_f32(
+        unknown.shape[0], unknown.shape[1], known.shape[1], _p(unknown), _p(known), _p(nn_d), _p(nn_i),
+        _p(ws) if ws_bytes else None, ctypes.c_size_t(ws_bytes), st))
     e = {"workload": "configs[2]a: three_nn unknown (16,16384,3) known (16,4096,3)", "metric": "queries/s",
-         "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall, "roofline": _roof_flops(pairs, 8, ev),
-         "pairs": pairs}
+         "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
+         "roofline": _roof_flops(executed, pairs, 8, ev, "three_nn"), "pairs": pairs}
     e["roofline"]["note"] += PRUNED_NOTE
+    e["all_pairs_kernel"] = _all_pairs_entry(lambda lib, st: lib.tpk_three_nn_f32(
+        unknown.shape[0], unknown.shape[1], known.shape[1], _p(unknown), _p(known), _p(nn_d), _p(nn_i), None,
+        ctypes.c_size_t(0), st), pairs, max(3, steps // 4), 1, "three_nn_kernel<4>")
     if ref is not None:
         sub = 4  # clouds
         secs = _cpu_time(lambda: ref.dense_knn(w["known"][:sub], w["unknown"][:sub], 3))
@@ -234,8 +445,7 @@ def bench_others(dev, steps, warmup, with_cpu):
     wall, ev = _time_gpu(lambda: nat.dense_knn(known, unknown, knn_k), steps, warmup)
     e = {"workload": "dense knn k=16, queries (16,16384,3), support (16,4096,3) (clouds of configs[2]a; not a BASELINE configuration)",
          "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
-         "roofline": _roof_flops(pairs, 8, ev), "pairs": pairs}
-    e["roofline"]["note"] += PRUNED_NOTE
+         "pairs": pairs, "algorithmic_rate_tflops": pairs * 8 / (ev * 1e-3) / 1e12}
     if ref is not None:
         sub = 4  # clouds
         secs = _cpu_time(lambda: ref.dense_knn(w["known"][:sub], w["unknown"][:sub], knn_k))
@@ -412,10 +622,22 @@ def bench_others(dev, steps, warmup, with_cpu):
     csteps = max(3, steps // 4)
     wall, ev = _time_gpu(lambda: nat.chamfer_dist(a, b), csteps, min(warmup, 2))
     pairs = W.pairs_chamfer()
+    cb, cn, cm = a.shape[0], a.shape[1], b.shape[1]
+    cd1, cd2 = torch.empty(cb, cn, device=dev), torch.empty(cb, cm, device=dev)
+    ci1 = torch.empty(cb, cn, dtype=torch.int32, device=dev)
+    ci2 = torch.empty(cb, cm, dtype=torch.int32, device=dev)
+    ws_bytes = _counting_lib().tpk_chamfer_fwd_workspace_bytes(cb, cn, cm)
+    ws = _ws(ws_bytes, dev)
+    executed = _executed(lambda lib, st: lib.tpk_chamfer_fwd_f32(
+        cb, cn, cm, _p(a), _p(b), _p(cd1), _p(cd2), _p(ci1), _p(ci2), _p(ws) if ws_bytes else None,
+        ctypes.c_size_t(ws_bytes), st))
     e = {"workload": "configs[4]: Chamfer forward B=32 16384x16384 (both directions)", "metric": "pairs/s",
-         "value": pairs / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall, "roofline": _roof_flops(pairs, 8, ev),
-         "pairs": pairs}
+         "value": pairs / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
+         "roofline": _roof_flops(executed, pairs, 8, ev, "chamfer_fwd"), "pairs": pairs}
     e["roofline"]["note"] += PRUNED_NOTE
+    e["all_pairs_kernel"] = _all_pairs_entry(lambda lib, st: lib.tpk_chamfer_fwd_f32(
+        cb, cn, cm, _p(a), _p(b), _p(cd1), _p(cd2), _p(ci1), _p(ci2), None, ctypes.c_size_t(0), st), pairs, 3, 1,
+        "chamfer_fwd_kernel<float, 4>")
     if with_cpu:
         import oracle
 
@@ -442,7 +664,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--ops", choices=["all", "headline"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-count", action="store_true",
+                    help="skip the runs through the counting build of the library (executed work is then reported as 0); "
+                         "for profiler runs, whose per-kernel averages those launches would enter")
     args = ap.parse_args()
+    global COUNT_WORK
+    COUNT_WORK = not args.no_count
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this library runs on ONE GPU (every operator is independent per cloud; nothing is "
                  "exchanged between GPUs), so only --gpus 1 is measured.")

@@ -33,6 +33,19 @@ def test_header_declares_the_expected_entry_points():
         assert want in names
 
 
+def test_counting_build_exports_the_same_abi_plus_its_reader():
+    """libtpk_hip_counting.so (measurement only) carries the whole C ABI and tpk_work_read_reset; the
+    shipping library carries no counter."""
+    path = LIB.replace("libtpk_hip.so", "libtpk_hip_counting.so")
+    assert os.path.exists(path), "libtpk_hip_counting.so is not built (run torch-points-kernels_amd/build.py)"
+    lib = ctypes.CDLL(path)
+    for name in _declared_symbols() + ["tpk_work_read_reset"]:
+        assert hasattr(lib, name), name
+    assert not hasattr(ctypes.CDLL(LIB), "tpk_work_read_reset")
+    text = open(os.path.join(ROOT, "include", "tpk_counting.h")).read()
+    assert "tpk_work_read_reset" in text
+
+
 def test_library_exports_every_declared_symbol():
     assert os.path.exists(LIB), "libtpk_hip.so is not built (run torch-points-kernels_amd/build.py)"
     lib = ctypes.CDLL(LIB)

@@ -2,6 +2,10 @@
 
   csrc/*.hip          -> torch_points_kernels/libtpk_hip.so   (HIP kernels + C ABI, no torch)
   csrc/points_cuda.cpp -> torch_points_kernels/points_cuda.so  (pybind11 module over the C ABI)
+  csrc/*.hip          -> torch_points_kernels/libtpk_hip_counting.so: the same library with the
+                         distance scans compiled -DTPK_COUNT_WORK (they count the pair
+                         evaluations they execute; include/tpk_counting.h).  Measurement only:
+                         the package never loads it.
 
 Run as ``python build.py`` (add ``--force`` to rebuild everything).  hipcc cross-compiles, so
 no GPU is needed to build.
@@ -50,24 +54,39 @@ def _run(cmd):
     return out
 
 
+# Translation units that hold distance scans (and the counters' reader): compiled a second time
+# with -DTPK_COUNT_WORK for the counting library; the other objects are shared.
+COUNTING_UNITS = ("status", "ball_query", "three_nn", "chamfer", "nn_grid", "fps")
+
+
 def build_kernels(force=False):
     os.makedirs(OBJ, exist_ok=True)
     headers = glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(INCLUDE, "*.h"))
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     lib = os.path.join(PKG, "libtpk_hip.so")
+    counting_lib = os.path.join(PKG, "libtpk_hip_counting.so")
     jobs = []
     objs = []
+    counting_objs = []
     for src in sources:
-        obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+        unit = os.path.basename(src)[:-4]
+        obj = os.path.join(OBJ, unit + ".o")
         objs.append(obj)
         if force or not _newer(obj, [src] + headers):
             jobs.append([HIPCC] + HIP_FLAGS + ["-c", src, "-o", obj])
+        if unit in COUNTING_UNITS:
+            obj = os.path.join(OBJ, unit + ".counting.o")
+            if force or not _newer(obj, [src] + headers):
+                jobs.append([HIPCC] + HIP_FLAGS + ["-DTPK_COUNT_WORK", "-c", src, "-o", obj])
+        counting_objs.append(obj)
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         for out in ex.map(_run, jobs):
             if out.strip():
                 print(out)
     if force or jobs or not _newer(lib, objs):
         _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs)
+    if force or jobs or not _newer(counting_lib, counting_objs):
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", counting_lib] + counting_objs)
     return lib
 
 

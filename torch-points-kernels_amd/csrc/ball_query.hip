@@ -64,6 +64,7 @@ __device__ __forceinline__ void scan_run(Tile& tile, const float* __restrict__ s
 {
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
+    TPK_WORK_DECL
 
     float r2q[BQ_Q];   // radius of a live query, -1 once it is finished / not in this run
     int cnt[BQ_Q];     // hits so far
@@ -123,6 +124,7 @@ __device__ __forceinline__ void scan_run(Tile& tile, const float* __restrict__ s
                 const float cy = tile.y[k0 + lane];
                 const float cz = tile.z[k0 + lane];
                 const int64_t pos = base + k0 + lane;
+                TPK_WORK_ADD(BQ_Q);
 #pragma unroll
                 for (int q = 0; q < BQ_Q; ++q)
                 {
@@ -155,6 +157,7 @@ __device__ __forceinline__ void scan_run(Tile& tile, const float* __restrict__ s
         }
     }
 
+    TPK_WORK_FLUSH
     // Unused slots.
 #pragma unroll
     for (int q = 0; q < BQ_Q; ++q)

@@ -106,6 +106,7 @@ __global__ __launch_bounds__(CH_THREADS) void chamfer_fwd_kernel(
         best[q] = tpk_inf<T>();
         bgroup[q] = 0;
     }
+    TPK_WORK_DECL
 
     for (int base = 0; base < nc; base += CH_TILE)
     {
@@ -147,6 +148,7 @@ __global__ __launch_bounds__(CH_THREADS) void chamfer_fwd_kernel(
                     mn[q] = c == 0 ? d : tpk_min(mn[q], d);
                 }
             }
+            TPK_WORK_ADD(CH_CHUNK * Q);
             const int group = base / CH_CHUNK + g;
 #pragma unroll
             for (int q = 0; q < Q; ++q)
@@ -158,6 +160,7 @@ __global__ __launch_bounds__(CH_THREADS) void chamfer_fwd_kernel(
         }
     }
 
+    TPK_WORK_FLUSH
     // Recover the index: first candidate of the winning group whose distance equals the
     // minimum (re-evaluated with the same operations, hence the same bits).
 #pragma unroll

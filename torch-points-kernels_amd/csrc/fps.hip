@@ -450,6 +450,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     int pending = -1; // sorted position of the previous round's sample while its index is unstored
     if (tid == 0)
         out[0] = 0;
+    TPK_WORK_DECL
 
     for (int j = 1; j < npoint; ++j)
     {
@@ -475,6 +476,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             {
                 if ((live >> gi) & 1u) // uniform over the wavefront
                 {
+                    TPK_WORK_ADD(GS);
 #pragma unroll
                     for (int e = 0; e < GS; ++e)
                     {
@@ -618,6 +620,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     }
     if (tid == 0 && pending >= 0)
         out[npoint - 1] = static_cast<int>(sort_keys[pending] & 0x3FFFu);
+    TPK_WORK_FLUSH
 }
 
 constexpr int FPS_CELL_WINDOW = CURVE_MAX_POINTS;            // points ordered together

@@ -48,7 +48,7 @@ struct Nearest
 // own 64-entry LDS buffer, through which every lane sees every candidate (broadcast reads).
 __device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, const float4* __restrict__ boxes,
                                           int cell, float4* stage, int lane, float qx, float qy, float qz,
-                                          Nearest& s)
+                                          Nearest& s TPK_WORK_PARAM)
 {
     stage[lane] = cand[cell * NG_CELL + lane];
     const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
@@ -74,6 +74,7 @@ __device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, const
             const float d = tpk_dist2(p.x, p.y, p.z, qx, qy, qz);
             mn = c == 0 ? d : fminf(mn, d);
         }
+        TPK_WORK_ADD(NG_CHUNK);
         const bool better = mn < s.best;
         const bool equal = mn == s.best;
         s.tie = better ? false : (s.tie || equal);
@@ -117,6 +118,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
     int32_t* __restrict__ iout = (second ? idx2 : idx1) + static_cast<int64_t>(cloud) * qcount;
     float4* const stage = stages[wave];
     float* const lows = lows_all + wave * ((max(cells1, cells2) + NG_CELL - 1) / NG_CELL * NG_CELL);
+    TPK_WORK_DECL
 
     const float4 query = qpts[qcell * NG_CELL + lane];
     const float qx = query.x, qy = query.y, qz = query.z;
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
         int seed = static_cast<int>(lowest & 63u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
         if (seed >= ccells) // no lane had a usable key (NaN boxes)
             seed = 0;
-        scan_cell(cpts, cbox, seed, stage, lane, qx, qy, qz, s);
+        scan_cell(cpts, cbox, seed, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
         if (lane == (seed & (NG_CELL - 1)))
             lows[seed] = __builtin_inff();
     }
@@ -182,7 +184,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
                         lows[c] = __builtin_inff();
                     continue;
                 }
-                scan_cell(cpts, cbox, c, stage, lane, qx, qy, qz, s);
+                scan_cell(cpts, cbox, c, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
                 if (lane == bit)
                     lows[c] = __builtin_inff();
                 if (phase)
@@ -221,9 +223,12 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
                 const int ci = __float_as_int(p.w);
                 bi = (s.tie && d == s.best && ci < bi) ? ci : bi;
             }
+            TPK_WORK_ADD(NG_CELL);
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     }
+    TPK_WORK_ADD(NG_CHUNK);
+    TPK_WORK_FLUSH
     if (qindex != 0x7FFFFFFF)
     {
         dout[qindex] = s.best;
@@ -253,7 +258,7 @@ __device__ __forceinline__ bool pair_less(float d, int ci, float b, int i)
 
 __device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, const float4* __restrict__ boxes,
                                            int cell, float4* stage, int lane, float qx, float qy, float qz,
-                                           Nearest3& s)
+                                           Nearest3& s TPK_WORK_PARAM)
 {
     stage[lane] = cand[cell * NG_CELL + lane];
     const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
@@ -278,8 +283,10 @@ __device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, cons
             const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
             mn = c == 0 ? d : fminf(mn, d);
         }
+        TPK_WORK_ADD(NG_CHUNK);
         if (__ballot(mn <= s.b3) == 0)
             continue; // no candidate of this group enters any lane's triple
+        TPK_WORK_ADD(NG_CHUNK); // (the distances of an admitted group are formed a second time)
 #pragma unroll
         for (int c = 0; c < NG_CHUNK; ++c)
         {
@@ -328,6 +335,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     idx += static_cast<int64_t>(cloud) * n * 3;
     float4* const stage = stages[wave];
     float* const lows = lows_all + wave * ((ccells + NG_CELL - 1) / NG_CELL * NG_CELL);
+    TPK_WORK_DECL
 
     const float4 query = qpts[qcell * NG_CELL + lane];
     const float qx = query.x, qy = query.y, qz = query.z;
@@ -361,7 +369,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
         int seed = static_cast<int>(lowest & 63u) * NG_CELL + __builtin_ctzll(__ballot(seed_key == lowest));
         if (seed >= ccells)
             seed = 0;
-        scan_cell3(cpts, cbox, seed, stage, lane, qx, qy, qz, s);
+        scan_cell3(cpts, cbox, seed, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
         if (lane == (seed & (NG_CELL - 1)))
             lows[seed] = __builtin_inff();
     }
@@ -379,7 +387,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
                 live &= live - 1;
                 const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
                 if (__ballot(lb * NG_MARGIN <= s.b3) != 0)
-                    scan_cell3(cpts, cbox, c, stage, lane, qx, qy, qz, s);
+                    scan_cell3(cpts, cbox, c, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
                 if (lane == bit)
                     lows[c] = __builtin_inff(); // scanned, or useless now and ever after
                 if (phase)
@@ -389,6 +397,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
                 }
             }
         }
+    TPK_WORK_FLUSH
     if (qindex != 0x7FFFFFFF)
     {
         dist2[qindex * 3 + 0] = s.b1;
@@ -650,6 +659,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     int s0, s1;
     wave_equal_range(batch_x, size_x, cloud, lane, s0, s1);
     const int64_t out = q * nsample;
+    TPK_WORK_DECL
 
     // The walk is laid out so that dependent loads are few: all windows at once (one lane each),
     // then all (window, bin) pairs at once, then the candidates 64 at a time.
@@ -711,6 +721,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 const float4 p = sorted_x[has ? at_x : 0];
                 const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+                TPK_WORK_ADD(1);
                 const int row = __float_as_int(p.w);
                 const bool hit = has && d <= radius2 && row >= s0 && row < s1;
                 const unsigned long long mask = __ballot(hit);
@@ -751,6 +762,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
             idx[out + s] = -1;
             dist[out + s] = -1.0f;
         }
+        TPK_WORK_FLUSH
         return;
     }
 
@@ -774,6 +786,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
         {
             const int pos = base + u * TPK_WAVE + lane;
             const float d = tpk_dist2(qx, qy, qz, px[u], py[u], pz[u]);
+            TPK_WORK_ADD(1);
             const bool hit = pos < s1 && d <= radius2;
             const unsigned long long mask = __ballot(hit);
             const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
@@ -790,6 +803,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
         idx[out + s] = -1;
         dist[out + s] = -1.0f;
     }
+    TPK_WORK_FLUSH
 }
 
 struct GridLayout

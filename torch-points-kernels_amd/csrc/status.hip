@@ -27,3 +27,41 @@ extern "C" const char* tpk_status_string(int status)
         return hipGetErrorString(static_cast<hipError_t>(status));
     return "unknown status";
 }
+
+#ifdef TPK_COUNT_WORK
+// Counting build only: the per-translation-unit work counters (tpk_device.h) and their sum.
+#include <vector>
+
+namespace {
+std::vector<int (*)(unsigned long long*)>& work_readers()
+{
+    static std::vector<int (*)(unsigned long long*)> readers;
+    return readers;
+}
+} // namespace
+
+extern "C" void tpk_work_register(int (*read_reset)(unsigned long long*))
+{
+    work_readers().push_back(read_reset);
+}
+
+// Waits for the device, returns the pair evaluations counted since the last call in *pairs and
+// sets the counters back to zero.
+extern "C" int tpk_work_read_reset(unsigned long long* pairs)
+{
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    unsigned long long total = 0;
+    for (auto reader : work_readers())
+    {
+        unsigned long long part = 0;
+        const int st = reader(&part);
+        if (st != 0)
+            return st;
+        total += part;
+    }
+    *pairs = total;
+    return TPK_OK;
+}
+#endif

@@ -52,6 +52,7 @@ __global__ __launch_bounds__(NN_THREADS) void three_nn_kernel(
         b1[q] = b2[q] = b3[q] = __builtin_inff();
         i1[q] = i2[q] = i3[q] = 0;
     }
+    TPK_WORK_DECL
 
     for (int base = 0; base < m; base += NN_TILE)
     {
@@ -75,6 +76,7 @@ __global__ __launch_bounds__(NN_THREADS) void three_nn_kernel(
         __syncthreads();
 
         const int cnt4 = (cnt + 3) & ~3;
+        TPK_WORK_ADD(cnt4 * Q);
 #pragma unroll 4
         for (int k = 0; k < cnt4; ++k)
         {
@@ -100,6 +102,7 @@ __global__ __launch_bounds__(NN_THREADS) void three_nn_kernel(
         }
     }
 
+    TPK_WORK_FLUSH
 #pragma unroll
     for (int q = 0; q < Q; ++q)
     {

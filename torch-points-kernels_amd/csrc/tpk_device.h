@@ -153,3 +153,43 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Work counters.  The library is also built a second time with -DTPK_COUNT_WORK
+// (libtpk_hip_counting.so): there the distance scans add up the pair evaluations their lanes
+// execute (one count = one lane forming one squared distance, or one running minimum updated by
+// furthest point sampling), so that a benchmark can divide EXECUTED work by time.  Every
+// translation unit has its own device counter, registered with the reader in status.hip.  In the
+// shipping build all of this expands to nothing.
+// ---------------------------------------------------------------------------------------------
+#ifdef TPK_COUNT_WORK
+namespace {
+__device__ unsigned long long tpk_work_cell;
+int tpk_work_cell_read_reset(unsigned long long* out)
+{
+    const unsigned long long zero = 0;
+    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(tpk_work_cell), sizeof(*out));
+    if (e == hipSuccess)
+        e = hipMemcpyToSymbol(HIP_SYMBOL(tpk_work_cell), &zero, sizeof(zero));
+    return static_cast<int>(e);
+}
+} // namespace
+extern "C" void tpk_work_register(int (*read_reset)(unsigned long long*));
+namespace {
+struct TpkWorkRegistration
+{
+    TpkWorkRegistration() { tpk_work_register(&tpk_work_cell_read_reset); }
+} tpk_work_registration;
+} // namespace
+#define TPK_WORK_DECL unsigned long long tpk_work = 0;
+#define TPK_WORK_ADD(n) (tpk_work += static_cast<unsigned long long>(n))
+#define TPK_WORK_FLUSH atomicAdd(&tpk_work_cell, tpk_work);
+#define TPK_WORK_PARAM , unsigned long long& tpk_work
+#define TPK_WORK_ARG , tpk_work
+#else
+#define TPK_WORK_DECL
+#define TPK_WORK_ADD(n) ((void)0)
+#define TPK_WORK_FLUSH
+#define TPK_WORK_PARAM
+#define TPK_WORK_ARG
+#endif
