@@ -226,9 +226,10 @@ int tpk_group_grad_f32(int b, int c, int n, int npoint, int nsample, const float
  * (tpk_chamfer_fwd_workspace_bytes() bytes - 0 for shapes it does not serve that way -, 256-byte
  * aligned, contents arbitrary before and after) and searches only nearby cells; with
  * workspace == NULL, and always in float64, it tests all pairs (same results, slower).
- * The backward pass inverts idx1 / idx2 into per-point lists held in `workspace`
- * (tpk_chamfer_bwd_workspace_bytes() bytes, 256-byte aligned, contents arbitrary before and
- * after); with workspace == NULL it scatters with hardware float atomics instead (slower).
+ * The backward pass needs no workspace (tpk_chamfer_bwd_workspace_bytes() returns 0; the
+ * arguments are kept for callers written against earlier versions and are ignored): the points
+ * that chose a point as nearest neighbour are chained to it in LDS.  Clouds of more than about
+ * 38000 points scatter with hardware float atomics instead.
  * ------------------------------------------------------------------------------------- */
 size_t tpk_chamfer_fwd_workspace_bytes(int b, int n, int m);
 int tpk_chamfer_fwd_f32(int b, int n, int m, const float* xyz1, const float* xyz2, float* dist1,

@@ -258,111 +258,153 @@ __global__ __launch_bounds__(256) void chamfer_bwd_scatter_kernel(
     }
 }
 
-// One lane per point of either cloud: own term, then the terms of the points that chose it.
-// lists_a: lists over the points of cloud 1 (built from idx2); lists_b: lists over the points
-// of cloud 2 (built from idx1).  A wavefront serves one block of lists, one lane per point:
-// in step i the lanes read slot i of their lists
-// (consecutive entries; padding entries carry an index past the other cloud and are skipped).
-template <typename T>
-__global__ __launch_bounds__(256) void chamfer_bwd_lists_kernel(
-    int n, int m, int clouds, const T* __restrict__ xyz1, const T* __restrict__ xyz2,
-    const int32_t* __restrict__ idx1, const int32_t* __restrict__ idx2,
-    const T* __restrict__ grad_dist1, const T* __restrict__ grad_dist2,
-    Lists<false> lists_a, Lists<false> lists_b, T* __restrict__ grad_xyz1, T* __restrict__ grad_xyz2)
-{
-    // A cloud pair takes blocks1 + blocks2 consecutive logical blocks: the n points of cloud 1
-    // first, then the m of cloud 2.  Logical blocks are numbered so that those of a pair run on
-    // one die: its L2 then serves the random reads into the pair's points and gradients.
-    const int blocks1 = (n + 255) / 256;
-    const int per_cloud = blocks1 + (m + 255) / 256;
-    const int64_t total = static_cast<int64_t>(per_cloud) * clouds;
-    const int lane = threadIdx.x & (TPK_WAVE - 1);
-    for (int64_t lin = xcd_local_block(blockIdx.x, gridDim.x); lin < total; lin += gridDim.x)
-    {
-        const int cloud = static_cast<int>(lin / per_cloud);
-        const int bx = static_cast<int>(lin % per_cloud);
-        const bool second = bx >= blocks1;
-        const int pos = (second ? bx - blocks1 : bx) * 256 + threadIdx.x;
-        const int npts = second ? m : n;
-        const int nother = second ? n : m;
-        if (pos - lane >= npts) // the whole wavefront lies past the cloud
-            continue;
-        const Lists<false>& lists = second ? lists_b : lists_a;
-        const int64_t nblocks = (npts + L_BLOCK - 1) / L_BLOCK;
-        const int k = pos;
-        const bool live = k < npts;
-        const int kk = live ? k : 0;
-        const T* __restrict__ own = (second ? xyz2 : xyz1) + static_cast<int64_t>(cloud) * npts * 3;
-        const T* __restrict__ other = (second ? xyz1 : xyz2) + static_cast<int64_t>(cloud) * nother * 3;
-        const int32_t* __restrict__ own_idx = (second ? idx2 : idx1) + static_cast<int64_t>(cloud) * npts;
-        const T* __restrict__ own_g = (second ? grad_dist2 : grad_dist1) + static_cast<int64_t>(cloud) * npts;
-        const T* __restrict__ other_g = (second ? grad_dist1 : grad_dist2) + static_cast<int64_t>(cloud) * nother;
-        const ListEntry<false>* __restrict__ ent = lists.entries + static_cast<int64_t>(cloud) * lists.capacity;
-        const ListBlock lb = list_block(lists.blocks + cloud * nblocks, pos / L_BLOCK);
+// Backward without float atomics and without workspace.  A workgroup owns a range of points
+// ("targets") of one cloud of one pair.  It first threads the points of the OTHER cloud that
+// chose one of its targets as nearest neighbour into per-target chains held in LDS: one LDS
+// integer exchange per point (head[target] <- point, next[point] <- old head).  Then one lane per
+// target adds the target's own term and walks its chain (most chains hold zero to two points).
+// Every output is written once, nothing is zero-filled.  The order of a chain is the order in
+// which the exchanges happened to be served, so - as with the reference's atomics - the sum of
+// a point with several terms may differ in the last bits from run to run.
+// dynamic LDS: (points of the larger cloud + targets per workgroup) ints.
+constexpr int CHB_THREADS = 1024;
+constexpr int CHB_LDS_INTS = 38912; // 152 KiB: chains of the other cloud's points + heads of a range
 
-        const T px = own[kk * 3 + 0], py = own[kk * 3 + 1], pz = own[kk * 3 + 2];
-        const int j2 = own_idx[kk];
-        const T g = own_g[kk] * 2;
-        T ax = g * (px - other[j2 * 3 + 0]);
-        T ay = g * (py - other[j2 * 3 + 1]);
-        T az = g * (pz - other[j2 * 3 + 2]);
-        auto add_entry = [&](int j) {
-            const T gj = other_g[j] * 2;
-            ax = ax + -(gj * (other[j * 3 + 0] - px));
-            ay = ay + -(gj * (other[j * 3 + 1] - py));
-            az = az + -(gj * (other[j * 3 + 2] - pz));
-        };
-        // Slots are fetched eight at a time, then the points they name.
-        for (int i = 0; i < lb.width; i += 8)
+template <typename T>
+__global__ __launch_bounds__(CHB_THREADS) void chamfer_bwd_chains_kernel(
+    int n, int m, int clouds, int splits, int range1, int range2, const T* __restrict__ xyz1,
+    const T* __restrict__ xyz2, const int32_t* __restrict__ idx1, const int32_t* __restrict__ idx2,
+    const T* __restrict__ grad_dist1, const T* __restrict__ grad_dist2, T* __restrict__ grad_xyz1,
+    T* __restrict__ grad_xyz2)
+{
+    extern __shared__ int chain_lds[];
+    // logical workgroup = ((cloud * 2 + direction) * splits + split); those of a pair run on one
+    // die, whose L2 then serves the random reads into the pair's points
+    const int lin = static_cast<int>(xcd_local_block(blockIdx.x, gridDim.x));
+    const int cloud = lin / (2 * splits);
+    const int rem = lin - cloud * 2 * splits;
+    const bool second = rem >= splits;
+    const int split = second ? rem - splits : rem;
+    const int npts = second ? m : n;
+    const int nother = second ? n : m;
+    const int range = second ? range2 : range1;
+    const int t0 = split * range;
+    const int t1 = min(t0 + range, npts);
+    if (t0 >= t1)
+        return; // (the whole workgroup: no barrier has been passed yet)
+    int* const next = chain_lds;
+    int* const head = chain_lds + nother;
+    const int tid = threadIdx.x;
+    const T* __restrict__ own = (second ? xyz2 : xyz1) + static_cast<int64_t>(cloud) * npts * 3;
+    const T* __restrict__ other = (second ? xyz1 : xyz2) + static_cast<int64_t>(cloud) * nother * 3;
+    const int32_t* __restrict__ own_idx = (second ? idx2 : idx1) + static_cast<int64_t>(cloud) * npts;
+    const int32_t* __restrict__ other_idx = (second ? idx1 : idx2) + static_cast<int64_t>(cloud) * nother;
+    const T* __restrict__ own_g = (second ? grad_dist2 : grad_dist1) + static_cast<int64_t>(cloud) * npts;
+    const T* __restrict__ other_g = (second ? grad_dist1 : grad_dist2) + static_cast<int64_t>(cloud) * nother;
+    T* __restrict__ out = (second ? grad_xyz2 : grad_xyz1) + static_cast<int64_t>(cloud) * npts * 3;
+
+    for (int t = tid; t < t1 - t0; t += CHB_THREADS)
+        head[t] = -1;
+    __syncthreads();
+    constexpr int BATCH = 8; // index loads in flight per thread
+    for (int j0 = tid; j0 < nother; j0 += BATCH * CHB_THREADS)
+    {
+        int k[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
         {
-            int j[8];
+            const int j = j0 + u * CHB_THREADS;
+            k[u] = j < nother ? other_idx[j] : -1;
+        }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                j[u] = i + u < lb.width ? ent[lb.start + (i + u) * L_BLOCK + lane].j : nother;
-            T gj[8], ox[8], oy[8], oz[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
+        for (int u = 0; u < BATCH; ++u)
+            if (k[u] >= t0 && k[u] < t1)
             {
-                const int jj = j[u] < nother ? j[u] : 0;
-                gj[u] = other_g[jj];
-                ox[u] = other[jj * 3 + 0];
-                oy[u] = other[jj * 3 + 1];
-                oz[u] = other[jj * 3 + 2];
+                const int j = j0 + u * CHB_THREADS;
+                next[j] = atomicExch(&head[k[u] - t0], j);
             }
+    }
+    __syncthreads();
+    // Several targets per lane at a time, so that their dependent reads (own index -> that point;
+    // chain head -> point -> next) travel together.
+    constexpr int TPT = 1;
+    for (int kb = t0 + tid; kb < t1; kb += TPT * CHB_THREADS)
+    {
+        T px[TPT], py[TPT], pz[TPT], g[TPT], ax[TPT], ay[TPT], az[TPT];
+        int j2[TPT], j[TPT];
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (j[u] < nother)
+        for (int u = 0; u < TPT; ++u)
+        {
+            const int k = min(kb + u * CHB_THREADS, t1 - 1);
+            px[u] = own[k * 3 + 0];
+            py[u] = own[k * 3 + 1];
+            pz[u] = own[k * 3 + 2];
+            j2[u] = own_idx[k];
+            g[u] = own_g[k] * 2;
+            j[u] = kb + u * CHB_THREADS < t1 ? head[k - t0] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < TPT; ++u)
+        {
+            ax[u] = g[u] * (px[u] - other[j2[u] * 3 + 0]);
+            ay[u] = g[u] * (py[u] - other[j2[u] * 3 + 1]);
+            az[u] = g[u] * (pz[u] - other[j2[u] * 3 + 2]);
+        }
+        // The chains are followed in LDS first, CHAIN links at a time, and the points they name are
+        // requested together: the reads from memory do not wait for one another.
+        constexpr int CHAIN = 2;
+        while (true)
+        {
+            bool any = false;
+#pragma unroll
+            for (int u = 0; u < TPT; ++u)
+                any = any || j[u] >= 0;
+            if (!any)
+                break;
+            int link[TPT][CHAIN];
+#pragma unroll
+            for (int u = 0; u < TPT; ++u)
+#pragma unroll
+                for (int l = 0; l < CHAIN; ++l)
                 {
-                    const T g2 = gj[u] * 2;
-                    ax = ax + -(g2 * (ox[u] - px));
-                    ay = ay + -(g2 * (oy[u] - py));
-                    az = az + -(g2 * (oz[u] - pz));
+                    link[u][l] = j[u];
+                    j[u] = j[u] >= 0 ? next[j[u]] : -1;
                 }
+            T gj[TPT][CHAIN], ox[TPT][CHAIN], oy[TPT][CHAIN], oz[TPT][CHAIN];
+#pragma unroll
+            for (int u = 0; u < TPT; ++u)
+#pragma unroll
+                for (int l = 0; l < CHAIN; ++l)
+                {
+                    const int jj = link[u][l] >= 0 ? link[u][l] : 0;
+                    gj[u][l] = other_g[jj] * 2;
+                    ox[u][l] = other[jj * 3 + 0];
+                    oy[u][l] = other[jj * 3 + 1];
+                    oz[u][l] = other[jj * 3 + 2];
+                }
+#pragma unroll
+            for (int u = 0; u < TPT; ++u)
+#pragma unroll
+                for (int l = 0; l < CHAIN; ++l)
+                    if (link[u][l] >= 0)
+                    {
+                        ax[u] = ax[u] + -(gj[u][l] * (ox[u][l] - px[u]));
+                        ay[u] = ay[u] + -(gj[u][l] * (oy[u][l] - py[u]));
+                        az[u] = az[u] + -(gj[u][l] * (oz[u][l] - pz[u]));
+                    }
         }
-        if (lb.longer)
+#pragma unroll
+        for (int u = 0; u < TPT; ++u)
         {
-            const int count = lists.counts[cloud * nblocks * L_BLOCK + pos];
-            int extra, extra_at;
-            list_extra(count, lb.width, extra, extra_at);
-            const ListEntry<false>* __restrict__ rest = ent + lb.start + lb.width * L_BLOCK + extra_at;
-            for (int p = 0; p < extra; ++p)
-                add_entry(rest[p].j);
-        }
-        if (live)
-        {
-            T* __restrict__ out = (second ? grad_xyz2 : grad_xyz1) + (static_cast<int64_t>(cloud) * npts + k) * 3;
-            out[0] = ax;
-            out[1] = ay;
-            out[2] = az;
+            const int k = kb + u * CHB_THREADS;
+            if (k < t1)
+            {
+                out[k * 3 + 0] = ax[u];
+                out[k * 3 + 1] = ay[u];
+                out[k * 3 + 2] = az[u];
+            }
         }
     }
-}
-
-// Workspace of the list-based backward: lists over cloud 1, then lists over cloud 2.
-size_t chamfer_lists_bytes(int b, int n, int m, size_t* second)
-{
-    *second = lists_bytes<false>(b, n, m);
-    return *second + lists_bytes<false>(b, m, n);
 }
 
 template <typename T>
@@ -437,31 +479,32 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
         hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(blocks), dim3(256), 0, s, p, count);
         return tpk_launch_status();
     }
-    size_t second;
-    const size_t need = chamfer_lists_bytes(b, n, m, &second);
-    if (workspace && workspace_bytes >= need && static_cast<int64_t>(n) * 3 <= 0x7fffffffLL &&
-        static_cast<int64_t>(m) * 3 <= 0x7fffffffLL)
+    (void)workspace;
+    (void)workspace_bytes;
+    // Chains in LDS (no workspace): as many target ranges per cloud as give the chip a few hundred
+    // workgroups, each of at least 1024 targets; clouds too large for LDS scatter with atomics.
     {
-        // lists over cloud-1 points: who in cloud 2 chose them (idx2); and the mirror image
-        const Lists<false> lists_a = lists_at<false>(workspace, b, n, m);
-        const Lists<false> lists_b = lists_at<false>(static_cast<char*>(workspace) + second, b, m, n);
-        ListJob<false, int32_t> job_a, job_b;
-        int st = make_list_job<1, false, int32_t>(b, n, m, m, m, 1, idx2, nullptr, lists_a, &job_a);
-        if (st == TPK_OK)
-            st = make_list_job<1, false, int32_t>(b, m, n, n, n, 1, idx1, nullptr, lists_b, &job_b);
-        if (st == TPK_OK)
-            st = launch_list_jobs<1, false, int32_t>(job_a, job_b, s);
-        if (st == TPK_OK)
+        const int larger = n > m ? n : m;
+        int splits = static_cast<int>(tpk_ceil_div(320, 2 * static_cast<int64_t>(b)));
+        const int most = static_cast<int>(tpk_ceil_div(larger, CHB_THREADS));
+        splits = splits > most ? most : splits;
+        splits = splits < 1 ? 1 : splits;
+        while (larger + tpk_ceil_div(larger, splits) > CHB_LDS_INTS && splits < most)
+            ++splits;
+        const int range1 = static_cast<int>(tpk_ceil_div(n, splits)), range2 = static_cast<int>(tpk_ceil_div(m, splits));
+        const int64_t groups = 2 * static_cast<int64_t>(b) * splits;
+        if (larger + (range1 > range2 ? range1 : range2) <= CHB_LDS_INTS && groups <= 0x7fffffffLL &&
+            static_cast<int64_t>(larger) * 3 <= 0x7fffffffLL)
         {
-            const int64_t blocks = (tpk_ceil_div(n, 256) + tpk_ceil_div(m, 256)) * static_cast<int64_t>(b);
-            hipLaunchKernelGGL(chamfer_bwd_lists_kernel<T>,
-                               dim3(static_cast<unsigned>(tpk_min64(blocks, 1 << 24))), dim3(256), 0, s, n, m, b, xyz1,
-                               xyz2, idx1, idx2, grad_dist1, grad_dist2, lists_a, lists_b,
-                               grad_xyz1, grad_xyz2);
+            const size_t lds = (static_cast<size_t>(larger) + (range1 > range2 ? range1 : range2)) * sizeof(int);
+            const int allowed = allow_lds(chamfer_bwd_chains_kernel<T>, lds);
+            if (allowed != TPK_OK)
+                return allowed;
+            hipLaunchKernelGGL(chamfer_bwd_chains_kernel<T>, dim3(static_cast<unsigned>(groups)), dim3(CHB_THREADS), lds, s,
+                               n, m, b, splits, range1, range2, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2, grad_xyz1,
+                               grad_xyz2);
             return tpk_launch_status();
         }
-        if (st != TPK_ERR_UNSUPPORTED)
-            return st;
     }
     const unsigned blocks =
         static_cast<unsigned>(tpk_min64(tpk_ceil_div(total1 + total2, 256), 1 << 20));
@@ -528,8 +571,8 @@ extern "C" int tpk_chamfer_bwd_f64(int b, int n, int m, const double* xyz1, cons
 
 extern "C" size_t tpk_chamfer_bwd_workspace_bytes(int b, int n, int m)
 {
-    if (b <= 0 || n <= 0 || m <= 0)
-        return 0;
-    size_t second;
-    return chamfer_lists_bytes(b, n, m, &second);
+    (void)b;
+    (void)n;
+    (void)m;
+    return 0; // the backward pass keeps its chains in LDS
 }

@@ -194,10 +194,9 @@ int launch_curve_cells(const PointSet& a, const PointSet& c, int* zero_word, hip
     if (windows_a + windows_c > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     const size_t lds = (2 * static_cast<size_t>(key_capacity) + CURVE_BINS) * sizeof(unsigned);
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(curve_cells_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    if (e != hipSuccess)
-        return static_cast<int>(e);
+    const int allowed = tpk_allow_lds(reinterpret_cast<const void*>(curve_cells_kernel), lds);
+    if (allowed != TPK_OK)
+        return allowed;
     hipLaunchKernelGGL(curve_cells_kernel, dim3(static_cast<unsigned>(windows_a + windows_c)),
                        dim3(NG_SORT_THREADS), lds, s, a, c, static_cast<int>(windows_a), key_capacity,
                        zero_word);

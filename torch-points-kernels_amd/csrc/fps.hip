@@ -902,11 +902,9 @@ int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float
     const int key_capacity = n > CURVE_BINS ? (n + 63) & ~63 : CURVE_BINS; // (the ordering borrows CURVE_BINS words)
     const size_t lds = (static_cast<size_t>(key_capacity) + static_cast<size_t>(PPT) * THREADS + CURVE_BINS) * sizeof(unsigned);
     auto kernel = fps_pruned_kernel<PPT, THREADS, GS>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       static_cast<int>(lds));
-    if (e != hipSuccess)
-        return static_cast<int>(e);
+    const int allowed = tpk_allow_lds(reinterpret_cast<const void*>(kernel), lds);
+    if (allowed != TPK_OK)
+        return allowed;
     hipLaunchKernelGGL(kernel, dim3(b), dim3(THREADS), lds, s, n, npoint, log2_bs, groups, key_capacity,
                        xyz, out);
     return tpk_launch_status();
@@ -997,10 +995,9 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
         if (st != TPK_OK)
             return st;
         const size_t lds = static_cast<size_t>(l.cells) * 48 + FPS_LIVE_CAPACITY * FPS_WAVES * sizeof(unsigned short);
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fps_cells_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-        if (e != hipSuccess)
-            return static_cast<int>(e);
+        st = tpk_allow_lds(reinterpret_cast<const void*>(fps_cells_kernel), lds);
+        if (st != TPK_OK)
+            return st;
         hipLaunchKernelGGL(fps_cells_kernel, dim3(b), dim3(FPS_THREADS), lds, s, n, npoint, log2_bs, groups, l.cells,
                            xyz, cloud.sorted, cloud.boxes, reinterpret_cast<float*>(w + l.temp), idx_out);
     }

@@ -350,10 +350,9 @@ int cubic_bwd(int b, int n_pts, int channels, int scale, int neighborhood_size, 
         if (blocks <= 0x7fffffffLL)
         {
             const size_t lds = static_cast<size_t>(group * cub) * sizeof(T);
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(cubic_scatter_lds_kernel<T>),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-            if (e != hipSuccess)
-                return static_cast<int>(e);
+            const int allowed = tpk_allow_lds(reinterpret_cast<const void*>(cubic_scatter_lds_kernel<T>), lds);
+            if (allowed != TPK_OK)
+                return allowed;
             hipLaunchKernelGGL(cubic_scatter_lds_kernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(CS_THREADS), lds, s, n_pts, static_cast<int>(nv), channels,
                                static_cast<int>(group), cub, grad_point_features, grid_pt_indexes, grad_cubic_features);
             return tpk_launch_status();

@@ -1,6 +1,6 @@
 // Inverted index ("lists"): for every target position of a cloud, the entries that refer to
 // it.  Shared by the backward passes that would otherwise scatter with float atomics
-// (three_interpolate, grouping, Chamfer): they gather along these lists instead.
+// (three_interpolate, grouping): they gather along these lists instead.
 #pragma once
 
 #include "tpk_device.h"
@@ -12,13 +12,13 @@ constexpr int G_THREADS = 1024;
 template <typename Kernel>
 int allow_lds(Kernel kernel, size_t bytes)
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       static_cast<int>(bytes));
-    return e == hipSuccess ? TPK_OK : static_cast<int>(e);
+    return tpk_allow_lds(reinterpret_cast<const void*>(kernel), bytes);
 }
 
-// One entry of a target's list: the column that references it and the weight it carries.
+// One entry of a target's list: the column that references it and the weight it carries.  The
+// column is stored the way the walker uses it: as the byte offset of that column's value in a
+// staged row that starts with four zeros, (column + 4) * 4 - so an all-zero entry, which is what
+// a lane without entry is given, points at a zero.
 template <bool WEIGHTED>
 struct ListEntry;
 template <>
@@ -35,26 +35,34 @@ struct ListEntry<false>
 
 constexpr int L_MAX_TARGETS = 15360; // targets whose bookkeeping fits in LDS (2 ints each)
 constexpr int L_BLOCK = TPK_WAVE;    // targets per block of lists: one per lane
-constexpr int L_SLACK = 576;         // entry slots a block owns beyond three per entry
-constexpr int L_WIDTH_STEP = 4;      // widths of the padded parts are multiples of 1, 2 or this (the walker's choice)
+constexpr int L_SLACK = 832;         // entry slots a block owns beyond three per entry
+constexpr int L_WIDTH_STEP = 8;      // widths of the slot-major parts are multiples of this
+constexpr int L_COUNT_BITS = 20;     // bits of a meta word that hold a list length
+constexpr int L_COUNT_MASK = (1 << L_COUNT_BITS) - 1;
 
 // Layout of the lists of one cloud ("sliced": made to be walked by one lane per target).
-// Targets are taken in blocks of 64; `counts` holds the length of every target's list (0 in the
-// unused positions of the last block).  Block b owns the entry slots from
+// Targets are taken in blocks of 64.  Inside a block the lanes serve the targets in order of
+// descending list length, so that in step i of a walk the lanes that still have an entry are
+// the first ones: a step requests one contiguous run of entries and nothing for the others.
+// `meta` holds one word per position p of a block:
+//   bits  0..19  length of the list served by LANE p
+//   bits 20..25  the target (position inside the block) that lane p serves
+//   bits 26..31  the lane that serves TARGET p
+// Block b owns the entry slots from
 //   start_b = 3 * (entries of all earlier targets) + L_SLACK * b
-// and stores slot i of its target L at start_b + i * 64 + L for i < width_b, so that the 64
-// lanes read consecutive entries in every step.  width_b = min(longest list of the block,
-// 2 * ceil(entries of the block / 64) + 4), rounded up to a multiple of at most 4; shorter lists are
-// padded with (pad_j, 0) entries.  The entries of a list beyond width_b follow the padded part,
-// list after list in target order.  Padded part <= 2 * entries + 574 slots, the rest <= entries:
-// a block never leaves its own slots, whatever the index looks like.
-//   counts[cloud][64 * blocks]
+// and stores slot i of lane L at start_b + i * 64 + L for i < width_b (only the slots a list
+// really has are written; the others are never read).  width_b = min(longest list of the
+// block, 2 * ceil(entries of the block / 64) + 4), rounded up to a multiple of 8.  The entries
+// of a list beyond width_b follow that part, list after list in lane order.  Slot-major part
+// <= 2 * entries + 830 slots, the rest <= entries: a block never leaves its own slots, whatever
+// the index looks like.
+//   meta[cloud][64 * blocks]
 //   blocks[cloud][b]         (start_b, width_b; bit 31 of the width: some list is longer)
 //   entries[cloud][capacity]
 template <bool WEIGHTED>
 struct Lists
 {
-    int* counts;
+    int* meta;
     int2* blocks;
     ListEntry<WEIGHTED>* entries;
     int64_t capacity; // entry slots per cloud
@@ -89,7 +97,7 @@ Lists<WEIGHTED> lists_at(void* workspace, int clouds, int m, int64_t total)
     const size_t positions = static_cast<size_t>(list_blocks(m)) * L_BLOCK;
     char* p = static_cast<char*>(workspace);
     Lists<WEIGHTED> l;
-    l.counts = reinterpret_cast<int*>(p);
+    l.meta = reinterpret_cast<int*>(p);
     p += list_align(c * positions * sizeof(int));
     l.blocks = reinterpret_cast<int2*>(p);
     p += list_align(c * static_cast<size_t>(list_blocks(m)) * sizeof(int2));
@@ -98,9 +106,8 @@ Lists<WEIGHTED> lists_at(void* workspace, int clouds, int m, int64_t total)
     return l;
 }
 
-// What a wavefront needs to walk the lists of block `block` of a cloud, lane L serving the
-// target block * 64 + L: start and width of the padded part, and whether longer
-// lists exist.
+// What a wavefront needs to walk the lists of block `block` of a cloud: start and width of the
+// slot-major part, and whether longer lists exist.
 struct ListBlock
 {
     int start;
@@ -112,10 +119,9 @@ __device__ __forceinline__ ListBlock list_block(const int2* __restrict__ cloud_b
     const int2 d = cloud_blocks[__builtin_amdgcn_readfirstlane(block)];
     return ListBlock{d.x, d.y & 0x7fffffff, d.y < 0};
 }
-// For a block with longer lists: how many entries of this lane's target lie beyond the padded
-// part (`extra`), and where they start relative to the end of the padded part (`extra_at`).
-// Every lane of the wavefront calls it; `count` is the length of the lane's list (0 for
-// lanes beyond the last target).
+// For a block with longer lists: how many entries of this lane's list lie beyond the slot-major
+// part (`extra`), and where they start relative to its end (`extra_at`).  Every lane of the
+// wavefront calls it; `count` is the length of the lane's list.
 __device__ __forceinline__ void list_extra(int count, int width, int& extra, int& extra_at)
 {
     extra = max(count - width, 0);
@@ -129,34 +135,30 @@ __device__ __forceinline__ void list_extra(int count, int width, int& extra, int
 // workgroup builds the lists of the targets [split * span, (split + 1) * span) (span is a
 // multiple of 64): it reads every index entry of its part, counts those inside its span (LDS
 // integer atomics) and those below it (their number fixes where its blocks start), prefix-sums
-// the lengths, lays out its blocks and fills the lists in a second pass.  Workgroups never wait
-// for each other.  dynamic LDS: (2 * span + span / 32 + G_THREADS) ints.  Index values outside [0, m) are dropped.
-// One launch can carry two such jobs (the two directions of the Chamfer backward): the first
-// `workgroups` workgroups serve the first job, the rest the second.
+// the lengths, orders the lanes of its blocks and fills the lists in a second pass.  Workgroups
+// never wait for each other.  dynamic LDS: (2 * span + span / 32 + G_THREADS) ints.  Index values
+// outside [0, m) are dropped.
 template <bool WEIGHTED, typename IdxT>
 struct ListJob
 {
-    int m, cloud_total, parts, part_total, splits, span, pad_j, width_step, workgroups;
+    int m, cloud_total, parts, part_total, splits, span, workgroups;
     const IdxT* idx;
     const float* weight;
     Lists<WEIGHTED> lists;
 };
 
 template <int K, bool WEIGHTED, typename IdxT>
-__global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED, IdxT> first_job,
-                                                                ListJob<WEIGHTED, IdxT> second_job)
+__global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED, IdxT> job)
 {
-    const bool second = static_cast<int>(blockIdx.x) >= first_job.workgroups;
-    const ListJob<WEIGHTED, IdxT>& job = second ? second_job : first_job;
-    const int workgroup = second ? blockIdx.x - first_job.workgroups : blockIdx.x;
+    const int workgroup = blockIdx.x;
     const int m = job.m, cloud_total = job.cloud_total, parts = job.parts, part_total = job.part_total;
-    const int splits = job.splits, span = job.span, pad_j = job.pad_j, width_step = job.width_step;
+    const int splits = job.splits, span = job.span;
     const IdxT* __restrict__ idx = job.idx;
     const float* __restrict__ weight = job.weight;
     const Lists<WEIGHTED>& lists = job.lists;
 
     extern __shared__ int counters[];            // [span] list lengths, later fill cursors
-    int* const aux = counters + span;            // [span] list starts, later starts of the long parts
+    int* const aux = counters + span;            // [span] list starts, later (start of the long part | lane << 26)
     int* const block_start = aux + span;         // [span / 64]
     int* const block_width = block_start + span / L_BLOCK;
     int* const scan = block_width + span / L_BLOCK; // [G_THREADS]
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
     if (WEIGHTED)
         weight += first_entry;
     const int64_t cloud_blocks = (m + L_BLOCK - 1) / L_BLOCK;
-    int* __restrict__ counts = lists.counts + cloud_part * cloud_blocks * L_BLOCK;
+    int* __restrict__ meta = lists.meta + cloud_part * cloud_blocks * L_BLOCK;
     int2* __restrict__ blocks = lists.blocks + cloud_part * cloud_blocks;
     ListEntry<WEIGHTED>* __restrict__ entries = lists.entries + static_cast<int64_t>(cloud_part) * lists.capacity;
 
@@ -234,41 +236,44 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
     }
     __syncthreads();
 
-    // Layout of the blocks, one wavefront per block at a time; the padding entries are written
-    // here, the real ones in the second pass.
-    ListEntry<WEIGHTED> pad;
-    pad.j = pad_j;
-    if constexpr (WEIGHTED)
-        pad.w = 0.f;
+    // Layout of the blocks, one wavefront per block at a time.
     const int nblocks = (width + L_BLOCK - 1) / L_BLOCK;
     for (int blk = wave; blk < nblocks; blk += G_THREADS / TPK_WAVE)
     {
         const int t = blk * L_BLOCK + lane;
-        const int count = t < width ? counters[t] : 0;
+        const int count = t < width ? min(counters[t], L_COUNT_MASK) : 0;
         const int first = aux[blk * L_BLOCK];
         const int before = wave_exclusive_sum(count);
         const int block_entries = __builtin_amdgcn_readlane(before + count, TPK_WAVE - 1);
         const int longest = wave_max_i32(count);
-        const int w = (min(longest, 2 * ((block_entries + L_BLOCK - 1) / L_BLOCK) + 4) + width_step - 1) &
-                      ~(width_step - 1);
+        const int w = (min(longest, 2 * ((block_entries + L_BLOCK - 1) / L_BLOCK) + 4) + L_WIDTH_STEP - 1) &
+                      ~(L_WIDTH_STEP - 1);
         const int start = 3 * first + L_SLACK * (i0 / L_BLOCK + blk);
+        // the lane that serves this target: its rank by descending length (equal lengths in order)
+        int serving = 0;
+        for (int other = 0; other < TPK_WAVE; ++other)
+        {
+            const int oc = __builtin_amdgcn_readlane(count, other);
+            serving += (oc > count || (oc == count && other < lane)) ? 1 : 0;
+        }
+        // what lane `lane` serves: the target and the length sent to it by that target's position
+        const int served = __builtin_amdgcn_ds_permute(serving * 4, lane);
+        const int served_count = __builtin_amdgcn_ds_permute(serving * 4, count);
         int extra, extra_at;
-        list_extra(count, w, extra, extra_at);
+        list_extra(served_count, w, extra, extra_at);
+        const int my_extra_at = __builtin_amdgcn_ds_bpermute(serving * 4, extra_at); // of the lane that serves this target
         if (t < width)
         {
-            aux[t] = extra_at;
+            aux[t] = my_extra_at | (serving << 26);
             counters[t] = 0;
         }
-        counts[i0 + t] = count;
+        meta[i0 + t] = served_count | (served << L_COUNT_BITS) | (serving << 26);
         if (lane == 0)
         {
             block_start[blk] = start;
             block_width[blk] = w;
             blocks[i0 / L_BLOCK + blk] = make_int2(start, longest > w ? w | static_cast<int>(0x80000000u) : w);
         }
-        for (int i = 0; i < w; ++i)
-            if (i >= count)
-                entries[start + i * L_BLOCK + lane] = pad;
     }
     __syncthreads();
 
@@ -302,15 +307,19 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
             const int t = slot[u] >= 0 ? static_cast<int>(iv[u]) - i0 : 0;
             const int blk = t / L_BLOCK;
             const int w = block_width[blk];
+            const int a = aux[t];
+            const int serving = static_cast<int>(static_cast<unsigned>(a) >> 26);
             at[u] = block_start[blk] +
-                    (slot[u] < w ? slot[u] * L_BLOCK + (t & (L_BLOCK - 1)) : w * L_BLOCK + aux[t] + (slot[u] - w));
+                    (slot[u] < w ? slot[u] * L_BLOCK + serving : w * L_BLOCK + (a & 0x3FFFFFF) + (slot[u] - w));
+            if (slot[u] >= L_COUNT_MASK) // (a list longer than a meta word can say is cut there)
+                slot[u] = -1;
         }
 #pragma unroll
         for (int u = 0; u < BATCH; ++u)
             if (slot[u] >= 0)
             {
                 ListEntry<WEIGHTED> entry;
-                entry.j = (e0 + u * G_THREADS) / K;
+                entry.j = ((e0 + u * G_THREADS) / K + 4) * 4;
                 if constexpr (WEIGHTED)
                     entry.w = wv[u];
                 entries[at[u]] = entry;
@@ -320,24 +329,25 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
 
 // Describes the job of building the lists of `clouds` clouds of `m` targets and `cloud_total`
 // index entries each, in parts of `part_total` entries (`lists` sized for clouds * parts clouds
-// of part_total entries); padding entries refer to column `pad_j`, padded widths are multiples of
-// `width_step`.  Returns TPK_ERR_UNSUPPORTED
-// when a span of targets would not fit in LDS or entry positions would not fit an int.
+// of part_total entries).  Returns TPK_ERR_UNSUPPORTED when a span of targets would not fit in
+// LDS or entry positions would not fit their fields.
 template <int K, bool WEIGHTED, typename IdxT>
-int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, int pad_j, int width_step,
-                  const IdxT* idx, const float* weight, const Lists<WEIGHTED>& lists, ListJob<WEIGHTED, IdxT>* job)
+int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, const IdxT* idx, const float* weight,
+                  const Lists<WEIGHTED>& lists, ListJob<WEIGHTED, IdxT>* job)
 {
     *job = ListJob<WEIGHTED, IdxT>{};
     if (clouds <= 0 || m <= 0 || cloud_total <= 0)
         return TPK_OK; // nothing to build: no workgroups
-    if (part_total <= 0 || part_total % K != 0 || (width_step != 1 && width_step != 2 && width_step != L_WIDTH_STEP))
+    if (part_total <= 0 || part_total % K != 0)
         return TPK_ERR_INVALID_ARG;
     const int64_t parts = tpk_ceil_div(cloud_total, part_total);
-    if (list_capacity(m, part_total) > 0x7fffffffLL || cloud_total > 0x7fffffffLL ||
+    // (a list holds at most part_total entries: lengths must fit a meta word, positions in the
+    // long part 26 bits, byte offsets of entries 32 bits)
+    if (part_total >= L_COUNT_MASK || list_capacity(m, part_total) * 8 > 0xffffffffLL || cloud_total > 0x7fffffffLL ||
         clouds * parts > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    // Enough workgroups to occupy a good part of the chip; spans of a multiple of 64 targets.
-    int splits = static_cast<int>(tpk_ceil_div(128, clouds * parts));
+    // Enough workgroups to occupy the chip; spans of a multiple of 64 targets.
+    int splits = static_cast<int>(tpk_ceil_div(256, clouds * parts));
     if (splits > 16)
         splits = 16;
     if (splits < tpk_ceil_div(m, L_MAX_TARGETS))
@@ -352,8 +362,6 @@ int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, in
     job->part_total = static_cast<int>(part_total);
     job->splits = splits;
     job->span = span;
-    job->pad_j = pad_j;
-    job->width_step = width_step;
     job->workgroups = static_cast<int>(clouds * parts * splits);
     job->idx = idx;
     job->weight = weight;
@@ -361,30 +369,21 @@ int make_list_job(int clouds, int m, int64_t cloud_total, int64_t part_total, in
     return TPK_OK;
 }
 
-// Launches build_lists_kernel for one or two jobs.
 template <int K, bool WEIGHTED, typename IdxT>
-int launch_list_jobs(const ListJob<WEIGHTED, IdxT>& first, const ListJob<WEIGHTED, IdxT>& second, hipStream_t s)
-{
-    const int workgroups = first.workgroups + second.workgroups;
-    if (workgroups == 0)
-        return TPK_OK;
-    const int span = first.span > second.span ? first.span : second.span;
-    const size_t lds = (2 * static_cast<size_t>(span) + 2 * (span / L_BLOCK) + G_THREADS) * sizeof(int);
-    auto build = build_lists_kernel<K, WEIGHTED, IdxT>;
-    int st = allow_lds(build, lds);
-    if (st != TPK_OK)
-        return st;
-    hipLaunchKernelGGL(build, dim3(static_cast<unsigned>(workgroups)), dim3(G_THREADS), lds, s, first, second);
-    return tpk_launch_status();
-}
-
-template <int K, bool WEIGHTED, typename IdxT>
-int launch_build_lists(int clouds, int m, int64_t cloud_total, int64_t part_total, int pad_j, const IdxT* idx,
+int launch_build_lists(int clouds, int m, int64_t cloud_total, int64_t part_total, const IdxT* idx,
                        const float* weight, const Lists<WEIGHTED>& lists, hipStream_t s)
 {
-    ListJob<WEIGHTED, IdxT> job, none{};
-    const int st = make_list_job<K, WEIGHTED, IdxT>(clouds, m, cloud_total, part_total, pad_j, L_WIDTH_STEP, idx, weight, lists, &job);
-    return st == TPK_OK ? launch_list_jobs<K, WEIGHTED, IdxT>(job, none, s) : st;
+    ListJob<WEIGHTED, IdxT> job;
+    const int st = make_list_job<K, WEIGHTED, IdxT>(clouds, m, cloud_total, part_total, idx, weight, lists, &job);
+    if (st != TPK_OK || job.workgroups == 0)
+        return st;
+    const size_t lds = (2 * static_cast<size_t>(job.span) + 2 * (job.span / L_BLOCK) + G_THREADS) * sizeof(int);
+    auto build = build_lists_kernel<K, WEIGHTED, IdxT>;
+    const int allowed = allow_lds(build, lds);
+    if (allowed != TPK_OK)
+        return allowed;
+    hipLaunchKernelGGL(build, dim3(static_cast<unsigned>(job.workgroups)), dim3(G_THREADS), lds, s, job);
+    return tpk_launch_status();
 }
 
 } // namespace

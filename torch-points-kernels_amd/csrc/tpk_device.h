@@ -10,6 +10,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "../../include/tpk.h"
 
 #pragma clang fp contract(off)
@@ -29,6 +33,39 @@ static inline int tpk_launch_status()
 {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TPK_OK : static_cast<int>(e);
+}
+
+// Lets `kernel` use up to `bytes` of dynamic LDS on the current device.  The runtime call behind it
+// is made once per kernel and device (again only when a larger size is asked for): a launch on
+// the hot path does a table look-up instead of a driver call.
+static inline int tpk_allow_lds(const void* kernel, size_t bytes)
+{
+    static std::mutex lock;
+    static std::map<std::pair<const void*, int>, size_t> allowed;
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    std::lock_guard<std::mutex> guard(lock);
+    size_t& have = allowed[std::make_pair(kernel, device)];
+    if (bytes <= have)
+        return TPK_OK;
+    // (sizes are rounded up so that slightly larger requests later seldom come back here)
+    size_t ask = (bytes + 16383) & ~static_cast<size_t>(16383);
+    if (ask > TPK_LDS_BYTES)
+        ask = bytes > TPK_LDS_BYTES ? bytes : TPK_LDS_BYTES;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(ask));
+    if (e != hipSuccess && ask != bytes)
+    {
+        // (the rounded size did not fit next to the kernel's static LDS: the exact one)
+        (void)hipGetLastError();
+        ask = bytes;
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(ask));
+    }
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    have = ask;
+    return TPK_OK;
 }
 
 static inline int64_t tpk_ceil_div(int64_t a, int64_t b)
