@@ -87,8 +87,10 @@ def test_library_exports_every_declared_symbol():
     # entry slots (3 per index entry + 832 per block of 64 targets; 8 B weighted, 4 B plain), per column piece
     lib.tpk_three_interpolate_grad_workspace_bytes.restype = ctypes.c_size_t
     assert lib.tpk_three_interpolate_grad_workspace_bytes(2, 1000, 100) == up(2 * 128 * 4) + up(2 * 2 * 8) + up(2 * (3 * 3000 + 832 * 2) * 8)
-    # 20000 columns: one row at a time in pieces of 16384 columns -> 2 pieces per cloud
-    assert lib.tpk_three_interpolate_grad_workspace_bytes(1, 20000, 64) == up(2 * 64 * 4) + up(2 * 1 * 8) + up(2 * (3 * 49152 + 832) * 8)
+    # 20000 columns: four rows at a time in pieces of 8192 columns -> 3 pieces per cloud, lists of 3 * 8192 entries each
+    assert lib.tpk_three_interpolate_grad_workspace_bytes(1, 20000, 64) == up(3 * 64 * 4) + up(3 * 1 * 8) + up(3 * (3 * 24576 + 832) * 8)
+    # 40000 columns: one row at a time in pieces of 32768 columns -> 2 pieces per cloud
+    assert lib.tpk_three_interpolate_grad_workspace_bytes(1, 40000, 64) == up(2 * 64 * 4) + up(2 * 1 * 8) + up(2 * (3 * 98304 + 832) * 8)
     lib.tpk_group_grad_workspace_bytes.restype = ctypes.c_size_t
     assert lib.tpk_group_grad_workspace_bytes(3, 70, 16, 8) == up(3 * 128 * 4) + up(3 * 2 * 8) + up(3 * (3 * 128 + 832 * 2) * 4)
     lib.tpk_chamfer_bwd_workspace_bytes.restype = ctypes.c_size_t
