@@ -9,7 +9,11 @@ checkout.
 
 Cases are chosen where the reference's CPU and CUDA paths compute the same thing (no equal
 distances, clouds away from the origin for FPS): nearest-neighbour searches, the sorted radius
-search, FPS started at point 0, three_interpolate.
+search, FPS started at point 0, three_interpolate.  For the package's host module (CPU tensors)
+the fixture also holds: the complete hit lists of the radius searches (what an unsorted search
+must draw its rows from), FPS with the random start the Python layer asks for (under a fixed seed
+of torch's default generator, which is where the reference draws the start from), the gradient of
+the interpolation, and a float64 search.
 """
 import os
 import sys
@@ -57,6 +61,27 @@ def main():
     w = w / w.sum(dim=2, keepdim=True)
     out.update(interp_features=feats, interp_idx=nn_idx, interp_weight=w,
                interp_out=ref.knn_interpolate(feats, nn_idx, w))  # cpu/src/interpolate.cpp
+
+    # --- added for the host module; everything above keeps its draws from the generator
+    idx, dist = ref.dense_ball_query(query, support, 0.15, 64, 0, True)  # wide enough for every hit list
+    assert int((dist[..., -1] >= 0).sum()) == 0, "64 columns must hold every hit"
+    out.update(ball_all_idx=idx, ball_all_dist=dist)
+    idx, dist = ref.batch_ball_query(x, y, bx, by, 0.12, 64, 0, True)
+    assert int((dist[..., -1] >= 0).sum()) == 0
+    out.update(packed_all_idx=idx, packed_all_dist=dist)
+
+    torch.manual_seed(4242)  # the reference draws the start point from torch's default generator (cpu/src/fps.cpp:24-25)
+    out.update(fps_random_seed=np.int64(4242), fps_random_idx=ref.fps(cloud, 64, True))
+
+    grad_out = torch.randn(2, 5, 300, generator=g)
+    out.update(interp_grad_out=grad_out, interp_grad=ref.knn_interpolate_grad(grad_out, nn_idx, w, 80))
+
+    support64 = torch.rand(2, 300, 3, generator=g, dtype=torch.float64)
+    query64 = torch.rand(2, 40, 3, generator=g, dtype=torch.float64)
+    idx, dist2 = ref.dense_knn(support64, query64, 5)
+    out.update(knn64_support=support64, knn64_query=query64, knn64_idx=idx, knn64_dist2=dist2)
+    idx, dist = ref.dense_ball_query(query64, support64, 0.2, 10, 0, True)
+    out.update(ball64_radius=np.float32(0.2), ball64_idx=idx, ball64_dist=dist)
 
     arrays = {k: (v.numpy() if isinstance(v, torch.Tensor) else np.asarray(v)) for k, v in out.items()}
     path = os.path.join(HERE, "reference_cpu_vectors.npz")

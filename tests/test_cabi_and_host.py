@@ -158,21 +158,36 @@ def test_python_api_errors_match_the_reference(tpk):
         ChamferFunction.apply(x, x)
 
 
-def test_cpu_tensors_raise_instead_of_falling_back(tpk):
+def test_tensors_are_served_by_the_module_of_their_device(tpk, monkeypatch):
+    """CPU tensors go to points_cpu, never to the HIP extension; and a GPU tensor whose extension is missing raises
+    instead of being served by the host module (checked by making the loader fail: the dispatch looks at is_cuda only)."""
+    from torch_points_kernels import _native, torchpoints
+
     x = torch.rand(1, 16, 3)
-    with pytest.raises(NotImplementedError):
-        tpk.ball_query(0.5, 4, x, x)
-    with pytest.raises(NotImplementedError):
-        tpk.furthest_point_sample(x, 4)
-    with pytest.raises(NotImplementedError):
-        tpk.three_nn(x, x)
-    with pytest.raises(NotImplementedError):
-        tpk.three_interpolate(torch.rand(1, 2, 16), torch.zeros(1, 16, 3, dtype=torch.int32), torch.rand(1, 16, 3))
-    with pytest.raises(NotImplementedError):
-        tpk.grouping_operation(torch.rand(1, 2, 16), torch.zeros(1, 4, 2, dtype=torch.long))
+    idx, dist = tpk.ball_query(0.5, 4, x, x, sort=True)
+    assert idx.dtype == torch.int64 and not idx.is_cuda and idx[0, :, 0].tolist() == list(range(16))
+    assert tpk.furthest_point_sample(x, 4).dtype == torch.int64  # the reference's CPU convention
+    assert tpk.three_nn(x, x)[1].dtype == torch.int64
+
+    class FakeGpuTensor:
+        is_cuda = True
+        shape = (1, 16, 3)
+
+    def missing():
+        raise ImportError("points_cuda is not built")
+
+    monkeypatch.setattr(torchpoints, "native", missing)
+    monkeypatch.setattr(torchpoints, "host", lambda: pytest.fail("a GPU tensor must not reach the host module"))
+    with pytest.raises(ImportError):
+        tpk.furthest_point_sample(FakeGpuTensor(), 4)
+    with pytest.raises(ImportError):
+        torchpoints.ball_query_dense(0.5, 4, FakeGpuTensor(), FakeGpuTensor())
+    with pytest.raises(ImportError):
+        torchpoints.ball_query_partial_dense(0.5, 4, FakeGpuTensor(), FakeGpuTensor(), None, None)
+    assert _native.native is not missing
 
 
-def test_added_operators_raise_for_cpu_tensors_and_bad_shapes(tpk):
+def test_gpu_only_operators_raise_for_cpu_tensors_and_bad_shapes(tpk):
     from torch_points_kernels.cluster import grow_proximity, region_grow
     from torch_points_kernels.cubic_feature_sampling import cubic_feature_sampling
     from torch_points_kernels.gridding import gridding
@@ -180,20 +195,16 @@ def test_added_operators_raise_for_cpu_tensors_and_bad_shapes(tpk):
 
     pos = torch.rand(20, 3)
     batch = torch.zeros(20, dtype=torch.long)
-    with pytest.raises(NotImplementedError):
-        tpk.knn(pos.unsqueeze(0), pos.unsqueeze(0), 3)
-    with pytest.raises(NotImplementedError):
-        tpk.ball_query(0.5, 4, pos.unsqueeze(0), pos.unsqueeze(0), sort=True)
-    with pytest.raises(NotImplementedError):
-        grow_proximity(pos, batch)
-    with pytest.raises(NotImplementedError):
-        region_grow(pos, torch.zeros(20, dtype=torch.long), batch)
     with pytest.raises(AssertionError):
         region_grow(pos, torch.zeros(20, 1, dtype=torch.long), batch)  # reference cluster.py:71
     with pytest.raises(ValueError):
         grow_proximity(pos, batch, member_order="sorted")
+    # the operators the reference has no CPU path for refuse CPU tensors (reference: chamfer_dist.py:10-11; its
+    # gridding.py and cubic_feature_sampling.py call the CUDA module unconditionally)
     with pytest.raises(NotImplementedError):
-        instance_iou([torch.tensor([0, 1])], torch.tensor([1, 1, 0]))
+        gridding(torch.rand(1, 10, 3), 4)
+    with pytest.raises(NotImplementedError):
+        cubic_feature_sampling(torch.rand(1, 10, 3), torch.rand(1, 2, 4, 4, 4))
     # reference gridding.py:50-51, cubic_feature_sampling.py:53-54
     with pytest.raises(ValueError):
         gridding(torch.rand(10, 3), 4)

@@ -701,8 +701,7 @@ def test_knn_ties_and_errors(tpk, oracle, dev):
     assert tpk.knn(support, query, 2)[0].tolist() == [[[0, 1]]]
     with pytest.raises(RuntimeError):
         tpk.knn(support, query, 5)
-    with pytest.raises(NotImplementedError):
-        tpk.knn(support.cpu(), query.cpu(), 2)
+    assert tpk.knn(support.cpu(), query.cpu(), 2)[0].tolist() == [[[0, 1]]]  # CPU tensors: the host module
     # equal distances everywhere: tripled points, lattices, a collapsed cloud; small and large clouds
     g = torch.Generator().manual_seed(8)
     base = torch.rand(1, 400, 3, generator=g)
@@ -756,8 +755,7 @@ def test_kat_region_grow(tpk, dev):
         assert all(c.is_cuda and c.dtype == torch.int64 for c in clusters)
         clusters = region_grow(pos, labels, batch, ignore_labels=[1, 10], radius=2, min_cluster_size=1, member_order=order)
         assert [c.tolist() for c in clusters] == [[0, 1], [4]]
-    with pytest.raises(NotImplementedError):
-        grow_proximity(pos.cpu(), batch.cpu(), radius=2)
+    assert grow_proximity(pos.cpu(), batch.cpu(), radius=2, min_cluster_size=1) == [[0, 1, 2], [3], [4, 5, 6], [7]]  # host module
     with pytest.raises(ValueError):
         grow_proximity(pos, batch, radius=2, member_order="sorted")
 
@@ -837,8 +835,8 @@ def test_kat_instance_iou(tpk, dev):
     ious = instance_iou([torch.tensor([0, 1]).to(dev), torch.tensor([3, 4]).to(dev), torch.tensor([5]).to(dev)], gt, batch=batch)
     want = torch.tensor([[0.5, 0.5, 0, 0, 0], [0, 0, 0, 1, 0], [0, 0, 0, 0, 1.0]])
     torch.testing.assert_close(ious.cpu(), want, rtol=1e-4, atol=1e-5)
-    with pytest.raises(NotImplementedError):
-        instance_iou([torch.tensor([0, 2])], gt.cpu())
+    host_ious = instance_iou([torch.tensor([0, 2])], gt.cpu())  # CPU tensors: the host module
+    assert host_ious.tolist() == [[1.0, 0.0, 0.0]] and not host_ious.is_cuda
 
 
 @pytest.mark.parametrize("samples,points,instances,proposals,longest", [(1, 1000, 9, 20, 50), (3, 5000, 40, 300, 700),

@@ -2,6 +2,7 @@
 
   csrc/*.hip          -> torch_points_kernels/libtpk_hip.so   (HIP kernels + C ABI, no torch)
   csrc/points_cuda.cpp -> torch_points_kernels/points_cuda.so  (pybind11 module over the C ABI)
+  csrc/points_cpu.cpp  -> torch_points_kernels/points_cpu.so   (operators for CPU tensors; host code only, no HIP)
   csrc/*.hip          -> torch_points_kernels/libtpk_hip_counting.so: the same library with the
                          distance scans compiled -DTPK_COUNT_WORK (they count the pair
                          evaluations they execute; include/tpk_counting.h).  Measurement only:
@@ -117,9 +118,33 @@ def build_extension(force=False):
     return out
 
 
+def build_cpu_extension(force=False):
+    """The module that serves CPU tensors: plain host C++ (g++), linked against torch only."""
+    import torch
+    from torch.utils import cpp_extension
+
+    src = os.path.join(CSRC, "points_cpu.cpp")
+    out = os.path.join(PKG, "points_cpu.so")
+    deps = [src] + glob.glob(os.path.join(CSRC, "cpu", "*.h"))
+    if not force and _newer(out, deps):
+        return out
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    # -ffp-contract=off: distances round every operation on its own, as in the GPU kernels
+    cmd = ["g++", "-O3", "-std=c++17", "-fPIC", "-shared", "-w", "-fopenmp", "-ffp-contract=off",
+           "-DTORCH_EXTENSION_NAME=points_cpu", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-I" + CSRC]
+    for inc in cpp_extension.include_paths(device_type="cpu") + [sysconfig.get_paths()["include"]]:
+        cmd.append("-I" + inc)
+    cmd += [src, "-o", out, "-L" + torch_lib, "-Wl,-rpath," + torch_lib,
+            "-lc10", "-ltorch_cpu", "-ltorch", "-ltorch_python"]
+    _run(cmd)
+    return out
+
+
 def build(force=False):
     lib = build_kernels(force)
     ext = build_extension(force)
+    build_cpu_extension(force)
     return lib, ext
 
 

@@ -2,8 +2,9 @@
 torch-points3d/torch-points-kernels (furthest point sampling, ball query, three_nn /
 three_interpolate, grouping, Chamfer distance, dense knn, region growing, instance IoU, GRNet's gridding and cubic feature sampling) on hand-written HIP kernels.
 
-Same names and call signatures as the reference package (torch_points_kernels/__init__.py);
-GPU tensors only.
+Same names and call signatures as the reference package (torch_points_kernels/__init__.py).  GPU
+tensors run on the HIP kernels (points_cuda); CPU tensors are served by the host module (points_cpu)
+for the operators the reference serves on the CPU.
 """
 from .torchpoints import (
     ThreeInterpolate,

@@ -1,5 +1,5 @@
 """Dense k nearest neighbours (API of the reference's torch_points_kernels/knn.py)."""
-from ._native import native, require_gpu
+from ._native import host, native
 
 
 def knn(pos_support, pos, k):
@@ -9,10 +9,12 @@ def knn(pos_support, pos, k):
     Returns (idx (B, M, k) int64, dist2 (B, M, k) squared distances), nearest first; equal distances
     keep the lower index first.
 
-    The reference (knn.py:4-18) serves CPU tensors only and raises for CUDA tensors; this build serves
-    GPU tensors only.
+    The reference (knn.py:4-18) serves CPU tensors only and raises for CUDA tensors; here CPU tensors go
+    to the host module and GPU tensors to the HIP kernels.
     """
     assert pos_support.dim() == 3 and pos.dim() == 3
-    require_gpu(pos_support, "knn")
-    require_gpu(pos, "knn")
-    return native().dense_knn(pos_support, pos, k)
+    if pos_support.is_cuda != pos.is_cuda:
+        raise ValueError("pos_support and pos must live on the same device")
+    if pos_support.is_cuda:
+        return native().dense_knn(pos_support, pos, k)
+    return host().dense_knn(pos_support, pos, k)

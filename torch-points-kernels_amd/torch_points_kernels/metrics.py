@@ -3,7 +3,7 @@ from typing import List, Optional
 
 import torch
 
-from ._native import native, require_gpu
+from ._native import host, native
 
 
 def instance_iou(
@@ -19,9 +19,9 @@ def instance_iou(
     Returns float32 (number of proposals, ground-truth instances of all samples); a proposal is compared
     with the instances of the sample its first point belongs to, the other columns are 0.
 
-    Reference: metrics.py:37-104; GPU tensors only here.
+    Reference: metrics.py:37-104.  As there, the GPU kernel adds 1e-5 to the union and the host routine
+    does not.
     """
-    require_gpu(gt_instances, "instance_iou")
     if batch is None:
         batch = torch.zeros_like(gt_instances)
 
@@ -49,6 +49,15 @@ def instance_iou(
         instance_offsets.append(cum_offset)
 
     instance_idx = torch.cat(instance_idx) if len(instance_idx) else torch.zeros(0, dtype=torch.long, device=device)
+    if not gt_instances.is_cuda:
+        return host().instance_iou(
+            instance_idx.long().contiguous(),
+            torch.tensor(instance_offsets, dtype=torch.long),
+            gt_instances.long().contiguous(),
+            gt_instance_sizes.long().contiguous(),
+            num_gt_instances,
+            batch.long().contiguous(),
+        )
     return native().instance_iou_cuda(
         instance_idx.to(device).long().contiguous(),
         torch.tensor(instance_offsets, dtype=torch.long, device=device),
