@@ -1159,6 +1159,134 @@ def test_c_abi_direct_call(oracle, dev):
     assert st == -3
 
 
+def test_c_abi_direct_call_every_family(oracle, dev):
+    """One call per family of entry points through ctypes (no extension in between): furthest point sampling, ball query
+    in both layouts with and without workspace, the gathers forward and backward, Chamfer forward and backward -
+    compared with the checker like the calls through the Python layer."""
+    import ctypes
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = ctypes.CDLL(os.path.join(root, "torch-points-kernels_amd", "torch_points_kernels", "libtpk_hip.so"))
+    for name in ("tpk_fps_workspace_bytes", "tpk_ball_query_partial_workspace_bytes", "tpk_three_interpolate_grad_workspace_bytes",
+                 "tpk_group_grad_workspace_bytes", "tpk_chamfer_fwd_workspace_bytes"):
+        getattr(lib, name).restype = ctypes.c_size_t
+    lib.tpk_ball_query_partial_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    F = ctypes.c_float
+    Z = ctypes.c_size_t
+    L = ctypes.c_int64
+    stream = torch.cuda.Stream()
+    S = ctypes.c_void_p(stream.cuda_stream)
+    g = torch.Generator().manual_seed(31)
+
+    def workspace(nbytes):
+        return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=dev)
+
+    def run(call):
+        stream.wait_stream(torch.cuda.current_stream())
+        assert call() == 0
+        stream.synchronize()
+
+    # furthest point sampling: a cloud held in registers, and one that needs the workspace
+    for n, npoint in ((3000, 100), (20000, 40)):
+        xyz = torch.rand(2, n, 3, generator=g) + 0.2
+        d = xyz.to(dev)
+        out = torch.full((2, npoint), -1, dtype=torch.int32, device=dev)
+        nbytes = lib.tpk_fps_workspace_bytes(2, n)
+        ws = workspace(nbytes)
+        run(lambda: lib.tpk_fps_f32(2, n, npoint, P(d), P(ws) if nbytes else None, Z(nbytes), P(out), S))
+        np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.numpy(), npoint))
+
+    # ball query, dense layout
+    xyz, centres = torch.rand(2, 2500, 3, generator=g), torch.rand(2, 300, 3, generator=g)
+    dx, dc = xyz.to(dev), centres.to(dev)
+    idx = torch.full((2, 300, 12), -7, dtype=torch.int64, device=dev)
+    dist = torch.full((2, 300, 12), -7.0, device=dev)
+    run(lambda: lib.tpk_ball_query_dense_f32(2, 2500, 300, F(0.12), 12, P(dc), P(dx), P(idx), P(dist), S))
+    wi, wd = oracle.ball_query_dense(0.12, 12, xyz.numpy(), centres.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist), wd)
+
+    # ball query, packed layout: all pairs (no workspace) and the walk over bins (workspace)
+    sizes = [9000, 400, 12000]
+    x = torch.rand(sum(sizes), 3, generator=g)
+    bx = torch.repeat_interleave(torch.arange(3), torch.tensor(sizes))
+    pick = torch.sort(torch.randperm(sum(sizes), generator=g)[:5000])[0]
+    y, by = x[pick].contiguous(), bx[pick].contiguous()
+    dxp, dyp, dbx, dby = x.to(dev), y.to(dev), bx.to(dev), by.to(dev)
+    wi, wd = oracle.ball_query_partial_dense(0.05, 16, x.numpy(), y.numpy(), bx.numpy(), by.numpy())
+    nbytes = lib.tpk_ball_query_partial_workspace_bytes(L(x.shape[0]), L(y.shape[0]), 16)
+    assert nbytes > 0
+    ws = workspace(nbytes)
+    for ws_ptr, ws_bytes in ((None, 0), (P(ws), nbytes)):
+        idx = torch.full((y.shape[0], 16), -7, dtype=torch.int64, device=dev)
+        dist = torch.full((y.shape[0], 16), -7.0, device=dev)
+        run(lambda: lib.tpk_ball_query_partial_f32(L(x.shape[0]), L(y.shape[0]), F(0.05), 16, P(dxp), P(dyp), P(dbx), P(dby),
+                                                   P(idx), P(dist), ws_ptr, Z(ws_bytes), S))
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist), wd)
+
+    # three_interpolate forward and backward (lists in the workspace, then global atomics without it)
+    b, c, m, n = 2, 9, 700, 5000
+    feats = torch.randn(b, c, m, generator=g)
+    nn = torch.randint(0, m, (b, n, 3), generator=g).int()
+    w = torch.rand(b, n, 3, generator=g)
+    gout = torch.randn(b, c, n, generator=g)
+    df, dn, dw, dg = feats.to(dev), nn.to(dev), w.to(dev), gout.to(dev)
+    out = torch.empty(b, c, n, device=dev)
+    run(lambda: lib.tpk_three_interpolate_f32(b, c, m, n, P(df), P(dn), P(dw), P(out), S))
+    np.testing.assert_array_equal(_np(out), oracle.three_interpolate(feats.numpy(), nn.numpy(), w.numpy()))
+    want = oracle.three_interpolate_grad(gout.numpy(), nn.numpy(), w.numpy(), m)
+    abs_sum = oracle.three_interpolate_grad(gout.abs().numpy(), nn.numpy(), w.numpy(), m)
+    nbytes = lib.tpk_three_interpolate_grad_workspace_bytes(b, n, m)
+    assert nbytes > 0
+    ws = workspace(nbytes)
+    for ws_ptr, ws_bytes in ((P(ws), nbytes), (None, 0)):
+        grad = torch.full((b, c, m), 7.0, device=dev)
+        run(lambda: lib.tpk_three_interpolate_grad_f32(b, c, n, m, P(dg), P(dn), P(dw), P(grad), ws_ptr, Z(ws_bytes), S))
+        _assert_scatter_sum_close(_np(grad), want, abs_sum)
+
+    # grouping forward and backward
+    b, c, n, npoint, nsample = 2, 6, 900, 300, 8
+    feats = torch.randn(b, c, n, generator=g)
+    gi = torch.randint(0, n, (b, npoint, nsample), generator=g)
+    gout = torch.randn(b, c, npoint, nsample, generator=g)
+    df, di, dg = feats.to(dev), gi.to(dev), gout.to(dev)
+    out = torch.empty(b, c, npoint, nsample, device=dev)
+    run(lambda: lib.tpk_group_f32(b, c, n, npoint, nsample, P(df), P(di), P(out), S))
+    np.testing.assert_array_equal(_np(out), oracle.grouping_operation(feats.numpy(), gi.numpy()))
+    nbytes = lib.tpk_group_grad_workspace_bytes(b, n, npoint, nsample)
+    ws = workspace(nbytes)
+    grad = torch.full((b, c, n), 7.0, device=dev)
+    run(lambda: lib.tpk_group_grad_f32(b, c, n, npoint, nsample, P(dg), P(di), P(grad), P(ws), Z(nbytes), S))
+    _assert_scatter_sum_close(_np(grad), oracle.grouping_operation_grad(gout.numpy(), gi.numpy(), n),
+                              oracle.grouping_operation_grad(gout.abs().numpy(), gi.numpy(), n))
+
+    # Chamfer forward (all pairs, then the cell search) and backward
+    b, n, m = 2, 3000, 2100
+    a, c2 = torch.rand(b, n, 3, generator=g), torch.rand(b, m, 3, generator=g)
+    da, dc2 = a.to(dev), c2.to(dev)
+    w1, w2, wi1, wi2 = oracle.chamfer_fwd(a.numpy(), c2.numpy())
+    nbytes = lib.tpk_chamfer_fwd_workspace_bytes(b, n, m)
+    assert nbytes > 0
+    ws = workspace(nbytes)
+    for ws_ptr, ws_bytes in ((None, 0), (P(ws), nbytes)):
+        d1, d2 = torch.empty(b, n, device=dev), torch.empty(b, m, device=dev)
+        i1 = torch.empty(b, n, dtype=torch.int32, device=dev)
+        i2 = torch.empty(b, m, dtype=torch.int32, device=dev)
+        run(lambda: lib.tpk_chamfer_fwd_f32(b, n, m, P(da), P(dc2), P(d1), P(d2), P(i1), P(i2), ws_ptr, Z(ws_bytes), S))
+        for got, want in ((d1, w1), (d2, w2), (i1, wi1), (i2, wi2)):
+            np.testing.assert_array_equal(_np(got), want)
+    g1, g2 = torch.randn(b, n, generator=g), torch.randn(b, m, generator=g)
+    dg1, dg2 = g1.to(dev), g2.to(dev)
+    ga, gb = torch.full((b, n, 3), 7.0, device=dev), torch.full((b, m, 3), 7.0, device=dev)
+    run(lambda: lib.tpk_chamfer_bwd_f32(b, n, m, P(da), P(dc2), P(i1), P(i2), P(dg1), P(dg2), P(ga), P(gb), None, Z(0), S))
+    wa, wb = oracle.chamfer_bwd(a.numpy(), c2.numpy(), wi1, wi2, g1.numpy(), g2.numpy())
+    np.testing.assert_allclose(_np(ga), wa, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(_np(gb), wb, rtol=RTOL, atol=ATOL)
+
+
 def test_counting_build_counts_executed_pairs(oracle, dev):
     """The counting build of the library returns the same results and counts the pair evaluations its lanes
     execute: a brute-force three_nn of 256 queries against 100 points = 256 lanes x 100 candidates; the search
