@@ -1114,6 +1114,20 @@ def test_chamfer_full_config5(tpk, oracle, dev):
 # ------------------------------------------------------------------ the C ABI called directly
 
 
+def test_gridding_last_cell_matches_the_reference_formula_inside_the_grid(tpk, dev):
+    """Vertices inside the grid carry the index and weight of the reference's formula (gridding_gpu.cu:17-20, 43-131);
+    the vertices of a point in the last cell that lie outside get -1 and deposit nothing, where the reference adds
+    their weight to a wrapped cell (y, z) or beyond the cloud's grid (x)."""
+    from tests.test_oracle_pinning import check_last_cell_behaviour
+    from torch_points_kernels._native import native
+
+    def gridding(points, scale):
+        g, w, i = native().gridding(-scale, scale - 1, -scale, scale - 1, -scale, scale - 1, torch.from_numpy(points).to(dev))
+        return _np(g), _np(w), _np(i)
+
+    check_last_cell_behaviour(gridding)
+
+
 def test_c_abi_direct_call(oracle, dev):
     """libtpk_hip.so used without the extension: ctypes + raw device pointers + a stream."""
     import ctypes

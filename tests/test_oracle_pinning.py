@@ -647,6 +647,61 @@ def test_gridding_matches_trilinear_closed_form(oracle):
     np.testing.assert_allclose(oracle.gridding(inner, scale)[0].sum(), 40, rtol=1e-12)
 
 
+def reference_formula_vertices(point, scale):
+    """The 8 (linear index, weight) pairs gridding_gpu.cu:43-131 forms for one point in grid units: floor / ceil per
+    axis (ceil + 1 on a vertex), offsets from -scale, index = (ox * len + oy) * len + oz formed WITHOUT a range check,
+    weight = product of 1 - |p - vertex| per axis.  Order LLL, LLU, LUL, LUU, ULL, ULU, UUL, UUU."""
+    side = 2 * scale
+    lo = np.floor(point).astype(int)
+    hi = np.ceil(point).astype(int)
+    hi = np.where(hi == lo, lo + 1, hi)
+    out = []
+    for cx in (lo[0], hi[0]):
+        for cy in (lo[1], hi[1]):
+            for cz in (lo[2], hi[2]):
+                index = ((cx + scale) * side + (cy + scale)) * side + (cz + scale)
+                weight = (1 - abs(point[0] - cx)) * (1 - abs(point[1] - cy)) * (1 - abs(point[2] - cz))
+                inside = all(0 <= c + scale < side for c in (cx, cy, cz))
+                out.append((index, weight, inside))
+    return out
+
+
+LAST_CELL_POINTS = {
+    # a point in the last cell of one axis: its upper vertices on that axis lie outside the grid
+    "z": np.array([0.25, -1.5, 2.6]), "y": np.array([-2.75, 2.3, 0.5]), "x": np.array([2.4, 1.25, -0.5]),
+}
+
+
+def check_last_cell_behaviour(gridding, scale=3):
+    """For a vertex outside the grid the reference's formula still yields an index: past the last z it is the cell
+    (x, y + 1, 0), past the last y the cell (x + 1, 0, z) - the weight lands in a cell far from the point - and past
+    the last x it lies beyond the cloud's grid (the next cloud's memory).  Here such a vertex gets index -1 and deposits
+    nothing; every vertex inside the grid has exactly the reference formula's index and weight."""
+    for axis, point in LAST_CELL_POINTS.items():
+        grid, weights, indexes = gridding(point[None, None, :].astype(np.float64), scale)
+        want = np.zeros((2 * scale) ** 3)
+        outside = 0
+        for v, (index, weight, inside) in enumerate(reference_formula_vertices(point, scale)):
+            if inside:
+                assert indexes[0, 0, v] == index, (axis, v)
+                want[index] += weight
+            else:
+                outside += 1
+                assert indexes[0, 0, v] == -1, (axis, v)
+                if axis != "x":  # where the reference would have added it: a cell of the grid, not next to the point
+                    assert 0 <= index < want.size and want[index] == 0
+                else:
+                    assert index >= want.size
+            np.testing.assert_allclose(weights[0, 0, v].prod(), weight, rtol=1e-12)
+        assert outside == 4, axis
+        np.testing.assert_allclose(grid[0], want, rtol=1e-12, atol=1e-15)
+        assert abs(grid.sum() - sum(w for _, w, ins in reference_formula_vertices(point, scale) if ins)) < 1e-12
+
+
+def test_gridding_last_cell_drops_the_vertices_outside(oracle):
+    check_last_cell_behaviour(oracle.gridding)
+
+
 def test_gridding_grad_matches_finite_differences(oracle):
     rng = np.random.default_rng(2)
     scale = 3
