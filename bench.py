@@ -38,9 +38,9 @@ VALU_FILE = os.path.join(PROFILES, "distance_scans_valu_utilisation.txt")
 TRAFFIC_KERNELS = {
     "fps": ["fps_pruned_kernel<32, 512, 4>"],
     "three_interpolate_fwd": ["gather_fwd_lds_kernel<3, true, int, true>"],
-    "three_interpolate_bwd": ["build_lists_kernel<3, true, int>", "gather_bwd_lists_kernel<3, true, 4, true>"],
+    "three_interpolate_bwd": ["build_lists_kernel<3, true, int>", "gather_bwd_lists_kernel<3, true, 2>"],
     "grouping_fwd": ["gather_fwd_lds_kernel<1, false, long, false>"],
-    "grouping_bwd": ["build_lists_kernel<1, false, long>", "gather_bwd_lists_kernel<1, false, 4, true>"],
+    "grouping_bwd": ["build_lists_kernel<1, false, long>", "gather_bwd_lists_kernel<1, false, 1>"],
     "chamfer_bwd": ["chamfer_bwd_chains_kernel<float>"],
 }
 # Kernels whose VALU counters describe a distance scan.

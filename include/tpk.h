@@ -183,8 +183,10 @@ int tpk_knn_f32(int b, int n_support, int m_query, int k, const float* support, 
  *   grad_points (b, c, m) += grad_out (b, c, n) scattered back (fully written, no pre-zero)
  * The backward pass inverts the index into per-target lists held in `workspace`
  * (tpk_three_interpolate_grad_workspace_bytes() bytes, 256-byte aligned; contents need not
- * be initialised and are garbage afterwards).  With workspace == NULL, or for shapes
- * the lists do not serve, it falls back to global float atomics - same result to rounding, much slower.
+ * be initialised and are garbage afterwards; about one entry of 8 bytes per index entry and
+ * per target).  With workspace == NULL, or for shapes the lists do not serve (m above about
+ * 36000: the sums of one row then leave no room in LDS; tpk_..._workspace_bytes() returns 0),
+ * it falls back to global float atomics - same result to rounding, much slower.
  * Index values outside [0, m) are ignored by the list path.
  * ------------------------------------------------------------------------------------- */
 int tpk_three_interpolate_f32(int b, int c, int m, int n, const float* points,

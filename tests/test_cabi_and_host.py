@@ -83,16 +83,19 @@ def test_library_exports_every_declared_symbol():
     assert fn(2, 4096, 100) == support_only(2, 4096)
     assert fn(2, 200000, 1000) == support_only(2, 200000)
     assert fn(2, 700, 900) == sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((11, 1024), (15, 1024), (11, 160), (15, 160)))
-    # list-based backward passes: counts (4 B per target, blocks of 64), block descriptions (8 B per block),
-    # entry slots (3 per index entry + 832 per block of 64 targets; 8 B weighted, 4 B plain), per column piece
+    # list-based backward passes, per cloud part (a part = up to 32768 columns): 16 regions (16 B each), the first
+    # target of 16 x 64 lanes (4 B each), and entry slots for every index entry, one empty entry per target, the
+    # rounding to rows of 64 and the gaps between the 16 regions (8 B weighted, 4 B plain)
+    slots = lambda m, total: -(-(total + m) // 64) * 64 + 128 * 16 + 64
+    lists = lambda parts, m, total, size: up(parts * 16 * 16) + up(parts * 16 * 64 * 4) + up(parts * slots(m, total) * size)
     lib.tpk_three_interpolate_grad_workspace_bytes.restype = ctypes.c_size_t
-    assert lib.tpk_three_interpolate_grad_workspace_bytes(2, 1000, 100) == up(2 * 128 * 4) + up(2 * 2 * 8) + up(2 * (3 * 3000 + 832 * 2) * 8)
-    # 20000 columns: four rows at a time in pieces of 8192 columns -> 3 pieces per cloud, lists of 3 * 8192 entries each
-    assert lib.tpk_three_interpolate_grad_workspace_bytes(1, 20000, 64) == up(3 * 64 * 4) + up(3 * 1 * 8) + up(3 * (3 * 24576 + 832) * 8)
-    # 40000 columns: one row at a time in pieces of 32768 columns -> 2 pieces per cloud
-    assert lib.tpk_three_interpolate_grad_workspace_bytes(1, 40000, 64) == up(2 * 64 * 4) + up(2 * 1 * 8) + up(2 * (3 * 98304 + 832) * 8)
+    assert lib.tpk_three_interpolate_grad_workspace_bytes(2, 1000, 100) == lists(2, 100, 3000, 8)
+    # 20000 columns: one part of 20000 columns (rows go one at a time)
+    assert lib.tpk_three_interpolate_grad_workspace_bytes(1, 20000, 64) == lists(1, 64, 60000, 8)
+    # 40000 columns: two parts of 32768 columns
+    assert lib.tpk_three_interpolate_grad_workspace_bytes(1, 40000, 64) == lists(2, 64, 3 * 32768, 8)
     lib.tpk_group_grad_workspace_bytes.restype = ctypes.c_size_t
-    assert lib.tpk_group_grad_workspace_bytes(3, 70, 16, 8) == up(3 * 128 * 4) + up(3 * 2 * 8) + up(3 * (3 * 128 + 832 * 2) * 4)
+    assert lib.tpk_group_grad_workspace_bytes(3, 70, 16, 8) == lists(3, 70, 128, 4)
     lib.tpk_chamfer_bwd_workspace_bytes.restype = ctypes.c_size_t
     # the Chamfer backward keeps its chains in LDS: no workspace
     assert lib.tpk_chamfer_bwd_workspace_bytes(2, 300, 515) == 0

@@ -15,14 +15,14 @@
 // about 190 cycles whatever the address pattern, against 8 for a random LDS read), so the
 // scatter is turned into a gather: a first kernel inverts the index of each cloud into
 // per-target lists (for target position i the columns j that reference it, with their
-// weights) using LDS *integer* atomics, which are fast, and an LDS prefix sum, laid out so that
-// one lane per target can walk them with coalesced reads (lists.h); the main kernel then
-// stages rows of grad_out in LDS - four rows in pieces of 8192 columns, or one longer row in
-// pieces of 16384 columns, with lists per piece - and every lane sums the listed columns of
-// its target.  No float atomics, no zero fill, each output written by one lane.  The lists cost
-// about 3 entries of 8 bytes (4 unweighted) per index entry of workspace, passed in by the
-// caller.  The order in which a target's terms are added differs from run to run only through
-// the order of its list, as with the reference's global atomics
+// weights) using LDS *integer* atomics, which are fast, and deals the sorted entries to the
+// lanes of sixteen wavefronts in equally long runs (lists.h); the main kernel then stages
+// whole rows of grad_out in LDS - four, two or one at a time, whatever leaves room for the
+// sums -, every lane adds up its run, one random LDS read per entry and row, and the sums
+// leave as contiguous stores.  No float atomics, no zero fill, each output written once.  The
+// lists cost about one entry of 8 bytes (4 unweighted) per index entry and target of
+// workspace, passed in by the caller.  The order in which a target's terms are added differs
+// from run to run only through the order of its list, as with the reference's global atomics
 // (cuda/src/interpolate_gpu.cu:122-152): results agree to rounding.
 //
 // Forward rows too long for LDS, or a backward call without workspace, take a direct path:
@@ -169,252 +169,105 @@ __global__ __launch_bounds__(G_THREADS) void gather_fwd_lds_kernel(
     }
 }
 
-constexpr int GB_STAGE_FLOATS = 32768; // floats of grad_out a workgroup keeps in LDS (128 KiB)
-constexpr int GB_WAVES = G_THREADS / TPK_WAVE;
-constexpr int GB_WALK_WAVES = GB_WAVES;
+constexpr int GB_LDS_FLOATS = TPK_LDS_BYTES / 4; // floats of LDS a workgroup of the backward walk may use (all 160 KiB)
+constexpr int GB_STAGE_FLOATS = 32768; // at most this many of them hold the staged piece of grad_out (128 KiB)
 constexpr int GB_FETCH = GB_STAGE_FLOATS / 4 / G_THREADS; // 16-byte loads per lane that bring in a piece: 8
-constexpr int GB_KEPT_BLOCKS = 4;      // blocks of 64 targets per wavefront whose sums stay in registers
-constexpr int GB_STEPS = L_WIDTH_STEP / 2; // list slots requested together (widths are multiples of twice that)
+constexpr int GB_AHEAD = 8;            // rows of list entries a wavefront has requested ahead of the one it adds
 
 typedef int int2_vec __attribute__((ext_vector_type(2)));
 
-// The entries of a cloud's lists as a buffer resource: a load whose offset lies beyond the buffer
-// returns zero and fetches nothing, so a lane without an entry in some step is given such an
-// offset instead of a branch around the load.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t entry_buffer(const void* base, uint32_t bytes)
+// A run of device memory as a buffer resource: a load whose offset lies beyond it returns zero and
+// fetches nothing, a store beyond it is dropped.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t memory_buffer(const void* base, uint32_t bytes)
 {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
 }
-constexpr uint32_t GB_NO_ENTRY = 0x80000000u; // a byte offset beyond every entry buffer (and below 2^32 with a round's offsets added)
 
-// What a walking wavefront does for one piece (see gather_bwd_lists_kernel): the sums of the lists of
-// its blocks (block walker + 16 b) over the columns of the piece.  KEEP: added to `kept` (lane = target)
-// and stored after the unit's last part; otherwise added to what the parts before stored.
-// STRIDE: floats from one staged row to the next when known at compile time, else 0 (`stride`).
-// `between(b)` is called once per block position b = 0 .. GB_KEPT_BLOCKS - 1 (KEEP) after that block's first
-// entries have been requested: the place for other memory requests that should not hold the walk up.
-template <int K, bool WEIGHTED, int R, bool KEEP, unsigned STRIDE, typename Between>
-__device__ __forceinline__ void walk_piece(const float* rows, unsigned stride, int piece, int unit0, int parts,
-                                           int row_groups, int c, int m, int nblocks, int walker, int lane,
-                                           const Lists<WEIGHTED>& lists, float* __restrict__ grad_src,
-                                           float (*kept)[R], Between&& between)
+// Sum over the lanes before this one, back to and including the nearest lane whose `starts` is set
+// (all lanes before it if there is none): what the lists that began in earlier lanes' runs carry into
+// this lane's run.  `open` = what a lane's run adds to the list that is still open at its end;
+// `starts` = the run ended at least one list, so that `open` begins a new sum.
+template <int R>
+__device__ __forceinline__ void carried_in(const float (&open)[R], bool starts, int lane, float (&carry)[R])
 {
-    const unsigned row_bytes = (STRIDE ? STRIDE : stride) * 4u;
-    const char* const staged = reinterpret_cast<const char*>(rows);
-    constexpr int STEPS = GB_STEPS; // list slots requested per round
-    constexpr uint32_t ENTRY_BYTES = sizeof(ListEntry<WEIGHTED>);
-    const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
-    const int cloud = unit / row_groups, c0 = (unit - cloud * row_groups) * R;
-    const int nrows = min(R, c - c0);
-    float* __restrict__ d = grad_src + (static_cast<int64_t>(cloud) * c + c0) * m;
-    const int64_t cloud_part = static_cast<int64_t>(cloud) * parts + part;
-    const int* __restrict__ meta = lists.meta + cloud_part * nblocks * L_BLOCK;
-    const int2* __restrict__ blocks = lists.blocks + cloud_part * nblocks;
-    const ListEntry<WEIGHTED>* __restrict__ entries = lists.entries + cloud_part * lists.capacity;
-    const __amdgpu_buffer_rsrc_t ebuf = entry_buffer(entries, static_cast<uint32_t>(lists.capacity) * ENTRY_BYTES);
-
-    // (the lane's offset decides whether the load is inside the buffer; `uniform` is added to the address)
-    auto load_entry = [&](uint32_t offset, uint32_t uniform) __attribute__((always_inline)) {
-        ListEntry<WEIGHTED> e;
-        if constexpr (WEIGHTED)
-        {
-            const int2_vec v = __builtin_amdgcn_raw_buffer_load_b64(ebuf, offset, uniform, 0);
-            e.j = v.x;
-            e.w = __int_as_float(v.y);
-        }
-        else
-            e.j = __builtin_amdgcn_raw_buffer_load_b32(ebuf, offset, uniform, 0);
-        return e;
-    };
-    // The staged value an entry refers to, in row r (a lane without entry was given the entry (0, 0): it
-    // reads the zero in front of the row).  Rows in pairs: an LDS instruction's own offset reaches the
-    // next row, not the one after.
-    auto staged_value = [&](const ListEntry<WEIGHTED>& e, int r) __attribute__((always_inline)) {
-        const char* const pair = staged + static_cast<unsigned>(e.j) + static_cast<unsigned>(r / 2) * (2u * row_bytes);
-        return *reinterpret_cast<const float*>(pair + static_cast<unsigned>(r % 2) * row_bytes);
-    };
-    auto add_value = [&](const ListEntry<WEIGHTED>& e, float v, float& sum) __attribute__((always_inline)) {
-        if constexpr (WEIGHTED)
-            sum = __builtin_fmaf(v, e.w, sum); // (one rounding instead of the reference's two: within its tolerance)
-        else
-            sum += v;
-    };
-    auto add_entry = [&](const ListEntry<WEIGHTED>& e, float (&sum)[R]) __attribute__((always_inline)) {
+    float val[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-            add_value(e, staged_value(e, r), sum[r]);
-    };
-    // Sums of the lists of a block over this piece, lane = position in the block's lane order.
-    auto walk_block = [&](int word, const ListBlock& lb, float (&sum)[R], auto&& after_first_request) __attribute__((always_inline)) {
-        const int count = word & L_COUNT_MASK;
-        const int slots = min(count, lb.width); // entries of this lane in the slot-major part
-        const uint32_t first = (static_cast<uint32_t>(lb.start) + static_cast<uint32_t>(lane)) * ENTRY_BYTES;
-        auto request = [&](int i, ListEntry<WEIGHTED> (&ent)[STEPS]) __attribute__((always_inline)) {
-            const uint32_t round = first + static_cast<uint32_t>(i) * (L_BLOCK * ENTRY_BYTES);
+    for (int r = 0; r < R; ++r)
+        val[r] = open[r];
+    int flag = starts ? 1 : 0;
+    // inside rows of 16 lanes: row_shr:1, 2, 4, 8 (a source outside the row reads as zero / no flag)
+#define TPK_ROW_SHR(x, d)                                                                  \
+    ((d) == 0   ? __builtin_amdgcn_update_dpp(0, (x), 0x111, 0xF, 0xF, false)              \
+     : (d) == 1 ? __builtin_amdgcn_update_dpp(0, (x), 0x112, 0xF, 0xF, false)              \
+     : (d) == 2 ? __builtin_amdgcn_update_dpp(0, (x), 0x114, 0xF, 0xF, false)              \
+                : __builtin_amdgcn_update_dpp(0, (x), 0x118, 0xF, 0xF, false))
 #pragma unroll
-            for (int u = 0; u < STEPS; ++u)
-                ent[u] = load_entry(i + u < slots ? round : GB_NO_ENTRY, static_cast<uint32_t>(u) * (L_BLOCK * ENTRY_BYTES));
-        };
-        // (all reads of a round are issued before the first sum; the compiler is kept from mixing the
-        // phases of a round, which would make every read wait for the one before)
-        auto add_round = [&](const ListEntry<WEIGHTED> (&ent)[STEPS]) __attribute__((always_inline)) {
-            float v[STEPS][R];
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int u = 0; u < STEPS; ++u)
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    v[u][r] = staged_value(ent[u], r);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int u = 0; u < STEPS; ++u)
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    add_value(ent[u], v[u][r], sum[r]);
-            __builtin_amdgcn_sched_barrier(0);
-        };
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-            sum[r] = 0.f;
-        // Two sets of registers take turns: while one round's entries are used, the next round's are
-        // on their way (beyond the width every lane asks for nothing and is given zeros).
-        ListEntry<WEIGHTED> even[STEPS], odd[STEPS];
-        request(0, even);
-        after_first_request();
-        for (int i = 0; i < lb.width; i += 2 * STEPS) // (widths are multiples of 2 * STEPS)
-        {
-            request(i + STEPS, odd);
-            add_round(even);
-            request(i + 2 * STEPS, even);
-            add_round(odd);
-        }
-        if (lb.longer)
-        {
-            int extra, extra_at;
-            list_extra(count, lb.width, extra, extra_at);
-            const uint32_t rest = (static_cast<uint32_t>(lb.start) + static_cast<uint32_t>(lb.width) * L_BLOCK) * ENTRY_BYTES;
-            for (unsigned long long todo = __ballot(extra > 0); todo; todo &= todo - 1)
-            {
-                const int owner = __builtin_ctzll(todo);
-                const int number = __builtin_amdgcn_readlane(extra, owner);
-                const int at = __builtin_amdgcn_readlane(extra_at, owner);
-                float rest_sum[R];
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    rest_sum[r] = 0.f;
-                for (int p = lane; p < number; p += TPK_WAVE)
-                    add_entry(load_entry(rest + static_cast<uint32_t>(at + p) * ENTRY_BYTES, 0u), rest_sum);
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                {
-                    const float total = wave_sum_f32(rest_sum[r]);
-                    if (lane == owner)
-                        sum[r] += total;
-                }
-            }
-        }
-    };
-
-    if constexpr (KEEP)
+    for (int d = 0; d < 4; ++d)
     {
-        const bool last_part = part == parts - 1;
-        // (the descriptions of all blocks are requested together)
-        int words[GB_KEPT_BLOCKS];
-        ListBlock lbs[GB_KEPT_BLOCKS];
+        const int pf = TPK_ROW_SHR(flag, d);
 #pragma unroll
-        for (int b = 0; b < GB_KEPT_BLOCKS; ++b)
+        for (int r = 0; r < R; ++r)
         {
-            const int blk = min(walker + b * GB_WALK_WAVES, nblocks - 1);
-            words[b] = meta[blk * L_BLOCK + lane];
-            lbs[b] = list_block(blocks, blk);
+            const int pv = TPK_ROW_SHR(__float_as_int(val[r]), d);
+            val[r] += flag ? 0.f : __int_as_float(pv);
         }
+        flag |= pf;
+    }
+#undef TPK_ROW_SHR
+    // across the rows, one after the other: the sum at the end of the row before is final by then
 #pragma unroll
-        for (int b = 0; b < GB_KEPT_BLOCKS; ++b)
+    for (int k = 1; k < 4; ++k)
+    {
+        const bool take = (lane >> 4) == k && flag == 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
         {
-            const int blk = walker + b * GB_WALK_WAVES;
-            if (blk >= nblocks)
-                between(b);
-            if (blk < nblocks)
-            {
-                float sum[R];
-                walk_block(words[b], lbs[b], sum, [&]() __attribute__((always_inline)) { between(b); });
-                // from the block's lane order to target order: lane T takes the sums of the lane that served target T
-                const int serving = static_cast<int>(static_cast<unsigned>(words[b]) >> 26);
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    kept[b][r] += __int_as_float(__builtin_amdgcn_ds_bpermute(serving * 4, __float_as_int(sum[r])));
-                if (last_part)
-                {
-                    const int tgt = blk * L_BLOCK + lane;
-#pragma unroll
-                    for (int r = 0; r < R; ++r)
-                    {
-                        if (tgt < m && r < nrows)
-                            d[static_cast<int64_t>(r) * m + tgt] = kept[b][r];
-                        kept[b][r] = 0.f;
-                    }
-                }
-            }
+            const float before = tpk_read_lane(val[r], 16 * k - 1);
+            val[r] += take ? before : 0.f;
         }
     }
-    else
+#pragma unroll
+    for (int r = 0; r < R; ++r)
     {
-        between(0);
-        for (int blk = walker; blk < nblocks; blk += GB_WALK_WAVES)
-        {
-            const int word = meta[blk * L_BLOCK + lane];
-            const ListBlock lb = list_block(blocks, blk);
-            const int tgt = blk * L_BLOCK + lane;
-            // (what the parts before stored for these targets is requested now, needed at the end)
-            float old[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                old[r] = part > 0 && tgt < m && r < nrows ? d[static_cast<int64_t>(r) * m + tgt] : 0.f;
-            float sum[R];
-            walk_block(word, lb, sum, [] {});
-            const int serving = static_cast<int>(static_cast<unsigned>(word) >> 26);
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-            {
-                const float mine = __int_as_float(__builtin_amdgcn_ds_bpermute(serving * 4, __float_as_int(sum[r])));
-                if (tgt < m && r < nrows)
-                    d[static_cast<int64_t>(r) * m + tgt] = old[r] + mine;
-            }
-        }
+        const float up = __shfl_up(val[r], 1);
+        carry[r] = lane == 0 ? 0.f : up;
     }
 }
 
 // grid: workgroups that each take `units_per_group` consecutive units; a unit = R feature rows
-// (c0 .. c0 + R - 1) of one cloud.  A unit is processed in `parts` pieces of `part_len` columns
-// (the lists are built per part, lists.h).  For a piece the workgroup holds the R x part_len
-// values of grad_out in LDS, and every wavefront takes blocks of 64 targets, one target per lane
-// (in the block's order of descending list length): in step i the lanes that still have an entry
-// read slot i of their lists - one contiguous run - and the staged values these refer to.  Two
-// sets of registers take turns, so the entries of a round are requested a round ahead.  The few
-// lists longer than the block's slot-major part are then summed by the whole wavefront.
+// (c0 .. c0 + R - 1) of one cloud.  A unit is processed in `parts` pieces of `part_len` columns (the
+// lists are built per part, lists.h).  For a piece the workgroup holds the R x part_len values of
+// grad_out in LDS; wavefront s walks the lists of span s of the targets: every lane adds up its run
+// of consecutive list entries, one entry per step - the entries of a step are one contiguous row,
+// requested GB_AHEAD steps ahead - and reads the staged values they refer to (an entry that refers
+// to nothing carries an address beyond the LDS, which reads as zero).  Where an entry ends a list the
+// lane puts its sum into the span's output row in LDS, at the target it has counted up to, and starts
+// the next sum.  The first list a lane ends may have begun in the runs of the lanes before it: when
+// the walk is over one scan over the lanes tells every lane what was carried into its run, and the
+// lane adds that to the first sum it put.  Then the span's sums leave as contiguous stores - every
+// target has at least one entry (lists.h), so the first part writes every output element; later
+// parts (rows longer than the LDS holds) add to what is there, the same wavefront at the same place.
 //
-// grad_out streams from memory while the lists are walked: every lane requests its eight 16-byte
-// loads of the NEXT piece (1024 lanes x 8 = the 128 KiB of a piece) into registers during the walk
-// and writes them to LDS between the two barriers that end a piece.  A wavefront's loads complete in
-// order, so the entry requests that follow those loads wait for them: each wavefront issues them
-// during one of its blocks only, a different one from wavefront to wavefront, and at any time
-// most wavefronts walk while some wait for memory.
-//
-// KEEP: the sums of every block stay in registers across the parts of a unit and are stored
-// once (m <= 64 * 16 * GB_KEPT_BLOCKS targets); otherwise a block's sums of one part are added
-// to what the parts before stored.
-// dynamic LDS: R * (part_len + 4) floats.
-template <int K, bool WEIGHTED, int R, bool KEEP>
+// grad_out streams from memory while the lists are walked: every lane requests its 16-byte loads of
+// the NEXT piece into registers during the walk (a wavefront's loads complete in order, so the entry
+// requests behind them wait for them: every wavefront does this at another point of its walk) and
+// writes them to LDS between the two barriers that end the piece.
+// dynamic LDS: R * part_len floats (the piece) + R * L_SPANS * span floats (the sums).
+template <int K, bool WEIGHTED, int R>
 __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
-    int c, int m, int64_t n, int parts, int part_len, int row_groups, int units, int units_per_group, bool vector_loads,
-    const float* __restrict__ grad_out, Lists<WEIGHTED> lists, float* __restrict__ grad_src)
+    int c, int m, int64_t n, int parts, int part_len, int span, int row_groups, int units, int units_per_group,
+    bool vector_loads, const float* __restrict__ grad_out, Lists<WEIGHTED> lists, float* __restrict__ grad_src)
 {
     extern __shared__ float rows[];
-    const unsigned stride = static_cast<unsigned>(part_len) + 4u;
+    const unsigned row_bytes = static_cast<unsigned>(part_len) * 4u;
     const unsigned tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE); // (a scalar for the compiler)
-    const int nblocks = (m + L_BLOCK - 1) / L_BLOCK;
+    constexpr uint32_t ENTRY_BYTES = sizeof(ListEntry<WEIGHTED>);
+    // the sums of this wavefront's span: sums[(target - t0) * R + r]
+    float* const sums = rows + static_cast<unsigned>(R) * static_cast<unsigned>(part_len) +
+                        static_cast<unsigned>(wave) * static_cast<unsigned>(span) * R;
+    const int t0 = min(wave * span, m), width = min(span, m - t0);
 
     // consecutive workgroups of a die work on consecutive units: one cloud's lists per L2
     const int group = static_cast<int>(xcd_local_block(blockIdx.x, gridDim.x));
@@ -422,56 +275,29 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
     const int unit1 = min(unit0 + units_per_group, units);
     const int pieces = (unit1 - unit0) * parts;
 
-    // what a lane without entry reads: four zeros in front of every staged row
-    for (unsigned t = tid; t < R * 4u; t += G_THREADS)
-        rows[(t >> 2) * stride + (t & 3u)] = 0.f;
-
-    float kept[KEEP ? GB_KEPT_BLOCKS : 1][R]; // sums of this wavefront's blocks over the parts so far, lane = target
-#pragma unroll
-    for (int b = 0; b < (KEEP ? GB_KEPT_BLOCKS : 1); ++b)
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-            kept[b][r] = 0.f;
-
-    if (!vector_loads)
-    {
-        // Rows that do not start on 16-byte boundaries, or pieces shorter than the LDS holds: the
-        // piece is staged before its walk, nothing overlaps.
-        for (int piece = 0; piece < pieces; ++piece)
-        {
-            const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
-            const int cloud = unit / row_groups, c0 = (unit - cloud * row_groups) * R;
-            const int64_t col0 = static_cast<int64_t>(part) * part_len;
-            __syncthreads();
-            stage_rows_by<G_THREADS, 4>(rows + 4, stride, grad_out + (static_cast<int64_t>(cloud) * c + c0) * n + col0, n,
-                                        static_cast<unsigned>(min(R, c - c0)),
-                                        static_cast<unsigned>(tpk_min64(part_len, n - col0)), tid);
-            __syncthreads();
-            walk_piece<K, WEIGHTED, R, KEEP, 0>(rows, stride, piece, unit0, parts, row_groups, c, m, nblocks, wave, lane, lists,
-                                                grad_src, kept, [](int) {});
-        }
-        return;
-    }
-
-    // (on this path part_len = GB_STAGE_FLOATS / R: load k of a lane lies in row k / CHUNKS of the
-    // piece, at a column that is the same for the whole workgroup plus four times the lane's number)
-    constexpr unsigned PART = GB_STAGE_FLOATS / R;
-    constexpr unsigned CHUNK = G_THREADS * 4; // columns covered by one load of all lanes
-    constexpr unsigned CHUNKS = PART / CHUNK;
+    // The next piece on its way into registers: 16-byte load k of a lane covers the floats
+    // (k * G_THREADS + tid) * 4 .. + 3 of the piece's R x part_len values (part_len is a multiple of 4 here).
+    const unsigned per_row = static_cast<unsigned>(part_len) >> 2;
     float4 fetched[GB_FETCH];
+    auto piece_source = [&](int piece, int& nrows, unsigned& len) __attribute__((always_inline)) {
+        const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
+        const int cloud = unit / row_groups, c0 = (unit - cloud * row_groups) * R;
+        nrows = min(R, c - c0);
+        const int64_t col0 = static_cast<int64_t>(part) * part_len;
+        len = static_cast<unsigned>(tpk_min64(part_len, n - col0));
+        return grad_out + (static_cast<int64_t>(cloud) * c + c0) * n + col0;
+    };
     auto fetch = [&](int piece) __attribute__((always_inline)) {
         if (piece >= pieces)
             return;
-        const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
-        const int cloud = unit / row_groups, c0 = (unit - cloud * row_groups) * R;
-        const int nrows = min(R, c - c0);
-        const int64_t col0 = static_cast<int64_t>(part) * PART;
-        const unsigned len = static_cast<unsigned>(tpk_min64(PART, n - col0));
-        const float* __restrict__ src = grad_out + (static_cast<int64_t>(cloud) * c + c0) * n + col0;
+        int nrows;
+        unsigned len;
+        const float* __restrict__ src = piece_source(piece, nrows, len);
 #pragma unroll
         for (int k = 0; k < GB_FETCH; ++k)
         {
-            const unsigned r = static_cast<unsigned>(k) / CHUNKS, col = (static_cast<unsigned>(k) % CHUNKS) * CHUNK + tid * 4u;
+            const unsigned i = static_cast<unsigned>(k) * G_THREADS + tid;
+            const unsigned r = R > 1 ? i / per_row : 0u, col = (i - r * per_row) * 4u;
             fetched[k] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (r < static_cast<unsigned>(nrows) && col < len)
                 fetched[k] = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(r) * n + col);
@@ -481,23 +307,145 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
 #pragma unroll
         for (int k = 0; k < GB_FETCH; ++k)
         {
-            const unsigned r = static_cast<unsigned>(k) / CHUNKS, col = (static_cast<unsigned>(k) % CHUNKS) * CHUNK + tid * 4u;
-            *reinterpret_cast<float4*>(rows + r * (PART + 4u) + 4u + col) = fetched[k];
+            const unsigned i = static_cast<unsigned>(k) * G_THREADS + tid;
+            const unsigned r = R > 1 ? i / per_row : 0u, col = (i - r * per_row) * 4u;
+            if (r < static_cast<unsigned>(R) && col < static_cast<unsigned>(part_len))
+                *reinterpret_cast<float4*>(rows + r * static_cast<unsigned>(part_len) + col) = fetched[k];
         }
     };
-    fetch(0);
-    stage_fetched();
-    const int my_turn = KEEP ? (wave & (GB_KEPT_BLOCKS - 1)) : 0; // the block position during which this wavefront fetches
+    auto stage_slowly = [&](int piece) __attribute__((always_inline)) {
+        int nrows;
+        unsigned len;
+        const float* __restrict__ src = piece_source(piece, nrows, len);
+        for (unsigned i = tid; i < R * static_cast<unsigned>(part_len); i += G_THREADS)
+        {
+            const unsigned r = i / static_cast<unsigned>(part_len), col = i - r * static_cast<unsigned>(part_len);
+            rows[i] = (r < static_cast<unsigned>(nrows) && col < len) ? src[static_cast<int64_t>(r) * n + col] : 0.f;
+        }
+    };
+
+    if (vector_loads)
+    {
+        fetch(0);
+        stage_fetched();
+    }
     for (int piece = 0; piece < pieces; ++piece)
     {
+        const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
+        const int cloud = unit / row_groups, c0 = (unit - cloud * row_groups) * R;
+        const int nrows = min(R, c - c0);
+        const int64_t cloud_part = static_cast<int64_t>(cloud) * parts + part;
+
+        // this wavefront's span of the lists of (cloud, part)
+        const int4 region = lists.regions[cloud_part * L_SPANS + wave];
+        const int base = __builtin_amdgcn_readfirstlane(region.x);
+        const int steps = __builtin_amdgcn_readfirstlane(region.z);
+        // where this lane puts its next sum: the target of its first entry, as a byte offset into `sums`
+        const int first_slot = (lists.first_target[(cloud_part * L_SPANS + wave) * TPK_WAVE + lane] - t0) * (R * 4);
+        const __amdgpu_buffer_rsrc_t ebuf =
+            memory_buffer(lists.entries + cloud_part * lists.capacity, static_cast<uint32_t>(lists.capacity) * ENTRY_BYTES);
+        const uint32_t first = (static_cast<uint32_t>(base) + static_cast<uint32_t>(lane)) * ENTRY_BYTES;
+        auto request = [&](int i) __attribute__((always_inline)) {
+            // (rows behind the last are never used: the last row again)
+            const uint32_t row = static_cast<uint32_t>(min(i, steps - 1)) * (TPK_WAVE * ENTRY_BYTES); // wave-uniform
+            ListEntry<WEIGHTED> e;
+            if constexpr (WEIGHTED)
+            {
+                const int2_vec v = __builtin_amdgcn_raw_buffer_load_b64(ebuf, first, row, 0);
+                e.j = v.x;
+                e.w = __int_as_float(v.y);
+            }
+            else
+                e.j = __builtin_amdgcn_raw_buffer_load_b32(ebuf, first, row, 0);
+            return e;
+        };
+        // (list entries do not depend on the staged values: the first rows are requested before the barrier)
+        ListEntry<WEIGHTED> ahead[GB_AHEAD];
+        if (steps > 0)
+        {
+#pragma unroll
+            for (int u = 0; u < GB_AHEAD; ++u)
+                ahead[u] = request(u);
+        }
+
+        if (!vector_loads)
+        {
+            // rows that do not start on 16-byte boundaries: the piece is staged before its walk, nothing overlaps
+            __syncthreads();
+            stage_slowly(piece);
+        }
         lds_barrier(); // the piece is in LDS
-        walk_piece<K, WEIGHTED, R, KEEP, PART + 4>(rows, stride, piece, unit0, parts, row_groups, c, m, nblocks, wave, lane, lists,
-                                                   grad_src, kept, [&](int b) __attribute__((always_inline)) {
-                                                       if (b == my_turn)
-                                                           fetch(piece + 1);
-                                                   });
+        const int fetch_at = vector_loads ? ((wave * steps / L_SPANS) / GB_AHEAD) * GB_AHEAD : -1;
+        if (vector_loads && steps == 0)
+            fetch(piece + 1);
+
+        const char* const staged = reinterpret_cast<const char*>(rows);
+        char* const put_at = reinterpret_cast<char*>(sums);
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            acc[r] = 0.f;
+        int slot = first_slot;
+        for (int i0 = 0; i0 < steps; i0 += GB_AHEAD)
+        {
+            if (i0 == fetch_at) // (wave-uniform)
+                fetch(piece + 1);
+#pragma unroll
+            for (int u = 0; u < GB_AHEAD; ++u)
+            {
+                if (i0 + u >= steps) // (wave-uniform)
+                    break;
+                const ListEntry<WEIGHTED> e = ahead[u];
+                ahead[u] = request(i0 + u + GB_AHEAD);
+                const unsigned at = static_cast<unsigned>(e.j) & 0x7fffffffu;
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                {
+                    const float v = *reinterpret_cast<const float*>(staged + at + static_cast<unsigned>(r) * row_bytes);
+                    if constexpr (WEIGHTED)
+                        acc[r] = __builtin_fmaf(v, e.w, acc[r]); // (one rounding instead of the reference's two: within its tolerance)
+                    else
+                        acc[r] += v;
+                }
+                const bool ends = e.j < 0; // the entry ends a list
+                if (ends)
+                {
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        *reinterpret_cast<float*>(put_at + slot + r * 4) = acc[r];
+                }
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    acc[r] = ends ? 0.f : acc[r];
+                slot += ends ? R * 4 : 0;
+            }
+        }
+        // the first list every lane ended, with what the lanes before carried into it
+        float carry[R];
+        const bool ended_one = slot != first_slot;
+        carried_in<R>(acc, ended_one, lane, carry);
+        if (ended_one)
+        {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                *reinterpret_cast<float*>(put_at + first_slot + r * 4) += carry[r];
+        }
+        // the span's sums leave in order (a wavefront's LDS accesses are executed in order: no barrier needed)
+        float* __restrict__ d = grad_src + (static_cast<int64_t>(cloud) * c + c0) * m + t0;
+        for (int t = lane; t < width; t += TPK_WAVE)
+        {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (r < nrows)
+                {
+                    const float v = sums[t * R + r];
+                    float* const at = d + static_cast<int64_t>(r) * m + t;
+                    *at = part == 0 ? v : *at + v;
+                }
+        }
         lds_barrier(); // everybody is done with the piece
-        stage_fetched();
+        if (vector_loads)
+            stage_fetched();
     }
 }
 
@@ -610,23 +558,37 @@ int gather_fwd(int b, int c, int m, int64_t n, const float* src, const IdxT* idx
     return tpk_launch_status();
 }
 
-// Rows of grad_out staged together and columns per part, for rows of n floats.
+// Rows of grad_out staged together and columns per part, for rows of n floats and m targets.
 struct BwdShape
 {
-    int rows;
+    int rows;     // 0: the shape does not fit (too many targets)
     int part_len;
     int parts;
+    int span;     // targets per wavefront
 };
-BwdShape bwd_shape(int64_t n)
+BwdShape bwd_shape(int64_t n, int m)
 {
     BwdShape sh;
-    // 128 KiB of LDS hold rows x part_len values.  Rows of up to 16384 floats go four at a time in
-    // pieces of 8192 columns (the lists of a piece are read once per four rows), rows of up to
-    // 32768 floats two at a time in pieces of 16384 columns, longer rows one at a time.
-    sh.rows = n <= GB_STAGE_FLOATS ? 4 : 1;
+    // The LDS holds rows x part_len staged values and rows x (16 spans) sums.  As many rows at a time as
+    // leave room for whole rows of grad_out (the lists are read once per row group): four, two or one; rows
+    // longer than that go one at a time in parts.
+    sh.span = static_cast<int>(tpk_ceil_div(m, L_SPANS));
+    const int64_t sums = static_cast<int64_t>(sh.span) * L_SPANS;
     const int64_t n4 = (n + 3) & ~static_cast<int64_t>(3);
-    sh.part_len = static_cast<int>(tpk_min64(n4, GB_STAGE_FLOATS / sh.rows));
-    sh.parts = static_cast<int>(tpk_min64(tpk_ceil_div(n, sh.part_len), 0x7fffffff));
+    sh.rows = 0;
+    sh.part_len = 0;
+    sh.parts = 0;
+    for (int r = 4; r >= 1; r /= 2)
+    {
+        const int64_t room = tpk_min64(GB_LDS_FLOATS / r - sums, GB_STAGE_FLOATS / r) & ~static_cast<int64_t>(3);
+        if (room >= n4 || (r == 1 && room >= 4096))
+        {
+            sh.rows = r;
+            sh.part_len = static_cast<int>(tpk_min64(n4, room));
+            sh.parts = static_cast<int>(tpk_min64(tpk_ceil_div(n, sh.part_len), 0x7fffffff));
+            break;
+        }
+    }
     return sh;
 }
 
@@ -636,13 +598,13 @@ size_t lists_workspace_bytes(int b, int m, int64_t n)
 {
     if (b <= 0 || m <= 0 || n <= 0)
         return 0;
-    const BwdShape sh = bwd_shape(n);
-    if (static_cast<int64_t>(b) * sh.parts > 0x7fffffffLL)
+    const BwdShape sh = bwd_shape(n, m);
+    if (sh.rows == 0 || static_cast<int64_t>(b) * sh.parts > 0x7fffffffLL)
         return 0;
-    return lists_bytes<WEIGHTED>(b * sh.parts, m, static_cast<int64_t>(sh.part_len) * K);
+    return lists_bytes<WEIGHTED>(static_cast<int64_t>(b) * sh.parts, m, static_cast<int64_t>(sh.part_len) * K);
 }
 
-template <int K, bool WEIGHTED, int R, bool KEEP>
+template <int K, bool WEIGHTED, int R>
 int launch_bwd_lists(int b, int c, int m, int64_t n, const BwdShape& sh, const float* grad_out,
                      const Lists<WEIGHTED>& lists, float* grad_src, hipStream_t s)
 {
@@ -654,28 +616,17 @@ int launch_bwd_lists(int b, int c, int m, int64_t n, const BwdShape& sh, const f
     // number of consecutive units, so that it can request its next piece while it works.
     const int per_group = static_cast<int>(tpk_ceil_div(units, 256));
     const int groups = static_cast<int>(tpk_ceil_div(units, per_group));
-    const size_t lds = static_cast<size_t>(R) * (sh.part_len + 4) * sizeof(float);
+    const size_t lds = static_cast<size_t>(R) * (static_cast<size_t>(sh.part_len) + static_cast<size_t>(sh.span) * L_SPANS) * sizeof(float);
     // 16-byte loads need rows that start on 16-byte boundaries
-    // the fetching wavefronts need rows that start on 16-byte boundaries and full-size pieces
-    const bool vector_loads = (n & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_out) & 15u) == 0 &&
-                              static_cast<int64_t>(sh.part_len) * R == GB_STAGE_FLOATS;
-    auto kernel = gather_bwd_lists_kernel<K, WEIGHTED, R, KEEP>;
+    const bool vector_loads = (n & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_out) & 15u) == 0;
+    auto kernel = gather_bwd_lists_kernel<K, WEIGHTED, R>;
     int st = allow_lds(kernel, lds);
     if (st != TPK_OK)
         return st;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups)), dim3(G_THREADS), lds, s, c, m, n, sh.parts,
-                       sh.part_len, row_groups, static_cast<int>(units), per_group, vector_loads, grad_out, lists,
+                       sh.part_len, sh.span, row_groups, static_cast<int>(units), per_group, vector_loads, grad_out, lists,
                        grad_src);
     return tpk_launch_status();
-}
-
-template <int K, bool WEIGHTED, int R>
-int launch_bwd_lists_rows(int b, int c, int m, int64_t n, const BwdShape& sh, const float* grad_out,
-                          const Lists<WEIGHTED>& lists, float* grad_src, hipStream_t s)
-{
-    if (list_blocks(m) <= GB_KEPT_BLOCKS * GB_WALK_WAVES)
-        return launch_bwd_lists<K, WEIGHTED, R, true>(b, c, m, n, sh, grad_out, lists, grad_src, s);
-    return launch_bwd_lists<K, WEIGHTED, R, false>(b, c, m, n, sh, grad_out, lists, grad_src, s);
 }
 
 template <int K, bool WEIGHTED, typename IdxT>
@@ -690,22 +641,22 @@ int gather_bwd(int b, int c, int m, int64_t n, const float* grad_out, const IdxT
     if (!grad_src || (n > 0 && (!grad_out || !idx || (WEIGHTED && !weight))))
         return TPK_ERR_INVALID_ARG;
     // The list path needs entry positions that fit an int, and the workspace.
-    const BwdShape sh = bwd_shape(n > 0 ? n : 1);
-    const bool fits = n > 0 && n * K <= 0x7fffffffLL &&
+    const BwdShape sh = bwd_shape(n > 0 ? n : 1, m);
+    const bool fits = n > 0 && sh.rows > 0 && n * K <= 0x7fffffffLL &&
                       static_cast<int64_t>(b) * sh.parts <= 0x7fffffffLL;
     const size_t need = lists_workspace_bytes<K, WEIGHTED>(b, m, n);
     if (fits && workspace && need > 0 && workspace_bytes >= need)
     {
         const int64_t part_total = static_cast<int64_t>(sh.part_len) * K;
-        const Lists<WEIGHTED> lists = lists_at<WEIGHTED>(workspace, b * sh.parts, m, part_total);
+        const Lists<WEIGHTED> lists = lists_at<WEIGHTED>(workspace, static_cast<int64_t>(b) * sh.parts, m, part_total);
         int st = launch_build_lists<K, WEIGHTED, IdxT>(b, m, n * K, part_total, idx, weight, lists, s);
         if (st == TPK_OK)
         {
             if (sh.rows == 4)
-                return launch_bwd_lists_rows<K, WEIGHTED, 4>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+                return launch_bwd_lists<K, WEIGHTED, 4>(b, c, m, n, sh, grad_out, lists, grad_src, s);
             if (sh.rows == 2)
-                return launch_bwd_lists_rows<K, WEIGHTED, 2>(b, c, m, n, sh, grad_out, lists, grad_src, s);
-            return launch_bwd_lists_rows<K, WEIGHTED, 1>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+                return launch_bwd_lists<K, WEIGHTED, 2>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+            return launch_bwd_lists<K, WEIGHTED, 1>(b, c, m, n, sh, grad_out, lists, grad_src, s);
         }
         if (st != TPK_ERR_UNSUPPORTED)
             return st;
