@@ -46,7 +46,7 @@ TRAFFIC_KERNELS = {
 # Kernels whose VALU counters describe a distance scan.
 VALU_KERNELS = {
     "fps": "fps_pruned_kernel<32, 512, 4>",
-    "ball_query_dense": "ball_query_dense_kernel",
+    "ball_query_dense": "ball_query_dense_kernel<2>",
     "ball_query_partial_dense": "ball_query_bins_kernel",
     "three_nn": "three_nn_grid_kernel",
     "chamfer_fwd": "chamfer_grid_kernel",

@@ -27,6 +27,7 @@ constexpr int BQ_WAVES = 4;
 constexpr int BQ_THREADS = BQ_WAVES * TPK_WAVE;
 constexpr int BQ_Q = 8;                    // queries per wavefront
 constexpr int BQ_BLOCK_Q = BQ_WAVES * BQ_Q; // queries per workgroup
+constexpr int BQ_Q_FEW = 2;                // queries per wavefront when the whole call has few queries
 constexpr int BQ_TILE = 2048;              // support points per LDS tile (24 KiB)
 
 struct Tile
@@ -54,7 +55,7 @@ __device__ __forceinline__ int64_t lower_bound_i64(const int64_t* __restrict__ a
 
 // Scan support[s0, s1) for the wavefront's queries.  in_run_mask: bit q set when query q
 // of this wavefront takes part.  row0: output row of the wavefront's query 0.
-template <bool PARTIAL>
+template <bool PARTIAL, int BQ_Q>
 __device__ __forceinline__ void scan_run(Tile& tile, const float* __restrict__ support,
                                          int64_t s0, int64_t s1, unsigned in_run_mask,
                                          const float (&qx)[BQ_Q], const float (&qy)[BQ_Q],
@@ -174,6 +175,10 @@ __device__ __forceinline__ void scan_run(Tile& tile, const float* __restrict__ s
     }
 }
 
+// BQ_Q queries per wavefront: 8 amortise the reads of the candidates best; a call with few queries (the usual
+// case: a few thousand ball centres) takes 2, so that it still spreads over four wavefronts per SIMD - one
+// wavefront per SIMD issues at half the rate.
+template <int BQ_Q>
 __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
     int n, int m, int blocks_per_cloud, float radius2, int nsample,
     const float* __restrict__ new_xyz, const float* __restrict__ xyz, int64_t* __restrict__ idx,
@@ -183,7 +188,7 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
     const int cloud = blockIdx.x / blocks_per_cloud;
     const int blk = blockIdx.x - cloud * blocks_per_cloud;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TPK_WAVE);
-    const int jq0 = blk * BQ_BLOCK_Q + wave * BQ_Q; // first query of this wavefront
+    const int jq0 = (blk * BQ_WAVES + wave) * BQ_Q; // first query of this wavefront
 
     new_xyz += static_cast<int64_t>(cloud) * m * 3;
     xyz += static_cast<int64_t>(cloud) * n * 3;
@@ -202,8 +207,8 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
         qz[q] = to_vector_register(new_xyz[jj * 3 + 2]);
         in_run |= ok ? (1u << q) : 0u;
     }
-    scan_run<false>(tile, xyz, 0, n, in_run, qx, qy, qz, radius2, nsample,
-                    static_cast<int64_t>(cloud) * m + jq0, idx, dist);
+    scan_run<false, BQ_Q>(tile, xyz, 0, n, in_run, qx, qy, qz, radius2, nsample,
+                          static_cast<int64_t>(cloud) * m + jq0, idx, dist);
 }
 
 __global__ __launch_bounds__(BQ_THREADS) void ball_query_partial_kernel(
@@ -249,7 +254,7 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_partial_kernel(
             const int64_t j = jq0 + q;
             in_run |= (j >= run_start && j < run_end && qc[q] == c) ? (1u << q) : 0u;
         }
-        scan_run<true>(tile, x, s0, s1, in_run, qx, qy, qz, radius2, nsample, jq0, idx, dist);
+        scan_run<true, BQ_Q>(tile, x, s0, s1, in_run, qx, qy, qz, radius2, nsample, jq0, idx, dist);
         run_start = run_end;
     }
 }
@@ -268,14 +273,19 @@ extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int n
         return TPK_ERR_INVALID_ARG;
     if (static_cast<int64_t>(n) * 3 > 0x7fffffffLL || static_cast<int64_t>(m) * 3 > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    const int64_t bpc = tpk_ceil_div(m, BQ_BLOCK_Q);
+    // fewer than four workgroups per compute unit with 8 queries per wavefront: 2 per wavefront
+    const bool few = tpk_ceil_div(m, BQ_BLOCK_Q) * b < 1024;
+    const int64_t bpc = tpk_ceil_div(m, few ? BQ_WAVES * BQ_Q_FEW : BQ_BLOCK_Q);
     const int64_t blocks = bpc * b;
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     const float radius2 = radius * radius; // fp32 product, as the reference kernel forms it
-    hipLaunchKernelGGL(ball_query_dense_kernel, dim3(static_cast<unsigned>(blocks)),
-                       dim3(BQ_THREADS), 0, tpk_stream(stream), n, m, static_cast<int>(bpc),
-                       radius2, nsample, new_xyz, xyz, idx, dist);
+    if (few)
+        hipLaunchKernelGGL(ball_query_dense_kernel<BQ_Q_FEW>, dim3(static_cast<unsigned>(blocks)), dim3(BQ_THREADS), 0,
+                           tpk_stream(stream), n, m, static_cast<int>(bpc), radius2, nsample, new_xyz, xyz, idx, dist);
+    else
+        hipLaunchKernelGGL(ball_query_dense_kernel<BQ_Q>, dim3(static_cast<unsigned>(blocks)), dim3(BQ_THREADS), 0,
+                           tpk_stream(stream), n, m, static_cast<int>(bpc), radius2, nsample, new_xyz, xyz, idx, dist);
     return tpk_launch_status();
 }
 

@@ -46,15 +46,24 @@ __host__ __device__ inline int64_t set_windows(const PointSet& s)
 
 // One workgroup orders one window: the first windows_a blocks those of set_a, the rest set_b.
 // `zero_word` (optional) is cleared by the first block: a counter used by the kernel that follows.
+// The window's points are read once and stay in registers (16 per thread): bounding box, curve
+// position of each point's cell of the 16^3 grid (a table in LDS), histogram and prefix sum over the
+// 4096 bins, and then every thread takes a place in its points' bins (LDS integer atomics) and stores
+// the records straight to their final positions.  The boxes of the cells are formed from the records
+// read back in order (one more trip to the L2 instead of random gathers of the coordinates).
+// Inside a bin (1/16 of the window's extent per axis) the order is that in which the atomics were
+// served; it decides where a point sits inside its bin, never what a search over the cells returns.
+// dynamic LDS: (2 * CURVE_BINS + 24 * cells) words.
 __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet set_a, PointSet set_b,
-                                                                      int windows_a, int key_capacity,
-                                                                      int* zero_word)
+                                                                      int windows_a, int* zero_word)
 {
-    extern __shared__ unsigned sort_keys[];
-    unsigned* const unsorted = sort_keys + key_capacity;
-    int* const bins = reinterpret_cast<int*>(unsorted + key_capacity);
+    extern __shared__ unsigned bin_of_cell[];  // [CURVE_BINS] curve position of every cell of the 16^3 grid
+    int* const bins = reinterpret_cast<int*>(bin_of_cell) + CURVE_BINS; // [CURVE_BINS]
+    int* const run_boxes = bins + CURVE_BINS;  // [cells * 4][6] ordered ints: boxes of the runs of 16 records
     __shared__ int cloud_box[6];
     __shared__ int wave_totals[NG_SORT_THREADS / TPK_WAVE];
+    constexpr int PER = CURVE_MAX_POINTS / NG_SORT_THREADS; // points per thread
+    static_assert(CURVE_BINS % NG_SORT_THREADS == 0, "every thread scans the same number of bins");
 
     const bool first_set = static_cast<int>(blockIdx.x) < windows_a;
     const PointSet set = first_set ? set_a : set_b;
@@ -65,62 +74,175 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     const int n = static_cast<int>(tpk_min64(set.stride, set.cloud_points - in_cloud));
     const int cells = set_cells(set);
     const float* __restrict__ xyz = set.xyz + start * 3;
+    const int64_t* __restrict__ group = set.group ? set.group + start : nullptr;
     float4* __restrict__ sorted = set.sorted + window * cells * NG_CELL;
     float4* __restrict__ boxes = set.boxes ? set.boxes + window * cells * NG_BOX : nullptr;
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
     if (zero_word && blockIdx.x == 0 && tid == 0)
         *zero_word = 0;
 
-    curve_order<NG_SORT_THREADS>(xyz, n, sort_keys, unsorted, bins, cloud_box, wave_totals,
-                                 set.group ? set.group + start : nullptr);
-
-    // Every wavefront writes whole cells; a batch of gathers is issued before any is used.
-    int* const run_boxes = reinterpret_cast<int*>(unsorted); // (free now) [cells * 4][6] ordered ints
-    constexpr int BATCH = 4;
-    const int padded = cells * NG_CELL;
-    for (int q0 = tid; q0 < padded; q0 += NG_SORT_THREADS * BATCH)
+    // the points of this thread: tid, tid + 1024, ... (all loads issued before the first is used)
+    float p[PER][3];
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
     {
-        int k[BATCH];
-        float v[BATCH][3];
+        const int k = min(tid + u * NG_SORT_THREADS, n - 1);
 #pragma unroll
-        for (int u = 0; u < BATCH; ++u)
+        for (int a = 0; a < 3; ++a)
+            p[u][a] = xyz[k * 3 + a];
+    }
+    // (with cloud ids: how far a point's id lies above the window's first, cut at 7)
+    int id_offset[PER];
+    if (group)
+    {
+        const int64_t first_group = group[0];
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            id_offset[u] = static_cast<int>(tpk_min64(group[min(tid + u * NG_SORT_THREADS, n - 1)] - first_group, 7));
+    }
+
+    const int empty_lo = float_to_ordered_int(__builtin_inff());
+    const int empty_hi = float_to_ordered_int(-__builtin_inff());
+    if (tid < 6)
+        cloud_box[tid] = tid < 3 ? empty_lo : empty_hi;
+    for (int i = tid; i < CURVE_BINS; i += NG_SORT_THREADS)
+    {
+        bins[i] = 0;
+        bin_of_cell[i] = curve_bin_of_cell(i & 15, (i >> 4) & 15, i >> 8);
+    }
+    __syncthreads();
+    {
+        // box of the window (only to quantise coordinates for the curve); the clamped loads repeat a real point
+        float lo[3], hi[3];
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
         {
-            const int q = q0 + u * NG_SORT_THREADS;
-            k[u] = q < n ? static_cast<int>(sort_keys[q] & 0x3FFFu) : -1;
-            const int kk = k[u] < 0 ? 0 : k[u];
+            lo[a] = hi[a] = p[0][a];
 #pragma unroll
-            for (int a = 0; a < 3; ++a)
-                v[u][a] = xyz[kk * 3 + a];
-        }
-#pragma unroll
-        for (int u = 0; u < BATCH; ++u)
-        {
-            const int q = q0 + u * NG_SORT_THREADS;
-            if (q >= padded) // uniform over the wavefront: cells are whole
-                continue;
-            const bool real = k[u] >= 0;
-            const float inf = __builtin_inff();
-            sorted[q] = real ? make_float4(v[u][0], v[u][1], v[u][2], __int_as_float(static_cast<int>(in_cloud) + k[u]))
-                             : make_float4(inf, inf, inf, __int_as_float(0x7FFFFFFF));
-            if (!boxes) // uniform
-                continue;
-            // boxes of the four runs of 16 points (DPP row reductions), left in LDS
-            int lo[3], hi[3];
-#pragma unroll
-            for (int a = 0; a < 3; ++a)
+            for (int u = 1; u < PER; ++u)
             {
-                lo[a] = ~row_all_max_i32(~float_to_ordered_int(real ? v[u][a] : inf));
-                hi[a] = row_all_max_i32(float_to_ordered_int(real ? v[u][a] : -inf));
+                lo[a] = fminf(lo[a], p[u][a]);
+                hi[a] = fmaxf(hi[a], p[u][a]);
             }
-            if ((lane & 15) == 0)
+            const int wave_lo = wave_min_i32(float_to_ordered_int(lo[a]));
+            const int wave_hi = wave_max_i32(float_to_ordered_int(hi[a]));
+            if (lane == 0)
             {
-                int* const run_box = run_boxes + (q / 16) * 6;
+                atomicMin(&cloud_box[a], wave_lo);
+                atomicMax(&cloud_box[3 + a], wave_hi);
+            }
+        }
+    }
+    __syncthreads();
+
+    // the bin of every point: position on the curve of its cell of the 16^3 grid (with cloud ids: the
+    // first 7 distinct-id offsets come first, one id after the other, each in curve order; the rest together)
+    int bin[PER];
+    {
+        const CurveGrid grid = curve_grid(cloud_box);
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            unsigned cell[3];
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+                cell[a] = curve_grid_cell(p[u][a], grid.lo[a], grid.scale[a]);
+            unsigned b = bin_of_cell[(cell[0] >> 2) | ((cell[1] >> 2) << 4) | ((cell[2] >> 2) << 8)];
+            if (group)
+            {
+                b = (static_cast<unsigned>(id_offset[u]) << 9) | (b >> 3);
+            }
+            bin[u] = static_cast<int>(b);
+            if (tid + u * NG_SORT_THREADS < n)
+                atomicAdd(&bins[b], 1);
+        }
+    }
+    __syncthreads();
+    {
+        // exclusive prefix sum over the bins: where every bin starts
+        int count[CURVE_BINS / NG_SORT_THREADS];
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < CURVE_BINS / NG_SORT_THREADS; ++i)
+        {
+            count[i] = bins[tid * (CURVE_BINS / NG_SORT_THREADS) + i];
+            sum += count[i];
+        }
+        const int before_in_wave = wave_exclusive_sum(sum);
+        if (lane == TPK_WAVE - 1)
+            wave_totals[wave] = before_in_wave + sum;
+        __syncthreads();
+        int run = before_in_wave;
+        for (int w = 0; w < wave; ++w)
+            run += wave_totals[w];
+#pragma unroll
+        for (int i = 0; i < CURVE_BINS / NG_SORT_THREADS; ++i)
+        {
+            bins[tid * (CURVE_BINS / NG_SORT_THREADS) + i] = run;
+            run += count[i];
+        }
+    }
+    __syncthreads();
+    // every point takes the next place of its bin; its record goes straight there
+    {
+        int place[PER];
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            place[u] = tid + u * NG_SORT_THREADS < n ? atomicAdd(&bins[bin[u]], 1) : -1;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            if (place[u] >= 0)
+                sorted[place[u]] = make_float4(p[u][0], p[u][1], p[u][2],
+                                               __int_as_float(static_cast<int>(in_cloud) + tid + u * NG_SORT_THREADS));
+    }
+    const int padded = cells * NG_CELL;
+    {
+        // records behind the last point: infinitely far away
+        const float inf = __builtin_inff();
+        for (int q = n + tid; q < padded; q += NG_SORT_THREADS)
+            sorted[q] = make_float4(inf, inf, inf, __int_as_float(0x7FFFFFFF));
+    }
+    // Every place is taken: `bins` now holds the end of every bin, and the records have been stored.  The barrier
+    // orders memory at workgroup scope, which is all the read-back below needs: the wavefronts of a workgroup share
+    // one L1, which holds no older copy of these lines (a wider fence would write the whole L2 back: 20 us).
+    __syncthreads();
+    if (boxes)
+    {
+        // The records in order, as the other wavefronts stored them: boxes of the runs of 16 (DPP row reductions).
+        constexpr int BATCH = 4;
+        for (int q0 = tid; q0 < padded; q0 += NG_SORT_THREADS * BATCH)
+        {
+            float4 rec[BATCH];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+                rec[u] = sorted[min(q0 + u * NG_SORT_THREADS, padded - 1)];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+            {
+                const int q = q0 + u * NG_SORT_THREADS;
+                if (q >= padded) // uniform over the wavefront: cells are whole
+                    continue;
+                const bool real = __float_as_int(rec[u].w) != 0x7FFFFFFF;
+                const float inf = __builtin_inff();
+                const float v[3] = {rec[u].x, rec[u].y, rec[u].z};
+                int lo[3], hi[3];
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
                 {
-                    run_box[a] = lo[a];
-                    run_box[3 + a] = hi[a];
+                    lo[a] = ~row_all_max_i32(~float_to_ordered_int(real ? v[a] : inf));
+                    hi[a] = row_all_max_i32(float_to_ordered_int(real ? v[a] : -inf));
+                }
+                if ((lane & 15) == 0)
+                {
+                    int* const run_box = run_boxes + (q / 16) * 6;
+#pragma unroll
+                    for (int a = 0; a < 3; ++a)
+                    {
+                        run_box[a] = lo[a];
+                        run_box[3 + a] = hi[a];
+                    }
                 }
             }
         }
@@ -189,17 +311,18 @@ __device__ __forceinline__ float point_box_dist2(float x, float y, float z, floa
 int launch_curve_cells(const PointSet& a, const PointSet& c, int* zero_word, hipStream_t s)
 {
     const int largest = a.stride > c.stride ? a.stride : c.stride;
-    const int key_capacity = largest > CURVE_BINS ? (largest + 63) & ~63 : CURVE_BINS; // (the ordering borrows CURVE_BINS words)
+    if (largest > CURVE_MAX_POINTS)
+        return TPK_ERR_UNSUPPORTED; // (a thread holds 16 points of a window: windows of at most 16384 points)
     const int64_t windows_a = set_windows(a), windows_c = set_windows(c);
     if (windows_a + windows_c > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    const size_t lds = (2 * static_cast<size_t>(key_capacity) + CURVE_BINS) * sizeof(unsigned);
+    const size_t most_cells = static_cast<size_t>((largest + NG_CELL - 1) / NG_CELL);
+    const size_t lds = (2 * static_cast<size_t>(CURVE_BINS) + 24 * most_cells) * sizeof(unsigned);
     const int allowed = tpk_allow_lds(reinterpret_cast<const void*>(curve_cells_kernel), lds);
     if (allowed != TPK_OK)
         return allowed;
     hipLaunchKernelGGL(curve_cells_kernel, dim3(static_cast<unsigned>(windows_a + windows_c)),
-                       dim3(NG_SORT_THREADS), lds, s, a, c, static_cast<int>(windows_a), key_capacity,
-                       zero_word);
+                       dim3(NG_SORT_THREADS), lds, s, a, c, static_cast<int>(windows_a), zero_word);
     return tpk_launch_status();
 }
 
