@@ -969,20 +969,22 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
     const int log2_bs = reference_log2_block(n);
     const int groups = static_cast<int>(tpk_ceil_div(n, 1 << log2_bs));
 
-    // Tiny clouds: one point per lane, no sorting.  Up to 16384 points: registers of a
-    // 512-lane workgroup, curve order and pruning (cells of 64, 128 or 256 points).
+    // Tiny clouds: one point per lane, no sorting.  Up to 16384 points: registers of a workgroup of 512 or
+    // 1024 lanes, curve order and pruning (cells of 64, 128 or 256 points).  Shapes as measured: sixteen
+    // wavefronts with half as many points each shorten a round (fewer cells per wavefront to update, fewer
+    // groups for the winner to search) except between 4097 and 8192 points.
     if (n <= 512)
         launch_resident<1, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 2)
         return launch_pruned<2, 512, 1>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 4)
-        return launch_pruned<4, 512, 1>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<2, 1024, 2>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 8)
-        return launch_pruned<8, 512, 2>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<4, 1024, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 16)
         return launch_pruned<16, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_REGISTER_POINTS)
-        return launch_pruned<32, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<16, 1024, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_CELL_POINTS && workspace && workspace_bytes >= cell_layout(b, n).total)
     {
         // Cells of 64 points in memory, their summaries in LDS.
