@@ -110,7 +110,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     for (int i = tid; i < CURVE_BINS; i += NG_SORT_THREADS)
     {
         bins[i] = 0;
-        bin_of_cell[i] = curve_bin_of_cell(i & 15, (i >> 4) & 15, i >> 8);
+        bin_of_cell[i] = curve_bin_table.bin[i]; // (= curve_bin_of_cell(i & 15, (i >> 4) & 15, i >> 8))
     }
     __syncthreads();
     {
@@ -145,6 +145,9 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
 #pragma unroll
         for (int u = 0; u < PER; ++u)
         {
+            bin[u] = 0;
+            if (u * NG_SORT_THREADS >= n) // (uniform over the workgroup: a short window has fewer rounds)
+                continue;
             unsigned cell[3];
 #pragma unroll
             for (int a = 0; a < 3; ++a)
@@ -211,7 +214,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     if (boxes)
     {
         // The records in order, as the other wavefronts stored them: boxes of the runs of 16 (DPP row reductions).
-        constexpr int BATCH = 4;
+        constexpr int BATCH = 16; // (all records of a thread are requested before the first is used: one trip to the L2)
         for (int q0 = tid; q0 < padded; q0 += NG_SORT_THREADS * BATCH)
         {
             float4 rec[BATCH];
@@ -227,12 +230,14 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
                 const bool real = __float_as_int(rec[u].w) != 0x7FFFFFFF;
                 const float inf = __builtin_inff();
                 const float v[3] = {rec[u].x, rec[u].y, rec[u].z};
+                (void)inf;
                 int lo[3], hi[3];
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
                 {
-                    lo[a] = ~row_all_max_i32(~float_to_ordered_int(real ? v[a] : inf));
-                    hi[a] = row_all_max_i32(float_to_ordered_int(real ? v[a] : -inf));
+                    const int ordered = float_to_ordered_int(v[a]);
+                    lo[a] = row_all_min_i32(real ? ordered : 0x7FFFFFFF);
+                    hi[a] = row_all_max_i32(real ? ordered : INT_MIN);
                 }
                 if ((lane & 15) == 0)
                 {
@@ -253,17 +258,16 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
         __syncthreads();
         for (int c = tid; c < cells; c += NG_SORT_THREADS)
         {
+            // (an empty run keeps (INT_MAX, INT_MIN), which map to NaN patterns: written as (+inf, -inf))
+            auto as_lo = [](int o) { return o == 0x7FFFFFFF ? __builtin_inff() : ordered_int_to_float(o); };
+            auto as_hi = [](int o) { return o == INT_MIN ? -__builtin_inff() : ordered_int_to_float(o); };
             int lo[3] = {0x7FFFFFFF, 0x7FFFFFFF, 0x7FFFFFFF}, hi[3] = {INT_MIN, INT_MIN, INT_MIN};
 #pragma unroll
             for (int r = 0; r < 4; ++r)
             {
                 const int* const run_box = run_boxes + (c * 4 + r) * 6;
-                boxes[c * NG_BOX + 2 + r * 2 + 0] =
-                    make_float4(ordered_int_to_float(run_box[0]), ordered_int_to_float(run_box[1]),
-                                ordered_int_to_float(run_box[2]), 0.f);
-                boxes[c * NG_BOX + 2 + r * 2 + 1] =
-                    make_float4(ordered_int_to_float(run_box[3]), ordered_int_to_float(run_box[4]),
-                                ordered_int_to_float(run_box[5]), 0.f);
+                boxes[c * NG_BOX + 2 + r * 2 + 0] = make_float4(as_lo(run_box[0]), as_lo(run_box[1]), as_lo(run_box[2]), 0.f);
+                boxes[c * NG_BOX + 2 + r * 2 + 1] = make_float4(as_hi(run_box[3]), as_hi(run_box[4]), as_hi(run_box[5]), 0.f);
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
                 {
@@ -271,10 +275,8 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
                     hi[a] = max(hi[a], run_box[3 + a]);
                 }
             }
-            boxes[c * NG_BOX + 0] = make_float4(ordered_int_to_float(lo[0]), ordered_int_to_float(lo[1]),
-                                                ordered_int_to_float(lo[2]), 0.f);
-            boxes[c * NG_BOX + 1] = make_float4(ordered_int_to_float(hi[0]), ordered_int_to_float(hi[1]),
-                                                ordered_int_to_float(hi[2]), 0.f);
+            boxes[c * NG_BOX + 0] = make_float4(as_lo(lo[0]), as_lo(lo[1]), as_lo(lo[2]), 0.f);
+            boxes[c * NG_BOX + 1] = make_float4(as_hi(hi[0]), as_hi(hi[1]), as_hi(hi[2]), 0.f);
         }
     }
     if (set.bin_ends)

@@ -18,6 +18,16 @@ __device__ __forceinline__ unsigned row_all_min_u32(unsigned v)
     return v;
 }
 
+// Minimum over each row of 16 lanes, in every lane of the row (built like row_all_max_i32).
+__device__ __forceinline__ int row_all_min_i32(int v)
+{
+    v = min(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));
+    v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));
+    v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, true));
+    v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true));
+    return v;
+}
+
 __device__ __forceinline__ int wave_min_i32(int v)
 {
     return ~wave_max_i32(~v);
@@ -78,6 +88,52 @@ __device__ __forceinline__ unsigned curve_bin_of_cell(unsigned bx, unsigned by, 
 {
     return hilbert_code<4>(bx, by, bz);
 }
+
+// The same position computed at compile time, and the table of all 4096 cells of the 16^3 grid (the ordering
+// kernel copies it to LDS instead of computing 4096 positions per window).
+constexpr unsigned spread_bits_6_const(unsigned v)
+{
+    v &= 0x3Fu;
+    v = (v | (v << 8)) & 0x300Fu;
+    v = (v | (v << 4)) & 0x30C3u;
+    v = (v | (v << 2)) & 0x9249u;
+    return v;
+}
+constexpr unsigned hilbert_code_const(int bits, unsigned x0, unsigned x1, unsigned x2)
+{
+    unsigned x[3] = {x0, x1, x2};
+    for (unsigned q = 1u << (bits - 1); q > 1u; q >>= 1)
+    {
+        const unsigned p = q - 1u;
+        for (int i = 0; i < 3; ++i)
+        {
+            const bool high = (x[i] & q) != 0;
+            const unsigned t = (x[0] ^ x[i]) & p;
+            const unsigned first = high ? x[0] ^ p : x[0] ^ t;
+            if (i)
+                x[i] = high ? x[i] : x[i] ^ t;
+            x[0] = first;
+        }
+    }
+    x[1] ^= x[0];
+    x[2] ^= x[1];
+    unsigned t = 0;
+    for (unsigned q = 1u << (bits - 1); q > 1u; q >>= 1)
+        t ^= (x[2] & q) ? q - 1u : 0u;
+    return (spread_bits_6_const(x[0] ^ t) << 2) | (spread_bits_6_const(x[1] ^ t) << 1) | spread_bits_6_const(x[2] ^ t);
+}
+struct CurveBinTable
+{
+    unsigned short bin[4096]; // [bx | by << 4 | bz << 8]
+};
+constexpr CurveBinTable make_curve_bin_table()
+{
+    CurveBinTable t{};
+    for (unsigned i = 0; i < 4096; ++i)
+        t.bin[i] = static_cast<unsigned short>(hilbert_code_const(4, i & 15u, (i >> 4) & 15u, i >> 8));
+    return t;
+}
+__device__ const CurveBinTable curve_bin_table = make_curve_bin_table();
 
 // Order-preserving map of a float to a signed integer (for integer atomic min / max).
 __device__ __forceinline__ int float_to_ordered_int(float f)
