@@ -105,7 +105,7 @@ def test_library_exports_every_declared_symbol():
     assert lib.tpk_ball_query_partial_workspace_bytes(8191, 100, 16) == 0
     assert lib.tpk_ball_query_partial_workspace_bytes(40000, 100, 0) == 0
     windows = 3  # 40000 support points in windows of 16384
-    assert lib.tpk_ball_query_partial_workspace_bytes(40000, 100, 16) == windows * (16384 * 16 + 4096 * 4) + 256
+    assert lib.tpk_ball_query_partial_workspace_bytes(40000, 100, 16) == windows * (16384 * 16 + 4096 * 4) + 256 + 1024  # + the queries' cloud rows, 8 bytes each
 
 
 def test_argument_errors_are_reported_without_a_gpu():

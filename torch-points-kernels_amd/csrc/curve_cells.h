@@ -44,6 +44,72 @@ __host__ __device__ inline int64_t set_windows(const PointSet& s)
     return s.total > 0 ? (s.total / s.cloud_points) * set_windows_per_cloud(s) : 0;
 }
 
+// The equal range [first, last) of value v in sorted a[0..len), found by the whole wavefront: 64
+// samples per round instead of one, and both ends in the same rounds, so that their loads
+// travel together.
+__device__ __forceinline__ void wave_equal_range(const int64_t* __restrict__ a, int len, int64_t v, int lane,
+                                                 int& first, int& last)
+{
+    int lo0 = 0, hi0 = len, lo1 = 0, hi1 = len;
+    while (hi0 > lo0 || hi1 > lo1)
+    {
+        const int step0 = (hi0 - lo0 + TPK_WAVE - 1) / TPK_WAVE, step1 = (hi1 - lo1 + TPK_WAVE - 1) / TPK_WAVE;
+        const int pos0 = lo0 + lane * step0, pos1 = lo1 + lane * step1;
+        const bool in0 = pos0 < hi0, in1 = pos1 < hi1;
+        const int64_t sample0 = a[in0 ? pos0 : 0], sample1 = a[in1 ? pos1 : 0];
+        const unsigned long long ge0 = __ballot(!in0 || sample0 >= v);
+        const unsigned long long ge1 = __ballot(!in1 || sample1 > v);
+        if (hi0 > lo0)
+        {
+            const int f = ge0 ? __builtin_ctzll(ge0) : TPK_WAVE;
+            const int next_lo = f > 0 ? lo0 + (f - 1) * step0 + 1 : lo0;
+            hi0 = f < TPK_WAVE ? min(lo0 + f * step0, hi0) : hi0;
+            lo0 = next_lo;
+        }
+        if (hi1 > lo1)
+        {
+            const int f = ge1 ? __builtin_ctzll(ge1) : TPK_WAVE;
+            const int next_lo = f > 0 ? lo1 + (f - 1) * step1 + 1 : lo1;
+            hi1 = f < TPK_WAVE ? min(lo1 + f * step1, hi1) : hi1;
+            lo1 = next_lo;
+        }
+    }
+    first = lo0;
+    last = lo1;
+}
+
+// Work that rides along with an ordering launch, in workgroups of its own behind those of the
+// windows: for every query of a packed call, the rows [x, y) of the support points that carry
+// the query's cloud id (both id arrays sorted).  A wavefront takes 64 consecutive queries and
+// searches once per distinct id among them - nearly always one.
+struct CloudRows
+{
+    const int64_t* batch_x;
+    const int64_t* batch_y;
+    int size_x;
+    int64_t size_y;
+    int2* rows;
+};
+
+__device__ __forceinline__ void cloud_rows_job(const CloudRows& job, int64_t group, int tid)
+{
+    const int lane = tid & (TPK_WAVE - 1);
+    const int64_t q = (group * (NG_SORT_THREADS / TPK_WAVE) + tid / TPK_WAVE) * TPK_WAVE + lane;
+    const bool has = q < job.size_y;
+    const int64_t mine = has ? job.batch_y[q] : 0;
+    unsigned long long todo = __ballot(has);
+    while (todo != 0)
+    {
+        const int64_t id = __shfl(mine, __builtin_ctzll(todo));
+        int first, last;
+        wave_equal_range(job.batch_x, job.size_x, id, lane, first, last);
+        const bool same = has && mine == id;
+        if (same)
+            job.rows[q] = make_int2(first, last);
+        todo &= ~__ballot(same); // (the lane that gave the id is among them: the loop ends)
+    }
+}
+
 // One workgroup orders one window: the first windows_a blocks those of set_a, the rest set_b.
 // `zero_word` (optional) is cleared by the first block: a counter used by the kernel that follows.
 // The window's points are read once and stay in registers (16 per thread): bounding box, curve
@@ -55,7 +121,8 @@ __host__ __device__ inline int64_t set_windows(const PointSet& s)
 // served; it decides where a point sits inside its bin, never what a search over the cells returns.
 // dynamic LDS: (2 * CURVE_BINS + 24 * cells) words.
 __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet set_a, PointSet set_b,
-                                                                      int windows_a, int* zero_word)
+                                                                      int windows_a, int windows, int* zero_word,
+                                                                      CloudRows rows_job)
 {
     extern __shared__ unsigned bin_of_cell[];  // [CURVE_BINS] curve position of every cell of the 16^3 grid
     int* const bins = reinterpret_cast<int*>(bin_of_cell) + CURVE_BINS; // [CURVE_BINS]
@@ -65,6 +132,11 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     constexpr int PER = CURVE_MAX_POINTS / NG_SORT_THREADS; // points per thread
     static_assert(CURVE_BINS % NG_SORT_THREADS == 0, "every thread scans the same number of bins");
 
+    if (static_cast<int>(blockIdx.x) >= windows)
+    {
+        cloud_rows_job(rows_job, static_cast<int>(blockIdx.x) - windows, threadIdx.x);
+        return;
+    }
     const bool first_set = static_cast<int>(blockIdx.x) < windows_a;
     const PointSet set = first_set ? set_a : set_b;
     const int64_t window = first_set ? blockIdx.x : blockIdx.x - windows_a;
@@ -310,21 +382,24 @@ __device__ __forceinline__ float point_box_dist2(float x, float y, float z, floa
     return __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz));
 }
 
-int launch_curve_cells(const PointSet& a, const PointSet& c, int* zero_word, hipStream_t s)
+int launch_curve_cells(const PointSet& a, const PointSet& c, int* zero_word, hipStream_t s,
+                       const CloudRows& rows_job = CloudRows{nullptr, nullptr, 0, 0, nullptr})
 {
     const int largest = a.stride > c.stride ? a.stride : c.stride;
     if (largest > CURVE_MAX_POINTS)
         return TPK_ERR_UNSUPPORTED; // (a thread holds 16 points of a window: windows of at most 16384 points)
     const int64_t windows_a = set_windows(a), windows_c = set_windows(c);
-    if (windows_a + windows_c > 0x7fffffffLL)
+    const int64_t row_groups = tpk_ceil_div(rows_job.size_y, NG_SORT_THREADS);
+    if (windows_a + windows_c + row_groups > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     const size_t most_cells = static_cast<size_t>((largest + NG_CELL - 1) / NG_CELL);
     const size_t lds = (2 * static_cast<size_t>(CURVE_BINS) + 24 * most_cells) * sizeof(unsigned);
     const int allowed = tpk_allow_lds(reinterpret_cast<const void*>(curve_cells_kernel), lds);
     if (allowed != TPK_OK)
         return allowed;
-    hipLaunchKernelGGL(curve_cells_kernel, dim3(static_cast<unsigned>(windows_a + windows_c)),
-                       dim3(NG_SORT_THREADS), lds, s, a, c, static_cast<int>(windows_a), zero_word);
+    hipLaunchKernelGGL(curve_cells_kernel, dim3(static_cast<unsigned>(windows_a + windows_c + row_groups)),
+                       dim3(NG_SORT_THREADS), lds, s, a, c, static_cast<int>(windows_a),
+                       static_cast<int>(windows_a + windows_c), zero_word, rows_job);
     return tpk_launch_status();
 }
 

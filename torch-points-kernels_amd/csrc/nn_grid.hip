@@ -576,8 +576,9 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
 // The support array is cut into windows of CURVE_MAX_POINTS consecutive rows, each ordered on its
 // own (curve_cells_kernel), which groups a window's points by the cell of a 16^3 grid over the
 // window's bounding box; the ordering kernel also leaves where each such bin ends.  One
-// wavefront serves one query: it finds the support rows of the query's cloud (the windows they
-// lie in), and in every window the bins that the cube around the ball touches - a handful
+// wavefront serves one query: it reads which support rows belong to the query's cloud (found for
+// every query by workgroups that ride along with the ordering launch), and so the windows they
+// lie in, and finds in every window the bins that the cube around the ball touches - a handful
 // when the radius is small against the cloud - and tests their points, 64 per step, one per
 // lane.  A candidate is a hit when its squared distance is <= radius^2 and its row lies in the
 // query's cloud.  The hits (at most 64) are collected in LDS, ranked by row, and written in
@@ -589,40 +590,6 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
 // neighbourhoods, where the scan ends soon.
 // ---------------------------------------------------------------------------------------
 constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
-
-// The equal range [first, last) of value v in sorted a[0..len), found by the whole wavefront: 64
-// samples per round instead of one, and both ends in the same rounds, so that their loads
-// travel together.
-__device__ __forceinline__ void wave_equal_range(const int64_t* __restrict__ a, int len, int64_t v, int lane,
-                                                 int& first, int& last)
-{
-    int lo0 = 0, hi0 = len, lo1 = 0, hi1 = len;
-    while (hi0 > lo0 || hi1 > lo1)
-    {
-        const int step0 = (hi0 - lo0 + TPK_WAVE - 1) / TPK_WAVE, step1 = (hi1 - lo1 + TPK_WAVE - 1) / TPK_WAVE;
-        const int pos0 = lo0 + lane * step0, pos1 = lo1 + lane * step1;
-        const bool in0 = pos0 < hi0, in1 = pos1 < hi1;
-        const int64_t sample0 = a[in0 ? pos0 : 0], sample1 = a[in1 ? pos1 : 0];
-        const unsigned long long ge0 = __ballot(!in0 || sample0 >= v);
-        const unsigned long long ge1 = __ballot(!in1 || sample1 > v);
-        if (hi0 > lo0)
-        {
-            const int f = ge0 ? __builtin_ctzll(ge0) : TPK_WAVE;
-            const int next_lo = f > 0 ? lo0 + (f - 1) * step0 + 1 : lo0;
-            hi0 = f < TPK_WAVE ? min(lo0 + f * step0, hi0) : hi0;
-            lo0 = next_lo;
-        }
-        if (hi1 > lo1)
-        {
-            const int f = ge1 ? __builtin_ctzll(ge1) : TPK_WAVE;
-            const int next_lo = f > 0 ? lo1 + (f - 1) * step1 + 1 : lo1;
-            hi1 = f < TPK_WAVE ? min(lo1 + f * step1, hi1) : hi1;
-            lo1 = next_lo;
-        }
-    }
-    first = lo0;
-    last = lo1;
-}
 
 // Range of 16^3-grid cells along one axis that [v - r, v + r] can touch.  The interval is widened
 // by a few ulps of its ends so that a point the fp32 radius test accepts is never left out.
@@ -636,8 +603,8 @@ __device__ __forceinline__ void bin_range(float v, float r, float lo, float scal
 __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     int size_x, int size_y, float radius, float radius2, int nsample, const float* __restrict__ x,
     const float* __restrict__ y, const float4* __restrict__ sorted_x, const int* __restrict__ bin_ends,
-    const float4* __restrict__ grids, const int64_t* __restrict__ batch_x,
-    const int64_t* __restrict__ batch_y, int64_t* __restrict__ idx, float* __restrict__ dist)
+    const float4* __restrict__ grids, const int2* __restrict__ cloud_rows, int64_t* __restrict__ idx,
+    float* __restrict__ dist)
 {
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
     __shared__ int hit_rows[WAVES][BQB_HITS];
@@ -655,9 +622,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
 
     const float ux = y[q * 3 + 0], uy = y[q * 3 + 1], uz = y[q * 3 + 2];
     const float qx = to_vector_register(ux), qy = to_vector_register(uy), qz = to_vector_register(uz);
-    const int64_t cloud = batch_y[q];
-    int s0, s1;
-    wave_equal_range(batch_x, size_x, cloud, lane, s0, s1);
+    const int2 cloud = cloud_rows[q]; // the support rows of the query's cloud
+    const int s0 = cloud.x, s1 = cloud.y;
     const int64_t out = q * nsample;
     TPK_WORK_DECL
 
@@ -1223,10 +1189,10 @@ namespace {
 
 struct BallLayout
 {
-    size_t sorted_x, bin_ends, grids, total;
+    size_t sorted_x, bin_ends, grids, cloud_rows, total;
 };
 
-BallLayout ball_layout(int64_t size_x)
+BallLayout ball_layout(int64_t size_x, int64_t size_y)
 {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
     const size_t wx = static_cast<size_t>((size_x + CURVE_MAX_POINTS - 1) / CURVE_MAX_POINTS);
@@ -1238,6 +1204,8 @@ BallLayout ball_layout(int64_t size_x)
     pos = up(pos + wx * CURVE_BINS * sizeof(int));
     l.grids = pos;
     pos = up(pos + wx * 2 * sizeof(float4));
+    l.cloud_rows = pos;
+    pos = up(pos + static_cast<size_t>(size_y) * sizeof(int2));
     l.total = pos;
     return l;
 }
@@ -1252,7 +1220,7 @@ bool ball_bins_supported(int64_t size_x, int64_t size_y, int nsample)
 
 size_t tpk_grid_ball_query_workspace_bytes(int64_t size_x, int64_t size_y, int nsample)
 {
-    return ball_bins_supported(size_x, size_y, nsample) ? ball_layout(size_x).total : 0;
+    return ball_bins_supported(size_x, size_y, nsample) ? ball_layout(size_x, size_y).total : 0;
 }
 
 int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample,
@@ -1262,7 +1230,7 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
 {
     if (!ball_bins_supported(size_x, size_y, nsample))
         return TPK_ERR_UNSUPPORTED;
-    const BallLayout l = ball_layout(size_x);
+    const BallLayout l = ball_layout(size_x, size_y);
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
@@ -1270,7 +1238,8 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
     PointSet px{x, nullptr, size_x, size_x, CURVE_MAX_POINTS, reinterpret_cast<float4*>(w + l.sorted_x), nullptr,
                 reinterpret_cast<int*>(w + l.bin_ends), reinterpret_cast<float4*>(w + l.grids)};
     PointSet none{nullptr, nullptr, 0, 1, CURVE_MAX_POINTS, nullptr, nullptr, nullptr, nullptr};
-    int st = launch_curve_cells(px, none, nullptr, s);
+    const CloudRows rows{batch_x, batch_y, static_cast<int>(size_x), size_y, reinterpret_cast<int2*>(w + l.cloud_rows)};
+    int st = launch_curve_cells(px, none, nullptr, s, rows);
     if (st != TPK_OK)
         return st;
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
@@ -1279,6 +1248,6 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
         return TPK_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(ball_query_bins_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
                        static_cast<int>(size_x), static_cast<int>(size_y), std::fabs(radius), radius2, nsample, x, y,
-                       px.sorted, px.bin_ends, px.grid, batch_x, batch_y, idx, dist);
+                       px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
     return tpk_launch_status();
 }
