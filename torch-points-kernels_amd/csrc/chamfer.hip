@@ -481,11 +481,12 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
     }
     (void)workspace;
     (void)workspace_bytes;
-    // Chains in LDS (no workspace): as many target ranges per cloud as give the chip a few hundred
-    // workgroups, each of at least 1024 targets; clouds too large for LDS scatter with atomics.
+    // Chains in LDS (no workspace): as many target ranges per cloud as give every compute unit one
+    // workgroup and none a second (config 5: 256 workgroups 19.7 us, 320 or 1024: 24 us, 512: 20.4 us),
+    // each of at least 1024 targets; clouds too large for LDS scatter with atomics.
     {
         const int larger = n > m ? n : m;
-        int splits = static_cast<int>(tpk_ceil_div(320, 2 * static_cast<int64_t>(b)));
+        int splits = TPK_COMPUTE_UNITS / (2 * b);
         const int most = static_cast<int>(tpk_ceil_div(larger, CHB_THREADS));
         splits = splits > most ? most : splits;
         splits = splits < 1 ? 1 : splits;

@@ -23,6 +23,9 @@
 // LDS a workgroup may use on gfx950 (160 KiB); the kernels stay below it.
 #define TPK_LDS_BYTES 163840
 
+// Compute units of an MI355X (8 dies of 32).
+#define TPK_COMPUTE_UNITS 256
+
 static inline hipStream_t tpk_stream(void* s)
 {
     return reinterpret_cast<hipStream_t>(s);
