@@ -655,36 +655,42 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
         serial = __ballot(nbins > TPK_WAVE) != 0 || pairs > 8 * TPK_WAVE;
         // 64 (window, bin) pairs at a time; nearly always there are no more than that
         auto walk_pairs = [&](int pair0) __attribute__((always_inline)) {
-            // one descriptor per pair, written by the window's lane
+            // one descriptor per pair, written by the window's lane: a window's block holds a few bins, so a loop
+            // is cheaper here than the marks used for the candidates below (64.6 against 62 us on 58750 queries)
+            // (volatile: what a lane reads back was written by other lanes)
+            volatile int* const marks = slots;
             for (int i = max(0, pair0 - pairs_before); i < nbins && pairs_before + i < pair0 + TPK_WAVE; ++i)
-                slots[pairs_before + i - pair0] = block | (i << 20);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                marks[pairs_before + i - pair0] = block | (i << 20);
             // lane p: where the points of pair pair0 + p start in the ordered array, and how many
             int start = 0, size = 0;
             if (pair0 + lane < pairs)
             {
-                const int d = slots[lane];
+                const int d = marks[lane];
+                const int i = (d >> 20) & 63, window = (d >> 26) & 63;
                 const int fx = d & 15, fy = (d >> 4) & 15, fz = (d >> 8) & 15;
                 const int nx = ((d >> 12) & 15) + 1, ny = ((d >> 16) & 15) + 1;
-                const int i = (d >> 20) & 63, wx = wx0 + ((d >> 26) & 63);
-                const unsigned bin = curve_bin_of_cell(fx + i % nx, fy + (i / nx) % ny, fz + i / (nx * ny));
+                const int wx = wx0 + window;
+                // (the table of the ordering kernel: 8 KiB that every wavefront reads, at home in the caches)
+                const unsigned bin = curve_bin_table.bin[(fx + i % nx) | ((fy + (i / nx) % ny) << 4) | ((fz + i / (nx * ny)) << 8)];
                 const int* __restrict__ ends = bin_ends + static_cast<int64_t>(wx) * CURVE_BINS;
                 start = bin ? ends[bin - 1] : 0;
                 size = ends[bin] - start;
                 start += wx * CURVE_MAX_POINTS;
             }
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             const int before = wave_exclusive_sum(size);
             const int total = __builtin_amdgcn_readlane(before + size, TPK_WAVE - 1);
+            const int origin = start - before; // candidate c of this walk lies at origin + c, for the c of this lane's pair
             for (int c0 = 0; c0 < total && !serial; c0 += TPK_WAVE)
             {
-                // the pairs' lanes hand out the addresses of candidates c0 .. c0 + 63
-                for (int i = max(0, c0 - before); i < size && before + i < c0 + TPK_WAVE; ++i)
-                    slots[before + i - c0] = start + i;
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                // Which pair does candidate c0 + lane belong to?  Every pair's lane marks the slot of its first
+                // candidate in this step with its own number; a running maximum over the slots carries the
+                // number on to the pair's other candidates.
+                marks[lane] = 0;
+                if (size > 0 && before < c0 + TPK_WAVE && before + size > c0)
+                    marks[max(before - c0, 0)] = lane;
+                const int mark = marks[lane];
                 const bool has = c0 + lane < total;
-                const int at_x = has ? slots[lane] : start;
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const int at_x = __shfl(origin, wave_inclusive_max_i32(mark)) + c0 + lane;
                 const float4 p = sorted_x[has ? at_x : 0];
                 const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
                 TPK_WORK_ADD(1);

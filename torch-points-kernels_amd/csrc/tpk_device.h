@@ -171,6 +171,20 @@ __device__ __forceinline__ int wave_exclusive_sum(int v)
     return s - v;
 }
 
+// Largest of the values v >= 0 of this lane and the lanes below it (the same steps with a maximum).
+__device__ __forceinline__ int wave_inclusive_max_i32(int v)
+{
+    int s = v;
+    s = max(s, __builtin_amdgcn_update_dpp(0, s, 0x111, 0xF, 0xF, false)); // row_shr:1
+    s = max(s, __builtin_amdgcn_update_dpp(0, s, 0x112, 0xF, 0xF, false)); // row_shr:2
+    s = max(s, __builtin_amdgcn_update_dpp(0, s, 0x114, 0xF, 0xF, false)); // row_shr:4
+    s = max(s, __builtin_amdgcn_update_dpp(0, s, 0x118, 0xF, 0xF, false)); // row_shr:8
+    const int r0 = __builtin_amdgcn_readlane(s, 15);
+    const int r1 = max(r0, __builtin_amdgcn_readlane(s, 31));
+    const int r2 = max(r1, __builtin_amdgcn_readlane(s, 47));
+    const int row = (threadIdx.x & (TPK_WAVE - 1)) >> 4;
+    return max(s, row == 0 ? 0 : row == 1 ? r0 : row == 2 ? r1 : r2);
+}
 
 // Sum of v over the wavefront, the same value in every lane (row rotations, then the four row
 // totals added in lane order: the result does not depend on which lanes call it).
