@@ -84,6 +84,41 @@ __device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, const
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The same for a cell that only a few queries of the wavefront still ask for (an outlier among the
+// queries keeps admitting cells that the other 63 have long turned down): one query at a time, the
+// 64 candidates of the cell side by side in the lanes.  `want`: the lanes whose queries ask.
+// A minimum reached in the cell by several groups of NG_CHUNK candidates, or equal to the query's
+// answer so far, sets the tie flag exactly as the scan above would.
+constexpr int NG_FEW = 8; // (the scan above costs about as much as 14 queries served this way; 16: the same time, 24: slower)
+__device__ __forceinline__ void scan_cell_few(const float4* __restrict__ cand, int cell, unsigned long long want,
+                                              int lane, float qx, float qy, float qz, Nearest& s TPK_WORK_PARAM)
+{
+    const float4 p = cand[cell * NG_CELL + lane];
+    while (want != 0)
+    {
+        const int q = __builtin_ctzll(want);
+        want &= want - 1;
+        TPK_WORK_ADD(1);
+        const float ux = tpk_read_lane(qx, q), uy = tpk_read_lane(qy, q), uz = tpk_read_lane(qz, q);
+        const float d = tpk_dist2(p.x, p.y, p.z, ux, uy, uz); // (a padding candidate lies at infinity)
+        // distances are >= +0: their bit patterns order like integers (a NaN sorts above infinity)
+        const float mn = __int_as_float(wave_min_i32(__float_as_int(d)));
+        const unsigned long long at = __ballot(d == mn);
+        if (at == 0)
+            continue; // nothing but NaN
+        const int first = __builtin_ctzll(at);
+        const bool several = (at & ~(0xFFull << (first & ~(NG_CHUNK - 1)))) != 0;
+        if (lane == q)
+        {
+            const bool better = mn < s.best;
+            const bool equal = mn == s.best;
+            s.tie = better ? several : (s.tie || equal);
+            s.chunk = better ? cell * (NG_CELL / NG_CHUNK) + first / NG_CHUNK : s.chunk;
+            s.best = better ? mn : s.best;
+        }
+    }
+}
+
 // One wavefront = the 64 queries of one cell.  Logical wavefront number (after the die-local
 // block mapping) = cloud * (cells1 + cells2) + cell; the cells of cloud 1 query cloud 2 and
 // write dist1 / idx1, those of cloud 2 the other way round.
@@ -177,16 +212,16 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
                 const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
-                if (__ballot(lb * NG_MARGIN <= s.best) == 0)
-                {
-                    // no lane can improve here now, and answers only get better: never again
-                    if (lane == bit)
-                        lows[c] = __builtin_inff();
-                    continue;
-                }
-                scan_cell(cpts, cbox, c, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
+                const unsigned long long want = __ballot(lb * NG_MARGIN <= s.best);
+                // scanned, or no lane can improve here now - and answers only get better: never again
                 if (lane == bit)
                     lows[c] = __builtin_inff();
+                if (want == 0)
+                    continue;
+                if (__builtin_popcountll(want) <= NG_FEW)
+                    scan_cell_few(cpts, c, want, lane, qx, qy, qz, s TPK_WORK_ARG);
+                else
+                    scan_cell(cpts, cbox, c, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
                 if (phase)
                 {
                     bound = __int_as_float(wave_max_i32(__float_as_int(s.best)));
@@ -206,26 +241,29 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
         const int ci = __float_as_int(p.w);
         bi = (d == s.best && ci < bi) ? ci : bi;
     }
-    if (__ballot(s.tie) != 0)
+    // Several groups reached a query's minimum (about one query in 10^5 on random clouds, every query on a
+    // lattice): the lowest index over all cells that can hold that distance.  One such query at a time: the
+    // lanes test the boxes of all cells side by side, then the candidates of every cell that passes.
+    for (unsigned long long tied = __ballot(s.tie); tied != 0; tied &= tied - 1)
     {
-        // Several groups reached the minimum (rare): lowest index over all cells that can hold it.
-        for (int c = 0; c < ccells; ++c)
+        const int q = __builtin_ctzll(tied);
+        const float ux = tpk_read_lane(qx, q), uy = tpk_read_lane(qy, q), uz = tpk_read_lane(qz, q);
+        const float ub = tpk_read_lane(s.best, q);
+        int lowest = 0x7FFFFFFF;
+        for (int g = 0; g < groups; ++g)
         {
-            const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
-            if (__ballot(s.tie && lb * NG_MARGIN <= s.best) == 0)
-                continue;
-            stage[lane] = cpts[c * NG_CELL + lane];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            for (int k = 0; k < NG_CELL; ++k)
+            const int c = g * NG_CELL + lane;
+            const int cc = c < ccells ? c : 0;
+            const float lb = point_box_dist2(ux, uy, uz, cbox[cc * NG_BOX + 0], cbox[cc * NG_BOX + 1]);
+            for (unsigned long long cells = __ballot(c < ccells && lb * NG_MARGIN <= ub); cells != 0; cells &= cells - 1)
             {
-                const float4 p = stage[k];
-                const float d = tpk_dist2(p.x, p.y, p.z, qx, qy, qz);
-                const int ci = __float_as_int(p.w);
-                bi = (s.tie && d == s.best && ci < bi) ? ci : bi;
+                const float4 p = cpts[(g * NG_CELL + __builtin_ctzll(cells)) * NG_CELL + lane];
+                const float d = tpk_dist2(p.x, p.y, p.z, ux, uy, uz);
+                TPK_WORK_ADD(1);
+                lowest = min(lowest, wave_min_i32(d == ub ? __float_as_int(p.w) : 0x7FFFFFFF));
             }
-            TPK_WORK_ADD(NG_CELL);
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
+        bi = lane == q ? min(bi, lowest) : bi;
     }
     TPK_WORK_ADD(NG_CHUNK);
     TPK_WORK_FLUSH
@@ -380,12 +418,24 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
             float bound = __int_as_float(wave_max_i32(__float_as_int(s.b3)));
             unsigned long long live =
                 __ballot(lw < __builtin_inff() && (phase == 0 ? lw == 0.f : lw * NG_MARGIN <= bound));
+            // (the box of the next cell is requested before this one is dealt with: a wavefront left with
+            // an outlier among its queries turns down cell after cell and would wait for memory at each)
+            int boxed = live != 0 ? g * NG_CELL + __builtin_ctzll(live) : 0;
+            float4 next_lo = cbox[boxed * NG_BOX + 0], next_hi = cbox[boxed * NG_BOX + 1];
             while (live != 0)
             {
                 const int bit = __builtin_ctzll(live);
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
-                const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
+                const bool have = c == boxed; // (else that cell has been turned down since, by a better bound)
+                const float4 lo = have ? next_lo : cbox[c * NG_BOX + 0], hi = have ? next_hi : cbox[c * NG_BOX + 1];
+                if (live != 0)
+                {
+                    boxed = g * NG_CELL + __builtin_ctzll(live);
+                    next_lo = cbox[boxed * NG_BOX + 0];
+                    next_hi = cbox[boxed * NG_BOX + 1];
+                }
+                const float lb = point_box_dist2(qx, qy, qz, lo, hi);
                 if (__ballot(lb * NG_MARGIN <= s.b3) != 0)
                     scan_cell3(cpts, cbox, c, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
                 if (lane == bit)
@@ -541,12 +591,24 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
             float bound = __int_as_float(wave_max_i32(__float_as_int(s.worst())));
             unsigned long long live =
                 __ballot(lw < __builtin_inff() && (phase == 0 ? lw == 0.f : lw * NG_MARGIN <= bound));
+            // (the box of the next cell is requested before this one is dealt with: a wavefront left with
+            // an outlier among its queries turns down cell after cell and would wait for memory at each)
+            int boxed = live != 0 ? g * NG_CELL + __builtin_ctzll(live) : 0;
+            float4 next_lo = cbox[boxed * NG_BOX + 0], next_hi = cbox[boxed * NG_BOX + 1];
             while (live != 0)
             {
                 const int bit = __builtin_ctzll(live);
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
-                const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
+                const bool have = c == boxed; // (else that cell has been turned down since, by a better bound)
+                const float4 lo = have ? next_lo : cbox[c * NG_BOX + 0], hi = have ? next_hi : cbox[c * NG_BOX + 1];
+                if (live != 0)
+                {
+                    boxed = g * NG_CELL + __builtin_ctzll(live);
+                    next_lo = cbox[boxed * NG_BOX + 0];
+                    next_hi = cbox[boxed * NG_BOX + 1];
+                }
+                const float lb = point_box_dist2(qx, qy, qz, lo, hi);
                 if (__ballot(lb * NG_MARGIN <= s.worst()) != 0)
                     scan_cell_k<K>(cpts, cbox, c, stage, lane, qx, qy, qz, s);
                 if (lane == bit)
