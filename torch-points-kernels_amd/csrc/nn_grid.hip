@@ -418,24 +418,12 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
             float bound = __int_as_float(wave_max_i32(__float_as_int(s.b3)));
             unsigned long long live =
                 __ballot(lw < __builtin_inff() && (phase == 0 ? lw == 0.f : lw * NG_MARGIN <= bound));
-            // (the box of the next cell is requested before this one is dealt with: a wavefront left with
-            // an outlier among its queries turns down cell after cell and would wait for memory at each)
-            int boxed = live != 0 ? g * NG_CELL + __builtin_ctzll(live) : 0;
-            float4 next_lo = cbox[boxed * NG_BOX + 0], next_hi = cbox[boxed * NG_BOX + 1];
             while (live != 0)
             {
                 const int bit = __builtin_ctzll(live);
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
-                const bool have = c == boxed; // (else that cell has been turned down since, by a better bound)
-                const float4 lo = have ? next_lo : cbox[c * NG_BOX + 0], hi = have ? next_hi : cbox[c * NG_BOX + 1];
-                if (live != 0)
-                {
-                    boxed = g * NG_CELL + __builtin_ctzll(live);
-                    next_lo = cbox[boxed * NG_BOX + 0];
-                    next_hi = cbox[boxed * NG_BOX + 1];
-                }
-                const float lb = point_box_dist2(qx, qy, qz, lo, hi);
+                const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
                 if (__ballot(lb * NG_MARGIN <= s.b3) != 0)
                     scan_cell3(cpts, cbox, c, stage, lane, qx, qy, qz, s TPK_WORK_ARG);
                 if (lane == bit)
@@ -591,24 +579,12 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
             float bound = __int_as_float(wave_max_i32(__float_as_int(s.worst())));
             unsigned long long live =
                 __ballot(lw < __builtin_inff() && (phase == 0 ? lw == 0.f : lw * NG_MARGIN <= bound));
-            // (the box of the next cell is requested before this one is dealt with: a wavefront left with
-            // an outlier among its queries turns down cell after cell and would wait for memory at each)
-            int boxed = live != 0 ? g * NG_CELL + __builtin_ctzll(live) : 0;
-            float4 next_lo = cbox[boxed * NG_BOX + 0], next_hi = cbox[boxed * NG_BOX + 1];
             while (live != 0)
             {
                 const int bit = __builtin_ctzll(live);
                 const int c = g * NG_CELL + bit;
                 live &= live - 1;
-                const bool have = c == boxed; // (else that cell has been turned down since, by a better bound)
-                const float4 lo = have ? next_lo : cbox[c * NG_BOX + 0], hi = have ? next_hi : cbox[c * NG_BOX + 1];
-                if (live != 0)
-                {
-                    boxed = g * NG_CELL + __builtin_ctzll(live);
-                    next_lo = cbox[boxed * NG_BOX + 0];
-                    next_hi = cbox[boxed * NG_BOX + 1];
-                }
-                const float lb = point_box_dist2(qx, qy, qz, lo, hi);
+                const float lb = point_box_dist2(qx, qy, qz, cbox[c * NG_BOX + 0], cbox[c * NG_BOX + 1]);
                 if (__ballot(lb * NG_MARGIN <= s.worst()) != 0)
                     scan_cell_k<K>(cpts, cbox, c, stage, lane, qx, qy, qz, s);
                 if (lane == bit)
