@@ -1069,6 +1069,40 @@ def test_chamfer_cell_search_ties(tpk, oracle, dev):
         np.testing.assert_array_equal(_np(d2), w2)
 
 
+def test_cell_search_outliers(tpk, oracle, dev):
+    # A few far outliers in every group of 64 queries: the cells they keep admitting are served one query at a
+    # time (candidates side by side in the lanes) - also where those candidates are duplicated points or a
+    # lattice, so that equal distances meet on that path.
+    from torch_points_kernels._native import native
+    g = torch.Generator().manual_seed(11)
+    def with_outliers(cloud, share, spread):
+        cloud = cloud.clone()
+        pick = torch.rand(cloud.shape[:2], generator=g) < share
+        cloud[pick] += spread * torch.randn(int(pick.sum()), 3, generator=g)
+        return cloud
+    sphere = torch.nn.functional.normalize(torch.randn(2, 6000, 3, generator=g), dim=2)
+    base = torch.rand(1, 1500, 3, generator=g)
+    doubled = torch.cat([base, base, base.flip(1)], 1)[:, torch.randperm(4500, generator=g)]
+    ax = torch.arange(12, dtype=torch.float32) / 12
+    lattice = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(1, -1, 3)
+    cases = [(with_outliers(sphere, 0.05, 0.3), sphere.flip(1)),
+             (with_outliers(torch.rand(1, 3000, 3, generator=g), 0.03, 2.0), doubled),
+             (with_outliers(lattice, 0.04, 1.5), lattice[:, torch.randperm(1728, generator=g)]),
+             (with_outliers(torch.rand(1, 20000, 3, generator=g), 0.02, 1.0), torch.rand(1, 18000, 3, generator=g))]
+    for a, b in cases:
+        a, b = a.contiguous(), b.contiguous()
+        d1, d2, i1, i2 = native().chamfer_dist(a.to(dev), b.to(dev))
+        w1, w2, wi1, wi2 = oracle.chamfer_fwd(a.numpy(), b.numpy())
+        np.testing.assert_array_equal(_np(i1), wi1)
+        np.testing.assert_array_equal(_np(i2), wi2)
+        np.testing.assert_array_equal(_np(d1), w1)
+        np.testing.assert_array_equal(_np(d2), w2)
+        dist2, idx = native().three_nn(a.to(dev), b.to(dev))
+        wd, wi = oracle.three_nn(a.numpy(), b.numpy())
+        np.testing.assert_array_equal(_np(idx), wi)
+        np.testing.assert_array_equal(_np(dist2), wd)
+
+
 def test_chamfer_gradcheck_double(tpk, dev):
     # reference test/test_chamfer_dist.py:20-25
     from torch.autograd import gradcheck
