@@ -36,6 +36,23 @@ constexpr int NG_SCAN_THREADS = 256;         // 4 wavefronts, each searching on 
 constexpr float NG_MARGIN = 0.999998f;
 constexpr int NG_CHUNK = 8;
 
+// Box of the 64 queries of a wavefront (one query per lane; a padding lane - index 0x7FFFFFFF - holds none),
+// the same value in every lane.  The ordering kernel forms no boxes for a set that is only queried.
+__device__ __forceinline__ void query_box(float qx, float qy, float qz, bool real, float4& lo, float4& hi)
+{
+    const float v[3] = {qx, qy, qz};
+    float l[3], h[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+    {
+        const int ordered = float_to_ordered_int(v[a]);
+        l[a] = ordered_int_to_float(wave_min_i32(real ? ordered : float_to_ordered_int(__builtin_inff())));
+        h[a] = ordered_int_to_float(wave_max_i32(real ? ordered : float_to_ordered_int(-__builtin_inff())));
+    }
+    lo = make_float4(l[0], l[1], l[2], 0.f);
+    hi = make_float4(h[0], h[1], h[2], 0.f);
+}
+
 // State of one lane's nearest-neighbour search.
 struct Nearest
 {
@@ -402,8 +419,8 @@ __device__ __forceinline__ void scan_cell3_few(const float4* __restrict__ cand, 
 
 __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     int n, int m, int qcells, int ccells, int clouds, const float4* __restrict__ sorted_unknown,
-    const float4* __restrict__ sorted_known, const float4* __restrict__ boxes_unknown,
-    const float4* __restrict__ boxes_known, float* __restrict__ dist2, int32_t* __restrict__ idx)
+    const float4* __restrict__ sorted_known, const float4* __restrict__ boxes_known, float* __restrict__ dist2,
+    int32_t* __restrict__ idx)
 {
     __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
     extern __shared__ float lows_all[]; // [wavefronts][candidate cells, in whole groups of 64]
@@ -417,7 +434,6 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     const int cloud = static_cast<int>(task / qcells);
     const int qcell = static_cast<int>(task - static_cast<int64_t>(cloud) * qcells);
     const float4* __restrict__ qpts = sorted_unknown + static_cast<int64_t>(cloud) * qcells * NG_CELL;
-    const float4* __restrict__ qbox = boxes_unknown + static_cast<int64_t>(cloud) * qcells * NG_BOX;
     const float4* __restrict__ cpts = sorted_known + static_cast<int64_t>(cloud) * ccells * NG_CELL;
     const float4* __restrict__ cbox = boxes_known + static_cast<int64_t>(cloud) * ccells * NG_BOX;
     dist2 += static_cast<int64_t>(cloud) * n * 3;
@@ -431,7 +447,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     const int qindex = __float_as_int(query.w); // 0x7FFFFFFF: padding, nothing to store
     if (__ballot(qindex != 0x7FFFFFFF) == 0)
         return; // a cell without points (the last window of a cloud may have some)
-    const float4 qlo = qbox[qcell * NG_BOX + 0], qhi = qbox[qcell * NG_BOX + 1];
+    float4 qlo, qhi;
+    query_box(qx, qy, qz, qindex != 0x7FFFFFFF, qlo, qhi);
 
     const int groups = (ccells + NG_CELL - 1) / NG_CELL;
     unsigned seed_key = 0xFFFFFFFFu;
@@ -561,8 +578,7 @@ template <int K>
 __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
     int n, int k, int first, int count, float limit, int qcells, int ccells, int clouds,
     const float4* __restrict__ sorted_query, const float4* __restrict__ sorted_support,
-    const float4* __restrict__ boxes_query, const float4* __restrict__ boxes_support,
-    float* __restrict__ dist2, int64_t* __restrict__ idx)
+    const float4* __restrict__ boxes_support, float* __restrict__ dist2, int64_t* __restrict__ idx)
 {
     __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
     extern __shared__ float lows_all[]; // [wavefronts][candidate cells, in whole groups of 64]
@@ -576,7 +592,6 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
     const int cloud = static_cast<int>(task / qcells);
     const int qcell = static_cast<int>(task - static_cast<int64_t>(cloud) * qcells);
     const float4* __restrict__ qpts = sorted_query + static_cast<int64_t>(cloud) * qcells * NG_CELL;
-    const float4* __restrict__ qbox = boxes_query + static_cast<int64_t>(cloud) * qcells * NG_BOX;
     const float4* __restrict__ cpts = sorted_support + static_cast<int64_t>(cloud) * ccells * NG_CELL;
     const float4* __restrict__ cbox = boxes_support + static_cast<int64_t>(cloud) * ccells * NG_BOX;
     dist2 += static_cast<int64_t>(cloud) * n * k;
@@ -590,7 +605,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
     if (__ballot(qindex != 0x7FFFFFFF) == 0)
         return; // a cell without points (the last window of a cloud may have some)
     const bool real = qindex != 0x7FFFFFFF;
-    const float4 qlo = qbox[qcell * NG_BOX + 0], qhi = qbox[qcell * NG_BOX + 1];
+    float4 qlo, qhi;
+    query_box(qx, qy, qz, real, qlo, qhi);
 
     NearestK<K> s;
     {
@@ -963,8 +979,9 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
+    // (the unknown points are only queried: no boxes of their cells - the search forms the box of its 64 queries)
     PointSet a{unknown, nullptr, static_cast<int64_t>(b) * n, n, grid_stride(n), reinterpret_cast<float4*>(w + l.sorted_a),
-               reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
+               nullptr, nullptr, nullptr};
     PointSet c{known, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted_b),
                reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
     int st = launch_curve_cells(a, c, nullptr, s);
@@ -978,7 +995,7 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
     const size_t lds = static_cast<size_t>(NG_SCAN_THREADS / TPK_WAVE) * ((ccells + NG_CELL - 1) / NG_CELL * NG_CELL) *
                        sizeof(float);
     hipLaunchKernelGGL(three_nn_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
-                       m, qcells, ccells, b, a.sorted, c.sorted, a.boxes, c.boxes, dist2, idx);
+                       m, qcells, ccells, b, a.sorted, c.sorted, c.boxes, dist2, idx);
     return tpk_launch_status();
 }
 
@@ -1245,8 +1262,8 @@ int launch_knn_grid(int b, int n, int k, float limit, int qcells, int ccells, co
     for (int first = 0; first < k; first += K)
     {
         hipLaunchKernelGGL(knn_grid_kernel<K>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
-                           k, first, k - first < K ? k - first : K, limit, qcells, ccells, b, a.sorted, c.sorted, a.boxes,
-                           c.boxes, dist2, idx);
+                           k, first, k - first < K ? k - first : K, limit, qcells, ccells, b, a.sorted, c.sorted, c.boxes,
+                           dist2, idx);
         const int st = tpk_launch_status();
         if (st != TPK_OK)
             return st;
@@ -1267,7 +1284,7 @@ int tpk_grid_knn(int b, int n, int m, int k, float limit, const float* query, co
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
     PointSet a{query, nullptr, static_cast<int64_t>(b) * n, n, grid_stride(n), reinterpret_cast<float4*>(w + l.sorted_a),
-               reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
+               nullptr, nullptr, nullptr};
     PointSet c{support, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted_b),
                reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
     int st = launch_curve_cells(a, c, nullptr, s);
