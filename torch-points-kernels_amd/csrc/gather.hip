@@ -259,7 +259,6 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
     bool vector_loads, const float* __restrict__ grad_out, Lists<WEIGHTED> lists, float* __restrict__ grad_src)
 {
     extern __shared__ float rows[];
-    const unsigned row_bytes = static_cast<unsigned>(part_len) * 4u;
     const unsigned tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE); // (a scalar for the compiler)
@@ -275,9 +274,8 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
     const int unit1 = min(unit0 + units_per_group, units);
     const int pieces = (unit1 - unit0) * parts;
 
-    // The next piece on its way into registers: 16-byte load k of a lane covers the floats
-    // (k * G_THREADS + tid) * 4 .. + 3 of the piece's R x part_len values (part_len is a multiple of 4 here).
-    const unsigned per_row = static_cast<unsigned>(part_len) >> 2;
+    // The next piece on its way into registers: 16-byte load k of a lane covers the columns
+    // ((k / R) * G_THREADS + tid) * 4 .. + 3 of row k % R of the piece (part_len is a multiple of 4 here).
     float4 fetched[GB_FETCH];
     auto piece_source = [&](int piece, int& nrows, unsigned& len) __attribute__((always_inline)) {
         const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
@@ -296,21 +294,39 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
 #pragma unroll
         for (int k = 0; k < GB_FETCH; ++k)
         {
-            const unsigned i = static_cast<unsigned>(k) * G_THREADS + tid;
-            const unsigned r = R > 1 ? i / per_row : 0u, col = (i - r * per_row) * 4u;
+            const unsigned r = static_cast<unsigned>(k % R), col = (static_cast<unsigned>(k / R) * G_THREADS + tid) * 4u;
             fetched[k] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (r < static_cast<unsigned>(nrows) && col < len)
                 fetched[k] = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(r) * n + col);
         }
     };
     auto stage_fetched = [&]() __attribute__((always_inline)) {
+        // the R rows side by side: value (row r, column col) at rows[col * R + r], so that the walk reads the
+        // R values an entry refers to with one LDS instruction
+        static_assert(GB_FETCH % R == 0, "a lane holds all R rows of its columns");
 #pragma unroll
-        for (int k = 0; k < GB_FETCH; ++k)
+        for (int g = 0; g < GB_FETCH / R; ++g)
         {
-            const unsigned i = static_cast<unsigned>(k) * G_THREADS + tid;
-            const unsigned r = R > 1 ? i / per_row : 0u, col = (i - r * per_row) * 4u;
-            if (r < static_cast<unsigned>(R) && col < static_cast<unsigned>(part_len))
-                *reinterpret_cast<float4*>(rows + r * static_cast<unsigned>(part_len) + col) = fetched[k];
+            const unsigned col = (static_cast<unsigned>(g) * G_THREADS + tid) * 4u;
+            if (col >= static_cast<unsigned>(part_len))
+                continue;
+            float* const to = rows + col * R;
+            if constexpr (R == 1)
+                *reinterpret_cast<float4*>(to) = fetched[g];
+            else if constexpr (R == 2)
+            {
+                const float4 a = fetched[g * 2 + 0], b = fetched[g * 2 + 1];
+                *reinterpret_cast<float4*>(to + 0) = make_float4(a.x, b.x, a.y, b.y);
+                *reinterpret_cast<float4*>(to + 4) = make_float4(a.z, b.z, a.w, b.w);
+            }
+            else
+            {
+                const float4 a = fetched[g * 4 + 0], b = fetched[g * 4 + 1], cc = fetched[g * 4 + 2], d = fetched[g * 4 + 3];
+                *reinterpret_cast<float4*>(to + 0) = make_float4(a.x, b.x, cc.x, d.x);
+                *reinterpret_cast<float4*>(to + 4) = make_float4(a.y, b.y, cc.y, d.y);
+                *reinterpret_cast<float4*>(to + 8) = make_float4(a.z, b.z, cc.z, d.z);
+                *reinterpret_cast<float4*>(to + 12) = make_float4(a.w, b.w, cc.w, d.w);
+            }
         }
     };
     auto stage_slowly = [&](int piece) __attribute__((always_inline)) {
@@ -320,7 +336,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
         for (unsigned i = tid; i < R * static_cast<unsigned>(part_len); i += G_THREADS)
         {
             const unsigned r = i / static_cast<unsigned>(part_len), col = i - r * static_cast<unsigned>(part_len);
-            rows[i] = (r < static_cast<unsigned>(nrows) && col < len) ? src[static_cast<int64_t>(r) * n + col] : 0.f;
+            rows[col * R + r] = (r < static_cast<unsigned>(nrows) && col < len) ? src[static_cast<int64_t>(r) * n + col] : 0.f;
         }
     };
 
@@ -397,15 +413,31 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
                     break;
                 const ListEntry<WEIGHTED> e = ahead[u];
                 ahead[u] = request(i0 + u + GB_AHEAD);
-                const unsigned at = static_cast<unsigned>(e.j) & 0x7fffffffu;
+                const unsigned at = (static_cast<unsigned>(e.j) & 0x7fffffffu) * R; // (column * 4 bytes in the entry)
+                float v[R];
+                if constexpr (R == 1)
+                    v[0] = *reinterpret_cast<const float*>(staged + at);
+                else if constexpr (R == 2)
+                {
+                    const float2 both = *reinterpret_cast<const float2*>(staged + at);
+                    v[0] = both.x;
+                    v[1] = both.y;
+                }
+                else
+                {
+                    const float4 all = *reinterpret_cast<const float4*>(staged + at);
+                    v[0] = all.x;
+                    v[1] = all.y;
+                    v[2] = all.z;
+                    v[3] = all.w;
+                }
 #pragma unroll
                 for (int r = 0; r < R; ++r)
                 {
-                    const float v = *reinterpret_cast<const float*>(staged + at + static_cast<unsigned>(r) * row_bytes);
                     if constexpr (WEIGHTED)
-                        acc[r] = __builtin_fmaf(v, e.w, acc[r]); // (one rounding instead of the reference's two: within its tolerance)
+                        acc[r] = __builtin_fmaf(v[r], e.w, acc[r]); // (one rounding instead of the reference's two: within its tolerance)
                     else
-                        acc[r] += v;
+                        acc[r] += v[r];
                 }
                 const bool ends = e.j < 0; // the entry ends a list
                 if (ends)
