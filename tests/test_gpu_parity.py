@@ -267,6 +267,7 @@ def test_ball_query_full_config4(tpk, oracle, dev):
         ((9000, 500, 12000), 0.5, 0.06, 8),         # more neighbours than nsample for many queries
         ((16384, 16384), 0.1, 0.05, 1),
         (tuple([50] * 200), 1.0, 0.3, 16),          # many tiny clouds in one window
+        (tuple([50] * 200), 0.04, 0.3, 16),         # two queries per cloud: 32 clouds among 64 consecutive queries
         ((40000,), 0.3, 0.012, 32),                 # most balls hold the query point only
         ((90000, 20000), 0.05, 0.04, 32),           # 6 windows x 27 bins: more (window, bin) pairs than lanes
     ],
