@@ -331,24 +331,25 @@ __device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, cons
             }
         }
         float mn = 0.f;
-#pragma unroll
-        for (int c = 0; c < NG_CHUNK; ++c)
-        {
-            const float4 p = stage[ch * NG_CHUNK + c];
-            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-            mn = c == 0 ? d : fminf(mn, d);
-        }
-        TPK_WORK_ADD(NG_CHUNK);
-        if (__ballot(mn <= s.b3) == 0)
-            continue; // no candidate of this group enters any lane's triple
-        TPK_WORK_ADD(NG_CHUNK); // (the distances of an admitted group are formed a second time)
+        float ds[NG_CHUNK];
+        int cis[NG_CHUNK];
 #pragma unroll
         for (int c = 0; c < NG_CHUNK; ++c)
         {
             const float4 p = stage[ch * NG_CHUNK + c];
             // Operand order of the reference: (query - scanned).
-            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-            const int ci = __float_as_int(p.w);
+            ds[c] = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            cis[c] = __float_as_int(p.w);
+            mn = c == 0 ? ds[c] : fminf(mn, ds[c]);
+        }
+        TPK_WORK_ADD(NG_CHUNK);
+        if (__ballot(mn <= s.b3) == 0)
+            continue; // no candidate of this group enters any lane's triple
+#pragma unroll
+        for (int c = 0; c < NG_CHUNK; ++c)
+        {
+            const float d = ds[c];
+            const int ci = cis[c];
             const bool l3 = pair_less(d, ci, s.b3, s.i3);
             if (__ballot(l3) == 0)
                 continue;
