@@ -29,6 +29,8 @@ struct PointSet
     float4* boxes;        // [windows][cells][NG_BOX]: (lo.xyz, -), (hi.xyz, -) of the cell and of its quarters; or nullptr
     int* bin_ends;        // optional [windows][CURVE_BINS]: end of every bin of the counting sort
     float4* grid;         // optional [windows][2]: origin and scale of the window's 64^3 grid
+    int* wide_first;      // optional (with boxes) [windows][cells]: the window's cells, those with much wider boxes than
+                          // the window's average first - the cells whose queries take a search longest
 };
 
 __host__ __device__ inline int set_cells(const PointSet& s)
@@ -110,6 +112,8 @@ __device__ __forceinline__ void cloud_rows_job(const CloudRows& job, int64_t gro
     }
 }
 
+constexpr float CURVE_WIDE_FACTOR = 3.0f; // a cell is wide when its box's squared diagonal exceeds this many times the window's average
+
 // One workgroup orders one window: the first windows_a blocks those of set_a, the rest set_b.
 // `zero_word` (optional) is cleared by the first block: a counter used by the kernel that follows.
 // The window's points are read once and stay in registers (16 per thread): bounding box, curve
@@ -129,6 +133,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     int* const run_boxes = bins + CURVE_BINS;  // [cells * 4][6] ordered ints: boxes of the runs of 16 records
     __shared__ int cloud_box[6];
     __shared__ int wave_totals[NG_SORT_THREADS / TPK_WAVE];
+    __shared__ float wide_sums[NG_SORT_THREADS / TPK_WAVE];
     constexpr int PER = CURVE_MAX_POINTS / NG_SORT_THREADS; // points per thread
     static_assert(CURVE_BINS % NG_SORT_THREADS == 0, "every thread scans the same number of bins");
 
@@ -327,6 +332,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     if (boxes)
     {
         // one thread per cell: the boxes of its four runs, and their union, to memory
+        float diagonal2 = -1.f;
         __syncthreads();
         for (int c = tid; c < cells; c += NG_SORT_THREADS)
         {
@@ -349,6 +355,45 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
             }
             boxes[c * NG_BOX + 0] = make_float4(as_lo(lo[0]), as_lo(lo[1]), as_lo(lo[2]), 0.f);
             boxes[c * NG_BOX + 1] = make_float4(as_hi(hi[0]), as_hi(hi[1]), as_hi(hi[2]), 0.f);
+            if (c == tid && lo[0] != 0x7FFFFFFF) // (a cell that holds points: the squared diagonal of its box)
+            {
+                const float dx = as_hi(hi[0]) - as_lo(lo[0]), dy = as_hi(hi[1]) - as_lo(lo[1]), dz = as_hi(hi[2]) - as_lo(lo[2]);
+                diagonal2 = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz));
+            }
+        }
+        if (set.wide_first) // (cells <= 256: one cell per thread of the first four wavefronts)
+        {
+            // the average over the cells that hold points, then the wide cells first, both groups in curve order
+            const bool holds = diagonal2 >= 0.f;
+            const float wave_sum = wave_sum_f32(holds ? diagonal2 : 0.f);
+            const int wave_count = __builtin_popcountll(__ballot(holds));
+            if (lane == 0)
+            {
+                wide_sums[wave] = wave_sum;
+                wave_totals[wave] = wave_count;
+            }
+            __syncthreads();
+            float sum = 0.f;
+            int count = 0;
+            for (int w = 0; w < NG_SORT_THREADS / TPK_WAVE; ++w)
+            {
+                sum += wide_sums[w];
+                count += wave_totals[w];
+            }
+            const bool wide = holds && diagonal2 * count > CURVE_WIDE_FACTOR * sum;
+            const unsigned long long wide_lanes = __ballot(wide);
+            __syncthreads();
+            if (lane == 0)
+                wave_totals[wave] = __builtin_popcountll(wide_lanes);
+            __syncthreads();
+            int before = static_cast<int>(tpk_prefix_count(wide_lanes)), all_wide = 0;
+            for (int w = 0; w < NG_SORT_THREADS / TPK_WAVE; ++w)
+            {
+                before += w < wave ? wave_totals[w] : 0;
+                all_wide += wave_totals[w];
+            }
+            if (tid < cells)
+                set.wide_first[window * cells + (wide ? before : all_wide + tid - before)] = tid;
         }
     }
     if (set.bin_ends)

@@ -106,6 +106,7 @@ __device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, const
 // 64 candidates of the cell side by side in the lanes.  `want`: the lanes whose queries ask.
 // A minimum reached in the cell by several groups of NG_CHUNK candidates, or equal to the query's
 // answer so far, sets the tie flag exactly as the scan above would.
+constexpr int NG_DEAL = 8;   // windows whose cells are dealt out together, wide cells first
 constexpr int NG_FEW = 8; // (the scan above costs about as much as 14 queries served this way; 16: the same time, 24: slower)
 __device__ __forceinline__ void scan_cell_few(const float4* __restrict__ cand, int cell, unsigned long long want,
                                               int lane, float qx, float qy, float qz, Nearest& s TPK_WORK_PARAM)
@@ -143,7 +144,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
     int n, int m, int cells1, int cells2, int clouds, const float4* __restrict__ sorted1,
     const float4* __restrict__ sorted2, const float4* __restrict__ boxes1,
     const float4* __restrict__ boxes2, float* __restrict__ dist1, float* __restrict__ dist2,
-    int32_t* __restrict__ idx1, int32_t* __restrict__ idx2)
+    int32_t* __restrict__ idx1, int32_t* __restrict__ idx2, const int* __restrict__ wide1,
+    const int* __restrict__ wide2, int window_cells)
 {
     __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
     extern __shared__ float lows_all[]; // [wavefronts][largest number of candidate cells, in whole groups of 64]
@@ -155,8 +157,30 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void chamfer_grid_kernel(
                              (NG_SCAN_THREADS / TPK_WAVE) + wave;
     if (task >= static_cast<int64_t>(per_cloud) * clouds)
         return; // (no workgroup barrier anywhere in this kernel)
-    const int cloud = static_cast<int>(task / per_cloud);
-    const int r = static_cast<int>(task - static_cast<int64_t>(cloud) * per_cloud);
+    int cloud = static_cast<int>(task / per_cloud);
+    int r = static_cast<int>(task - static_cast<int64_t>(cloud) * per_cloud);
+    if (window_cells > 0)
+    {
+        // Wavefronts start in the order of their numbers, and the call lasts as long as the wavefront that ends
+        // last: the cells with the widest boxes - whose queries search longest - go first.  The cells of both
+        // clouds' windows are dealt out in groups of NG_DEAL windows, window after window, every window
+        // handing out its cells in the order the ordering kernel left: wide ones first.
+        const int per_cloud_windows = per_cloud / window_cells;
+        const int64_t all_windows = static_cast<int64_t>(per_cloud_windows) * clouds;
+        const int64_t group = task / (NG_DEAL * window_cells);
+        const int within = static_cast<int>(task - group * (NG_DEAL * window_cells));
+        const int dealt = static_cast<int>(tpk_min64(NG_DEAL, all_windows - group * NG_DEAL));
+        const int64_t window = group * NG_DEAL + within % dealt;
+        const int rank = within / dealt;
+        cloud = static_cast<int>(window / per_cloud_windows);
+        const int k = static_cast<int>(window - static_cast<int64_t>(cloud) * per_cloud_windows);
+        const int windows1 = cells1 / window_cells;
+        const bool in_second = k >= windows1;
+        const int own = in_second ? k - windows1 : k; // the window's number in its cloud
+        const int* __restrict__ order = in_second ? wide2 + (static_cast<int64_t>(cloud) * (per_cloud_windows - windows1) + own) * window_cells
+                                                  : wide1 + (static_cast<int64_t>(cloud) * windows1 + own) * window_cells;
+        r = (in_second ? cells1 : 0) + own * window_cells + order[rank];
+    }
     const bool second = r >= cells1;
     const int qcell = second ? r - cells1 : r;
     const int qcells = second ? cells2 : cells1;
@@ -889,7 +913,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
 
 struct GridLayout
 {
-    size_t sorted_a, sorted_b, boxes_a, boxes_b, total;
+    size_t sorted_a, sorted_b, boxes_a, boxes_b, wide_a, wide_b, total;
 };
 
 // Cells of a cloud of n points: ordered whole up to NG_WINDOW points, else in windows of NG_WINDOW
@@ -904,7 +928,7 @@ int grid_stride(int n)
     return n <= NG_WINDOW ? n : NG_WINDOW;
 }
 
-GridLayout grid_layout(int b, int n, int m)
+GridLayout grid_layout(int b, int n, int m, bool wide_first = false)
 {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
     const size_t cells_a = static_cast<size_t>(grid_cells(n));
@@ -919,6 +943,13 @@ GridLayout grid_layout(int b, int n, int m)
     pos = up(pos + static_cast<size_t>(b) * cells_a * NG_BOX * sizeof(float4));
     l.boxes_b = pos;
     pos = up(pos + static_cast<size_t>(b) * cells_b * NG_BOX * sizeof(float4));
+    l.wide_a = l.wide_b = pos;
+    if (wide_first) // (the Chamfer search: the cells of every window, wide ones first)
+    {
+        pos = up(pos + static_cast<size_t>(b) * cells_a * sizeof(int));
+        l.wide_b = pos;
+        pos = up(pos + static_cast<size_t>(b) * cells_b * sizeof(int));
+    }
     l.total = pos;
     return l;
 }
@@ -934,7 +965,7 @@ bool grid_supported(int b, int n, int m)
 
 size_t tpk_grid_chamfer_workspace_bytes(int b, int n, int m)
 {
-    return grid_supported(b, n, m) ? grid_layout(b, n, m).total : 0;
+    return grid_supported(b, n, m) ? grid_layout(b, n, m, true).total : 0;
 }
 
 int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xyz2, float* dist1,
@@ -943,14 +974,22 @@ int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xy
 {
     if (!grid_supported(b, n, m) || static_cast<int64_t>(b) * 2 > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    const GridLayout l = grid_layout(b, n, m);
+    const GridLayout l = grid_layout(b, n, m, true);
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
     PointSet a{xyz1, nullptr, static_cast<int64_t>(b) * n, n, grid_stride(n), reinterpret_cast<float4*>(w + l.sorted_a),
-               reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr};
+               reinterpret_cast<float4*>(w + l.boxes_a), nullptr, nullptr, nullptr};
     PointSet c{xyz2, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted_b),
-               reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
+               reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr, nullptr};
+    // Both clouds' windows hold the same number of cells (clouds of one size class, the usual case): the cells
+    // are handed to the wavefronts wide ones first.
+    const int window_cells = set_cells(a) == set_cells(c) ? set_cells(a) : 0;
+    if (window_cells > 0)
+    {
+        a.wide_first = reinterpret_cast<int*>(w + l.wide_a);
+        c.wide_first = reinterpret_cast<int*>(w + l.wide_b);
+    }
     int st = launch_curve_cells(a, c, nullptr, s);
     if (st != TPK_OK)
         return st;
@@ -962,7 +1001,8 @@ int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xy
     const size_t lds = static_cast<size_t>(NG_SCAN_THREADS / TPK_WAVE) *
                        ((std::max(cells1, cells2) + NG_CELL - 1) / NG_CELL * NG_CELL) * sizeof(float);
     hipLaunchKernelGGL(chamfer_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
-                       m, cells1, cells2, b, a.sorted, c.sorted, a.boxes, c.boxes, dist1, dist2, idx1, idx2);
+                       m, cells1, cells2, b, a.sorted, c.sorted, a.boxes, c.boxes, dist1, dist2, idx1, idx2, a.wide_first,
+                       c.wide_first, window_cells);
     return tpk_launch_status();
 }
 
