@@ -68,35 +68,39 @@ __device__ __forceinline__ void scan_cell(const float4* __restrict__ cand, const
                                           Nearest& s TPK_WORK_PARAM)
 {
     stage[lane] = cand[cell * NG_CELL + lane];
-    const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
+    // (the boxes of the cell's four runs are requested together with its candidates: one wait, not five)
+    float4 quarter[NG_BOX - 2];
+#pragma unroll
+    for (int i = 0; i < NG_BOX - 2; ++i)
+        quarter[i] = boxes[cell * NG_BOX + 2 + i];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); // LDS serves a wavefront's requests in order
-    for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
+#pragma unroll
+    for (int run = 0; run < NG_CELL / (2 * NG_CHUNK); ++run)
     {
         // a run of 16 candidates whose box no lane's answer reaches is passed over
-        if ((ch & 1) == 0)
-        {
-            const float lb = point_box_dist2(qx, qy, qz, quarter[ch], quarter[ch + 1]);
-            if (__ballot(lb * NG_MARGIN <= s.best) == 0)
-            {
-                ++ch;
-                continue;
-            }
-        }
-        float mn = 0.f;
+        const float lb = point_box_dist2(qx, qy, qz, quarter[2 * run], quarter[2 * run + 1]);
+        if (__ballot(lb * NG_MARGIN <= s.best) == 0)
+            continue;
 #pragma unroll
-        for (int c = 0; c < NG_CHUNK; ++c)
+        for (int half = 0; half < 2; ++half)
         {
-            const float4 p = stage[ch * NG_CHUNK + c];
-            // Operand order of the reference: (scanned - query), squares summed x, y, z.
-            const float d = tpk_dist2(p.x, p.y, p.z, qx, qy, qz);
-            mn = c == 0 ? d : fminf(mn, d);
+            const int ch = 2 * run + half;
+            float mn = 0.f;
+#pragma unroll
+            for (int c = 0; c < NG_CHUNK; ++c)
+            {
+                const float4 p = stage[ch * NG_CHUNK + c];
+                // Operand order of the reference: (scanned - query), squares summed x, y, z.
+                const float d = tpk_dist2(p.x, p.y, p.z, qx, qy, qz);
+                mn = c == 0 ? d : fminf(mn, d);
+            }
+            TPK_WORK_ADD(NG_CHUNK);
+            const bool better = mn < s.best;
+            const bool equal = mn == s.best;
+            s.tie = better ? false : (s.tie || equal);
+            s.chunk = better ? cell * (NG_CELL / NG_CHUNK) + ch : s.chunk;
+            s.best = better ? mn : s.best;
         }
-        TPK_WORK_ADD(NG_CHUNK);
-        const bool better = mn < s.best;
-        const bool equal = mn == s.best;
-        s.tie = better ? false : (s.tie || equal);
-        s.chunk = better ? cell * (NG_CELL / NG_CHUNK) + ch : s.chunk;
-        s.best = better ? mn : s.best;
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
@@ -340,20 +344,25 @@ __device__ __forceinline__ void scan_cell3(const float4* __restrict__ cand, cons
                                            Nearest3& s TPK_WORK_PARAM)
 {
     stage[lane] = cand[cell * NG_CELL + lane];
-    const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
+    // (the boxes of the cell's four runs are requested together with its candidates: one wait, not five)
+    float4 quarter[NG_BOX - 2];
+#pragma unroll
+    for (int i = 0; i < NG_BOX - 2; ++i)
+        quarter[i] = boxes[cell * NG_BOX + 2 + i];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    bool reached = true;
+#pragma unroll
     for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
     {
         // a run of 16 candidates whose box no lane's third best reaches is passed over
+        // (decided at the run's first group: `reached` carries it to the second)
         if ((ch & 1) == 0)
         {
             const float lb = point_box_dist2(qx, qy, qz, quarter[ch], quarter[ch + 1]);
-            if (__ballot(lb * NG_MARGIN <= s.b3) == 0)
-            {
-                ++ch;
-                continue;
-            }
+            reached = __ballot(lb * NG_MARGIN <= s.b3) != 0;
         }
+        if (!reached)
+            continue;
         float mn = 0.f;
         float ds[NG_CHUNK];
         int cis[NG_CHUNK];
