@@ -564,37 +564,44 @@ __device__ __forceinline__ void scan_cell_k(const float4* __restrict__ cand, con
                                             NearestK<K>& s)
 {
     stage[lane] = cand[cell * NG_CELL + lane];
-    const float4* __restrict__ quarter = boxes + cell * NG_BOX + 2;
     float worst = s.worst(); // distance of the lane's last entry
+    // The runs of 16 candidates whose box no lane's last entry reaches are passed over.  The four boxes are
+    // requested together with the candidates and tested before the scan: one wait, not five.
+    unsigned reached = 0;
+    {
+        float4 quarter[NG_BOX - 2];
+#pragma unroll
+        for (int i = 0; i < NG_BOX - 2; ++i)
+            quarter[i] = boxes[cell * NG_BOX + 2 + i];
+#pragma unroll
+        for (int run = 0; run < (NG_BOX - 2) / 2; ++run)
+        {
+            const float lb = point_box_dist2(qx, qy, qz, quarter[2 * run], quarter[2 * run + 1]);
+            reached |= __ballot(lb * NG_MARGIN <= worst) != 0 ? 1u << run : 0u;
+        }
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     for (int ch = 0; ch < NG_CELL / NG_CHUNK; ++ch)
     {
-        // a run of 16 candidates whose box no lane's last entry reaches is passed over
-        if ((ch & 1) == 0)
-        {
-            const float lb = point_box_dist2(qx, qy, qz, quarter[ch], quarter[ch + 1]);
-            if (__ballot(lb * NG_MARGIN <= worst) == 0)
-            {
-                ++ch;
-                continue;
-            }
-        }
+        if (((reached >> (ch >> 1)) & 1u) == 0)
+            continue;
         float mn = 0.f;
+        float ds[NG_CHUNK];
+        int cis[NG_CHUNK];
 #pragma unroll
         for (int c = 0; c < NG_CHUNK; ++c)
         {
             const float4 p = stage[ch * NG_CHUNK + c];
-            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-            mn = c == 0 ? d : fminf(mn, d);
+            ds[c] = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            cis[c] = __float_as_int(p.w);
+            mn = c == 0 ? ds[c] : fminf(mn, ds[c]);
         }
         if (__ballot(mn <= worst) == 0)
             continue; // no candidate of this group enters any lane's list
 #pragma unroll
         for (int c = 0; c < NG_CHUNK; ++c)
         {
-            const float4 p = stage[ch * NG_CHUNK + c];
-            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-            const unsigned long long cand = knn_key(d, __float_as_int(p.w));
+            const unsigned long long cand = knn_key(ds[c], cis[c]);
             const bool in = s.admits(cand);
             if (__ballot(in) == 0)
                 continue;
