@@ -404,7 +404,7 @@ def bench_others(dev, steps, warmup, with_cpu):
     e = {"workload": "ball_query partial_dense sort=True on configs[3] (the reference has this mode for CPU tensors only)",
          "metric": "queries/s", "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
          "pairs": pairs, "algorithmic_rate_tflops": pairs * 8 / (ev * 1e-3) / 1e12,
-         "note": "the clouds are searched one after the other, after one wait for the stream"}
+         "note": "the bin walk of the unsorted packed query with a selection of the nearest in place of its hit list"}
     if ref is not None:
         secs = _cpu_time(lambda: ref.batch_ball_query(w["x"], w["y"], w["batch_x"], w["batch_y"], w["radius"],
                                                       w["nsample"], 0, True))

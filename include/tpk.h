@@ -5,7 +5,7 @@
  * Every entry point takes plain device pointers and sizes, launches on the HIP stream
  * passed as `stream` (a hipStream_t cast to void*; NULL = the null stream), never
  * allocates, never synchronises the host (exceptions, documented below: tpk_grow_proximity and
- * tpk_ball_query_sorted_partial_f32 with a workspace) and keeps no state between calls.  The caller
+ * tpk_ball_query_sorted_partial_f32 with a workspace and nsample > 64) and keeps no state between calls.  The caller
  * owns all memory.  All arrays are dense row-major ("contiguous").  Outputs need not be
  * initialised: every element of every output array is written by the call.
  *
@@ -106,9 +106,10 @@ int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int
  * shapes not served that way -, 256-byte aligned) the support points are ordered along a
  * space filling curve and a query only visits cells within its radius (clouds of 512 support
  * points or more; up to 64 neighbours one wavefront serves a query), same results as the all
- * pairs scan used otherwise.  In the packed layout this is done cloud by cloud (clouds of up
- * to 163840 points, cloud ids below 1024; others by all pairs), and the call then waits for
- * the stream once, to read where the clouds start.
+ * pairs scan used otherwise.  In the packed layout up to 64 neighbours are found by the walk
+ * over bins of tpk_ball_query_partial_f32 (no wait for the stream); more than 64 cloud by
+ * cloud (clouds of up to 163840 points, cloud ids below 1024; others by all pairs), and only
+ * then the call waits for the stream once, to read where the clouds start.
  * ------------------------------------------------------------------------------------- */
 size_t tpk_ball_query_sorted_dense_workspace_bytes(int b, int n, int m);
 int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius, int nsample,

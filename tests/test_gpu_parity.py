@@ -337,7 +337,11 @@ def test_ball_query_sorted_ties_and_boundary(tpk, oracle, dev):
 
 @pytest.mark.parametrize("sizes,qfrac,r,ns", [((50, 70, 10), 0.5, 0.3, 8), ((3000, 1, 2100, 4500), 0.25, 0.1, 16),
                                                ((2048, 2049), 0.1, 0.2, 64), ((700,), 1.0, 0.5, 100),
-                                               ((20000, 300), 0.05, 0.05, 12)])
+                                               ((20000, 300), 0.05, 0.05, 12),
+                                               # balls over most of a cloud (too many bins to walk), more
+                                               # neighbours than a wavefront keeps (cloud by cloud), many windows
+                                               ((3000, 4000), 0.2, 0.6, 32), ((9000, 5000), 0.1, 0.1, 70),
+                                               ((70000,), 0.02, 0.03, 64), (tuple([40] * 150), 0.3, 0.4, 5)])
 def test_ball_query_sorted_partial_parity(tpk, oracle, dev, sizes, qfrac, r, ns):
     x, y, bx, by = _packed_case(17 + len(sizes), sizes, qfrac, 0.01)
     idx, dist = tpk.ball_query(r, ns, x.to(dev), y.to(dev), mode="partial_dense", batch_x=bx.to(dev), batch_y=by.to(dev), sort=True)

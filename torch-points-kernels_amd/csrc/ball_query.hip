@@ -313,7 +313,7 @@ extern "C" int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float 
     if (workspace)
     {
         // Search over curve-ordered cells where it applies; otherwise all pairs.
-        const int st = tpk_grid_ball_query_partial(size_x, size_y, radius, radius2, nsample, x, y, batch_x, batch_y, idx,
+        const int st = tpk_grid_ball_query_partial(size_x, size_y, radius, radius2, nsample, false, x, y, batch_x, batch_y, idx,
                                                    dist, workspace, workspace_bytes, tpk_stream(stream));
         if (st != TPK_ERR_UNSUPPORTED)
             return st;

@@ -417,7 +417,10 @@ extern "C" size_t tpk_ball_query_sorted_partial_workspace_bytes(int64_t size_x, 
     const size_t lists = tpk_grid_knn_workspace_bytes(1, static_cast<int>(tpk_min64(size_y, NP_GRID_POINTS)), most_x);
     const size_t waves = tpk_grid_ball_sorted_workspace_bytes(1, most_x);
     const size_t grid = waves > lists ? waves : lists;
-    return grid ? NP_RANGES_BYTES + grid : 0;
+    // (up to 64 neighbours the packed array is searched as a whole, bins of windows of consecutive rows: no wait)
+    const size_t bins = tpk_grid_ball_query_workspace_bytes(size_x, size_y, TPK_WAVE);
+    const size_t cloudwise = grid ? NP_RANGES_BYTES + grid : 0;
+    return bins > cloudwise ? bins : cloudwise;
 }
 
 extern "C" int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y, float radius, int nsample,
@@ -443,6 +446,15 @@ extern "C" int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y,
     }
     if (workspace_bytes < wanted || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
+    if (nsample <= TPK_WAVE)
+    {
+        // One launch over the whole packed array (windows of consecutive rows, bins of a 16^3 grid per window,
+        // the rows of every query's cloud found on the device): no wait for the stream.
+        const int st = tpk_grid_ball_query_partial(size_x, size_y, radius, limit, nsample, true, x, y, batch_x, batch_y,
+                                                   idx, dist, workspace, workspace_bytes, s);
+        if (st != TPK_ERR_UNSUPPORTED)
+            return st;
+    }
 
     // Where every cloud starts in both arrays.
     static_assert(NP_MAX_CLOUDS + 1 <= 5 * KNN_THREADS, "one thread per cloud id");

@@ -37,9 +37,10 @@ int tpk_grid_ball_sorted(int b, int n, int m, int nsample, float limit, bool pac
 
 // Ball query, packed layout (a hit has squared distance <= radius2 = radius * radius as the caller
 // rounds it): same conventions.  Queries with dense neighbourhoods are answered by a scan in
-// index order inside the same kernel.
+// index order inside the same kernel.  `sorted`: the nsample (<= 64) nearest points with squared
+// distance < radius2 instead, nearest first (equal distances: lower row first), -1 behind them.
 size_t tpk_grid_ball_query_workspace_bytes(int64_t size_x, int64_t size_y, int nsample);
-int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample,
+int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample, bool sorted,
                                 const float* x, const float* y, const int64_t* batch_x,
                                 const int64_t* batch_y, int64_t* idx, float* dist, void* workspace,
                                 size_t workspace_bytes, hipStream_t stream);

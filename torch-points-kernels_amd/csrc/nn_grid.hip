@@ -719,6 +719,45 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
     }
 }
 
+using u64 = unsigned long long;
+constexpr int NG_RUN = 16; // consecutive cells that share a second-level box in the wavefront-per-query search
+
+// The 64 keys of a wavefront sorted across its lanes (bitonic network; lane i ends with the i-th
+// smallest, or the i-th largest when `descending`).
+__device__ __forceinline__ u64 wave_sort_keys(u64 key, int lane, bool descending)
+{
+#pragma unroll
+    for (int k = 2; k <= TPK_WAVE; k <<= 1)
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1)
+        {
+            const u64 other = __shfl_xor(key, j, TPK_WAVE);
+            const bool up = ((lane & k) == 0) != descending;
+            const bool keep_min = ((lane & j) == 0) == up;
+            key = (keep_min == (key < other)) ? key : other;
+        }
+    return key;
+}
+
+// A bitonic sequence across the lanes put into ascending order.
+__device__ __forceinline__ u64 wave_merge_ascending(u64 key, int lane)
+{
+#pragma unroll
+    for (int j = TPK_WAVE / 2; j > 0; j >>= 1)
+    {
+        const u64 other = __shfl_xor(key, j, TPK_WAVE);
+        key = (((lane & j) == 0) == (key < other)) ? key : other;
+    }
+    return key;
+}
+
+__device__ __forceinline__ u64 read_lane_key(u64 key, int from)
+{
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<int>(key & 0xFFFFFFFFu), from);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<int>(key >> 32), from);
+    return (static_cast<u64>(hi) << 32) | lo;
+}
+
 // ---------------------------------------------------------------------------------------
 // Ball query over bins, packed layout (several clouds back to back, sorted cloud id per point).
 //
@@ -749,6 +788,11 @@ __device__ __forceinline__ void bin_range(float v, float r, float lo, float scal
     last = static_cast<int>(curve_grid_cell((v + r) + slack, lo, scale) >> 2);
 }
 
+// SORTED: the nsample (<= 64) NEAREST points with squared distance < radius2, nearest first, instead of the
+// first nsample in row order with squared distance <= radius2: the wavefront keeps its 64 best (distance, row)
+// keys sorted across the lanes and merges the hits of a step into them (as the wavefront-per-query kernel
+// further down does with the points of a cell).
+template <bool SORTED>
 __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     int size_x, int size_y, float radius, float radius2, int nsample, const float* __restrict__ x,
     const float* __restrict__ y, const float4* __restrict__ sorted_x, const int* __restrict__ bin_ends,
@@ -779,6 +823,18 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     // The walk is laid out so that dependent loads are few: all windows at once (one lane each),
     // then all (window, bin) pairs at once, then the candidates 64 at a time.
     int cnt = 0;
+    // SORTED: lane i holds the i-th smallest (distance, row) key so far; a hit must beat the nsample-th
+    constexpr u64 NONE = ~0ull;
+    u64 best = NONE, admit = NONE;
+    auto offer = [&](bool hit, float d, int row) __attribute__((always_inline)) {
+        u64 cand = hit ? knn_key(d, row) : NONE;
+        cand = cand < admit ? cand : NONE;
+        if (__ballot(cand != NONE) == 0)
+            return;
+        cand = wave_sort_keys(cand, lane, true);
+        best = wave_merge_ascending(best < cand ? best : cand, lane);
+        admit = read_lane_key(best, nsample - 1);
+    };
     const int wx0 = s0 / CURVE_MAX_POINTS;
     const int windows = s1 > s0 ? (s1 - 1) / CURVE_MAX_POINTS - wx0 + 1 : 0;
     bool serial = windows > TPK_WAVE; // answer by the scan in index order instead
@@ -844,6 +900,11 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
                 TPK_WORK_ADD(1);
                 const int row = __float_as_int(p.w);
+                if constexpr (SORTED)
+                {
+                    offer(has && d < radius2 && row >= s0 && row < s1, d, row);
+                    continue;
+                }
                 const bool hit = has && d <= radius2 && row >= s0 && row < s1;
                 const unsigned long long mask = __ballot(hit);
                 if (mask == 0)
@@ -864,6 +925,42 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
             walk_pairs(pair0);
     }
 
+    if constexpr (SORTED)
+    {
+        if (serial)
+        {
+            // too many windows or bins for the walk: every row of the cloud, 64 per step
+            constexpr int BATCH = 4;
+            for (int base = s0; base < s1; base += BATCH * TPK_WAVE)
+            {
+                float px[BATCH], py[BATCH], pz[BATCH];
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u)
+                {
+                    const int64_t pos = min(base + u * TPK_WAVE + lane, s1 - 1);
+                    px[u] = x[pos * 3 + 0];
+                    py[u] = x[pos * 3 + 1];
+                    pz[u] = x[pos * 3 + 2];
+                }
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u)
+                {
+                    const int pos = base + u * TPK_WAVE + lane;
+                    const float d = tpk_dist2(qx, qy, qz, px[u], py[u], pz[u]);
+                    TPK_WORK_ADD(1);
+                    offer(pos < s1 && d < radius2, d, pos);
+                }
+            }
+        }
+        if (lane < nsample)
+        {
+            const bool found = best != NONE;
+            idx[out + lane] = found ? static_cast<int64_t>(best & 0xFFFFFFFFu) : -1;
+            dist[out + lane] = found ? __int_as_float(static_cast<int>(best >> 32)) : -1.0f;
+        }
+        TPK_WORK_FLUSH
+        return;
+    }
     if (!serial)
     {
         // rank of every hit among the hits (rows are distinct), then hits in order, then -1
@@ -1057,45 +1154,6 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
 }
 
 namespace {
-
-using u64 = unsigned long long;
-constexpr int NG_RUN = 16; // consecutive cells that share a second-level box in the wavefront-per-query search
-
-// The 64 keys of a wavefront sorted across its lanes (bitonic network; lane i ends with the i-th
-// smallest, or the i-th largest when `descending`).
-__device__ __forceinline__ u64 wave_sort_keys(u64 key, int lane, bool descending)
-{
-#pragma unroll
-    for (int k = 2; k <= TPK_WAVE; k <<= 1)
-#pragma unroll
-        for (int j = k >> 1; j > 0; j >>= 1)
-        {
-            const u64 other = __shfl_xor(key, j, TPK_WAVE);
-            const bool up = ((lane & k) == 0) != descending;
-            const bool keep_min = ((lane & j) == 0) == up;
-            key = (keep_min == (key < other)) ? key : other;
-        }
-    return key;
-}
-
-// A bitonic sequence across the lanes put into ascending order.
-__device__ __forceinline__ u64 wave_merge_ascending(u64 key, int lane)
-{
-#pragma unroll
-    for (int j = TPK_WAVE / 2; j > 0; j >>= 1)
-    {
-        const u64 other = __shfl_xor(key, j, TPK_WAVE);
-        key = (((lane & j) == 0) == (key < other)) ? key : other;
-    }
-    return key;
-}
-
-__device__ __forceinline__ u64 read_lane_key(u64 key, int from)
-{
-    const unsigned lo = __builtin_amdgcn_readlane(static_cast<int>(key & 0xFFFFFFFFu), from);
-    const unsigned hi = __builtin_amdgcn_readlane(static_cast<int>(key >> 32), from);
-    return (static_cast<u64>(hi) << 32) | lo;
-}
 
 // Ball query with sorted neighbours, one wavefront per query: the nsample (<= 64) nearest support
 // points with squared distance < limit.  The support points lie in curve-ordered cells of 64; a
@@ -1395,12 +1453,12 @@ size_t tpk_grid_ball_query_workspace_bytes(int64_t size_x, int64_t size_y, int n
     return ball_bins_supported(size_x, size_y, nsample) ? ball_layout(size_x, size_y).total : 0;
 }
 
-int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample,
+int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample, bool sorted,
                                 const float* x, const float* y, const int64_t* batch_x,
                                 const int64_t* batch_y, int64_t* idx, float* dist, void* workspace,
                                 size_t workspace_bytes, hipStream_t s)
 {
-    if (!ball_bins_supported(size_x, size_y, nsample))
+    if (!ball_bins_supported(size_x, size_y, nsample) || (sorted && nsample > TPK_WAVE))
         return TPK_ERR_UNSUPPORTED;
     const BallLayout l = ball_layout(size_x, size_y);
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
@@ -1418,8 +1476,13 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
     const int64_t blocks = tpk_ceil_div(size_y, WAVES);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(ball_query_bins_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
-                       static_cast<int>(size_x), static_cast<int>(size_y), std::fabs(radius), radius2, nsample, x, y,
-                       px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
+    if (sorted)
+        hipLaunchKernelGGL(ball_query_bins_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+                           static_cast<int>(size_x), static_cast<int>(size_y), std::fabs(radius), radius2, nsample, x, y,
+                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
+    else
+        hipLaunchKernelGGL(ball_query_bins_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+                           static_cast<int>(size_x), static_cast<int>(size_y), std::fabs(radius), radius2, nsample, x, y,
+                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
     return tpk_launch_status();
 }
