@@ -46,7 +46,7 @@ TRAFFIC_KERNELS = {
 # Kernels whose VALU counters describe a distance scan.
 VALU_KERNELS = {
     "fps": "fps_pruned_kernel<16, 1024, 4>",
-    "ball_query_dense": "ball_query_dense_kernel<2>",
+    "ball_query_dense": "ball_query_dense_cells_kernel",
     "ball_query_partial_dense": "ball_query_bins_kernel",
     "three_nn": "three_nn_grid_kernel",
     "chamfer_fwd": "chamfer_grid_kernel",
@@ -351,6 +351,7 @@ def bench_others(dev, steps, warmup, with_cpu):
     e = {"workload": "configs[0]: ball_query dense B=8 N=4096 M=1024 r=0.1 nsample=32", "metric": "queries/s",
          "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
          "roofline": _roof_flops(executed, pairs, 8, ev, "ball_query_dense"), "pairs_upper_bound": pairs}
+    e["roofline"]["note"] += PRUNED_NOTE
     if ref is not None:
         secs = _cpu_time(lambda: ref.dense_ball_query(w["new_xyz"], w["xyz"], w["radius"], w["nsample"], 0, False))
         e["cpu_baseline"] = {"value": nq / secs, "unit": "queries/s", "cores": 1, "kind": "reference",

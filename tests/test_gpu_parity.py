@@ -173,6 +173,46 @@ def test_ball_query_dense_boundary_and_empty(tpk, oracle, dev):
     assert (idx == 0).all() and (dist == -1).all()
 
 
+@pytest.mark.parametrize("kind", ["uniform", "clusters", "flat", "one_point", "outlier", "queries_outside", "non_finite", "line"])
+@pytest.mark.parametrize("B,N,M,r,ns", [(2, 512, 100, 0.2, 8), (4, 8192, 300, 0.05, 16), (1, 4096, 1030, 0.1, 100),
+                                        (3, 1500, 17, 0.02, 4), (2, 6000, 64, 0.35, 32)])
+def test_ball_query_dense_over_cells(tpk, oracle, dev, kind, B, N, M, r, ns):
+    # clouds of 512 .. 8192 support points are binned into cells of at least one radius: shapes of clouds that
+    # stress the grid (no extent along an axis, everything in one cell, a far point that makes all cells wide,
+    # queries outside the box, coordinates that are not finite), checked against the scan in index order
+    g = torch.Generator().manual_seed(7 * N + M)
+    xyz = torch.rand(B, N, 3, generator=g)
+    new_xyz = xyz[:, torch.randperm(N, generator=g)[:M] % N].clone() + 0.01 * torch.randn(B, M, 3, generator=g)
+    if kind == "clusters":
+        centres = torch.rand(B, 5, 3, generator=g)
+        xyz = centres[:, torch.randint(0, 5, (N,), generator=g)] + 0.03 * torch.randn(B, N, 3, generator=g)
+        new_xyz = xyz[:, :M].clone() + 0.005
+    elif kind == "flat":
+        xyz[..., 2] = 0.25
+        new_xyz[..., 2] = 0.25 + 0.5 * r
+    elif kind == "one_point":
+        xyz[:] = 0.5
+        new_xyz[:, ::2] = 0.5
+    elif kind == "outlier":
+        xyz[:, N // 3] = torch.tensor([400.0, -300.0, 1e6])
+    elif kind == "queries_outside":
+        new_xyz[:, ::3] += 2.0
+        new_xyz[:, 1::3, 0] = -r * 0.5
+    elif kind == "non_finite":
+        xyz[:, 5, 0] = float("nan")
+        xyz[:, 77, 1] = float("inf")
+        xyz[:, 300, 2] = -float("inf")
+        new_xyz[:, 3, 1] = float("nan")
+        new_xyz[:, 4, 2] = float("inf")
+    elif kind == "line":
+        xyz[..., 1:] = 0.0
+        new_xyz[..., 1:] = 0.0
+    idx, dist = tpk.ball_query(r, ns, xyz.to(dev), new_xyz.contiguous().to(dev), mode="dense")
+    want_idx, want_dist = oracle.ball_query_dense(r, ns, xyz.numpy(), new_xyz.numpy())
+    np.testing.assert_array_equal(_np(idx), want_idx)
+    np.testing.assert_array_equal(_np(dist), want_dist)
+
+
 def _packed_case(seed, sizes, qfrac, jitter):
     g = torch.Generator().manual_seed(seed)
     xs, ys, bx, by = [], [], [], []

@@ -211,6 +211,332 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
                           static_cast<int64_t>(cloud) * m + jq0, idx, dist);
 }
 
+// ---------------------------------------------------------------------------------------
+// Dense layout over cells: clouds of BQC_MIN_POINTS .. BQC_MAX_POINTS support points.
+//
+// Testing every support point costs n / 64 steps per query whatever the radius.  Here a workgroup
+// of 16 wavefronts first bins its cloud in LDS: bounding box, a grid of up to 16 cells per axis
+// whose cells are at least one radius wide, a count per cell (LDS atomics that also hand every
+// point its place inside its cell), a prefix sum, and the points (x, y, z, index) written cell by
+// cell.  All workgroups of a cloud repeat this (a few microseconds; the cloud comes from the L2),
+// which is cheaper than a launch that does it once.  Then every wavefront answers queries, one at
+// a time: the cells that the cube around the ball touches form, for every (y, z), one run of
+// consecutive places - cells are numbered x first - so lane r takes row r's run, and the
+// candidates of all runs are dealt to the lanes 64 at a time.  A candidate with d2 < radius^2 is
+// a hit; the hits (at most 64) are ranked by index and written in ascending index order, which
+// is what the scan in index order produces (cuda/src/ball_query_gpu.cu:9-52).  A query with more
+// than 64 hits, or whose cube holds more than BQC_MAX_CANDIDATES points (a ball that covers much
+// of its cloud), is answered by that scan itself, 64 points per step from global memory with
+// early exit: with so many hits it ends soon.
+// ---------------------------------------------------------------------------------------
+constexpr int BQC_THREADS = 1024;
+constexpr int BQC_WAVES = BQC_THREADS / TPK_WAVE;
+constexpr int BQC_MIN_POINTS = 512;
+constexpr int BQC_MAX_POINTS = 8192;
+constexpr int BQC_PER_THREAD = BQC_MAX_POINTS / BQC_THREADS;
+constexpr int BQC_GRID = 16;
+constexpr int BQC_CELLS = BQC_GRID * BQC_GRID * BQC_GRID;
+constexpr int BQC_STARTS = BQC_CELLS + TPK_WAVE; // the cells' first places, one more for the end, padded
+constexpr int BQC_HITS = TPK_WAVE;
+constexpr int BQC_MAX_CANDIDATES = 8 * TPK_WAVE;
+
+struct CellWave
+{
+    int rows[BQC_HITS];
+    float dists[BQC_HITS];
+    int marks[TPK_WAVE];
+};
+
+size_t bqc_lds_bytes(int n)
+{
+    return static_cast<size_t>(n) * sizeof(float4) + BQC_STARTS * sizeof(int) + BQC_WAVES * sizeof(CellWave);
+}
+
+// Smallest / largest v of every 16-lane row, in all lanes of the row.
+__device__ __forceinline__ float row_all_min_f32(float v)
+{
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true)));
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true)));
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, true)));
+    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true)));
+    return v;
+}
+__device__ __forceinline__ float wave_min_f32(float v)
+{
+    v = row_all_min_f32(v);
+    return fminf(fminf(tpk_read_lane(v, 0), tpk_read_lane(v, 16)), fminf(tpk_read_lane(v, 32), tpk_read_lane(v, 48)));
+}
+
+// Cell along one axis: monotone in v (so the cells of [v - r, v + r] enclose the cell of every point in
+// that interval), clamped to the grid; NaN goes to cell 0.
+__device__ __forceinline__ int bqc_cell(float v, float lo, float inv, int cells)
+{
+    return min(cells - 1, max(0, static_cast<int>((v - lo) * inv)));
+}
+
+__global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
+    int n, int m, int blocks_per_cloud, int queries_per_block, float radius, float radius2, int nsample,
+    const float* __restrict__ new_xyz, const float* __restrict__ xyz, int64_t* __restrict__ idx,
+    float* __restrict__ dist)
+{
+    extern __shared__ __align__(16) unsigned char bqc_lds[];
+    float4* const sorted = reinterpret_cast<float4*>(bqc_lds); // [n] x, y, z, index; cell by cell
+    int* const starts = reinterpret_cast<int*>(sorted + n);    // [BQC_STARTS] counts, then first places
+    CellWave* const waves = reinterpret_cast<CellWave*>(starts + BQC_STARTS);
+    __shared__ float box_parts[6][BQC_WAVES]; // per wavefront: -min x, y, z then max x, y, z
+    __shared__ float box[6];
+    __shared__ int wave_totals[BQC_WAVES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
+    const int cloud = blockIdx.x / blocks_per_cloud;
+    const int blk = blockIdx.x - cloud * blocks_per_cloud;
+    new_xyz += static_cast<int64_t>(cloud) * m * 3;
+    xyz += static_cast<int64_t>(cloud) * n * 3;
+    TPK_WORK_DECL
+
+    // ---- the cloud's points and bounding box (finite coordinates only) ----
+    float px[BQC_PER_THREAD], py[BQC_PER_THREAD], pz[BQC_PER_THREAD];
+#pragma unroll
+    for (int u = 0; u < BQC_PER_THREAD; ++u)
+    {
+        const int t = min(tid + u * BQC_THREADS, n - 1);
+        px[u] = xyz[t * 3 + 0];
+        py[u] = xyz[t * 3 + 1];
+        pz[u] = xyz[t * 3 + 2];
+    }
+    for (int c = tid; c < BQC_STARTS; c += BQC_THREADS)
+        starts[c] = 0;
+    {
+        const float inf = __builtin_inff();
+        float ends[6] = {inf, inf, inf, inf, inf, inf}; // (minima of -max: one kind of reduction)
+#pragma unroll
+        for (int u = 0; u < BQC_PER_THREAD; ++u)
+        {
+            // (rows past the end repeat the last point: no effect on the box)
+            const float v[3] = {px[u], py[u], pz[u]};
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+                if (fabsf(v[a]) < inf)
+                {
+                    ends[a] = fminf(ends[a], v[a]);
+                    ends[3 + a] = fminf(ends[3 + a], -v[a]);
+                }
+        }
+#pragma unroll
+        for (int a = 0; a < 6; ++a)
+        {
+            const float e = wave_min_f32(ends[a]);
+            if (lane == 0)
+                box_parts[a][wave] = e;
+        }
+    }
+    __syncthreads();
+    if (wave == 0)
+    {
+#pragma unroll
+        for (int a = 0; a < 6; ++a)
+        {
+            const float e = row_all_min_f32(box_parts[a][lane & (BQC_WAVES - 1)]);
+            if (lane == 0)
+                box[a] = e;
+        }
+    }
+    __syncthreads();
+
+    // ---- the grid: per axis as many cells (16 at most) as are at least one radius wide ----
+    const float reach = fabsf(radius); // (the test itself uses radius * radius)
+    float lo[3], inv[3];
+    int cells[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+    {
+        lo[a] = box[a];
+        const float extent = -box[3 + a] - lo[a]; // (NaN or -inf for a cloud without finite coordinates)
+        const float fit = fminf(extent / reach, static_cast<float>(BQC_GRID));
+        cells[a] = fit >= 1.0f ? static_cast<int>(fit) : 1;
+        inv[a] = extent > 0.0f ? static_cast<float>(cells[a]) / extent : 0.0f;
+        lo[a] = extent > 0.0f ? lo[a] : 0.0f;
+    }
+
+    // ---- count per cell; the count before a point's own increment is its place inside the cell ----
+    int placed[BQC_PER_THREAD];
+#pragma unroll
+    for (int u = 0; u < BQC_PER_THREAD; ++u)
+        if (tid + u * BQC_THREADS < n)
+        {
+            const int c = bqc_cell(px[u], lo[0], inv[0], cells[0]) +
+                          cells[0] * (bqc_cell(py[u], lo[1], inv[1], cells[1]) + cells[1] * bqc_cell(pz[u], lo[2], inv[2], cells[2]));
+            placed[u] = (c << 16) | atomicAdd(&starts[c], 1);
+        }
+    __syncthreads();
+    {
+        // exclusive prefix sum over the cells, four per thread
+        int4 c4 = reinterpret_cast<int4*>(starts)[tid];
+        const int own = c4.x + c4.y + c4.z + c4.w;
+        const int before = wave_exclusive_sum(own);
+        if (lane == TPK_WAVE - 1)
+            wave_totals[wave] = before + own;
+        __syncthreads();
+        const int total = lane < BQC_WAVES ? wave_totals[lane] : 0;
+        int at = __builtin_amdgcn_readlane(wave_exclusive_sum(total), wave) + before;
+        int4 s4;
+        s4.x = at;
+        s4.y = at += c4.x;
+        s4.z = at += c4.y;
+        s4.w = at += c4.z;
+        reinterpret_cast<int4*>(starts)[tid] = s4;
+        if (tid == BQC_THREADS - 1)
+            starts[BQC_CELLS] = at + c4.w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < BQC_PER_THREAD; ++u)
+        if (tid + u * BQC_THREADS < n)
+            sorted[starts[placed[u] >> 16] + (placed[u] & 0xFFFF)] =
+                make_float4(px[u], py[u], pz[u], __int_as_float(tid + u * BQC_THREADS));
+    __syncthreads();
+
+    // ---- queries: one wavefront each, no workgroup barrier from here on ----
+    int* const rows = waves[wave].rows;
+    float* const dists = waves[wave].dists;
+    volatile int* const marks = waves[wave].marks; // (volatile: a lane reads what other lanes wrote)
+    const int q_end = min(m, (blk + 1) * queries_per_block);
+    for (int j = blk * queries_per_block + wave; j < q_end; j += BQC_WAVES)
+    {
+        const float ux = new_xyz[j * 3 + 0], uy = new_xyz[j * 3 + 1], uz = new_xyz[j * 3 + 2];
+        const float qx = to_vector_register(ux), qy = to_vector_register(uy), qz = to_vector_register(uz);
+        const int64_t out = (static_cast<int64_t>(cloud) * m + j) * nsample;
+        const float u[3] = {ux, uy, uz};
+        int first[3], count[3];
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+        {
+            // (the interval is widened by a few ulps of its ends: a point that the fp32 radius test accepts
+            // is never left out)
+            const float slack = (fabsf(u[a]) + reach) * 1e-6f + 1e-30f;
+            first[a] = bqc_cell((u[a] - reach) - slack, lo[a], inv[a], cells[a]);
+            count[a] = bqc_cell((u[a] + reach) + slack, lo[a], inv[a], cells[a]) - first[a] + 1;
+        }
+        const int runs = count[1] * count[2];
+        int cnt = 0;
+        bool serial = runs > TPK_WAVE;
+        if (!serial)
+        {
+            // lane r: the places of run r (the cells first[0] .. first[0] + count[0] - 1 of one (y, z))
+            int start = 0, size = 0;
+            if (lane < runs)
+            {
+                const int c = first[0] + cells[0] * ((first[1] + lane % count[1]) + cells[1] * (first[2] + lane / count[1]));
+                start = starts[c];
+                size = starts[c + count[0]] - start;
+            }
+            const int before = wave_exclusive_sum(size);
+            const int total = __builtin_amdgcn_readlane(before + size, TPK_WAVE - 1);
+            const int origin = start - before; // candidate c lies at origin + c, for the c of this lane's run
+            serial = total > BQC_MAX_CANDIDATES;
+            for (int c0 = 0; c0 < total && !serial; c0 += TPK_WAVE)
+            {
+                // Which run does candidate c0 + lane belong to?  Every run's lane marks the slot of its first
+                // candidate in this step with its own number; a running maximum carries it to the others.
+                marks[lane] = 0;
+                if (size > 0 && before < c0 + TPK_WAVE && before + size > c0)
+                    marks[max(before - c0, 0)] = lane;
+                const int mark = marks[lane];
+                const bool has = c0 + lane < total;
+                const int at = __shfl(origin, wave_inclusive_max_i32(mark)) + c0 + lane;
+                const float4 p = sorted[has ? at : 0];
+                const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+                TPK_WORK_ADD(1);
+                const bool hit = has && d < radius2;
+                const unsigned long long mask = __ballot(hit);
+                if (mask == 0ull)
+                    continue;
+                const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
+                if (hit && slot < BQC_HITS)
+                {
+                    rows[slot] = __float_as_int(p.w);
+                    dists[slot] = d;
+                }
+                cnt += __builtin_popcountll(mask);
+                serial = cnt > BQC_HITS;
+            }
+        }
+        if (!serial)
+        {
+            // rank of every hit among the hits (indices are distinct), hits in that order, then the padding
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            const int my_row = rows[lane < cnt ? lane : 0];
+            const float my_dist = dists[lane < cnt ? lane : 0];
+            int rank = 0, lowest = cnt > 0 ? 0x7fffffff : 0;
+            for (int h = 0; h < cnt; ++h)
+            {
+                const int other = rows[h];
+                rank += other < my_row ? 1 : 0;
+                lowest = min(lowest, other);
+            }
+            if (lane < cnt && rank < nsample)
+            {
+                idx[out + rank] = my_row;
+                dist[out + rank] = my_dist;
+            }
+            for (int s = cnt + lane; s < nsample; s += TPK_WAVE)
+            {
+                idx[out + s] = lowest;
+                dist[out + s] = -1.0f;
+            }
+            // (the next query's hits overwrite rows / dists: all lanes have read theirs above)
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            continue;
+        }
+
+        // The scan in index order itself: lanes hold 64 consecutive points; ballot + prefix count give the
+        // hits their slots; stop after nsample hits.
+        cnt = 0;
+        int64_t lowest = 0;
+        constexpr int BATCH = 4; // loads of four steps in flight
+        for (int base = 0; base < n && cnt < nsample; base += BATCH * TPK_WAVE)
+        {
+            float sx[BATCH], sy[BATCH], sz[BATCH];
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b)
+            {
+                const int pos = min(base + b * TPK_WAVE + lane, n - 1);
+                sx[b] = xyz[pos * 3 + 0];
+                sy[b] = xyz[pos * 3 + 1];
+                sz[b] = xyz[pos * 3 + 2];
+            }
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b)
+            {
+                const int pos = base + b * TPK_WAVE + lane;
+                const float d = tpk_dist2(qx, qy, qz, sx[b], sy[b], sz[b]);
+                TPK_WORK_ADD(1);
+                const bool hit = pos < n && d < radius2;
+                const unsigned long long mask = __ballot(hit);
+                if (mask == 0ull)
+                    continue;
+                const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
+                if (hit && slot < nsample)
+                {
+                    idx[out + slot] = pos;
+                    dist[out + slot] = d;
+                }
+                if (cnt == 0)
+                    lowest = base + b * TPK_WAVE + __builtin_ctzll(mask);
+                cnt += __builtin_popcountll(mask);
+            }
+        }
+        for (int s = cnt + lane; s < nsample; s += TPK_WAVE)
+        {
+            idx[out + s] = lowest;
+            dist[out + s] = -1.0f;
+        }
+    }
+    TPK_WORK_FLUSH
+}
+
 __global__ __launch_bounds__(BQ_THREADS) void ball_query_partial_kernel(
     int64_t size_x, int64_t size_y, float radius2, int nsample, const float* __restrict__ x,
     const float* __restrict__ y, const int64_t* __restrict__ batch_x,
@@ -280,6 +606,21 @@ extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int n
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     const float radius2 = radius * radius; // fp32 product, as the reference kernel forms it
+    if (n >= BQC_MIN_POINTS && n <= BQC_MAX_POINTS)
+    {
+        // over cells; one workgroup per compute unit where the queries allow it (every workgroup bins its cloud)
+        const int64_t per_cloud = std::max<int64_t>(1, std::min<int64_t>(tpk_ceil_div(m, BQC_WAVES), TPK_COMPUTE_UNITS / b));
+        const int per_block = static_cast<int>(tpk_ceil_div(m, per_cloud));
+        const int64_t cell_bpc = tpk_ceil_div(m, per_block);
+        const size_t lds = bqc_lds_bytes(n);
+        const int st = tpk_allow_lds(reinterpret_cast<const void*>(&ball_query_dense_cells_kernel), lds);
+        if (st != TPK_OK)
+            return st;
+        hipLaunchKernelGGL(ball_query_dense_cells_kernel, dim3(static_cast<unsigned>(cell_bpc * b)), dim3(BQC_THREADS), lds,
+                           tpk_stream(stream), n, m, static_cast<int>(cell_bpc), per_block, radius, radius2, nsample, new_xyz,
+                           xyz, idx, dist);
+        return tpk_launch_status();
+    }
     if (few)
         hipLaunchKernelGGL(ball_query_dense_kernel<BQ_Q_FEW>, dim3(static_cast<unsigned>(blocks)), dim3(BQ_THREADS), 0,
                            tpk_stream(stream), n, m, static_cast<int>(bpc), radius2, nsample, new_xyz, xyz, idx, dist);
