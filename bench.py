@@ -351,7 +351,8 @@ def bench_others(dev, steps, warmup, with_cpu):
     e = {"workload": "configs[0]: ball_query dense B=8 N=4096 M=1024 r=0.1 nsample=32", "metric": "queries/s",
          "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
          "roofline": _roof_flops(executed, pairs, 8, ev, "ball_query_dense"), "pairs_upper_bound": pairs}
-    e["roofline"]["note"] += PRUNED_NOTE
+    e["roofline"]["note"] += ("; every workgroup bins its cloud into cells at least one radius wide and a query tests "
+                              "the cells around its ball only")
     if ref is not None:
         secs = _cpu_time(lambda: ref.dense_ball_query(w["new_xyz"], w["xyz"], w["radius"], w["nsample"], 0, False))
         e["cpu_baseline"] = {"value": nq / secs, "unit": "queries/s", "cores": 1, "kind": "reference",

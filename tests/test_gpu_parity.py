@@ -173,13 +173,14 @@ def test_ball_query_dense_boundary_and_empty(tpk, oracle, dev):
     assert (idx == 0).all() and (dist == -1).all()
 
 
-@pytest.mark.parametrize("kind", ["uniform", "clusters", "flat", "one_point", "outlier", "queries_outside", "non_finite", "line"])
+@pytest.mark.parametrize("kind", ["uniform", "clusters", "flat", "one_point", "outlier", "queries_outside", "non_finite", "line",
+                                  "offset_3e4", "offset_1e6", "negative"])
 @pytest.mark.parametrize("B,N,M,r,ns", [(2, 512, 100, 0.2, 8), (4, 8192, 300, 0.05, 16), (1, 4096, 1030, 0.1, 100),
                                         (3, 1500, 17, 0.02, 4), (2, 6000, 64, 0.35, 32)])
 def test_ball_query_dense_over_cells(tpk, oracle, dev, kind, B, N, M, r, ns):
-    # clouds of 512 .. 8192 support points are binned into cells of at least one radius: shapes of clouds that
-    # stress the grid (no extent along an axis, everything in one cell, a far point that makes all cells wide,
-    # queries outside the box, coordinates that are not finite), checked against the scan in index order
+    # clouds of 512 .. 8192 support points are hung into buckets of cells: shapes of clouds that stress the
+    # cells (no extent along an axis, everything in one cell, a far point, queries away from the cloud,
+    # coordinates that are not finite or far from the origin), checked against the scan in index order
     g = torch.Generator().manual_seed(7 * N + M)
     xyz = torch.rand(B, N, 3, generator=g)
     new_xyz = xyz[:, torch.randperm(N, generator=g)[:M] % N].clone() + 0.01 * torch.randn(B, M, 3, generator=g)
@@ -207,6 +208,11 @@ def test_ball_query_dense_over_cells(tpk, oracle, dev, kind, B, N, M, r, ns):
     elif kind == "line":
         xyz[..., 1:] = 0.0
         new_xyz[..., 1:] = 0.0
+    elif kind.startswith("offset"):
+        # coordinates far from the origin: their rounding is no longer small against the radius
+        xyz, new_xyz = xyz + float(kind[7:]), new_xyz + float(kind[7:])
+    elif kind == "negative":
+        xyz, new_xyz = xyz * 3.0 - 2.0, new_xyz * 3.0 - 2.0
     idx, dist = tpk.ball_query(r, ns, xyz.to(dev), new_xyz.contiguous().to(dev), mode="dense")
     want_idx, want_dist = oracle.ball_query_dense(r, ns, xyz.numpy(), new_xyz.numpy())
     np.testing.assert_array_equal(_np(idx), want_idx)

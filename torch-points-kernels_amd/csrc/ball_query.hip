@@ -215,63 +215,54 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
 // Dense layout over cells: clouds of BQC_MIN_POINTS .. BQC_MAX_POINTS support points.
 //
 // Testing every support point costs n / 64 steps per query whatever the radius.  Here a workgroup
-// of 16 wavefronts first bins its cloud in LDS: bounding box, a grid of up to 16 cells per axis
-// whose cells are at least one radius wide, a count per cell (LDS atomics that also hand every
-// point its place inside its cell), a prefix sum, and the points (x, y, z, index) written cell by
-// cell.  All workgroups of a cloud repeat this (a few microseconds; the cloud comes from the L2),
-// which is cheaper than a launch that does it once.  Then every wavefront answers queries, one at
-// a time: the cells that the cube around the ball touches form, for every (y, z), one run of
-// consecutive places - cells are numbered x first - so lane r takes row r's run, and the
-// candidates of all runs are dealt to the lanes 64 at a time.  A candidate with d2 < radius^2 is
-// a hit; the hits (at most 64) are ranked by index and written in ascending index order, which
-// is what the scan in index order produces (cuda/src/ball_query_gpu.cu:9-52).  A query with more
-// than 64 hits, or whose cube holds more than BQC_MAX_CANDIDATES points (a ball that covers much
-// of its cloud), is answered by that scan itself, 64 points per step from global memory with
-// early exit: with so many hits it ends soon.
+// of 16 wavefronts first hangs its cloud into 4096 buckets in LDS: space is cut into cells 0.7
+// radii wide, cell (i, j, k) belongs to bucket (i mod 16, j mod 16, k mod 16), and every point
+// is pushed onto its bucket's chain (one LDS exchange per point; the points stay in index order
+// in LDS and carry the link to the next one).  No bounding box, no counting, no sorting: two
+// barriers, and a far outlier or a tiny radius costs nothing.  All workgroups of a cloud repeat
+// this (the cloud comes from the L2), which is cheaper than a launch that does it once.  Then
+// every wavefront answers queries, one at a time: [q - r, q + r] touches at most four cells per
+// axis (five when an end of the interval falls within rounding of a cell's edge), lane c takes
+// cell c and walks its bucket's chain, all lanes in step.  Points of other cells that share
+// the bucket fail the distance test like any other; no two cells of one query share a bucket.
+// A candidate with d2 < radius^2 is a hit; the hits (at most 64) are ranked by index and written
+// in ascending index order, which is what the scan in index order produces
+// (cuda/src/ball_query_gpu.cu:9-52).  A query with more than 64 hits, with chains longer than
+// BQC_MAX_CHAIN in all, or whose interval is wider than five cells (coordinates so large that
+// rounding dwarfs the radius) is answered by that scan itself, 64 points per step from global
+// memory with early exit: with so many hits it ends soon.
 // ---------------------------------------------------------------------------------------
 constexpr int BQC_THREADS = 1024;
 constexpr int BQC_WAVES = BQC_THREADS / TPK_WAVE;
 constexpr int BQC_MIN_POINTS = 512;
 constexpr int BQC_MAX_POINTS = 8192;
 constexpr int BQC_PER_THREAD = BQC_MAX_POINTS / BQC_THREADS;
-constexpr int BQC_GRID = 16;
-constexpr int BQC_CELLS = BQC_GRID * BQC_GRID * BQC_GRID;
-constexpr int BQC_STARTS = BQC_CELLS + TPK_WAVE; // the cells' first places, one more for the end, padded
+constexpr int BQC_BUCKETS = 4096;    // 16 x 16 x 16
+constexpr float BQC_CELL = 0.7f;     // cell width in radii
+constexpr int BQC_SPAN = 5;          // cells per axis a query may touch
 constexpr int BQC_HITS = TPK_WAVE;
-constexpr int BQC_MAX_CANDIDATES = 8 * TPK_WAVE;
+constexpr int BQC_MAX_CHAIN = 48;    // steps of the chain walk per query
 
 struct CellWave
 {
     int rows[BQC_HITS];
     float dists[BQC_HITS];
-    int marks[TPK_WAVE];
 };
 
 size_t bqc_lds_bytes(int n)
 {
-    return static_cast<size_t>(n) * sizeof(float4) + BQC_STARTS * sizeof(int) + BQC_WAVES * sizeof(CellWave);
+    return static_cast<size_t>(n) * sizeof(float4) + BQC_BUCKETS * sizeof(int) + BQC_WAVES * sizeof(CellWave);
 }
 
-// Smallest / largest v of every 16-lane row, in all lanes of the row.
-__device__ __forceinline__ float row_all_min_f32(float v)
+// Cell along one axis: monotone in v, so the cells of [v - r, v + r] enclose the cell of every point in
+// that interval (the conversion saturates; NaN goes to cell 0).
+__device__ __forceinline__ int bqc_cell(float v, float inv)
 {
-    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true)));
-    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true)));
-    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, true)));
-    v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true)));
-    return v;
+    return static_cast<int>(floorf(v * inv));
 }
-__device__ __forceinline__ float wave_min_f32(float v)
+__device__ __forceinline__ int bqc_bucket(int i, int j, int k)
 {
-    v = row_all_min_f32(v);
-    return fminf(fminf(tpk_read_lane(v, 0), tpk_read_lane(v, 16)), fminf(tpk_read_lane(v, 32), tpk_read_lane(v, 48)));
-}
-
-// Cell along one axis: monotone in v (so the cells of [v - r, v + r] enclose the cell of every point in
-// that interval), clamped to the grid; NaN goes to cell 0.
-__device__ __forceinline__ int bqc_cell(float v, float lo, float inv, int cells)
-{
-    return min(cells - 1, max(0, static_cast<int>((v - lo) * inv)));
+    return (i & 15) | ((j & 15) << 4) | ((k & 15) << 8);
 }
 
 __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
@@ -280,12 +271,9 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
     float* __restrict__ dist)
 {
     extern __shared__ __align__(16) unsigned char bqc_lds[];
-    float4* const sorted = reinterpret_cast<float4*>(bqc_lds); // [n] x, y, z, index; cell by cell
-    int* const starts = reinterpret_cast<int*>(sorted + n);    // [BQC_STARTS] counts, then first places
-    CellWave* const waves = reinterpret_cast<CellWave*>(starts + BQC_STARTS);
-    __shared__ float box_parts[6][BQC_WAVES]; // per wavefront: -min x, y, z then max x, y, z
-    __shared__ float box[6];
-    __shared__ int wave_totals[BQC_WAVES];
+    float4* const points = reinterpret_cast<float4*>(bqc_lds); // [n] x, y, z, next point of the bucket's chain
+    int* const heads = reinterpret_cast<int*>(points + n);     // [BQC_BUCKETS] first point of the chain, -1: none
+    CellWave* const waves = reinterpret_cast<CellWave*>(heads + BQC_BUCKETS);
 
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
@@ -296,7 +284,7 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
     xyz += static_cast<int64_t>(cloud) * n * 3;
     TPK_WORK_DECL
 
-    // ---- the cloud's points and bounding box (finite coordinates only) ----
+    // ---- the cloud's points onto the chains of their buckets ----
     float px[BQC_PER_THREAD], py[BQC_PER_THREAD], pz[BQC_PER_THREAD];
 #pragma unroll
     for (int u = 0; u < BQC_PER_THREAD; ++u)
@@ -306,102 +294,27 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
         py[u] = xyz[t * 3 + 1];
         pz[u] = xyz[t * 3 + 2];
     }
-    for (int c = tid; c < BQC_STARTS; c += BQC_THREADS)
-        starts[c] = 0;
-    {
-        const float inf = __builtin_inff();
-        float ends[6] = {inf, inf, inf, inf, inf, inf}; // (minima of -max: one kind of reduction)
-#pragma unroll
-        for (int u = 0; u < BQC_PER_THREAD; ++u)
-        {
-            // (rows past the end repeat the last point: no effect on the box)
-            const float v[3] = {px[u], py[u], pz[u]};
-#pragma unroll
-            for (int a = 0; a < 3; ++a)
-                if (fabsf(v[a]) < inf)
-                {
-                    ends[a] = fminf(ends[a], v[a]);
-                    ends[3 + a] = fminf(ends[3 + a], -v[a]);
-                }
-        }
-#pragma unroll
-        for (int a = 0; a < 6; ++a)
-        {
-            const float e = wave_min_f32(ends[a]);
-            if (lane == 0)
-                box_parts[a][wave] = e;
-        }
-    }
-    __syncthreads();
-    if (wave == 0)
-    {
-#pragma unroll
-        for (int a = 0; a < 6; ++a)
-        {
-            const float e = row_all_min_f32(box_parts[a][lane & (BQC_WAVES - 1)]);
-            if (lane == 0)
-                box[a] = e;
-        }
-    }
-    __syncthreads();
-
-    // ---- the grid: per axis as many cells (16 at most) as are at least one radius wide ----
+    static_assert(BQC_BUCKETS == 4 * BQC_THREADS, "one int4 of heads per thread");
+    reinterpret_cast<int4*>(heads)[tid] = make_int4(-1, -1, -1, -1);
     const float reach = fabsf(radius); // (the test itself uses radius * radius)
-    float lo[3], inv[3];
-    int cells[3];
-#pragma unroll
-    for (int a = 0; a < 3; ++a)
-    {
-        lo[a] = box[a];
-        const float extent = -box[3 + a] - lo[a]; // (NaN or -inf for a cloud without finite coordinates)
-        const float fit = fminf(extent / reach, static_cast<float>(BQC_GRID));
-        cells[a] = fit >= 1.0f ? static_cast<int>(fit) : 1;
-        inv[a] = extent > 0.0f ? static_cast<float>(cells[a]) / extent : 0.0f;
-        lo[a] = extent > 0.0f ? lo[a] : 0.0f;
-    }
-
-    // ---- count per cell; the count before a point's own increment is its place inside the cell ----
-    int placed[BQC_PER_THREAD];
+    const float inv = reach > 0.0f ? 1.0f / (BQC_CELL * reach) : 0.0f;
+    lds_barrier();
 #pragma unroll
     for (int u = 0; u < BQC_PER_THREAD; ++u)
-        if (tid + u * BQC_THREADS < n)
+    {
+        const int t = tid + u * BQC_THREADS;
+        if (t < n)
         {
-            const int c = bqc_cell(px[u], lo[0], inv[0], cells[0]) +
-                          cells[0] * (bqc_cell(py[u], lo[1], inv[1], cells[1]) + cells[1] * bqc_cell(pz[u], lo[2], inv[2], cells[2]));
-            placed[u] = (c << 16) | atomicAdd(&starts[c], 1);
+            const int bucket = bqc_bucket(bqc_cell(px[u], inv), bqc_cell(py[u], inv), bqc_cell(pz[u], inv));
+            const int next = atomicExch(&heads[bucket], t);
+            points[t] = make_float4(px[u], py[u], pz[u], __int_as_float(next));
         }
-    __syncthreads();
-    {
-        // exclusive prefix sum over the cells, four per thread
-        int4 c4 = reinterpret_cast<int4*>(starts)[tid];
-        const int own = c4.x + c4.y + c4.z + c4.w;
-        const int before = wave_exclusive_sum(own);
-        if (lane == TPK_WAVE - 1)
-            wave_totals[wave] = before + own;
-        __syncthreads();
-        const int total = lane < BQC_WAVES ? wave_totals[lane] : 0;
-        int at = __builtin_amdgcn_readlane(wave_exclusive_sum(total), wave) + before;
-        int4 s4;
-        s4.x = at;
-        s4.y = at += c4.x;
-        s4.z = at += c4.y;
-        s4.w = at += c4.z;
-        reinterpret_cast<int4*>(starts)[tid] = s4;
-        if (tid == BQC_THREADS - 1)
-            starts[BQC_CELLS] = at + c4.w;
     }
-    __syncthreads();
-#pragma unroll
-    for (int u = 0; u < BQC_PER_THREAD; ++u)
-        if (tid + u * BQC_THREADS < n)
-            sorted[starts[placed[u] >> 16] + (placed[u] & 0xFFFF)] =
-                make_float4(px[u], py[u], pz[u], __int_as_float(tid + u * BQC_THREADS));
     __syncthreads();
 
     // ---- queries: one wavefront each, no workgroup barrier from here on ----
     int* const rows = waves[wave].rows;
     float* const dists = waves[wave].dists;
-    volatile int* const marks = waves[wave].marks; // (volatile: a lane reads what other lanes wrote)
     const int q_end = min(m, (blk + 1) * queries_per_block);
     for (int j = blk * queries_per_block + wave; j < q_end; j += BQC_WAVES)
     {
@@ -416,66 +329,76 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
             // (the interval is widened by a few ulps of its ends: a point that the fp32 radius test accepts
             // is never left out)
             const float slack = (fabsf(u[a]) + reach) * 1e-6f + 1e-30f;
-            first[a] = bqc_cell((u[a] - reach) - slack, lo[a], inv[a], cells[a]);
-            count[a] = bqc_cell((u[a] + reach) + slack, lo[a], inv[a], cells[a]) - first[a] + 1;
+            first[a] = bqc_cell((u[a] - reach) - slack, inv);
+            // (as a difference of 64-bit values: the ends may lie at the two ends of the int range)
+            const long long span = static_cast<long long>(bqc_cell((u[a] + reach) + slack, inv)) - first[a] + 1;
+            count[a] = static_cast<int>(span < BQC_SPAN + 1 ? span : BQC_SPAN + 1);
         }
-        const int runs = count[1] * count[2];
         int cnt = 0;
-        bool serial = runs > TPK_WAVE;
+        bool serial = count[0] > BQC_SPAN || count[1] > BQC_SPAN || count[2] > BQC_SPAN;
         if (!serial)
         {
-            // lane r: the places of run r (the cells first[0] .. first[0] + count[0] - 1 of one (y, z))
-            int start = 0, size = 0;
-            if (lane < runs)
+            const int cells = count[0] * count[1] * count[2];
+            const int plane = count[0] * count[1];
+            // (lane -> cell by float division: exact for these small numbers)
+            const float inv_plane = 1.0f / static_cast<float>(plane), inv_line = 1.0f / static_cast<float>(count[0]);
+            int steps = 0;
+            for (int c0 = 0; c0 < cells && !serial; c0 += TPK_WAVE)
             {
-                const int c = first[0] + cells[0] * ((first[1] + lane % count[1]) + cells[1] * (first[2] + lane / count[1]));
-                start = starts[c];
-                size = starts[c + count[0]] - start;
-            }
-            const int before = wave_exclusive_sum(size);
-            const int total = __builtin_amdgcn_readlane(before + size, TPK_WAVE - 1);
-            const int origin = start - before; // candidate c lies at origin + c, for the c of this lane's run
-            serial = total > BQC_MAX_CANDIDATES;
-            for (int c0 = 0; c0 < total && !serial; c0 += TPK_WAVE)
-            {
-                // Which run does candidate c0 + lane belong to?  Every run's lane marks the slot of its first
-                // candidate in this step with its own number; a running maximum carries it to the others.
-                marks[lane] = 0;
-                if (size > 0 && before < c0 + TPK_WAVE && before + size > c0)
-                    marks[max(before - c0, 0)] = lane;
-                const int mark = marks[lane];
-                const bool has = c0 + lane < total;
-                const int at = __shfl(origin, wave_inclusive_max_i32(mark)) + c0 + lane;
-                const float4 p = sorted[has ? at : 0];
-                const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
-                TPK_WORK_ADD(1);
-                const bool hit = has && d < radius2;
-                const unsigned long long mask = __ballot(hit);
-                if (mask == 0ull)
-                    continue;
-                const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
-                if (hit && slot < BQC_HITS)
+                const int c = c0 + lane;
+                const int k = static_cast<int>((static_cast<float>(c) + 0.5f) * inv_plane);
+                const int rest = c - k * plane;
+                const int jj = static_cast<int>((static_cast<float>(rest) + 0.5f) * inv_line);
+                const int i = rest - jj * count[0];
+                int cur = c < cells ? heads[bqc_bucket(first[0] + i, first[1] + jj, first[2] + k)] : -1;
+                // all lanes walk their chains in step
+                while (__ballot(cur >= 0) != 0ull)
                 {
-                    rows[slot] = __float_as_int(p.w);
-                    dists[slot] = d;
+                    if (++steps > BQC_MAX_CHAIN)
+                    {
+                        serial = true;
+                        break;
+                    }
+                    const float4 p = points[max(cur, 0)];
+                    const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+                    TPK_WORK_ADD(1);
+                    const bool hit = cur >= 0 && d < radius2;
+                    const unsigned long long mask = __ballot(hit);
+                    if (mask != 0ull)
+                    {
+                        const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
+                        if (hit && slot < BQC_HITS)
+                        {
+                            rows[slot] = cur;
+                            dists[slot] = d;
+                        }
+                        cnt += __builtin_popcountll(mask);
+                        if (cnt > BQC_HITS)
+                        {
+                            serial = true;
+                            break;
+                        }
+                    }
+                    cur = cur >= 0 ? __float_as_int(p.w) : -1;
                 }
-                cnt += __builtin_popcountll(mask);
-                serial = cnt > BQC_HITS;
             }
         }
         if (!serial)
         {
             // rank of every hit among the hits (indices are distinct), hits in that order, then the padding
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            const int my_row = rows[lane < cnt ? lane : 0];
+            const int my_row = lane < cnt ? rows[lane] : 0x7fffffff;
             const float my_dist = dists[lane < cnt ? lane : 0];
             int rank = 0, lowest = cnt > 0 ? 0x7fffffff : 0;
-            for (int h = 0; h < cnt; ++h)
-            {
-                const int other = rows[h];
-                rank += other < my_row ? 1 : 0;
-                lowest = min(lowest, other);
-            }
+            // (four hits per turn; the lanes past the last hit hold the largest int, which counts for nothing)
+            for (int h = 0; h < cnt; h += 4)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    const int other = __builtin_amdgcn_readlane(my_row, h + g);
+                    rank += other < my_row ? 1 : 0;
+                    lowest = min(lowest, other);
+                }
             if (lane < cnt && rank < nsample)
             {
                 idx[out + rank] = my_row;
