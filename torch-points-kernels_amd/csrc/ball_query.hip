@@ -234,11 +234,11 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
 // ---------------------------------------------------------------------------------------
 constexpr int BQC_THREADS = 1024;
 constexpr int BQC_WAVES = BQC_THREADS / TPK_WAVE;
-constexpr int BQC_MIN_POINTS = 512;
+constexpr int BQC_MIN_POINTS = 1024;
 constexpr int BQC_MAX_POINTS = 8192;
 constexpr int BQC_PER_THREAD = BQC_MAX_POINTS / BQC_THREADS;
 constexpr int BQC_BUCKETS = 4096;    // 16 x 16 x 16
-constexpr float BQC_CELL = 0.7f;     // cell width in radii
+constexpr float BQC_CELL = 0.7f;     // cell width in radii (measured: 0.55 / 0.85 / 1.0 are 28 / 8 / 18 % slower)
 constexpr int BQC_SPAN = 5;          // cells per axis a query may touch
 constexpr int BQC_HITS = TPK_WAVE;
 constexpr int BQC_MAX_CHAIN = 48;    // steps of the chain walk per query
@@ -274,6 +274,7 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
     float4* const points = reinterpret_cast<float4*>(bqc_lds); // [n] x, y, z, next point of the bucket's chain
     int* const heads = reinterpret_cast<int*>(points + n);     // [BQC_BUCKETS] first point of the chain, -1: none
     CellWave* const waves = reinterpret_cast<CellWave*>(heads + BQC_BUCKETS);
+    __shared__ int occupied; // buckets with a chain
 
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
@@ -296,26 +297,111 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
     }
     static_assert(BQC_BUCKETS == 4 * BQC_THREADS, "one int4 of heads per thread");
     reinterpret_cast<int4*>(heads)[tid] = make_int4(-1, -1, -1, -1);
+    if (tid == 0)
+        occupied = 0;
     const float reach = fabsf(radius); // (the test itself uses radius * radius)
     const float inv = reach > 0.0f ? 1.0f / (BQC_CELL * reach) : 0.0f;
     lds_barrier();
+    int fresh = 0; // chains this wavefront started
 #pragma unroll
     for (int u = 0; u < BQC_PER_THREAD; ++u)
     {
         const int t = tid + u * BQC_THREADS;
+        int next = 0;
         if (t < n)
         {
             const int bucket = bqc_bucket(bqc_cell(px[u], inv), bqc_cell(py[u], inv), bqc_cell(pz[u], inv));
-            const int next = atomicExch(&heads[bucket], t);
+            next = atomicExch(&heads[bucket], t);
             points[t] = make_float4(px[u], py[u], pz[u], __int_as_float(next));
         }
+        fresh += __builtin_popcountll(__ballot(next < 0));
     }
+    if (lane == 0 && fresh > 0)
+        atomicAdd(&occupied, fresh);
     __syncthreads();
 
+    // Chains or the scan in index order for this cloud?  n / occupied points per cell stand for about 12 times
+    // as many in a ball (volumes 4.19 against 0.34 radii cubed).  A chain walk takes a step for every five
+    // points in the ball and is lost work when the ball holds more than 64.  The scan stops after nsample hits,
+    // 64 points a step, two queries a step; balls at the rim of a cloud hold a fraction of the points and scan
+    // far longer, hence the 4.  Both costs in units fitted to measurements on clouds of 1024 .. 8192 points and
+    // 2 .. 1100 points per ball.  (A query whose surroundings are denser than the cloud's average still falls
+    // back on its own.)
+    const float in_ball = 12.2f * static_cast<float>(n) / static_cast<float>(max(occupied, 1));
+    const float scan_steps = fminf(static_cast<float>(n), 4.0f * static_cast<float>(nsample) * static_cast<float>(n) / in_ball) * (1.0f / TPK_WAVE);
+    const bool scan_all = 1.6f + 0.24f * scan_steps < 2.0f + 0.2f * in_ball;
+
     // ---- queries: one wavefront each, no workgroup barrier from here on ----
+    const int q_end = min(m, (blk + 1) * queries_per_block);
+    if (scan_all)
+    {
+        // The scan in index order over the points in LDS, for two of the wavefront's queries at a time: lanes
+        // hold 64 consecutive points; a ballot of the radius test and a prefix count give the hits their slots;
+        // a query is switched off (radius -1) once it has nsample hits.
+        constexpr int QS = 2;
+        for (int j0 = blk * queries_per_block + wave; j0 < q_end; j0 += QS * BQC_WAVES)
+        {
+            float qx[QS], qy[QS], qz[QS], r2q[QS];
+            int cnt[QS], lowest[QS], live = 0;
+#pragma unroll
+            for (int t = 0; t < QS; ++t)
+            {
+                const bool on = j0 + t * BQC_WAVES < q_end;
+                const int j = on ? j0 + t * BQC_WAVES : j0;
+                qx[t] = to_vector_register(new_xyz[j * 3 + 0]);
+                qy[t] = to_vector_register(new_xyz[j * 3 + 1]);
+                qz[t] = to_vector_register(new_xyz[j * 3 + 2]);
+                r2q[t] = on ? radius2 : -1.0f;
+                cnt[t] = lowest[t] = 0;
+                live += on ? 1 : 0;
+            }
+            for (int base = 0; base < n && live > 0; base += TPK_WAVE)
+            {
+                const int pos = base + lane;
+                const float4 p = points[min(pos, n - 1)];
+                TPK_WORK_ADD(QS);
+#pragma unroll
+                for (int t = 0; t < QS; ++t)
+                {
+                    const float d = tpk_dist2(qx[t], qy[t], qz[t], p.x, p.y, p.z);
+                    const bool hit = pos < n && d < r2q[t];
+                    const unsigned long long mask = __ballot(hit);
+                    if (mask != 0ull)
+                    {
+                        const int slot = cnt[t] + static_cast<int>(tpk_prefix_count(mask));
+                        if (hit && slot < nsample)
+                        {
+                            const int64_t o = (static_cast<int64_t>(cloud) * m + j0 + t * BQC_WAVES) * nsample + slot;
+                            idx[o] = pos;
+                            dist[o] = d;
+                        }
+                        if (cnt[t] == 0)
+                            lowest[t] = base + __builtin_ctzll(mask);
+                        cnt[t] += __builtin_popcountll(mask);
+                        if (cnt[t] >= nsample)
+                        {
+                            cnt[t] = nsample;
+                            r2q[t] = -1.0f;
+                            --live;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < QS; ++t)
+                if (j0 + t * BQC_WAVES < q_end)
+                    for (int s = cnt[t] + lane; s < nsample; s += TPK_WAVE)
+                    {
+                        const int64_t o = (static_cast<int64_t>(cloud) * m + j0 + t * BQC_WAVES) * nsample + s;
+                        idx[o] = lowest[t];
+                        dist[o] = -1.0f;
+                    }
+        }
+        TPK_WORK_FLUSH
+        return;
+    }
     int* const rows = waves[wave].rows;
     float* const dists = waves[wave].dists;
-    const int q_end = min(m, (blk + 1) * queries_per_block);
     for (int j = blk * queries_per_block + wave; j < q_end; j += BQC_WAVES)
     {
         const float ux = new_xyz[j * 3 + 0], uy = new_xyz[j * 3 + 1], uz = new_xyz[j * 3 + 2];
@@ -414,42 +500,29 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
             continue;
         }
 
-        // The scan in index order itself: lanes hold 64 consecutive points; ballot + prefix count give the
-        // hits their slots; stop after nsample hits.
+        // The scan in index order itself, over the points in LDS: lanes hold 64 consecutive points; ballot +
+        // prefix count give the hits their slots; stop after nsample hits.
         cnt = 0;
-        int64_t lowest = 0;
-        constexpr int BATCH = 4; // loads of four steps in flight
-        for (int base = 0; base < n && cnt < nsample; base += BATCH * TPK_WAVE)
+        int lowest = 0;
+        for (int base = 0; base < n && cnt < nsample; base += TPK_WAVE)
         {
-            float sx[BATCH], sy[BATCH], sz[BATCH];
-#pragma unroll
-            for (int b = 0; b < BATCH; ++b)
+            const int pos = base + lane;
+            const float4 p = points[min(pos, n - 1)];
+            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+            TPK_WORK_ADD(1);
+            const bool hit = pos < n && d < radius2;
+            const unsigned long long mask = __ballot(hit);
+            if (mask == 0ull)
+                continue;
+            const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
+            if (hit && slot < nsample)
             {
-                const int pos = min(base + b * TPK_WAVE + lane, n - 1);
-                sx[b] = xyz[pos * 3 + 0];
-                sy[b] = xyz[pos * 3 + 1];
-                sz[b] = xyz[pos * 3 + 2];
+                idx[out + slot] = pos;
+                dist[out + slot] = d;
             }
-#pragma unroll
-            for (int b = 0; b < BATCH; ++b)
-            {
-                const int pos = base + b * TPK_WAVE + lane;
-                const float d = tpk_dist2(qx, qy, qz, sx[b], sy[b], sz[b]);
-                TPK_WORK_ADD(1);
-                const bool hit = pos < n && d < radius2;
-                const unsigned long long mask = __ballot(hit);
-                if (mask == 0ull)
-                    continue;
-                const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
-                if (hit && slot < nsample)
-                {
-                    idx[out + slot] = pos;
-                    dist[out + slot] = d;
-                }
-                if (cnt == 0)
-                    lowest = base + b * TPK_WAVE + __builtin_ctzll(mask);
-                cnt += __builtin_popcountll(mask);
-            }
+            if (cnt == 0)
+                lowest = base + __builtin_ctzll(mask);
+            cnt += __builtin_popcountll(mask);
         }
         for (int s = cnt + lane; s < nsample; s += TPK_WAVE)
         {
