@@ -105,7 +105,8 @@ int tpk_ball_query_partial_f32(int64_t size_x, int64_t size_y, float radius, int
  * both -1.  With a `workspace` (tpk_ball_query_sorted_*_workspace_bytes() bytes - 0 for
  * shapes not served that way -, 256-byte aligned) the support points are ordered along a
  * space filling curve and a query only visits cells within its radius (clouds of 512 support
- * points or more; up to 64 neighbours one wavefront serves a query), same results as the all
+ * points or more; up to 64 neighbours one wavefront serves a query; dense layout, clouds of
+ * 1024 .. 8192 points, up to 64 neighbours: buckets of cells in LDS, workspace not used), same results as the all
  * pairs scan used otherwise.  In the packed layout up to 64 neighbours are found by the walk
  * over bins of tpk_ball_query_partial_f32 (no wait for the stream); more than 64 cloud by
  * cloud (clouds of up to 163840 points, cloud ids below 1024; others by all pairs), and only

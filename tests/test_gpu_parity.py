@@ -175,8 +175,8 @@ def test_ball_query_dense_boundary_and_empty(tpk, oracle, dev):
 
 @pytest.mark.parametrize("kind", ["uniform", "clusters", "flat", "one_point", "outlier", "queries_outside", "non_finite", "line",
                                   "offset_3e4", "offset_1e6", "negative"])
-@pytest.mark.parametrize("B,N,M,r,ns", [(2, 512, 100, 0.2, 8), (4, 8192, 300, 0.05, 16), (1, 4096, 1030, 0.1, 100),
-                                        (3, 1500, 17, 0.02, 4), (2, 6000, 64, 0.35, 32)])
+@pytest.mark.parametrize("B,N,M,r,ns", [(2, 1024, 100, 0.2, 8), (4, 8192, 300, 0.05, 16), (1, 4096, 1030, 0.1, 100),
+                                        (3, 1500, 17, 0.02, 4), (2, 6000, 64, 0.35, 32), (2, 3000, 200, 0.15, 64)])
 def test_ball_query_dense_over_cells(tpk, oracle, dev, kind, B, N, M, r, ns):
     # clouds of 512 .. 8192 support points are hung into buckets of cells: shapes of clouds that stress the
     # cells (no extent along an axis, everything in one cell, a far point, queries away from the cloud,
@@ -215,6 +215,11 @@ def test_ball_query_dense_over_cells(tpk, oracle, dev, kind, B, N, M, r, ns):
         xyz, new_xyz = xyz * 3.0 - 2.0, new_xyz * 3.0 - 2.0
     idx, dist = tpk.ball_query(r, ns, xyz.to(dev), new_xyz.contiguous().to(dev), mode="dense")
     want_idx, want_dist = oracle.ball_query_dense(r, ns, xyz.numpy(), new_xyz.numpy())
+    np.testing.assert_array_equal(_np(idx), want_idx)
+    np.testing.assert_array_equal(_np(dist), want_dist)
+    # the nearest first (up to 64 neighbours the same buckets serve this)
+    idx, dist = tpk.ball_query(r, ns, xyz.to(dev), new_xyz.contiguous().to(dev), mode="dense", sort=True)
+    want_idx, want_dist = oracle.ball_query_sorted_dense(r, ns, xyz.numpy(), new_xyz.contiguous().numpy())
     np.testing.assert_array_equal(_np(idx), want_idx)
     np.testing.assert_array_equal(_np(dist), want_dist)
 

@@ -19,7 +19,9 @@
 // the equal range of c in batch_x, found by binary search on the device.  A workgroup
 // owns a block of consecutive queries; where the block straddles clouds it processes one
 // run of equal cloud id at a time.  Nothing is copied to the host.
+#include "ball_cells.h"
 #include "nn_grid.h"
+#include "topk.h"
 
 namespace {
 
@@ -231,6 +233,10 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_dense_kernel(
 // BQC_MAX_CHAIN in all, or whose interval is wider than five cells (coordinates so large that
 // rounding dwarfs the radius) is answered by that scan itself, 64 points per step from global
 // memory with early exit: with so many hits it ends soon.
+// SORTED (the nsample <= 64 NEAREST points inside the radius, nearest first; cpu/src/neighbors.cpp:8-136):
+// the same walk, the hits ranked by (distance, index) instead.  A query with more than 64 hits walks its
+// chains once more and keeps the 64 best (distance, index) keys sorted across the lanes, merging the hits
+// of every step into them; with an interval wider than five cells it does so over all points.
 // ---------------------------------------------------------------------------------------
 constexpr int BQC_THREADS = 1024;
 constexpr int BQC_WAVES = BQC_THREADS / TPK_WAVE;
@@ -265,6 +271,7 @@ __device__ __forceinline__ int bqc_bucket(int i, int j, int k)
     return (i & 15) | ((j & 15) << 4) | ((k & 15) << 8);
 }
 
+template <bool SORTED>
 __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
     int n, int m, int blocks_per_cloud, int queries_per_block, float radius, float radius2, int nsample,
     const float* __restrict__ new_xyz, const float* __restrict__ xyz, int64_t* __restrict__ idx,
@@ -333,7 +340,7 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
 
     // ---- queries: one wavefront each, no workgroup barrier from here on ----
     const int q_end = min(m, (blk + 1) * queries_per_block);
-    if (scan_all)
+    if (!SORTED && scan_all)
     {
         // The scan in index order over the points in LDS, for two of the wavefront's queries at a time: lanes
         // hold 64 consecutive points; a ballot of the radius test and a prefix count give the hits their slots;
@@ -421,22 +428,26 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
             count[a] = static_cast<int>(span < BQC_SPAN + 1 ? span : BQC_SPAN + 1);
         }
         int cnt = 0;
-        bool serial = count[0] > BQC_SPAN || count[1] > BQC_SPAN || count[2] > BQC_SPAN;
+        const bool wide = count[0] > BQC_SPAN || count[1] > BQC_SPAN || count[2] > BQC_SPAN;
+        bool serial = wide;
+        const int cells = count[0] * count[1] * count[2];
+        const int plane = count[0] * count[1];
+        // (lane -> cell by float division: exact for these small numbers)
+        const float inv_plane = 1.0f / static_cast<float>(plane), inv_line = 1.0f / static_cast<float>(count[0]);
+        // first point of the chain of cell c (-1 past the last cell)
+        auto chain_of = [&](int c) __attribute__((always_inline)) {
+            const int k = static_cast<int>((static_cast<float>(c) + 0.5f) * inv_plane);
+            const int rest = c - k * plane;
+            const int jj = static_cast<int>((static_cast<float>(rest) + 0.5f) * inv_line);
+            const int i = rest - jj * count[0];
+            return c < cells ? heads[bqc_bucket(first[0] + i, first[1] + jj, first[2] + k)] : -1;
+        };
         if (!serial)
         {
-            const int cells = count[0] * count[1] * count[2];
-            const int plane = count[0] * count[1];
-            // (lane -> cell by float division: exact for these small numbers)
-            const float inv_plane = 1.0f / static_cast<float>(plane), inv_line = 1.0f / static_cast<float>(count[0]);
             int steps = 0;
             for (int c0 = 0; c0 < cells && !serial; c0 += TPK_WAVE)
             {
-                const int c = c0 + lane;
-                const int k = static_cast<int>((static_cast<float>(c) + 0.5f) * inv_plane);
-                const int rest = c - k * plane;
-                const int jj = static_cast<int>((static_cast<float>(rest) + 0.5f) * inv_line);
-                const int i = rest - jj * count[0];
-                int cur = c < cells ? heads[bqc_bucket(first[0] + i, first[1] + jj, first[2] + k)] : -1;
+                int cur = chain_of(c0 + lane);
                 // all lanes walk their chains in step
                 while (__ballot(cur >= 0) != 0ull)
                 {
@@ -471,20 +482,38 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
         }
         if (!serial)
         {
-            // rank of every hit among the hits (indices are distinct), hits in that order, then the padding
+            // rank of every hit among the hits - by index, SORTED: by (distance, index); the keys are distinct -,
+            // hits in that order, then the padding
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             const int my_row = lane < cnt ? rows[lane] : 0x7fffffff;
             const float my_dist = dists[lane < cnt ? lane : 0];
             int rank = 0, lowest = cnt > 0 ? 0x7fffffff : 0;
-            // (four hits per turn; the lanes past the last hit hold the largest int, which counts for nothing)
-            for (int h = 0; h < cnt; h += 4)
+            // (four hits per turn; the lanes past the last hit hold the largest key, which counts for nothing)
+            if constexpr (SORTED)
+            {
+                const u64 my_key = lane < cnt ? knn_key(my_dist, my_row) : ~0ull;
+                u64 nearest = ~0ull;
+                for (int h = 0; h < cnt; h += 4)
 #pragma unroll
-                for (int g = 0; g < 4; ++g)
-                {
-                    const int other = __builtin_amdgcn_readlane(my_row, h + g);
-                    rank += other < my_row ? 1 : 0;
-                    lowest = min(lowest, other);
-                }
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        const u64 other = read_lane_key(my_key, h + g);
+                        rank += other < my_key ? 1 : 0;
+                        nearest = other < nearest ? other : nearest;
+                    }
+                lowest = cnt > 0 ? static_cast<int>(nearest & 0xFFFFFFFFu) : 0;
+            }
+            else
+            {
+                for (int h = 0; h < cnt; h += 4)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        const int other = __builtin_amdgcn_readlane(my_row, h + g);
+                        rank += other < my_row ? 1 : 0;
+                        lowest = min(lowest, other);
+                    }
+            }
             if (lane < cnt && rank < nsample)
             {
                 idx[out + rank] = my_row;
@@ -497,6 +526,54 @@ __global__ __launch_bounds__(BQC_THREADS) void ball_query_dense_cells_kernel(
             }
             // (the next query's hits overwrite rows / dists: all lanes have read theirs above)
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            continue;
+        }
+
+        if constexpr (SORTED)
+        {
+            // More hits than the buffer holds: lane i keeps the i-th smallest (distance, index) key so far; the
+            // hits of a step that beat the nsample-th are sorted the other way round and merged in.
+            constexpr u64 NONE = ~0ull;
+            u64 best = NONE, admit = NONE;
+            auto offer = [&](bool hit, float d, int row) __attribute__((always_inline)) {
+                u64 cand = hit ? knn_key(d, row) : NONE;
+                cand = cand < admit ? cand : NONE;
+                if (__ballot(cand != NONE) == 0ull)
+                    return;
+                cand = wave_sort_keys(cand, lane, true);
+                best = wave_merge_ascending(best < cand ? best : cand, lane);
+                admit = read_lane_key(best, nsample - 1);
+            };
+            if (wide)
+                for (int base = 0; base < n; base += TPK_WAVE)
+                {
+                    const int pos = base + lane;
+                    const float4 p = points[min(pos, n - 1)];
+                    const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+                    TPK_WORK_ADD(1);
+                    offer(pos < n && d < radius2, d, pos);
+                }
+            else
+                for (int c0 = 0; c0 < cells; c0 += TPK_WAVE)
+                {
+                    int cur = chain_of(c0 + lane);
+                    while (__ballot(cur >= 0) != 0ull)
+                    {
+                        const float4 p = points[max(cur, 0)];
+                        const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
+                        TPK_WORK_ADD(1);
+                        offer(cur >= 0 && d < radius2, d, cur);
+                        cur = cur >= 0 ? __float_as_int(p.w) : -1;
+                    }
+                }
+            const u64 nearest = read_lane_key(best, 0);
+            if (lane < nsample)
+            {
+                const bool found = best != NONE;
+                idx[out + lane] = found ? static_cast<int64_t>(best & 0xFFFFFFFFu)
+                                        : (nearest != NONE ? static_cast<int64_t>(nearest & 0xFFFFFFFFu) : 0);
+                dist[out + lane] = found ? __int_as_float(static_cast<int>(best >> 32)) : -1.0f;
+            }
             continue;
         }
 
@@ -583,6 +660,32 @@ __global__ __launch_bounds__(BQ_THREADS) void ball_query_partial_kernel(
 
 } // namespace
 
+int tpk_cells_ball_query_dense(int b, int n, int m, float radius, float radius2, int nsample, bool sorted,
+                               const float* new_xyz, const float* xyz, int64_t* idx, float* dist, hipStream_t s)
+{
+    if (n < BQC_MIN_POINTS || n > BQC_MAX_POINTS || (sorted && nsample > BQC_HITS))
+        return TPK_ERR_UNSUPPORTED;
+    // one workgroup per compute unit where the queries allow it (every workgroup hangs up its cloud)
+    const int64_t per_cloud = std::max<int64_t>(1, std::min<int64_t>(tpk_ceil_div(m, BQC_WAVES), TPK_COMPUTE_UNITS / b));
+    const int per_block = static_cast<int>(tpk_ceil_div(m, per_cloud));
+    const int64_t bpc = tpk_ceil_div(m, per_block);
+    if (bpc * b > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    const size_t lds = bqc_lds_bytes(n);
+    const void* kernel = sorted ? reinterpret_cast<const void*>(&ball_query_dense_cells_kernel<true>)
+                                : reinterpret_cast<const void*>(&ball_query_dense_cells_kernel<false>);
+    const int st = tpk_allow_lds(kernel, lds);
+    if (st != TPK_OK)
+        return st;
+    if (sorted)
+        hipLaunchKernelGGL(ball_query_dense_cells_kernel<true>, dim3(static_cast<unsigned>(bpc * b)), dim3(BQC_THREADS), lds, s,
+                           n, m, static_cast<int>(bpc), per_block, radius, radius2, nsample, new_xyz, xyz, idx, dist);
+    else
+        hipLaunchKernelGGL(ball_query_dense_cells_kernel<false>, dim3(static_cast<unsigned>(bpc * b)), dim3(BQC_THREADS), lds, s,
+                           n, m, static_cast<int>(bpc), per_block, radius, radius2, nsample, new_xyz, xyz, idx, dist);
+    return tpk_launch_status();
+}
+
 extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int nsample,
                                         const float* new_xyz, const float* xyz, int64_t* idx,
                                         float* dist, void* stream)
@@ -602,20 +705,10 @@ extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int n
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     const float radius2 = radius * radius; // fp32 product, as the reference kernel forms it
-    if (n >= BQC_MIN_POINTS && n <= BQC_MAX_POINTS)
     {
-        // over cells; one workgroup per compute unit where the queries allow it (every workgroup bins its cloud)
-        const int64_t per_cloud = std::max<int64_t>(1, std::min<int64_t>(tpk_ceil_div(m, BQC_WAVES), TPK_COMPUTE_UNITS / b));
-        const int per_block = static_cast<int>(tpk_ceil_div(m, per_cloud));
-        const int64_t cell_bpc = tpk_ceil_div(m, per_block);
-        const size_t lds = bqc_lds_bytes(n);
-        const int st = tpk_allow_lds(reinterpret_cast<const void*>(&ball_query_dense_cells_kernel), lds);
-        if (st != TPK_OK)
+        const int st = tpk_cells_ball_query_dense(b, n, m, radius, radius2, nsample, false, new_xyz, xyz, idx, dist, tpk_stream(stream));
+        if (st != TPK_ERR_UNSUPPORTED)
             return st;
-        hipLaunchKernelGGL(ball_query_dense_cells_kernel, dim3(static_cast<unsigned>(cell_bpc * b)), dim3(BQC_THREADS), lds,
-                           tpk_stream(stream), n, m, static_cast<int>(cell_bpc), per_block, radius, radius2, nsample, new_xyz,
-                           xyz, idx, dist);
-        return tpk_launch_status();
     }
     if (few)
         hipLaunchKernelGGL(ball_query_dense_kernel<BQ_Q_FEW>, dim3(static_cast<unsigned>(blocks)), dim3(BQ_THREADS), 0,

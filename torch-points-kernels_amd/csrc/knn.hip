@@ -12,6 +12,7 @@
 // (nn_grid.hip).  Otherwise all pairs are tested: one lane owns one query and keeps its list in
 // registers (topk.h); the support points of the cloud stream through LDS in tiles of float4, read
 // by all lanes at the same address.  k above 32 is served in rounds of 32 entries.
+#include "ball_cells.h"
 #include "nn_grid.h"
 #include "topk.h"
 
@@ -357,6 +358,12 @@ extern "C" int tpk_ball_query_sorted_dense_f32(int b, int n, int m, float radius
         return TPK_ERR_UNSUPPORTED;
     hipStream_t s = tpk_stream(stream);
     const float limit = radius * radius; // fp32 product (cpu/src/neighbors.cpp:19)
+    {
+        // clouds that fit in LDS, up to 64 neighbours: buckets of cells built by every workgroup, no workspace
+        const int cells = tpk_cells_ball_query_dense(b, n, m, radius, limit, nsample, true, new_xyz, xyz, idx, dist, s);
+        if (cells != TPK_ERR_UNSUPPORTED)
+            return cells; // (padding included)
+    }
     if (workspace)
     {
         const int direct = tpk_grid_ball_sorted(b, m, n, nsample, limit, false, 0, new_xyz, xyz, dist, idx, workspace,

@@ -719,44 +719,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void knn_grid_kernel(
     }
 }
 
-using u64 = unsigned long long;
 constexpr int NG_RUN = 16; // consecutive cells that share a second-level box in the wavefront-per-query search
-
-// The 64 keys of a wavefront sorted across its lanes (bitonic network; lane i ends with the i-th
-// smallest, or the i-th largest when `descending`).
-__device__ __forceinline__ u64 wave_sort_keys(u64 key, int lane, bool descending)
-{
-#pragma unroll
-    for (int k = 2; k <= TPK_WAVE; k <<= 1)
-#pragma unroll
-        for (int j = k >> 1; j > 0; j >>= 1)
-        {
-            const u64 other = __shfl_xor(key, j, TPK_WAVE);
-            const bool up = ((lane & k) == 0) != descending;
-            const bool keep_min = ((lane & j) == 0) == up;
-            key = (keep_min == (key < other)) ? key : other;
-        }
-    return key;
-}
-
-// A bitonic sequence across the lanes put into ascending order.
-__device__ __forceinline__ u64 wave_merge_ascending(u64 key, int lane)
-{
-#pragma unroll
-    for (int j = TPK_WAVE / 2; j > 0; j >>= 1)
-    {
-        const u64 other = __shfl_xor(key, j, TPK_WAVE);
-        key = (((lane & j) == 0) == (key < other)) ? key : other;
-    }
-    return key;
-}
-
-__device__ __forceinline__ u64 read_lane_key(u64 key, int from)
-{
-    const unsigned lo = __builtin_amdgcn_readlane(static_cast<int>(key & 0xFFFFFFFFu), from);
-    const unsigned hi = __builtin_amdgcn_readlane(static_cast<int>(key >> 32), from);
-    return (static_cast<u64>(hi) << 32) | lo;
-}
 
 // ---------------------------------------------------------------------------------------
 // Ball query over bins, packed layout (several clouds back to back, sorted cloud id per point).
