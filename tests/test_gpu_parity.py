@@ -587,6 +587,56 @@ def test_three_nn_cell_search_ties(tpk, oracle, dev):
         np.testing.assert_array_equal(_np(dist2), wd)
 
 
+@pytest.mark.parametrize("kind", ["uniform", "clusters", "flat", "one_point", "outlier", "queries_outside", "non_finite", "line",
+                                  "lattice", "tripled", "offset_1e5", "two_points"])
+@pytest.mark.parametrize("B,n,m", [(2, 700, 1024), (1, 5000, 4096), (3, 300, 8192), (300, 40, 1500), (1, 2100, 3000)])
+def test_three_nn_grid_in_lds(tpk, oracle, dev, kind, B, n, m):
+    # known clouds of 1024 .. 8192 points are sorted into the cells of a grid in LDS, one lane per query: clouds
+    # that stress the grid and the widening of the examined block (no extent along an axis, everything in one
+    # cell, a far point that makes all cells wide, queries far from the cloud, coordinates that are not finite)
+    # and equal distances in every triple (lattices, tripled points), against the scan in index order
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    g = torch.Generator().manual_seed(11 * n + m)
+    known = torch.rand(B, m, 3, generator=g)
+    unknown = torch.rand(B, n, 3, generator=g)
+    if kind == "clusters":
+        centres = torch.rand(B, 4, 3, generator=g)
+        known = centres[:, torch.randint(0, 4, (m,), generator=g)] + 0.004 * torch.randn(B, m, 3, generator=g)
+    elif kind == "flat":
+        known[..., 2] = 0.25
+    elif kind == "one_point":
+        known[:] = 0.5
+    elif kind == "outlier":
+        known[:, m // 3] = torch.tensor([400.0, -300.0, 1e6])
+    elif kind == "queries_outside":
+        unknown[:, ::3] += 5.0
+        unknown[:, 1::3, 1] = -40.0
+    elif kind == "non_finite":
+        known[:, 5, 0] = float("nan")
+        known[:, 77, 1] = float("inf")
+        known[:, 300, 2] = -float("inf")
+        unknown[:, 3, 1] = float("nan")
+        unknown[:, 4, 2] = float("inf")
+    elif kind == "line":
+        known[..., 1:] = 0.0
+    elif kind == "lattice":
+        known = torch.round(known * 12) / 4
+        unknown = torch.round(unknown * 12) / 4 + 0.125
+    elif kind == "tripled":
+        k = known[:, : m // 3]
+        known = torch.cat([k, k.flip(1), k, known[:, : m - 3 * (m // 3)]], 1)[:, torch.randperm(m, generator=g)]
+    elif kind == "offset_1e5":
+        known, unknown = known + 1e5, unknown + 1e5
+    elif kind == "two_points":
+        known[:, ::2] = 0.25
+        known[:, 1::2] = 0.75
+    unknown, known = unknown.contiguous(), known.contiguous()
+    dist2, idx = native.three_nn(unknown.to(dev), known.to(dev))
+    wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist2), wd)
+
+
 def test_three_nn_ties(tpk, oracle, dev):
     # duplicated known points: equal distances must keep the lower index first
     g = torch.Generator().manual_seed(3)
