@@ -69,11 +69,13 @@ def test_library_exports_every_declared_symbol():
         # (the Chamfer search also keeps the cells of every window in the order it hands them out: 4 bytes per cell)
         order = ((11, 4), (15, 4)) if "chamfer" in name else ()
         want = sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((11, 1024), (15, 1024), (11, 160), (15, 160)) + order)
-        assert fn(2, 700, 900) == want
+        # (three_nn: one word per cloud at the end, for the clouds that a kernel in front has not answered)
+        flags = 256 if "three_nn" in name else 0
+        assert fn(2, 700, 900) == want + flags
         # clouds above 16384 points: whole windows of 16384 points (256 cells each)
         order = ((512, 4), (15, 4)) if "chamfer" in name else ()
         want = sum(-(-2 * c * nbytes // 256) * 256 for c, nbytes in ((512, 1024), (15, 1024), (512, 160), (15, 160)) + order)
-        assert fn(2, 20000, 900) == want
+        assert fn(2, 20000, 900) == want + flags
     up = lambda v: -(-v // 256) * 256
     # sorted ball query (b, support points, queries): only the support points are ordered when one wavefront serves a
     # query (up to 64 neighbours); the size also covers the k-nearest lists that serve more neighbours

@@ -635,6 +635,21 @@ def test_three_nn_grid_in_lds(tpk, oracle, dev, kind, B, n, m):
     wd, wi = oracle.three_nn(unknown.numpy(), known.numpy())
     np.testing.assert_array_equal(_np(idx), wi)
     np.testing.assert_array_equal(_np(dist2), wd)
+    # without a workspace the grid has nothing to hand uneven clouds over to and answers them itself
+    import ctypes
+    import os
+
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "torch-points-kernels_amd",
+                                   "torch_points_kernels", "libtpk_hip.so"))
+    u, k = unknown.to(dev), known.to(dev)
+    dist2.fill_(-1.0)
+    idx.fill_(-1)
+    st = lib.tpk_three_nn_f32(B, n, m, ctypes.c_void_p(u.data_ptr()), ctypes.c_void_p(k.data_ptr()),
+                              ctypes.c_void_p(dist2.data_ptr()), ctypes.c_void_p(idx.data_ptr()), None, ctypes.c_size_t(0),
+                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist2), wd)
 
 
 def test_three_nn_ties(tpk, oracle, dev):

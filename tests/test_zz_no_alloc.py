@@ -18,10 +18,16 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
-def _three_nn_both_ways(lib, dev, b, n, m, seed):
+def _three_nn_both_ways(lib, dev, b, n, m, seed, clustered=False):
     g = torch.Generator().manual_seed(seed)
     unknown = torch.rand(b, n, 3, generator=g).to(dev)
-    known = torch.rand(b, m, 3, generator=g).to(dev)
+    known = torch.rand(b, m, 3, generator=g)
+    if clustered:
+        # uneven density: the grid in LDS gives such clouds up, and the search over curve-ordered cells, whose
+        # ordered copies and boxes fill the scratch array, answers them
+        centres = torch.rand(b, 4, 3, generator=g)
+        known = centres[:, torch.randint(0, 4, (m,), generator=g)] + 0.002 * torch.randn(b, m, 3, generator=g)
+    known = known.contiguous().to(dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     # the existing entry point, with a workspace the caller allocates
     ws_bytes = lib.tpk_three_nn_workspace_bytes(b, n, m)
@@ -53,6 +59,8 @@ def test_three_nn_without_allocation(dev):
     assert capacity == 8 << 20
     # first a problem that fills most of the array, then a smaller one that reuses its front part
     used = _three_nn_both_ways(lib, dev, 16, 16384, 4096, seed=21)
+    assert 0 < used <= capacity
+    used = _three_nn_both_ways(lib, dev, 16, 16384, 4096, seed=24, clustered=True)
     assert 0 < used <= capacity
     used = _three_nn_both_ways(lib, dev, 3, 1500, 700, seed=22)
     assert 0 < used <= capacity

@@ -31,6 +31,7 @@ struct PointSet
     float4* grid;         // optional [windows][2]: origin and scale of the window's 64^3 grid
     int* wide_first;      // optional (with boxes) [windows][cells]: the window's cells, those with much wider boxes than
                           // the window's average first - the cells whose queries take a search longest
+    const int* only;      // optional [clouds]: a cloud whose word is 0 is left out (dense layout)
 };
 
 __host__ __device__ inline int set_cells(const PointSet& s)
@@ -159,6 +160,8 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
     if (zero_word && blockIdx.x == 0 && tid == 0)
         *zero_word = 0;
+    if (set.only && set.only[window / per_cloud] == 0)
+        return; // (before the first barrier)
 
     // the points of this thread: tid, tid + 1024, ... (all loads issued before the first is used)
     float p[PER][3];

@@ -14,10 +14,13 @@ int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xy
                          float* dist2, int32_t* idx1, int32_t* idx2, void* workspace,
                          size_t workspace_bytes, hipStream_t stream);
 
-// three_nn, float32: same conventions.
+// three_nn, float32: same conventions.  The workspace ends with one word per cloud
+// (tpk_grid_three_nn_flags: its address, or nullptr when the workspace does not serve the shape); with
+// `flagged` only the clouds whose word is not 0 are searched - a kernel enqueued before has answered the others.
 size_t tpk_grid_three_nn_workspace_bytes(int b, int n, int m);
+int* tpk_grid_three_nn_flags(int b, int n, int m, void* workspace, size_t workspace_bytes);
 int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2,
-                      int32_t* idx, void* workspace, size_t workspace_bytes, hipStream_t stream);
+                      int32_t* idx, void* workspace, size_t workspace_bytes, bool flagged, hipStream_t stream);
 
 // k nearest neighbours, float32 (n queries, m support points per cloud; idx int64, both outputs
 // (b, n, k), ascending by (squared distance, index)): same conventions.  Only support points with

@@ -454,7 +454,7 @@ __device__ __forceinline__ void scan_cell3_few(const float4* __restrict__ cand, 
 __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     int n, int m, int qcells, int ccells, int clouds, const float4* __restrict__ sorted_unknown,
     const float4* __restrict__ sorted_known, const float4* __restrict__ boxes_known, float* __restrict__ dist2,
-    int32_t* __restrict__ idx)
+    int32_t* __restrict__ idx, const int* __restrict__ only)
 {
     __shared__ float4 stages[NG_SCAN_THREADS / TPK_WAVE][NG_CELL];
     extern __shared__ float lows_all[]; // [wavefronts][candidate cells, in whole groups of 64]
@@ -466,6 +466,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void three_nn_grid_kernel(
     if (task >= static_cast<int64_t>(qcells) * clouds)
         return; // (no workgroup barrier anywhere in this kernel)
     const int cloud = static_cast<int>(task / qcells);
+    if (only && only[cloud] == 0)
+        return; // (a cloud that another kernel has answered)
     const int qcell = static_cast<int>(task - static_cast<int64_t>(cloud) * qcells);
     const float4* __restrict__ qpts = sorted_unknown + static_cast<int64_t>(cloud) * qcells * NG_CELL;
     const float4* __restrict__ cpts = sorted_known + static_cast<int64_t>(cloud) * ccells * NG_CELL;
@@ -1082,25 +1084,35 @@ int tpk_grid_chamfer_fwd(int b, int n, int m, const float* xyz1, const float* xy
     return tpk_launch_status();
 }
 
+// (behind the ordered copies and boxes: one word per cloud, see tpk_grid_three_nn_flags)
 size_t tpk_grid_three_nn_workspace_bytes(int b, int n, int m)
 {
-    return grid_supported(b, n, m) ? grid_layout(b, n, m).total : 0;
+    return grid_supported(b, n, m) ? grid_layout(b, n, m).total + ((static_cast<size_t>(b) * sizeof(int) + 255) & ~static_cast<size_t>(255)) : 0;
+}
+
+int* tpk_grid_three_nn_flags(int b, int n, int m, void* workspace, size_t workspace_bytes)
+{
+    const size_t need = tpk_grid_three_nn_workspace_bytes(b, n, m);
+    if (!need || !workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return nullptr;
+    return reinterpret_cast<int*>(static_cast<char*>(workspace) + grid_layout(b, n, m).total);
 }
 
 int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2,
-                      int32_t* idx, void* workspace, size_t workspace_bytes, hipStream_t s)
+                      int32_t* idx, void* workspace, size_t workspace_bytes, bool flagged, hipStream_t s)
 {
     if (!grid_supported(b, n, m) || static_cast<int64_t>(b) * 2 > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     const GridLayout l = grid_layout(b, n, m);
-    if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    if (!workspace || workspace_bytes < tpk_grid_three_nn_workspace_bytes(b, n, m) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
+    const int* only = flagged ? reinterpret_cast<const int*>(w + l.total) : nullptr;
     // (the unknown points are only queried: no boxes of their cells - the search forms the box of its 64 queries)
     PointSet a{unknown, nullptr, static_cast<int64_t>(b) * n, n, grid_stride(n), reinterpret_cast<float4*>(w + l.sorted_a),
-               nullptr, nullptr, nullptr};
+               nullptr, nullptr, nullptr, nullptr, only};
     PointSet c{known, nullptr, static_cast<int64_t>(b) * m, m, grid_stride(m), reinterpret_cast<float4*>(w + l.sorted_b),
-               reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr};
+               reinterpret_cast<float4*>(w + l.boxes_b), nullptr, nullptr, nullptr, only};
     int st = launch_curve_cells(a, c, nullptr, s);
     if (st != TPK_OK)
         return st;
@@ -1112,7 +1124,7 @@ int tpk_grid_three_nn(int b, int n, int m, const float* unknown, const float* kn
     const size_t lds = static_cast<size_t>(NG_SCAN_THREADS / TPK_WAVE) * ((ccells + NG_CELL - 1) / NG_CELL * NG_CELL) *
                        sizeof(float);
     hipLaunchKernelGGL(three_nn_grid_kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), lds, s, n,
-                       m, qcells, ccells, b, a.sorted, c.sorted, c.boxes, dist2, idx);
+                       m, qcells, ccells, b, a.sorted, c.sorted, c.boxes, dist2, idx, only);
     return tpk_launch_status();
 }
 

@@ -159,9 +159,10 @@ constexpr int TNC_WAVES = TNC_THREADS / TPK_WAVE;
 constexpr int TNC_MIN_KNOWN = 1024;
 constexpr int TNC_MAX_KNOWN = 8192;
 constexpr int TNC_PER_THREAD = TNC_MAX_KNOWN / TNC_THREADS;
-constexpr int TNC_GRID = 16;
-constexpr int TNC_CELLS = TNC_GRID * TNC_GRID * TNC_GRID;
+constexpr int TNC_AXIS = 64;    // cells per axis at most
+constexpr int TNC_CELLS = 4096; // cells in all at most
 constexpr int TNC_STARTS = TNC_CELLS + TPK_WAVE; // the cells' first places, one more for the end, padded
+constexpr float TNC_CROWDED = 12.0f; // points per cell, as a point sees them, from which the grid is given up
 constexpr float TNC_PER_CELL = 2.0f;             // points per cell aimed at (1 / 1.5 / 3: 9 / 6 / 1 % slower)
 
 size_t tnc_lds_bytes(int m)
@@ -216,7 +217,7 @@ struct Best3
 
 __global__ __launch_bounds__(TNC_THREADS) void three_nn_cells_kernel(
     int n, int m, int blocks_per_cloud, int queries_per_block, const float* __restrict__ unknown,
-    const float* __restrict__ known, float* __restrict__ dist2, int32_t* __restrict__ idx)
+    const float* __restrict__ known, float* __restrict__ dist2, int32_t* __restrict__ idx, int* __restrict__ general)
 {
     extern __shared__ __align__(16) unsigned char tnc_lds[];
     float* const sx = reinterpret_cast<float*>(tnc_lds); // [m] each: the known points cell by cell
@@ -291,7 +292,8 @@ __global__ __launch_bounds__(TNC_THREADS) void three_nn_cells_kernel(
     }
     __syncthreads();
 
-    // ---- the grid: about TNC_PER_CELL points per cell, cells as cubic as 16 per axis allow ----
+    // ---- the grid: about TNC_PER_CELL points per cell, cells as cubic as TNC_AXIS per axis and TNC_CELLS in
+    // all allow (a flat cloud gets a flat grid of up to 64 x 64 cells) ----
     float lo[3], inv[3], width[3];
     int cells[3];
     {
@@ -304,18 +306,34 @@ __global__ __launch_bounds__(TNC_THREADS) void three_nn_cells_kernel(
             extent[a] = extent[a] > 0.0f ? extent[a] : 0.0f;
             longest = fmaxf(longest, extent[a]);
         }
-        // (an axis without extent counts as a thousandth of the longest: a flat cloud gets a flat grid)
-        float volume = 1.0f;
+        // cells per axis for `along` cells along the longest axis, and their product
+        auto fit = [&](float along, int (&count)[3]) __attribute__((always_inline)) {
+            int all = 1;
 #pragma unroll
-        for (int a = 0; a < 3; ++a)
-            volume *= fmaxf(extent[a], 1e-3f * longest) / fmaxf(longest, 1e-30f);
-        const float wanted = fminf(static_cast<float>(TNC_CELLS), static_cast<float>(m) / TNC_PER_CELL);
-        const float per_unit = cbrtf(wanted / volume); // cells along an axis as long as the longest
+            for (int a = 0; a < 3; ++a)
+            {
+                const float f = longest > 0.0f ? fminf(extent[a] / longest * along + 0.5f, static_cast<float>(TNC_AXIS)) : 1.0f;
+                count[a] = f >= 1.0f ? static_cast<int>(f) : 1;
+                all *= count[a];
+            }
+            return all;
+        };
+        // (the product grows with `along`: the largest value that stays within the cells wanted, by bisection)
+        const int wanted = static_cast<int>(fminf(static_cast<float>(TNC_CELLS), fmaxf(static_cast<float>(m) / TNC_PER_CELL, 1.0f)));
+        float few = 0.0f, many = 2.0f * TNC_AXIS;
+        for (int step = 0; step < 12; ++step)
+        {
+            const float mid = 0.5f * (few + many);
+            int count[3];
+            if (fit(mid, count) > wanted)
+                many = mid;
+            else
+                few = mid;
+        }
+        fit(few, cells);
 #pragma unroll
         for (int a = 0; a < 3; ++a)
         {
-            const float fit = longest > 0.0f ? fminf(extent[a] / longest * per_unit + 0.5f, static_cast<float>(TNC_GRID)) : 1.0f;
-            cells[a] = fit >= 1.0f ? static_cast<int>(fit) : 1;
             inv[a] = extent[a] > 0.0f ? static_cast<float>(cells[a]) / extent[a] : 0.0f;
             width[a] = extent[a] / static_cast<float>(cells[a]);
             lo[a] = extent[a] > 0.0f ? lo[a] : 0.0f;
@@ -369,8 +387,21 @@ __global__ __launch_bounds__(TNC_THREADS) void three_nn_cells_kernel(
             si[at] = tid + u * TNC_THREADS;
         }
     __syncthreads();
-    // (points per cell as a point sees them; 40 of them cost a lane what the whole cloud costs by broadcast reads)
-    const bool crowded = static_cast<float>(crowding) * 40.0f > static_cast<float>(m) * static_cast<float>(m);
+    // Points per cell as a point sees them (3 in a cloud of even density): above TNC_CROWDED the grid is a poor
+    // fit - dense cells cost their queries many candidates, empty ones many steps of widening - and, where the
+    // caller enqueues it behind this kernel, the search over curve-ordered cells answers the cloud instead.
+    // Without it: on with the grid; when 40 points cost a lane what the whole cloud costs by broadcast reads,
+    // every lane scans the cloud.
+    const float crowd = static_cast<float>(crowding) / static_cast<float>(m);
+    if (general)
+    {
+        const bool hand_over = crowd > TNC_CROWDED;
+        if (blk == 0 && tid == 0)
+            general[cloud] = hand_over ? 1 : 0;
+        if (hand_over)
+            return;
+    }
+    const bool crowded = crowd * 40.0f > static_cast<float>(m);
 
     // ---- queries: one lane each, no workgroup barrier from here on ----
     const int q_end = min(n, (blk + 1) * queries_per_block);
@@ -398,7 +429,7 @@ __global__ __launch_bounds__(TNC_THREADS) void three_nn_cells_kernel(
                 t[a] = (q[a] - lo[a]) * inv[a];
                 c[a] = tnc_cell(t[a], cells[a]);
                 // (what rounding may have moved a point's cell by, in cell widths)
-                slack[a] = 1e-5f * (fabsf(t[a]) + static_cast<float>(TNC_GRID));
+                slack[a] = 1e-5f * (fabsf(t[a]) + static_cast<float>(TNC_AXIS));
             }
             // Distance along axis a, in cell widths, from the query to cell k (0 for its own cell), a lower bound.
             auto to_cell = [&](int a, int k) __attribute__((always_inline)) {
@@ -513,7 +544,7 @@ __global__ __launch_bounds__(TNC_THREADS) void three_nn_cells_kernel(
 }
 
 int launch_three_nn_cells(int b, int n, int m, const float* unknown, const float* known, float* dist2, int32_t* idx,
-                          hipStream_t stream)
+                          int* general, hipStream_t stream)
 {
     // one workgroup per compute unit where the queries allow it (every workgroup sorts its cloud)
     const int64_t per_cloud = std::max<int64_t>(1, std::min<int64_t>(tpk_ceil_div(n, TNC_THREADS), TPK_COMPUTE_UNITS / b));
@@ -526,7 +557,7 @@ int launch_three_nn_cells(int b, int n, int m, const float* unknown, const float
     if (st != TPK_OK)
         return st;
     hipLaunchKernelGGL(three_nn_cells_kernel, dim3(static_cast<unsigned>(bpc * b)), dim3(TNC_THREADS), lds, stream, n, m,
-                       static_cast<int>(bpc), per_block, unknown, known, dist2, idx);
+                       static_cast<int>(bpc), per_block, unknown, known, dist2, idx, general);
     return tpk_launch_status();
 }
 
@@ -550,14 +581,20 @@ extern "C" int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const
     if (static_cast<int64_t>(n) * 3 > 0x7fffffffLL || static_cast<int64_t>(m) * 3 > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     hipStream_t s = tpk_stream(stream);
-#ifndef TNC_OFF
     if (m >= TNC_MIN_KNOWN && m <= TNC_MAX_KNOWN)
-        return launch_three_nn_cells(b, n, m, unknown, known, dist2, idx, s); // (the known cloud fits in LDS)
-#endif
+    {
+        // The known cloud fits in LDS: a grid there, one lane per query.  It notes the clouds it gives up (uneven
+        // density) in the workspace, and the search over curve-ordered cells, enqueued behind it, answers those.
+        int* const general = tpk_grid_three_nn_flags(b, n, m, workspace, workspace_bytes);
+        const int st = launch_three_nn_cells(b, n, m, unknown, known, dist2, idx, general, s);
+        if (st != TPK_OK || !general)
+            return st;
+        return tpk_grid_three_nn(b, n, m, unknown, known, dist2, idx, workspace, workspace_bytes, true, s);
+    }
     if (workspace)
     {
         // Search over curve-ordered cells where it applies; otherwise all pairs.
-        const int st = tpk_grid_three_nn(b, n, m, unknown, known, dist2, idx, workspace, workspace_bytes, s);
+        const int st = tpk_grid_three_nn(b, n, m, unknown, known, dist2, idx, workspace, workspace_bytes, false, s);
         if (st != TPK_ERR_UNSUPPORTED)
             return st;
     }
