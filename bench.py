@@ -48,7 +48,7 @@ VALU_KERNELS = {
     "fps": "fps_pruned_kernel<16, 1024, 4>",
     "ball_query_dense": "ball_query_dense_cells_kernel",
     "ball_query_partial_dense": "ball_query_bins_kernel",
-    "three_nn": "three_nn_grid_kernel",
+    "three_nn": "three_nn_cells_kernel",
     "chamfer_fwd": "chamfer_grid_kernel",
 }
 
@@ -228,7 +228,8 @@ def _all_pairs_entry(call, pairs, steps, warmup, valu_kernel):
         roof["valu"] = {"valu_busy_pct": table[valu_kernel].get("VALUBusy"),
                         "valu_lane_utilisation_pct": table[valu_kernel].get("VALUUtilization"),
                         "source": "profiles/" + os.path.basename(VALU_FILE), "measured_at_commit": commit}
-    return {"what": "the same configuration through the C ABI with workspace == NULL: every query scans its whole cloud "
+    return {"what": "the same configuration through the C ABI's scan of all pairs (workspace == NULL; three_nn: "
+                    "tpk_three_nn_all_pairs_f32): every query scans its whole cloud "
                     "(the kernel the north star describes); same results", "kernel_ms": ev, "wall_ms": wall, "roofline": roof}
 
 
@@ -430,10 +431,12 @@ def bench_others(dev, steps, warmup, with_cpu):
     e = {"workload": "configs[2]a: three_nn unknown (16,16384,3) known (16,4096,3)", "metric": "queries/s",
          "value": nq / (wall * 1e-3), "kernel_ms": ev, "wall_ms": wall,
          "roofline": _roof_flops(executed, pairs, 8, ev, "three_nn"), "pairs": pairs}
-    e["roofline"]["note"] += PRUNED_NOTE
-    e["all_pairs_kernel"] = _all_pairs_entry(lambda lib, st: lib.tpk_three_nn_f32(
-        unknown.shape[0], unknown.shape[1], known.shape[1], _p(unknown), _p(known), _p(nn_d), _p(nn_i), None,
-        ctypes.c_size_t(0), st), pairs, max(3, steps // 4), 1, "three_nn_kernel<4>")
+    e["roofline"]["note"] += ("; every workgroup sorts its known cloud into a grid in LDS and a query looks at the cells "
+                              "around it only; kernel_ms also covers the two launches behind it that would answer clouds "
+                              "of uneven density (here they return at once)")
+    e["all_pairs_kernel"] = _all_pairs_entry(lambda lib, st: lib.tpk_three_nn_all_pairs_f32(
+        unknown.shape[0], unknown.shape[1], known.shape[1], _p(unknown), _p(known), _p(nn_d), _p(nn_i), st),
+        pairs, max(3, steps // 4), 1, "three_nn_kernel<4>")
     if ref is not None:
         sub = 4  # clouds
         secs = _cpu_time(lambda: ref.dense_knn(w["known"][:sub], w["unknown"][:sub], 3))

@@ -130,22 +130,29 @@ int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y, float radi
  *   dist2 (b, n, 3) float32 squared distances, ascending   idx (b, n, 3) int32
  * Equal distances keep the lower index first; with m < 3 the missing entries are
  * (+inf, 0).
- * With a `workspace` (tpk_three_nn_workspace_bytes() bytes - 0 for shapes not served that way -,
- * 256-byte aligned, contents arbitrary before and after) both clouds are ordered along a space
- * filling curve and only nearby cells are searched; with workspace == NULL all pairs are tested
- * (same results, slower).
+ * Known clouds of 1024 .. 8192 points are sorted into a grid that every workgroup builds in its
+ * local memory, and a query looks at the cells around it only.  With a `workspace`
+ * (tpk_three_nn_workspace_bytes() bytes - 0 for shapes not served that way -, 256-byte aligned,
+ * contents arbitrary before and after) other shapes, and clouds whose density is too uneven for
+ * that grid, are ordered along a space filling curve and only nearby cells are searched; with
+ * workspace == NULL the grid answers uneven clouds as well (slower there), and for other shapes
+ * all pairs are tested.  Same results every way.
+ * tpk_three_nn_all_pairs_f32: the scan of all pairs itself, for any shape (what the reference
+ * kernel does; here for measurements and as a check).
  * ------------------------------------------------------------------------------------- */
 size_t tpk_three_nn_workspace_bytes(int b, int n, int m);
 int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const float* known,
                      float* dist2, int32_t* idx, void* workspace, size_t workspace_bytes,
                      void* stream);
+int tpk_three_nn_all_pairs_f32(int b, int n, int m, const float* unknown, const float* known,
+                               float* dist2, int32_t* idx, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Three nearest neighbours without any allocation.
  * No counterpart in the reference.  It is for callers that cannot allocate device memory (not
  * even a workspace to pass in): code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc.  Same arguments and results as tpk_three_nn_f32 with a workspace, but
- * the curve-ordered copies of both clouds live in an array of
+ * the workspace (curve-ordered copies of both clouds, a word per cloud) is an array of
  * TPK_THREE_NN_STATIC_SCRATCH_BYTES bytes of device memory that is part of the library (every GPU
  * the library runs on holds one until the process ends).  The call allocates and frees nothing.
  * Shapes whose workspace (tpk_three_nn_workspace_bytes()) exceeds the array are rejected with

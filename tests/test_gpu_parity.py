@@ -1315,6 +1315,17 @@ def test_c_abi_direct_call(oracle, dev):
         stream.synchronize()
         np.testing.assert_array_equal(_np(idx), wi)
         np.testing.assert_array_equal(_np(dist2), wd)
+    # the scan of all pairs by name
+    dist2.fill_(-1.0)
+    idx.fill_(-1)
+    stream.wait_stream(torch.cuda.current_stream())
+    st = lib.tpk_three_nn_all_pairs_f32(2, 700, 900, ctypes.c_void_p(u.data_ptr()), ctypes.c_void_p(k.data_ptr()),
+                                        ctypes.c_void_p(dist2.data_ptr()), ctypes.c_void_p(idx.data_ptr()),
+                                        ctypes.c_void_p(stream.cuda_stream))
+    assert st == 0
+    stream.synchronize()
+    np.testing.assert_array_equal(_np(idx), wi)
+    np.testing.assert_array_equal(_np(dist2), wd)
     # a workspace that is too small is refused before any launch
     st = lib.tpk_three_nn_f32(2, 700, 900, ctypes.c_void_p(u.data_ptr()), ctypes.c_void_p(k.data_ptr()),
                               ctypes.c_void_p(dist2.data_ptr()), ctypes.c_void_p(idx.data_ptr()),

@@ -598,6 +598,21 @@ extern "C" int tpk_three_nn_f32(int b, int n, int m, const float* unknown, const
         if (st != TPK_ERR_UNSUPPORTED)
             return st;
     }
+    return tpk_three_nn_all_pairs_f32(b, n, m, unknown, known, dist2, idx, stream);
+}
+
+extern "C" int tpk_three_nn_all_pairs_f32(int b, int n, int m, const float* unknown, const float* known,
+                                          float* dist2, int32_t* idx, void* stream)
+{
+    if (b < 0 || n < 0 || m < 0)
+        return TPK_ERR_INVALID_ARG;
+    if (b == 0 || n == 0)
+        return TPK_OK;
+    if (!unknown || !dist2 || !idx || (m > 0 && !known))
+        return TPK_ERR_INVALID_ARG;
+    if (static_cast<int64_t>(n) * 3 > 0x7fffffffLL || static_cast<int64_t>(m) * 3 > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    hipStream_t s = tpk_stream(stream);
     // Queries per lane: as many as still leave a few workgroups per compute unit.
     const int64_t queries = static_cast<int64_t>(b) * n;
     if (queries >= 4LL * NN_THREADS * 2048)
