@@ -341,7 +341,7 @@ __device__ __forceinline__ int sorted_position(int g, int wave, int e, int lane)
     return ((g * WAVES + wave) * GS + e) * TPK_WAVE + lane;
 }
 
-template <int PPT, int THREADS, int GS>
+template <int PPT, int THREADS, int GS, bool BATCHED>
 __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     int n, int npoint, int log2_bs, int ref_groups, int key_capacity,
     const float* __restrict__ xyz, int32_t* __restrict__ out)
@@ -452,6 +452,278 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         out[0] = 0;
     TPK_WORK_DECL
 
+    if constexpr (BATCHED)
+    {
+        // Several samples per round.  After a round's updates let c0 > c1 > c2 ... be the points in the order of
+        // their running minima.  c0 is the next sample.  If c1's minimum is not changed by c0 (c0 is no closer
+        // to it than its minimum), then after c0's update c1 still holds what it held, nothing holds more, and
+        // c1 is the sample after c0 - and so on: ck follows as long as none of c0 .. c(k-1) changes its minimum.
+        // Late in a sampling the largest minima sit in different corners of the cloud, far from each other, and
+        // nearly every round takes the FPB_T samples it may.  Every wavefront publishes its two best points and
+        // the largest minimum it does not publish; after ONE barrier every wavefront sorts out the same list:
+        // candidates above everything unpublished, strictly ordered (equal minima are left to the exact
+        // resolution below, one sample at a time), each unchanged by those before it.
+        constexpr int FPB_T = 8; // samples per round at most (8 x 8 pairs: one per lane)
+        __shared__ float4 cand_rec[2][WAVES * 2]; // x, y, z, sorted position of a wavefront's published points
+        __shared__ __align__(16) int cand_val[2][WAVES * 2]; // their running minima (INT_MIN: nothing published)
+        __shared__ int hidden[2][WAVES];          // per wavefront: the largest minimum not published
+        int g2[NG]; // per lane: second largest of each group (g: the largest)
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi)
+        {
+            int a1 = INT_MIN, a2 = INT_MIN;
+#pragma unroll
+            for (int e = 0; e < GS; ++e)
+            {
+                const int v = t[gi * GS + e];
+                a2 = max(a2, min(a1, v));
+                a1 = max(a1, v);
+            }
+            g2[gi] = a2;
+        }
+        // the samples whose updates are due: records published in the round before, chosen by wavefront 0
+        // (first: point 0)
+        struct Chosen
+        {
+            int count, bound; // samples taken (0: equal minima, see below); no running minimum exceeds `bound`
+            int pad0, pad1;
+            int from[FPB_T];  // their places in cand_rec
+        };
+        __shared__ Chosen chosen[2];
+        if (tid == 0)
+        {
+            cand_rec[0][0] = make_float4(p0x, p0y, p0z, 0.f);
+            chosen[0].count = 1;
+            chosen[0].bound = bound;
+            chosen[0].from[0] = 0;
+        }
+        __syncthreads();
+        int ns = 1, from = 0;
+        int j = 1;
+        for (int round = 1; j < npoint; ++round)
+        {
+            const int par = round & 1;
+            if (tid == 0)
+                words[0] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
+            // 1. the updates of the round before's samples.  Which groups can change?  The four rows of 16 lanes
+            // test four samples at a time (lane g of a row: group g), two passes for up to eight samples.
+            // (lane k < 8 fetches sample k; the others get it from there)
+            const float4 fetched = cand_rec[from][chosen[from].from[lane < ns ? lane : 0]];
+            unsigned long long live[FPB_T / 4];
+#pragma unroll
+            for (int pass = 0; pass < FPB_T / 4; ++pass)
+            {
+                const int k = pass * 4 + (lane >> 4);
+                float4 sample;
+                sample.x = __shfl(fetched.x, k, TPK_WAVE);
+                sample.y = __shfl(fetched.y, k, TPK_WAVE);
+                sample.z = __shfl(fetched.z, k, TPK_WAVE);
+                const float dx = fmaxf(fmaxf(blo[0] - sample.x, sample.x - bhi[0]), 0.f);
+                const float dy = fmaxf(fmaxf(blo[1] - sample.y, sample.y - bhi[1]), 0.f);
+                const float dz = fmaxf(fmaxf(blo[2] - sample.z, sample.z - bhi[2]), 0.f);
+                const float lb = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz)) * 0.999998f;
+                // an empty box gives lb = +inf (never live); NaN compares false -> live
+                live[pass] = __ballot(k < ns && !(lb >= __int_as_float(bound)));
+            }
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi)
+            {
+                // samples that reach group gi, one bit each
+                unsigned reach = 0;
+#pragma unroll
+                for (int pass = 0; pass < FPB_T / 4; ++pass)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        reach |= static_cast<unsigned>((live[pass] >> (r * 16 + gi)) & 1ull) << (pass * 4 + r);
+                if (reach == 0)
+                    continue; // (uniform over the wavefront)
+                while (reach != 0)
+                {
+                    const int k = __builtin_ctz(reach);
+                    reach &= reach - 1;
+                    const float sx = to_vector_register(tpk_read_lane(fetched.x, k)), sy = to_vector_register(tpk_read_lane(fetched.y, k));
+                    const float sz = to_vector_register(tpk_read_lane(fetched.z, k));
+                    TPK_WORK_ADD(GS);
+#pragma unroll
+                    for (int e = 0; e < GS; ++e)
+                    {
+                        const int i = gi * GS + e;
+                        t[i] = min(t[i], ordered_bits(tpk_dist2(x[i], y[i], z[i], sx, sy, sz)));
+                    }
+                }
+                int a1 = INT_MIN, a2 = INT_MIN;
+#pragma unroll
+                for (int e = 0; e < GS; ++e)
+                {
+                    const int v = t[gi * GS + e];
+                    a2 = max(a2, min(a1, v));
+                    a1 = max(a1, v);
+                }
+                g[gi] = a1;
+                g2[gi] = a2;
+            }
+            // 2. the lane's largest and second largest minimum
+            int b1 = INT_MIN, b2 = INT_MIN;
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi)
+            {
+                b2 = max(max(b2, min(b1, g[gi])), g2[gi]);
+                b1 = max(b1, g[gi]);
+            }
+            best = b1;
+            // 3. the wavefront's two best points (of different lanes) and the largest minimum it keeps to itself
+            const int w1 = wave_max_i32(b1);
+            const int l1 = __builtin_ctzll(__ballot(b1 == w1));
+            const int c2 = lane == l1 ? b2 : b1;
+            const int w2 = wave_max_i32(c2);
+            const int l2 = __builtin_ctzll(__ballot(c2 == w2));
+            const bool two = l2 != l1; // (else the second best is the first lane's other point: not published)
+            const int c3 = (lane == l1 || lane == l2) ? b2 : b1;
+            const int w3 = two ? wave_max_i32(c3) : w2;
+            // the slot of a lane's best point: group, then member (uniform indices into the registers)
+            auto publish = [&](int from_lane, int place) __attribute__((always_inline)) {
+                int my_grp = 0;
+#pragma unroll
+                for (int gi = NG - 1; gi >= 0; --gi)
+                    my_grp = g[gi] == b1 ? gi : my_grp;
+                const int grp = __builtin_amdgcn_readlane(my_grp, from_lane);
+                int my_e = 0;
+#pragma unroll
+                for (int e = GS - 1; e >= 0; --e)
+                    my_e = t[grp * GS + e] == b1 ? e : my_e;
+                const int ce = __builtin_amdgcn_readlane(my_e, from_lane);
+                const int slot = grp * GS + ce;
+                const float cx = x[slot], cy = y[slot], cz = z[slot];
+                if (lane == from_lane)
+                {
+                    cand_rec[par][place] = make_float4(cx, cy, cz, __int_as_float(sorted_position<WAVES, GS>(grp, wave, ce, lane)));
+                    cand_val[par][place] = b1;
+                }
+            };
+            publish(l1, wave * 2);
+            if (two)
+                publish(l2, wave * 2 + 1);
+            if (lane == 0)
+            {
+                if (!two)
+                    cand_val[par][wave * 2 + 1] = INT_MIN;
+                hidden[par][wave] = w3;
+            }
+            lds_barrier();
+            // 4. wavefront 0 sorts out the list, the others wait for it
+            if (wave == 0)
+            {
+                const int v = lane < 2 * WAVES ? cand_val[par][lane] : INT_MIN;
+                const int kept = wave_max_i32(lane < WAVES ? hidden[par][lane] : INT_MIN);
+                // place of this lane's candidate in descending order (equal values: lower lane first)
+                int place = 0;
+#pragma unroll
+                for (int o4 = 0; o4 < 2 * WAVES / 4; ++o4)
+                {
+                    const int4 others = reinterpret_cast<const int4*>(cand_val[par])[o4]; // (the same for all lanes)
+                    const int other[4] = {others.x, others.y, others.z, others.w};
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        place += (other[u] > v || (other[u] == v && o4 * 4 + u < lane)) ? 1 : 0;
+                }
+                // lane k: the candidate of place k (its value and where its record lies)
+                const int my_val = __builtin_amdgcn_ds_permute(place << 2, v);
+                const int my_src = __builtin_amdgcn_ds_permute(place << 2, lane);
+                // candidate k < FPB_T may follow when it is above everything unpublished, strictly above the one
+                // behind it (and so strictly below the one before), and a real minimum (>= 0)
+                const int behind = __shfl_down(my_val, 1, TPK_WAVE);
+                const bool fine = lane < FPB_T && lane < 2 * WAVES - 1 && my_val > kept && my_val > behind && my_val >= 0;
+                const int usable = __builtin_ctzll(~__ballot(fine));
+                // lane (k, i), i < k: does candidate i change candidate k's minimum?
+                int accept = usable;
+                {
+                    const int k = lane >> 3, i = lane & 7;
+                    const int from_k = __shfl(my_src, k, TPK_WAVE) & (2 * WAVES - 1), from_i = __shfl(my_src, i, TPK_WAVE) & (2 * WAVES - 1);
+                    const int val_k = __shfl(my_val, k, TPK_WAVE);
+                    const float4 rk = cand_rec[par][from_k], ri = cand_rec[par][from_i];
+                    const bool hits = i < k && k < usable && ordered_bits(tpk_dist2(rk.x, rk.y, rk.z, ri.x, ri.y, ri.z)) < val_k;
+                    const unsigned long long spoiled = __ballot(hits);
+                    if (spoiled != 0ull)
+                        accept = min(accept, static_cast<int>(__builtin_ctzll(spoiled)) >> 3);
+                }
+                accept = min(accept, npoint - j);
+                if (lane < accept)
+                    out[j + lane] = static_cast<int>(sort_keys[__float_as_int(cand_rec[par][my_src & (2 * WAVES - 1)].w)] & 0x3FFFu);
+                if (lane < FPB_T)
+                    chosen[par].from[lane] = my_src & (2 * WAVES - 1);
+                if (lane == 0)
+                {
+                    chosen[par].count = accept;
+                    // (no minimum exceeds the round's largest; the new samples still hold theirs until their own updates)
+                    chosen[par].bound = my_val;
+                }
+            }
+            lds_barrier();
+            const int accept = __builtin_amdgcn_readfirstlane(chosen[par].count);
+            if (accept > 0)
+            {
+                ns = accept;
+                from = par;
+                j += accept;
+                bound = __builtin_amdgcn_readfirstlane(chosen[par].bound);
+                continue;
+            }
+
+            // Equal minima at the top, or nothing eligible: one sample by the reference's tie key over all points
+            // that hold the maximum (the key comes from the original index kept in the sort keys).
+            const int row_best = row_all_max_i32(b1);
+            if (row_head)
+                lds_atomic_max_i32(&words[0].max_val, row_best);
+            lds_barrier();
+            const int gv = __builtin_amdgcn_readfirstlane(words[0].max_val);
+            if (gv < 0)
+            {
+                // No eligible point in the whole cloud: the reference's reduction yields index 0.
+                if (tid == 0)
+                {
+                    cand_rec[par][0] = make_float4(p0x, p0y, p0z, 0.f);
+                    out[j] = 0;
+                }
+            }
+            else
+            {
+                unsigned my_tk = 0xFFFFFFFFu;
+                int my_q = 0;
+#pragma unroll
+                for (int i = 0; i < PPT; ++i)
+                {
+                    const int q = sorted_position<WAVES, GS>(i / GS, wave, i % GS, lane);
+                    if (t[i] == gv && q < n)
+                    {
+                        const unsigned tk = tie_key(static_cast<int>(sort_keys[q] & 0x3FFFu), log2_bs, ref_groups);
+                        if (tk < my_tk)
+                        {
+                            my_tk = tk;
+                            my_q = q;
+                        }
+                    }
+                }
+                if (my_tk != 0xFFFFFFFFu)
+                    atomicMin(&words[0].min_tie, my_tk);
+                lds_barrier();
+                if (my_tk == words[0].min_tie) // tie keys are distinct: exactly one lane
+                {
+                    const int k = static_cast<int>(sort_keys[my_q] & 0x3FFFu);
+                    cand_rec[par][0] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2], __int_as_float(my_q));
+                    out[j] = k;
+                }
+            }
+            if (tid == 0)
+                chosen[par].from[0] = 0;
+            lds_barrier();
+            ns = 1;
+            from = par;
+            j += 1;
+            bound = gv < 0 ? bound : gv;
+        }
+        TPK_WORK_FLUSH
+        return;
+    }
     for (int j = 1; j < npoint; ++j)
     {
         const int par = j & 1;
@@ -895,13 +1167,13 @@ void launch_resident(int b, int n, int npoint, int log2_bs, int groups, const fl
 }
 
 
-template <int PPT, int THREADS, int GS>
+template <int PPT, int THREADS, int GS, bool BATCHED = false>
 int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float* xyz,
                   int32_t* out, hipStream_t s)
 {
     const int key_capacity = n > CURVE_BINS ? (n + 63) & ~63 : CURVE_BINS; // (the ordering borrows CURVE_BINS words)
     const size_t lds = (static_cast<size_t>(key_capacity) + static_cast<size_t>(PPT) * THREADS + CURVE_BINS) * sizeof(unsigned);
-    auto kernel = fps_pruned_kernel<PPT, THREADS, GS>;
+    auto kernel = fps_pruned_kernel<PPT, THREADS, GS, BATCHED>;
     const int allowed = tpk_allow_lds(reinterpret_cast<const void*>(kernel), lds);
     if (allowed != TPK_OK)
         return allowed;
@@ -984,7 +1256,7 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
     else if (n <= 512 * 16)
         return launch_pruned<16, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_REGISTER_POINTS)
-        return launch_pruned<16, 1024, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<16, 1024, 4, true>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_CELL_POINTS && workspace && workspace_bytes >= cell_layout(b, n).total)
     {
         // Cells of 64 points in memory, their summaries in LDS.

@@ -841,7 +841,12 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 const int nx = ((d >> 12) & 15) + 1, ny = ((d >> 16) & 15) + 1;
                 const int wx = wx0 + window;
                 // (the table of the ordering kernel: 8 KiB that every wavefront reads, at home in the caches)
-                const unsigned bin = curve_bin_table.bin[(fx + i % nx) | ((fy + (i / nx) % ny) << 4) | ((fz + i / (nx * ny)) << 8)];
+                // (i = ix + nx * (iy + ny * iz), taken apart by float division: exact for these small numbers)
+                const int iz = static_cast<int>((static_cast<float>(i) + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(nx * ny)));
+                const int in_plane = i - iz * nx * ny;
+                const int iy = static_cast<int>((static_cast<float>(in_plane) + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(nx)));
+                const int ix = in_plane - iy * nx;
+                const unsigned bin = curve_bin_table.bin[(fx + ix) | ((fy + iy) << 4) | ((fz + iz) << 8)];
                 const int* __restrict__ ends = bin_ends + static_cast<int64_t>(wx) * CURVE_BINS;
                 start = bin ? ends[bin - 1] : 0;
                 size = ends[bin] - start;
