@@ -520,6 +520,30 @@ def test_fps_ties_large_cloud(tpk, oracle, dev):
     np.testing.assert_array_equal(out, oracle.furthest_point_sample(tiny.numpy(), 5))
 
 
+@pytest.mark.parametrize("B,N,npoint,kind", [(2, 16384, 2, "uniform"), (1, 12000, 3, "clusters"), (2, 9000, 777, "clusters"),
+                                             (1, 16384, 5000, "uniform"), (1, 10000, 10000, "shell"), (3, 8200, 1001, "line"),
+                                             (1, 16000, 900, "two_scales")])
+def test_fps_several_samples_per_round(tpk, oracle, dev, B, N, npoint, kind):
+    # clouds of 8193 .. 16384 points take up to 16 samples per round (the points with the largest minima, as long
+    # as none changes the next one's minimum): sample counts that end inside a round, every point sampled,
+    # clouds whose largest minima lie close together (a line, dense clusters next to a sparse background)
+    g = torch.Generator().manual_seed(N + npoint)
+    xyz = torch.rand(B, N, 3, generator=g) + 0.1
+    if kind == "clusters":
+        centres = torch.rand(B, 6, 3, generator=g) * 4 + 0.5
+        xyz = centres[:, torch.randint(0, 6, (N,), generator=g)] + 0.05 * torch.randn(B, N, 3, generator=g)
+    elif kind == "shell":
+        p = torch.randn(B, N, 3, generator=g)
+        xyz = p / p.norm(dim=2, keepdim=True) * 2.0 + 3.0
+    elif kind == "line":
+        xyz[..., 1:] = 0.5
+    elif kind == "two_scales":
+        xyz[:, : N // 2] = xyz[:, : N // 2] * 0.01 + 1.0
+        xyz[:, N // 2 :] = xyz[:, N // 2 :] * 20.0
+    out = tpk.furthest_point_sample(xyz.contiguous().to(dev), npoint)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.contiguous().numpy(), npoint))
+
+
 def test_fps_full_config2(tpk, oracle, dev):
     w = W.cfg2_fps()
     xyz = w["xyz"].to(dev)

@@ -419,7 +419,9 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     }
     __syncthreads();
     // lane g of every 16-lane row tests this wavefront's group g; lanes beyond NG hold an empty box
-    const int my_group = lane & 15;
+    // (BATCHED: row g tests group g, its lane k against sample k of the round)
+    static_assert(!BATCHED || NG <= 4, "one row of lanes per group");
+    const int my_group = BATCHED ? lane >> 4 : lane & 15;
     float blo[3], bhi[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a)
@@ -458,12 +460,17 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         // their running minima.  c0 is the next sample.  If c1's minimum is not changed by c0 (c0 is no closer
         // to it than its minimum), then after c0's update c1 still holds what it held, nothing holds more, and
         // c1 is the sample after c0 - and so on: ck follows as long as none of c0 .. c(k-1) changes its minimum.
-        // Late in a sampling the largest minima sit in different corners of the cloud, far from each other, and
-        // nearly every round takes the FPB_T samples it may.  Every wavefront publishes its two best points and
-        // the largest minimum it does not publish; after ONE barrier every wavefront sorts out the same list:
-        // candidates above everything unpublished, strictly ordered (equal minima are left to the exact
-        // resolution below, one sample at a time), each unchanged by those before it.
-        constexpr int FPB_T = 8; // samples per round at most (8 x 8 pairs: one per lane)
+        // The largest minima sit in different corners of the cloud, far from each other, and a round takes eight
+        // samples on average.  Every wavefront publishes its two best points and the largest minimum it does
+        // not publish; after a barrier wavefront 0 sorts out the list - candidates above everything unpublished,
+        // strictly ordered (equal minima are left to the exact resolution below, one sample at a time), each
+        // unchanged by those before it - and after a second barrier all wavefronts apply the new samples'
+        // updates together: which of a wavefront's groups a sample can change is one box test per (group,
+        // sample), all of a round's in one instruction sequence.
+        constexpr int FPB_T = 16; // samples per round at most: one lane of a 16-lane row each in the box tests
+        static_assert(FPB_T <= 16 && TPK_WAVE % FPB_T == 0, "the pair tests take whole rows of lanes");
+        constexpr int CANDS = WAVES * 2;
+        static_assert((CANDS & (CANDS - 1)) == 0 && CANDS <= TPK_WAVE && CANDS > FPB_T, "one lane per published point");
         __shared__ float4 cand_rec[2][WAVES * 2]; // x, y, z, sorted position of a wavefront's published points
         __shared__ __align__(16) int cand_val[2][WAVES * 2]; // their running minima (INT_MIN: nothing published)
         __shared__ int hidden[2][WAVES];          // per wavefront: the largest minimum not published
@@ -505,36 +512,25 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             const int par = round & 1;
             if (tid == 0)
                 words[0] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
-            // 1. the updates of the round before's samples.  Which groups can change?  The four rows of 16 lanes
-            // test four samples at a time (lane g of a row: group g), two passes for up to eight samples.
-            // (lane k < 8 fetches sample k; the others get it from there)
+            // 1. the updates of the round before's samples.  Which groups can change?  Lane k < FPB_T fetches
+            // sample k; row g of the lanes tests its lane's sample against group g.
             const float4 fetched = cand_rec[from][chosen[from].from[lane < ns ? lane : 0]];
-            unsigned long long live[FPB_T / 4];
-#pragma unroll
-            for (int pass = 0; pass < FPB_T / 4; ++pass)
+            unsigned long long live;
             {
-                const int k = pass * 4 + (lane >> 4);
-                float4 sample;
-                sample.x = __shfl(fetched.x, k, TPK_WAVE);
-                sample.y = __shfl(fetched.y, k, TPK_WAVE);
-                sample.z = __shfl(fetched.z, k, TPK_WAVE);
-                const float dx = fmaxf(fmaxf(blo[0] - sample.x, sample.x - bhi[0]), 0.f);
-                const float dy = fmaxf(fmaxf(blo[1] - sample.y, sample.y - bhi[1]), 0.f);
-                const float dz = fmaxf(fmaxf(blo[2] - sample.z, sample.z - bhi[2]), 0.f);
+                const int k = lane & 15;
+                const float sx = __shfl(fetched.x, k, TPK_WAVE), sy = __shfl(fetched.y, k, TPK_WAVE), sz = __shfl(fetched.z, k, TPK_WAVE);
+                const float dx = fmaxf(fmaxf(blo[0] - sx, sx - bhi[0]), 0.f);
+                const float dy = fmaxf(fmaxf(blo[1] - sy, sy - bhi[1]), 0.f);
+                const float dz = fmaxf(fmaxf(blo[2] - sz, sz - bhi[2]), 0.f);
                 const float lb = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz)) * 0.999998f;
                 // an empty box gives lb = +inf (never live); NaN compares false -> live
-                live[pass] = __ballot(k < ns && !(lb >= __int_as_float(bound)));
+                live = __ballot(k < ns && !(lb >= __int_as_float(bound)));
             }
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi)
             {
                 // samples that reach group gi, one bit each
-                unsigned reach = 0;
-#pragma unroll
-                for (int pass = 0; pass < FPB_T / 4; ++pass)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        reach |= static_cast<unsigned>((live[pass] >> (r * 16 + gi)) & 1ull) << (pass * 4 + r);
+                unsigned reach = static_cast<unsigned>(live >> (gi * 16)) & 0xFFFFu;
                 if (reach == 0)
                     continue; // (uniform over the wavefront)
                 while (reach != 0)
@@ -611,46 +607,50 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             }
             lds_barrier();
             // 4. wavefront 0 sorts out the list, the others wait for it
+            int out_pos = 0;
             if (wave == 0)
             {
-                const int v = lane < 2 * WAVES ? cand_val[par][lane] : INT_MIN;
+                const int v = lane < CANDS ? cand_val[par][lane] : INT_MIN;
                 const int kept = wave_max_i32(lane < WAVES ? hidden[par][lane] : INT_MIN);
                 // place of this lane's candidate in descending order (equal values: lower lane first)
-                int place = 0;
+                int places[4] = {0, 0, 0, 0};
 #pragma unroll
-                for (int o4 = 0; o4 < 2 * WAVES / 4; ++o4)
+                for (int o4 = 0; o4 < CANDS / 4; ++o4)
                 {
                     const int4 others = reinterpret_cast<const int4*>(cand_val[par])[o4]; // (the same for all lanes)
                     const int other[4] = {others.x, others.y, others.z, others.w};
 #pragma unroll
                     for (int u = 0; u < 4; ++u)
-                        place += (other[u] > v || (other[u] == v && o4 * 4 + u < lane)) ? 1 : 0;
+                        places[u] += (other[u] > v || (other[u] == v && o4 * 4 + u < lane)) ? 1 : 0;
                 }
+                const int place = (places[0] + places[1]) + (places[2] + places[3]);
                 // lane k: the candidate of place k (its value and where its record lies)
                 const int my_val = __builtin_amdgcn_ds_permute(place << 2, v);
                 const int my_src = __builtin_amdgcn_ds_permute(place << 2, lane);
                 // candidate k < FPB_T may follow when it is above everything unpublished, strictly above the one
                 // behind it (and so strictly below the one before), and a real minimum (>= 0)
                 const int behind = __shfl_down(my_val, 1, TPK_WAVE);
-                const bool fine = lane < FPB_T && lane < 2 * WAVES - 1 && my_val > kept && my_val > behind && my_val >= 0;
+                const bool fine = lane < FPB_T && my_val > kept && my_val > behind && my_val >= 0;
                 const int usable = __builtin_ctzll(~__ballot(fine));
                 // lane (k, i), i < k: does candidate i change candidate k's minimum?
                 int accept = usable;
+                const float4 mine = cand_rec[par][my_src & (CANDS - 1)]; // lane k: candidate k
+#pragma unroll
+                for (int k0 = 0; k0 < FPB_T; k0 += TPK_WAVE / FPB_T)
                 {
-                    const int k = lane >> 3, i = lane & 7;
-                    const int from_k = __shfl(my_src, k, TPK_WAVE) & (2 * WAVES - 1), from_i = __shfl(my_src, i, TPK_WAVE) & (2 * WAVES - 1);
+                    const int k = k0 + lane / FPB_T, i = lane % FPB_T;
                     const int val_k = __shfl(my_val, k, TPK_WAVE);
-                    const float4 rk = cand_rec[par][from_k], ri = cand_rec[par][from_i];
-                    const bool hits = i < k && k < usable && ordered_bits(tpk_dist2(rk.x, rk.y, rk.z, ri.x, ri.y, ri.z)) < val_k;
+                    const float kx = __shfl(mine.x, k, TPK_WAVE), ky = __shfl(mine.y, k, TPK_WAVE), kz = __shfl(mine.z, k, TPK_WAVE);
+                    const float ix = __shfl(mine.x, i, TPK_WAVE), iy = __shfl(mine.y, i, TPK_WAVE), iz = __shfl(mine.z, i, TPK_WAVE);
+                    const bool hits = i < k && k < accept && ordered_bits(tpk_dist2(kx, ky, kz, ix, iy, iz)) < val_k;
                     const unsigned long long spoiled = __ballot(hits);
                     if (spoiled != 0ull)
-                        accept = min(accept, static_cast<int>(__builtin_ctzll(spoiled)) >> 3);
+                        accept = min(accept, k0 + static_cast<int>(__builtin_ctzll(spoiled)) / FPB_T);
                 }
                 accept = min(accept, npoint - j);
-                if (lane < accept)
-                    out[j + lane] = static_cast<int>(sort_keys[__float_as_int(cand_rec[par][my_src & (2 * WAVES - 1)].w)] & 0x3FFFu);
+                out_pos = __float_as_int(mine.w);
                 if (lane < FPB_T)
-                    chosen[par].from[lane] = my_src & (2 * WAVES - 1);
+                    chosen[par].from[lane] = my_src & (CANDS - 1);
                 if (lane == 0)
                 {
                     chosen[par].count = accept;
@@ -662,6 +662,8 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             const int accept = __builtin_amdgcn_readfirstlane(chosen[par].count);
             if (accept > 0)
             {
+                if (wave == 0 && lane < accept) // (the others are on their way already)
+                    out[j + lane] = static_cast<int>(sort_keys[out_pos] & 0x3FFFu);
                 ns = accept;
                 from = par;
                 j += accept;
