@@ -36,7 +36,7 @@ VALU_FILE = os.path.join(PROFILES, "distance_scans_valu_utilisation.txt")
 
 # Kernels whose HBM traffic adds up to one launch of an operator (names as rocprofv3 prints them).
 TRAFFIC_KERNELS = {
-    "fps": ["fps_pruned_kernel<16, 1024, 4>"],
+    "fps": ["fps_pruned_kernel<16, 1024, 4, true>"],
     "three_interpolate_fwd": ["gather_fwd_lds_kernel<3, true, int, true>"],
     "three_interpolate_bwd": ["build_lists_kernel<3, true, int>", "gather_bwd_lists_kernel<3, true, 2>"],
     "grouping_fwd": ["gather_fwd_lds_kernel<1, false, long, false>"],
@@ -45,7 +45,7 @@ TRAFFIC_KERNELS = {
 }
 # Kernels whose VALU counters describe a distance scan.
 VALU_KERNELS = {
-    "fps": "fps_pruned_kernel<16, 1024, 4>",
+    "fps": "fps_pruned_kernel<16, 1024, 4, true>",
     "ball_query_dense": "ball_query_dense_cells_kernel<false>",
     "ball_query_partial_dense": "ball_query_bins_kernel<false>",
     "three_nn": "three_nn_cells_kernel",

@@ -467,12 +467,13 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         // unchanged by those before it - and after a second barrier all wavefronts apply the new samples'
         // updates together: which of a wavefront's groups a sample can change is one box test per (group,
         // sample), all of a round's in one instruction sequence.
-        constexpr int FPB_T = 16; // samples per round at most: one lane of a 16-lane row each in the box tests
+        constexpr int FPB_T = WAVES >= 16 ? 16 : 8; // samples per round at most (16: one lane of a row each in the box tests)
         static_assert(FPB_T <= 16 && TPK_WAVE % FPB_T == 0, "the pair tests take whole rows of lanes");
-        constexpr int CANDS = WAVES * 2;
-        static_assert((CANDS & (CANDS - 1)) == 0 && CANDS <= TPK_WAVE && CANDS > FPB_T, "one lane per published point");
-        __shared__ float4 cand_rec[2][WAVES * 2]; // x, y, z, sorted position of a wavefront's published points
-        __shared__ __align__(16) int cand_val[2][WAVES * 2]; // their running minima (INT_MIN: nothing published)
+        constexpr int FPB_PUB = 2; // points a wavefront publishes per round (3: fewer rounds, each longer - no gain)
+        constexpr int CANDS = WAVES * FPB_PUB;
+        static_assert(CANDS % 4 == 0 && CANDS <= TPK_WAVE && CANDS > FPB_T, "one lane per published point");
+        __shared__ float4 cand_rec[2][CANDS];                // x, y, z, sorted position of the published points
+        __shared__ __align__(16) int cand_val[2][CANDS];     // their running minima (INT_MIN: nothing published)
         __shared__ int hidden[2][WAVES];          // per wavefront: the largest minimum not published
         int g2[NG]; // per lane: second largest of each group (g: the largest)
 #pragma unroll
@@ -494,15 +495,14 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         {
             int count, bound; // samples taken (0: equal minima, see below); no running minimum exceeds `bound`
             int pad0, pad1;
-            int from[FPB_T];  // their places in cand_rec
+            float4 rec[FPB_T]; // x, y, z, sorted position of each
         };
-        __shared__ Chosen chosen[2];
+        __shared__ __align__(16) Chosen chosen[2];
         if (tid == 0)
         {
-            cand_rec[0][0] = make_float4(p0x, p0y, p0z, 0.f);
             chosen[0].count = 1;
             chosen[0].bound = bound;
-            chosen[0].from[0] = 0;
+            chosen[0].rec[0] = make_float4(p0x, p0y, p0z, 0.f);
         }
         __syncthreads();
         int ns = 1, from = 0;
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 words[0] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
             // 1. the updates of the round before's samples.  Which groups can change?  Lane k < FPB_T fetches
             // sample k; row g of the lanes tests its lane's sample against group g.
-            const float4 fetched = cand_rec[from][chosen[from].from[lane < ns ? lane : 0]];
+            const float4 fetched = chosen[from].rec[lane < ns ? lane : 0];
             unsigned long long live;
             {
                 const int k = lane & 15;
@@ -567,15 +567,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 b1 = max(b1, g[gi]);
             }
             best = b1;
-            // 3. the wavefront's two best points (of different lanes) and the largest minimum it keeps to itself
-            const int w1 = wave_max_i32(b1);
-            const int l1 = __builtin_ctzll(__ballot(b1 == w1));
-            const int c2 = lane == l1 ? b2 : b1;
-            const int w2 = wave_max_i32(c2);
-            const int l2 = __builtin_ctzll(__ballot(c2 == w2));
-            const bool two = l2 != l1; // (else the second best is the first lane's other point: not published)
-            const int c3 = (lane == l1 || lane == l2) ? b2 : b1;
-            const int w3 = two ? wave_max_i32(c3) : w2;
+            // 3. the wavefront's FPB_PUB best points (of different lanes) and the largest minimum it keeps to itself
             // the slot of a lane's best point: group, then member (uniform indices into the registers)
             auto publish = [&](int from_lane, int place) __attribute__((always_inline)) {
                 int my_grp = 0;
@@ -596,14 +588,28 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                     cand_val[par][place] = b1;
                 }
             };
-            publish(l1, wave * 2);
-            if (two)
-                publish(l2, wave * 2 + 1);
-            if (lane == 0)
             {
-                if (!two)
-                    cand_val[par][wave * 2 + 1] = INT_MIN;
-                hidden[par][wave] = w3;
+                int left = b1;                   // the lane's best point not yet published
+                unsigned long long gone = 0ull;  // lanes whose best point is published
+                int most = wave_max_i32(left);
+#pragma unroll
+                for (int p = 0; p < FPB_PUB; ++p)
+                {
+                    const int from_lane = __builtin_ctzll(__ballot(left == most));
+                    // (a lane's second point is not published: with it the list ends)
+                    const bool fresh = ((gone >> from_lane) & 1ull) == 0ull;
+                    if (fresh)
+                    {
+                        publish(from_lane, wave * FPB_PUB + p);
+                        gone |= 1ull << from_lane;
+                        left = lane == from_lane ? b2 : left;
+                        most = wave_max_i32(left);
+                    }
+                    else if (lane == 0)
+                        cand_val[par][wave * FPB_PUB + p] = INT_MIN;
+                }
+                if (lane == 0)
+                    hidden[par][wave] = most;
             }
             lds_barrier();
             // 4. wavefront 0 sorts out the list, the others wait for it
@@ -634,14 +640,17 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 const int usable = __builtin_ctzll(~__ballot(fine));
                 // lane (k, i), i < k: does candidate i change candidate k's minimum?
                 int accept = usable;
-                const float4 mine = cand_rec[par][my_src & (CANDS - 1)]; // lane k: candidate k
+                const float4 mine = cand_rec[par][min(my_src, CANDS - 1)]; // lane k: candidate k
+                const int i = lane % FPB_T;
+                const float ix = __shfl(mine.x, i, TPK_WAVE), iy = __shfl(mine.y, i, TPK_WAVE), iz = __shfl(mine.z, i, TPK_WAVE);
 #pragma unroll
                 for (int k0 = 0; k0 < FPB_T; k0 += TPK_WAVE / FPB_T)
                 {
-                    const int k = k0 + lane / FPB_T, i = lane % FPB_T;
+                    if (k0 >= accept)
+                        break; // (uniform)
+                    const int k = k0 + lane / FPB_T;
                     const int val_k = __shfl(my_val, k, TPK_WAVE);
                     const float kx = __shfl(mine.x, k, TPK_WAVE), ky = __shfl(mine.y, k, TPK_WAVE), kz = __shfl(mine.z, k, TPK_WAVE);
-                    const float ix = __shfl(mine.x, i, TPK_WAVE), iy = __shfl(mine.y, i, TPK_WAVE), iz = __shfl(mine.z, i, TPK_WAVE);
                     const bool hits = i < k && k < accept && ordered_bits(tpk_dist2(kx, ky, kz, ix, iy, iz)) < val_k;
                     const unsigned long long spoiled = __ballot(hits);
                     if (spoiled != 0ull)
@@ -650,7 +659,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 accept = min(accept, npoint - j);
                 out_pos = __float_as_int(mine.w);
                 if (lane < FPB_T)
-                    chosen[par].from[lane] = my_src & (CANDS - 1);
+                    chosen[par].rec[lane] = mine;
                 if (lane == 0)
                 {
                     chosen[par].count = accept;
@@ -683,7 +692,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 // No eligible point in the whole cloud: the reference's reduction yields index 0.
                 if (tid == 0)
                 {
-                    cand_rec[par][0] = make_float4(p0x, p0y, p0z, 0.f);
+                    chosen[par].rec[0] = make_float4(p0x, p0y, p0z, 0.f);
                     out[j] = 0;
                 }
             }
@@ -711,12 +720,10 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 if (my_tk == words[0].min_tie) // tie keys are distinct: exactly one lane
                 {
                     const int k = static_cast<int>(sort_keys[my_q] & 0x3FFFu);
-                    cand_rec[par][0] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2], __int_as_float(my_q));
+                    chosen[par].rec[0] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2], __int_as_float(my_q));
                     out[j] = k;
                 }
             }
-            if (tid == 0)
-                chosen[par].from[0] = 0;
             lds_barrier();
             ns = 1;
             from = par;
@@ -1169,7 +1176,13 @@ void launch_resident(int b, int n, int npoint, int log2_bs, int groups, const fl
 }
 
 
-template <int PPT, int THREADS, int GS, bool BATCHED = false>
+#ifdef FPS_ONE_PER_ROUND
+constexpr bool FPS_BATCHED = false;
+#else
+constexpr bool FPS_BATCHED = true;
+#endif
+
+template <int PPT, int THREADS, int GS, bool BATCHED>
 int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float* xyz,
                   int32_t* out, hipStream_t s)
 {
@@ -1249,16 +1262,18 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
     // groups for the winner to search) except between 4097 and 8192 points.
     if (n <= 512)
         launch_resident<1, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+    // (FPS_BATCHED: several samples per round; a build with -DFPS_ONE_PER_ROUND keeps the loop that takes one, for
+    // comparison)
     else if (n <= 512 * 2)
-        return launch_pruned<2, 512, 1>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<2, 512, 1, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 4)
-        return launch_pruned<2, 1024, 2>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<2, 1024, 2, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 8)
-        return launch_pruned<4, 1024, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<4, 1024, 4, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 16)
-        return launch_pruned<16, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<16, 512, 4, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_REGISTER_POINTS)
-        return launch_pruned<16, 1024, 4, true>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<16, 1024, 4, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_CELL_POINTS && workspace && workspace_bytes >= cell_layout(b, n).total)
     {
         // Cells of 64 points in memory, their summaries in LDS.
