@@ -298,7 +298,9 @@ def bench_fps(dev, steps, warmup, with_cpu):
         roof["traffic_measured_at_commit"] = commit
     roof["note"] += "; here a pair = one running minimum updated (10 flop: 8 for the distance, min, max); algorithmic " \
                     "work = every point updated in every round, as the reference does; the kernel skips updates it " \
-                    "proves to be no-ops; the rounds of a cloud are sequential and one workgroup owns a cloud: 16 of 256 " \
+                    "proves to be no-ops and takes up to 16 samples per round (the points with the largest running minima, as " \
+                    "long as none changes the next one's minimum: the same samples in the same order); the rounds " \
+                    "of a cloud are sequential and one workgroup owns a cloud: 16 of 256 " \
                     "compute units are occupied by design, executed fraction of those 16 CUs' peak = %.4f, " \
                     "algorithmic %.4f" % (roof["frac"] * 256 / 16, roof["algorithmic_rate"] / PEAK_FP32_TFLOPS * 256 / 16)
     res = {"wall_ms": wall, "kernel_ms": ev, "roofline": roof, "point_updates": updates}
