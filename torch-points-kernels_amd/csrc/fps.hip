@@ -469,7 +469,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         // sample), all of a round's in one instruction sequence.
         constexpr int FPB_T = WAVES >= 16 ? 16 : 8; // samples per round at most (16: one lane of a row each in the box tests)
         static_assert(FPB_T <= 16 && TPK_WAVE % FPB_T == 0, "the pair tests take whole rows of lanes");
-        constexpr int FPB_PUB = 2; // points a wavefront publishes per round (3: fewer rounds, each longer - no gain)
+        constexpr int FPB_PUB = 2; // points a wavefront publishes per round (3: 1 % faster at best)
         constexpr int CANDS = WAVES * FPB_PUB;
         static_assert(CANDS % 4 == 0 && CANDS <= TPK_WAVE && CANDS > FPB_T, "one lane per published point");
         __shared__ float4 cand_rec[2][CANDS];                // x, y, z, sorted position of the published points
@@ -489,21 +489,15 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             }
             g2[gi] = a2;
         }
-        // the samples whose updates are due: records published in the round before, chosen by wavefront 0
-        // (first: point 0)
-        struct Chosen
-        {
-            int count, bound; // samples taken (0: equal minima, see below); no running minimum exceeds `bound`
-            int pad0, pad1;
-            float4 rec[FPB_T]; // x, y, z, sorted position of each
-        };
-        __shared__ __align__(16) Chosen chosen[2];
+        // the samples whose updates are due: the round before's published points in the order of their minima
+        // (first: point 0), and which of them may follow each other
+        static_assert(FPB_PUB * CANDS <= TPK_WAVE && FPB_T <= WAVES, "a wavefront ranks its points in one step; one wavefront per place");
+        __shared__ int order[2][CANDS];             // published point of every place
+        __shared__ __align__(16) float4 taken[2][FPB_T]; // x, y, z, sorted position of the point of place k
+        __shared__ int follows[2][FPB_T];           // 1: the point of place k may follow those before it
+        __shared__ int largest[2];                  // the round's largest minimum
         if (tid == 0)
-        {
-            chosen[0].count = 1;
-            chosen[0].bound = bound;
-            chosen[0].rec[0] = make_float4(p0x, p0y, p0z, 0.f);
-        }
+            taken[0][0] = make_float4(p0x, p0y, p0z, 0.f);
         __syncthreads();
         int ns = 1, from = 0;
         int j = 1;
@@ -514,7 +508,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 words[0] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
             // 1. the updates of the round before's samples.  Which groups can change?  Lane k < FPB_T fetches
             // sample k; row g of the lanes tests its lane's sample against group g.
-            const float4 fetched = chosen[from].rec[lane < ns ? lane : 0];
+            const float4 fetched = taken[from][lane < ns ? lane : 0];
             unsigned long long live;
             {
                 const int k = lane & 15;
@@ -612,71 +606,48 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                     hidden[par][wave] = most;
             }
             lds_barrier();
-            // 4. wavefront 0 sorts out the list, the others wait for it
-            int out_pos = 0;
-            if (wave == 0)
+            // 4. the list is sorted out by all wavefronts together, in two short steps.  First every wavefront
+            // finds the places of its own published points among all of them (lane (c, o): is point o above my
+            // point c? - equal values: the lower number first, so the places are distinct).
             {
-                const int v = lane < CANDS ? cand_val[par][lane] : INT_MIN;
+                const int c = lane / CANDS, o = lane % CANDS;
+                const int mine = wave * FPB_PUB + (c < FPB_PUB ? c : 0);
+                const int my_val = cand_val[par][mine], other = cand_val[par][o];
+                const unsigned long long above = __ballot(c < FPB_PUB && (other > my_val || (other == my_val && o < mine)));
+                if (o == 0 && c < FPB_PUB)
+                    order[par][__builtin_popcountll((above >> (c * CANDS)) & ((1ull << CANDS) - 1ull))] = mine;
+            }
+            lds_barrier();
+            // Then wavefront k looks at the point of place k: it may follow when its minimum is above everything
+            // unpublished, strictly above the next one's (equal minima are left to the exact resolution below)
+            // and a real minimum (>= 0), and when none of the points before it changes it (lane i: point i).
+            if (wave < FPB_T)
+            {
+                const int at = order[par][wave], next = order[par][wave + 1], before = order[par][lane < wave ? lane : 0];
+                const int val = cand_val[par][at], val_next = cand_val[par][next];
+                const float4 rec = cand_rec[par][at], earlier = cand_rec[par][before];
                 const int kept = wave_max_i32(lane < WAVES ? hidden[par][lane] : INT_MIN);
-                // place of this lane's candidate in descending order (equal values: lower lane first)
-                int places[4] = {0, 0, 0, 0};
-#pragma unroll
-                for (int o4 = 0; o4 < CANDS / 4; ++o4)
-                {
-                    const int4 others = reinterpret_cast<const int4*>(cand_val[par])[o4]; // (the same for all lanes)
-                    const int other[4] = {others.x, others.y, others.z, others.w};
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-                        places[u] += (other[u] > v || (other[u] == v && o4 * 4 + u < lane)) ? 1 : 0;
-                }
-                const int place = (places[0] + places[1]) + (places[2] + places[3]);
-                // lane k: the candidate of place k (its value and where its record lies)
-                const int my_val = __builtin_amdgcn_ds_permute(place << 2, v);
-                const int my_src = __builtin_amdgcn_ds_permute(place << 2, lane);
-                // candidate k < FPB_T may follow when it is above everything unpublished, strictly above the one
-                // behind it (and so strictly below the one before), and a real minimum (>= 0)
-                const int behind = __shfl_down(my_val, 1, TPK_WAVE);
-                const bool fine = lane < FPB_T && my_val > kept && my_val > behind && my_val >= 0;
-                const int usable = __builtin_ctzll(~__ballot(fine));
-                // lane (k, i), i < k: does candidate i change candidate k's minimum?
-                int accept = usable;
-                const float4 mine = cand_rec[par][min(my_src, CANDS - 1)]; // lane k: candidate k
-                const int i = lane % FPB_T;
-                const float ix = __shfl(mine.x, i, TPK_WAVE), iy = __shfl(mine.y, i, TPK_WAVE), iz = __shfl(mine.z, i, TPK_WAVE);
-#pragma unroll
-                for (int k0 = 0; k0 < FPB_T; k0 += TPK_WAVE / FPB_T)
-                {
-                    if (k0 >= accept)
-                        break; // (uniform)
-                    const int k = k0 + lane / FPB_T;
-                    const int val_k = __shfl(my_val, k, TPK_WAVE);
-                    const float kx = __shfl(mine.x, k, TPK_WAVE), ky = __shfl(mine.y, k, TPK_WAVE), kz = __shfl(mine.z, k, TPK_WAVE);
-                    const bool hits = i < k && k < accept && ordered_bits(tpk_dist2(kx, ky, kz, ix, iy, iz)) < val_k;
-                    const unsigned long long spoiled = __ballot(hits);
-                    if (spoiled != 0ull)
-                        accept = min(accept, k0 + static_cast<int>(__builtin_ctzll(spoiled)) / FPB_T);
-                }
-                accept = min(accept, npoint - j);
-                out_pos = __float_as_int(mine.w);
-                if (lane < FPB_T)
-                    chosen[par].rec[lane] = mine;
+                const bool spoiled = lane < wave && ordered_bits(tpk_dist2(rec.x, rec.y, rec.z, earlier.x, earlier.y, earlier.z)) < val;
+                const bool may = __ballot(spoiled) == 0ull && val > kept && val > val_next && val >= 0;
                 if (lane == 0)
                 {
-                    chosen[par].count = accept;
-                    // (no minimum exceeds the round's largest; the new samples still hold theirs until their own updates)
-                    chosen[par].bound = my_val;
+                    taken[par][wave] = rec;
+                    follows[par][wave] = may ? 1 : 0;
+                    if (wave == 0)
+                        largest[par] = val;
                 }
             }
             lds_barrier();
-            const int accept = __builtin_amdgcn_readfirstlane(chosen[par].count);
+            const int accept = min(static_cast<int>(__builtin_ctzll(~__ballot(lane < FPB_T && follows[par][lane < FPB_T ? lane : 0] != 0))), npoint - j);
             if (accept > 0)
             {
                 if (wave == 0 && lane < accept) // (the others are on their way already)
-                    out[j + lane] = static_cast<int>(sort_keys[out_pos] & 0x3FFFu);
+                    out[j + lane] = static_cast<int>(sort_keys[__float_as_int(taken[par][lane].w)] & 0x3FFFu);
                 ns = accept;
                 from = par;
                 j += accept;
-                bound = __builtin_amdgcn_readfirstlane(chosen[par].bound);
+                // (no minimum exceeds the round's largest; the new samples still hold theirs until their own updates)
+                bound = __builtin_amdgcn_readfirstlane(largest[par]);
                 continue;
             }
 
@@ -692,7 +663,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 // No eligible point in the whole cloud: the reference's reduction yields index 0.
                 if (tid == 0)
                 {
-                    chosen[par].rec[0] = make_float4(p0x, p0y, p0z, 0.f);
+                    taken[par][0] = make_float4(p0x, p0y, p0z, 0.f);
                     out[j] = 0;
                 }
             }
@@ -720,7 +691,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 if (my_tk == words[0].min_tie) // tie keys are distinct: exactly one lane
                 {
                     const int k = static_cast<int>(sort_keys[my_q] & 0x3FFFu);
-                    chosen[par].rec[0] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2], __int_as_float(my_q));
+                    taken[par][0] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2], __int_as_float(my_q));
                     out[j] = k;
                 }
             }
