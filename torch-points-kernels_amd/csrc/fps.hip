@@ -500,12 +500,14 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
             taken[0][0] = make_float4(p0x, p0y, p0z, 0.f);
         __syncthreads();
         int ns = 1, from = 0;
+        // Clouds with equal minima at the top in round after round (lattices, repeated points) gain nothing from the
+        // list: after a round that had to fall back on the exact resolution the next `pause` rounds go there at
+        // once, twice as many each time it happens again, until a round takes several samples.
+        int pause = 0, penalty = 1, which = 0;
         int j = 1;
         for (int round = 1; j < npoint; ++round)
         {
             const int par = round & 1;
-            if (tid == 0)
-                words[0] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
             // 1. the updates of the round before's samples.  Which groups can change?  Lane k < FPB_T fetches
             // sample k; row g of the lanes tests its lane's sample against group g.
             const float4 fetched = taken[from][lane < ns ? lane : 0];
@@ -561,103 +563,113 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 b1 = max(b1, g[gi]);
             }
             best = b1;
-            // 3. the wavefront's FPB_PUB best points (of different lanes) and the largest minimum it keeps to itself
-            // the slot of a lane's best point: group, then member (uniform indices into the registers)
-            auto publish = [&](int from_lane, int place) __attribute__((always_inline)) {
-                int my_grp = 0;
-#pragma unroll
-                for (int gi = NG - 1; gi >= 0; --gi)
-                    my_grp = g[gi] == b1 ? gi : my_grp;
-                const int grp = __builtin_amdgcn_readlane(my_grp, from_lane);
-                int my_e = 0;
-#pragma unroll
-                for (int e = GS - 1; e >= 0; --e)
-                    my_e = t[grp * GS + e] == b1 ? e : my_e;
-                const int ce = __builtin_amdgcn_readlane(my_e, from_lane);
-                const int slot = grp * GS + ce;
-                const float cx = x[slot], cy = y[slot], cz = z[slot];
-                if (lane == from_lane)
-                {
-                    cand_rec[par][place] = make_float4(cx, cy, cz, __int_as_float(sorted_position<WAVES, GS>(grp, wave, ce, lane)));
-                    cand_val[par][place] = b1;
-                }
-            };
+            if (pause == 0)
             {
-                int left = b1;                   // the lane's best point not yet published
-                unsigned long long gone = 0ull;  // lanes whose best point is published
-                int most = wave_max_i32(left);
+                // 3. the wavefront's FPB_PUB best points (of different lanes) and the largest minimum it keeps to itself
+                // the slot of a lane's best point: group, then member (uniform indices into the registers)
+                auto publish = [&](int from_lane, int place) __attribute__((always_inline)) {
+                    int my_grp = 0;
 #pragma unroll
-                for (int p = 0; p < FPB_PUB; ++p)
-                {
-                    const int from_lane = __builtin_ctzll(__ballot(left == most));
-                    // (a lane's second point is not published: with it the list ends)
-                    const bool fresh = ((gone >> from_lane) & 1ull) == 0ull;
-                    if (fresh)
+                    for (int gi = NG - 1; gi >= 0; --gi)
+                        my_grp = g[gi] == b1 ? gi : my_grp;
+                    const int grp = __builtin_amdgcn_readlane(my_grp, from_lane);
+                    int my_e = 0;
+#pragma unroll
+                    for (int e = GS - 1; e >= 0; --e)
+                        my_e = t[grp * GS + e] == b1 ? e : my_e;
+                    const int ce = __builtin_amdgcn_readlane(my_e, from_lane);
+                    const int slot = grp * GS + ce;
+                    const float cx = x[slot], cy = y[slot], cz = z[slot];
+                    if (lane == from_lane)
                     {
-                        publish(from_lane, wave * FPB_PUB + p);
-                        gone |= 1ull << from_lane;
-                        left = lane == from_lane ? b2 : left;
-                        most = wave_max_i32(left);
+                        cand_rec[par][place] = make_float4(cx, cy, cz, __int_as_float(sorted_position<WAVES, GS>(grp, wave, ce, lane)));
+                        cand_val[par][place] = b1;
                     }
-                    else if (lane == 0)
-                        cand_val[par][wave * FPB_PUB + p] = INT_MIN;
-                }
-                if (lane == 0)
-                    hidden[par][wave] = most;
-            }
-            lds_barrier();
-            // 4. the list is sorted out by all wavefronts together, in two short steps.  First every wavefront
-            // finds the places of its own published points among all of them (lane (c, o): is point o above my
-            // point c? - equal values: the lower number first, so the places are distinct).
-            {
-                const int c = lane / CANDS, o = lane % CANDS;
-                const int mine = wave * FPB_PUB + (c < FPB_PUB ? c : 0);
-                const int my_val = cand_val[par][mine], other = cand_val[par][o];
-                const unsigned long long above = __ballot(c < FPB_PUB && (other > my_val || (other == my_val && o < mine)));
-                if (o == 0 && c < FPB_PUB)
-                    order[par][__builtin_popcountll((above >> (c * CANDS)) & ((1ull << CANDS) - 1ull))] = mine;
-            }
-            lds_barrier();
-            // Then wavefront k looks at the point of place k: it may follow when its minimum is above everything
-            // unpublished, strictly above the next one's (equal minima are left to the exact resolution below)
-            // and a real minimum (>= 0), and when none of the points before it changes it (lane i: point i).
-            if (wave < FPB_T)
-            {
-                const int at = order[par][wave], next = order[par][wave + 1], before = order[par][lane < wave ? lane : 0];
-                const int val = cand_val[par][at], val_next = cand_val[par][next];
-                const float4 rec = cand_rec[par][at], earlier = cand_rec[par][before];
-                const int kept = wave_max_i32(lane < WAVES ? hidden[par][lane] : INT_MIN);
-                const bool spoiled = lane < wave && ordered_bits(tpk_dist2(rec.x, rec.y, rec.z, earlier.x, earlier.y, earlier.z)) < val;
-                const bool may = __ballot(spoiled) == 0ull && val > kept && val > val_next && val >= 0;
-                if (lane == 0)
+                };
                 {
-                    taken[par][wave] = rec;
-                    follows[par][wave] = may ? 1 : 0;
-                    if (wave == 0)
-                        largest[par] = val;
+                    int left = b1;                   // the lane's best point not yet published
+                    unsigned long long gone = 0ull;  // lanes whose best point is published
+                    int most = wave_max_i32(left);
+#pragma unroll
+                    for (int p = 0; p < FPB_PUB; ++p)
+                    {
+                        const int from_lane = __builtin_ctzll(__ballot(left == most));
+                        // (a lane's second point is not published: with it the list ends)
+                        const bool fresh = ((gone >> from_lane) & 1ull) == 0ull;
+                        if (fresh)
+                        {
+                            publish(from_lane, wave * FPB_PUB + p);
+                            gone |= 1ull << from_lane;
+                            left = lane == from_lane ? b2 : left;
+                            most = wave_max_i32(left);
+                        }
+                        else if (lane == 0)
+                            cand_val[par][wave * FPB_PUB + p] = INT_MIN;
+                    }
+                    if (lane == 0)
+                        hidden[par][wave] = most;
                 }
+                lds_barrier();
+                // 4. the list is sorted out by all wavefronts together, in two short steps.  First every wavefront
+                // finds the places of its own published points among all of them (lane (c, o): is point o above my
+                // point c? - equal values: the lower number first, so the places are distinct).
+                {
+                    const int c = lane / CANDS, o = lane % CANDS;
+                    const int mine = wave * FPB_PUB + (c < FPB_PUB ? c : 0);
+                    const int my_val = cand_val[par][mine], other = cand_val[par][o];
+                    const unsigned long long above = __ballot(c < FPB_PUB && (other > my_val || (other == my_val && o < mine)));
+                    if (o == 0 && c < FPB_PUB)
+                        order[par][__builtin_popcountll((above >> (c * CANDS)) & ((1ull << CANDS) - 1ull))] = mine;
+                }
+                lds_barrier();
+                // Then wavefront k looks at the point of place k: it may follow when its minimum is above everything
+                // unpublished, strictly above the next one's (equal minima are left to the exact resolution below)
+                // and a real minimum (>= 0), and when none of the points before it changes it (lane i: point i).
+                if (wave < FPB_T)
+                {
+                    const int at = order[par][wave], next = order[par][wave + 1], before = order[par][lane < wave ? lane : 0];
+                    const int val = cand_val[par][at], val_next = cand_val[par][next];
+                    const float4 rec = cand_rec[par][at], earlier = cand_rec[par][before];
+                    const int kept = wave_max_i32(lane < WAVES ? hidden[par][lane] : INT_MIN);
+                    const bool spoiled = lane < wave && ordered_bits(tpk_dist2(rec.x, rec.y, rec.z, earlier.x, earlier.y, earlier.z)) < val;
+                    const bool may = __ballot(spoiled) == 0ull && val > kept && val > val_next && val >= 0;
+                    if (lane == 0)
+                    {
+                        taken[par][wave] = rec;
+                        follows[par][wave] = may ? 1 : 0;
+                        if (wave == 0)
+                            largest[par] = val;
+                    }
+                }
+                lds_barrier();
+                const int accept = min(static_cast<int>(__builtin_ctzll(~__ballot(lane < FPB_T && follows[par][lane < FPB_T ? lane : 0] != 0))), npoint - j);
+                if (accept > 0)
+                {
+                    if (wave == 0 && lane < accept) // (the others are on their way already)
+                        out[j + lane] = static_cast<int>(sort_keys[__float_as_int(taken[par][lane].w)] & 0x3FFFu);
+                    ns = accept;
+                    from = par;
+                    j += accept;
+                    // (no minimum exceeds the round's largest; the new samples still hold theirs until their own updates)
+                    bound = __builtin_amdgcn_readfirstlane(largest[par]);
+                    penalty = accept > 1 ? 1 : penalty;
+                    continue;
+                }
+                pause = penalty;
+                penalty = min(2 * penalty, 32);
             }
-            lds_barrier();
-            const int accept = min(static_cast<int>(__builtin_ctzll(~__ballot(lane < FPB_T && follows[par][lane < FPB_T ? lane : 0] != 0))), npoint - j);
-            if (accept > 0)
-            {
-                if (wave == 0 && lane < accept) // (the others are on their way already)
-                    out[j + lane] = static_cast<int>(sort_keys[__float_as_int(taken[par][lane].w)] & 0x3FFFu);
-                ns = accept;
-                from = par;
-                j += accept;
-                // (no minimum exceeds the round's largest; the new samples still hold theirs until their own updates)
-                bound = __builtin_amdgcn_readfirstlane(largest[par]);
-                continue;
-            }
+            else
+                --pause;
 
             // Equal minima at the top, or nothing eligible: one sample by the reference's tie key over all points
             // that hold the maximum (the key comes from the original index kept in the sort keys).
+            if (tid == 0)
+                words[which ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0}; // (for the next time)
             const int row_best = row_all_max_i32(b1);
             if (row_head)
-                lds_atomic_max_i32(&words[0].max_val, row_best);
+                lds_atomic_max_i32(&words[which].max_val, row_best);
             lds_barrier();
-            const int gv = __builtin_amdgcn_readfirstlane(words[0].max_val);
+            const int gv = __builtin_amdgcn_readfirstlane(words[which].max_val);
             if (gv < 0)
             {
                 // No eligible point in the whole cloud: the reference's reduction yields index 0.
@@ -686,9 +698,9 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                     }
                 }
                 if (my_tk != 0xFFFFFFFFu)
-                    atomicMin(&words[0].min_tie, my_tk);
+                    atomicMin(&words[which].min_tie, my_tk);
                 lds_barrier();
-                if (my_tk == words[0].min_tie) // tie keys are distinct: exactly one lane
+                if (my_tk == words[which].min_tie) // tie keys are distinct: exactly one lane
                 {
                     const int k = static_cast<int>(sort_keys[my_q] & 0x3FFFu);
                     taken[par][0] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2], __int_as_float(my_q));
@@ -696,6 +708,7 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                 }
             }
             lds_barrier();
+            which ^= 1;
             ns = 1;
             from = par;
             j += 1;
