@@ -459,6 +459,12 @@ def test_fps_cells_in_memory_ties(tpk, oracle, dev):
     tiny[1, 18123] = 1.0
     np.testing.assert_array_equal(_np(tpk.furthest_point_sample(tiny.to(dev), 5)),
                                   oracle.furthest_point_sample(tiny.numpy(), 5))
+    # a handful of eligible points: once all are sampled, their minima are all 0 and the tie rule decides
+    for first in (0.001, 2.0):
+        few = torch.full((2, 20000, 3), 0.001)
+        few[:, 0] = first
+        few[:, [18123, 77, 4500, 4501, 16000], 0] = torch.tensor([1.0, 3.0, 4.5, 5.0, 9.0])
+        np.testing.assert_array_equal(_np(tpk.furthest_point_sample(few.to(dev), 12)), oracle.furthest_point_sample(few.numpy(), 12))
 
 
 def test_fps_streaming_path_parity(tpk, oracle, dev):
@@ -518,15 +524,27 @@ def test_fps_ties_large_cloud(tpk, oracle, dev):
     tiny[1, 8123] = 1.0
     out = _np(tpk.furthest_point_sample(tiny.to(dev), 5))
     np.testing.assert_array_equal(out, oracle.furthest_point_sample(tiny.numpy(), 5))
+    # a handful of eligible points, the first point among them or not: once all are sampled, their minima are
+    # all 0 and the tie rule decides among them
+    for first in (0.001, 2.0):
+        few = torch.full((2, 9000, 3), 0.001)
+        few[:, 0] = first
+        few[:, [8123, 77, 4500, 4501, 6000], 0] = torch.tensor([1.0, 3.0, 4.5, 5.0, 9.0])
+        np.testing.assert_array_equal(_np(tpk.furthest_point_sample(few.to(dev), 12)), oracle.furthest_point_sample(few.numpy(), 12))
 
 
 @pytest.mark.parametrize("B,N,npoint,kind", [(2, 16384, 2, "uniform"), (1, 12000, 3, "clusters"), (2, 9000, 777, "clusters"),
                                              (1, 16384, 5000, "uniform"), (1, 10000, 10000, "shell"), (3, 8200, 1001, "line"),
-                                             (1, 16000, 900, "two_scales")])
+                                             (1, 16000, 900, "two_scales"),
+                                             # clouds in cells in memory
+                                             (2, 16385, 3, "uniform"), (2, 40000, 3001, "uniform"), (1, 30000, 2000, "clusters"),
+                                             (1, 20000, 20000, "shell"), (2, 33000, 1500, "line"), (1, 50000, 1200, "two_scales"),
+                                             (1, 163840, 700, "uniform"), (2, 24000, 2500, "four_times")])
 def test_fps_several_samples_per_round(tpk, oracle, dev, B, N, npoint, kind):
-    # clouds of 8193 .. 16384 points take up to 16 samples per round (the points with the largest minima, as long
+    # clouds of 8193 .. 163840 points take up to 16 samples per round (the points with the largest minima, as long
     # as none changes the next one's minimum): sample counts that end inside a round, every point sampled,
-    # clouds whose largest minima lie close together (a line, dense clusters next to a sparse background)
+    # clouds whose largest minima lie close together (a line, dense clusters next to a sparse background), every
+    # point four times (each round's runner-up is its sample's twin)
     g = torch.Generator().manual_seed(N + npoint)
     xyz = torch.rand(B, N, 3, generator=g) + 0.1
     if kind == "clusters":
@@ -540,6 +558,8 @@ def test_fps_several_samples_per_round(tpk, oracle, dev, B, N, npoint, kind):
     elif kind == "two_scales":
         xyz[:, : N // 2] = xyz[:, : N // 2] * 0.01 + 1.0
         xyz[:, N // 2 :] = xyz[:, N // 2 :] * 20.0
+    elif kind == "four_times":
+        xyz = xyz[:, : N // 4].repeat(1, 4, 1)[:, torch.randperm(N, generator=g)]
     out = tpk.furthest_point_sample(xyz.contiguous().to(dev), npoint)
     np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.contiguous().numpy(), npoint))
 

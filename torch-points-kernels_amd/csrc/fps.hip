@@ -632,7 +632,8 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
                     const float4 rec = cand_rec[par][at], earlier = cand_rec[par][before];
                     const int kept = wave_max_i32(lane < WAVES ? hidden[par][lane] : INT_MIN);
                     const bool spoiled = lane < wave && ordered_bits(tpk_dist2(rec.x, rec.y, rec.z, earlier.x, earlier.y, earlier.z)) < val;
-                    const bool may = __ballot(spoiled) == 0ull && val > kept && val > val_next && val >= 0;
+                    // (after place 0 above 0: the samples before it drop to 0, and equal minima go by tie keys)
+                    const bool may = __ballot(spoiled) == 0ull && val > kept && val > val_next && val >= (wave == 0 ? 0 : 1);
                     if (lane == 0)
                     {
                         taken[par][wave] = rec;
@@ -1064,6 +1065,346 @@ __global__ __launch_bounds__(FPS_THREADS) void fps_cells_kernel(
 }
 
 
+// The same with several samples per round, as in fps_pruned_kernel: after a round's updates the points with the
+// largest running minima follow each other as samples as long as none of them changes the next one's minimum.
+// Here the order is by (minimum, then the reference's tie key), which is strict - equal minima need no separate
+// path - and a candidate's coordinates are at hand in LDS (the best point of its cell).  LDS also keeps every
+// cell's SECOND best point's minimum and key: what a wavefront does not publish - the best points of its other
+// cells, the second best of all its cells - must stay below a candidate for it to count.  A live cell is loaded
+// once per round and takes the updates of all samples that reach it.
+// dynamic LDS: 56 bytes per cell + FPS_LIVE_CAPACITY * 16 * 4.
+constexpr int FPC_T = 16;  // samples per round at most (one wavefront decides on each)
+constexpr int FPC_PUB = 2; // points a wavefront publishes per round
+constexpr int FPC_CANDS = FPS_WAVES * FPC_PUB;
+#ifndef FPC_CELL_BATCH_N
+#define FPC_CELL_BATCH_N 4
+#endif
+constexpr int FPC_CELL_BATCH = FPC_CELL_BATCH_N; // live cells in flight per wavefront
+static_assert(FPC_T <= FPS_WAVES && FPC_T < FPC_CANDS && FPC_PUB * FPC_CANDS <= TPK_WAVE, "one wavefront per place, one lane per pair");
+
+// (larger minimum first, among equals the smaller tie key)
+__device__ __forceinline__ bool fps_above(int v, unsigned t, int w, unsigned u)
+{
+    return v > w || (v == w && t < u);
+}
+
+__global__ __launch_bounds__(FPS_THREADS) void fps_cells_batched_kernel(
+    int n, int npoint, int log2_bs, int groups, int cells, const float* __restrict__ xyz,
+    const float4* __restrict__ sorted, const float4* __restrict__ boxes, float* __restrict__ temp,
+    int32_t* __restrict__ out)
+{
+    extern __shared__ float4 cell_best[];                                  // [cells] x, y, z, index
+    float* const box = reinterpret_cast<float*>(cell_best + cells);        // [6][cells] lo.xyz, hi.xyz
+    int* const cell_max = reinterpret_cast<int*>(box + 6 * cells);         // [cells] bits of the largest minimum
+    unsigned* const cell_tie = reinterpret_cast<unsigned*>(cell_max + cells); // [cells] its point's tie key
+    int* const cell_max2 = reinterpret_cast<int*>(cell_tie + cells);       // [cells] the same for the second best point
+    unsigned* const cell_tie2 = reinterpret_cast<unsigned*>(cell_max2 + cells);
+    unsigned* const live_all = cell_tie2 + cells;                          // per wavefront: live cell | samples that reach it << 16
+    __shared__ int cand_val[2][FPC_CANDS];      // published points: minimum, tie key, cell
+    __shared__ unsigned cand_tie[2][FPC_CANDS];
+    __shared__ int cand_cell[2][FPC_CANDS];
+    __shared__ int kept_val[2][FPS_WAVES];      // per wavefront: the best of what it does not publish
+    __shared__ unsigned kept_tie[2][FPS_WAVES];
+    __shared__ int order[2][FPC_CANDS];         // published point of every place
+    __shared__ __align__(16) float4 taken[2][FPC_T]; // x, y, z, index of the point of place k
+    __shared__ int follows[2][FPC_T];           // 1: the point of place k may follow those before it
+    __shared__ __align__(16) float4 lone[2][FPS_WAVES]; // rounds with one sample: every wavefront's best point
+
+    xyz += static_cast<int64_t>(blockIdx.x) * n * 3;
+    sorted += static_cast<int64_t>(blockIdx.x) * cells * NG_CELL;
+    boxes += static_cast<int64_t>(blockIdx.x) * cells * NG_BOX;
+    temp += static_cast<int64_t>(blockIdx.x) * cells * NG_CELL;
+    out += static_cast<int64_t>(blockIdx.x) * npoint;
+    const int tid = threadIdx.x;
+    const int lane = tid & (TPK_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
+    unsigned* const live = live_all + wave * FPS_LIVE_CAPACITY;
+    const int steps = (cells + FPS_THREADS - 1) / FPS_THREADS; // cells per lane
+    const unsigned bs_mask = (1u << log2_bs) - 1u;
+    auto tie_key = [&](unsigned k) __attribute__((always_inline)) {
+        const unsigned rev = log2_bs ? (__brev(k & bs_mask) >> (32 - log2_bs)) : 0u;
+        return rev * static_cast<unsigned>(groups) + (k >> log2_bs);
+    };
+
+    // Set-up: minima, boxes and largest minima (best points are found by the first update: it reaches every cell).
+    for (int c = wave; c < cells; c += FPS_WAVES)
+    {
+        const float4 r = sorted[c * NG_CELL + lane];
+        const bool takes_part = __float_as_int(r.w) != 0x7FFFFFFF && eligible(r.x, r.y, r.z);
+        temp[c * NG_CELL + lane] = takes_part ? 1e10f : -1.0f;
+        const bool any = __ballot(takes_part) != 0;
+        if (lane < 6)
+        {
+            const float4 b = boxes[c * NG_BOX + lane / 3];
+            const int a = lane % 3;
+            box[lane * cells + c] = a == 0 ? b.x : a == 1 ? b.y : b.z;
+        }
+        if (lane == 6)
+        {
+            cell_max[c] = ordered_bits(any ? 1e10f : -1.0f);
+            cell_tie[c] = 0xFFFFFFFFu;
+            cell_max2[c] = ordered_bits(-1.0f);
+            cell_tie2[c] = 0xFFFFFFFFu;
+        }
+    }
+    const float p0x = xyz[0], p0y = xyz[1], p0z = xyz[2];
+    if (tid == 0)
+    {
+        out[0] = 0;
+        taken[0][0] = make_float4(p0x, p0y, p0z, 0.f);
+    }
+    __syncthreads();
+
+    // Rounds in which only one point follows cost more this way than with one sample per round (two barriers
+    // more, second bests): from the second such round in a row on, the next 1, 2, 4 .. 32 rounds take one sample
+    // each, the plain way.
+    int ns = 1, j = 1, pause = 0, penalty = 0;
+    float4 fetched = taken[0][0]; // lane k < ns: sample k of the round before
+    for (int round = 1; j < npoint; ++round)
+    {
+        const int par = round & 1;
+        // 1. the live cells among this wavefront's, and which of the round before's samples reach each
+        int count = 0;
+        for (int step = 0; step < steps; ++step)
+        {
+            const int c = (step * TPK_WAVE + lane) * FPS_WAVES + wave;
+            unsigned reach = 0;
+            if (c < cells)
+            {
+                const float lx = box[0 * cells + c], ly = box[1 * cells + c], lz = box[2 * cells + c];
+                const float hx = box[3 * cells + c], hy = box[4 * cells + c], hz = box[5 * cells + c];
+                const float most = __int_as_float(cell_max[c]);
+                for (int k = 0; k < ns; ++k)
+                {
+                    const float sx = tpk_read_lane(fetched.x, k), sy = tpk_read_lane(fetched.y, k), sz = tpk_read_lane(fetched.z, k);
+                    const float dx = fmaxf(fmaxf(lx - sx, sx - hx), 0.f);
+                    const float dy = fmaxf(fmaxf(ly - sy, sy - hy), 0.f);
+                    const float dz = fmaxf(fmaxf(lz - sz, sz - hz), 0.f);
+                    const float lb = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz));
+                    reach |= lb * 0.999998f < most ? 1u << k : 0u;
+                }
+            }
+            const unsigned long long mask = __ballot(reach != 0);
+            if (reach != 0)
+                live[count + tpk_prefix_count(mask)] = static_cast<unsigned>(c) | (reach << 16);
+            count += __builtin_popcountll(mask);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
+        // 2. their points: new minima, and the cell's best and second best point
+        for (int i0 = 0; i0 < count; i0 += FPC_CELL_BATCH)
+        {
+            unsigned entry[FPC_CELL_BATCH];
+            float4 r[FPC_CELL_BATCH];
+            float m[FPC_CELL_BATCH];
+#pragma unroll
+            for (int u = 0; u < FPC_CELL_BATCH; ++u)
+            {
+                entry[u] = __builtin_amdgcn_readfirstlane(live[min(i0 + u, count - 1)]);
+                const int c = static_cast<int>(entry[u] & 0xFFFFu);
+                r[u] = sorted[c * NG_CELL + lane];
+                m[u] = temp[c * NG_CELL + lane];
+            }
+#pragma unroll
+            for (int u = 0; u < FPC_CELL_BATCH; ++u)
+            {
+                if (i0 + u >= count) // wave-uniform
+                    break;
+                const int c = static_cast<int>(entry[u] & 0xFFFFu);
+                const int old_bits = ordered_bits(m[u]);
+                int new_bits = old_bits;
+                for (unsigned reach = entry[u] >> 16; reach != 0; reach &= reach - 1)
+                {
+                    const int k = __builtin_ctz(reach);
+                    const float d = tpk_dist2(r[u].x, r[u].y, r[u].z, tpk_read_lane(fetched.x, k), tpk_read_lane(fetched.y, k),
+                                              tpk_read_lane(fetched.z, k));
+                    new_bits = min(ordered_bits(d), new_bits); // -1 stays -1
+                }
+                if (new_bits != old_bits)
+                    temp[c * NG_CELL + lane] = __int_as_float(new_bits);
+                const unsigned k = static_cast<unsigned>(__float_as_int(r[u].w));
+                const unsigned tk = tie_key(k);
+                int first_val, second_val;
+                const int first = winning_lane(new_bits, tk, first_val);
+                const int second = winning_lane(lane == first ? INT_MIN : new_bits, tk, second_val);
+                if (lane == first)
+                {
+                    cell_max[c] = first_val;
+                    cell_tie[c] = tk;
+                    cell_best[c] = make_float4(r[u].x, r[u].y, r[u].z, __int_as_float(static_cast<int>(k)));
+                }
+                if (lane == second)
+                {
+                    cell_max2[c] = second_val;
+                    cell_tie2[c] = tk;
+                }
+            }
+        }
+
+        // 3. the two best of this wavefront's cells, and the best of what it keeps to itself: per lane the best
+        // cell (b1) and the best of everything else the lane knows of (b2: its other cells' best points and all
+        // its cells' second best points)
+        int b1v = INT_MIN, b2v = INT_MIN, b1c = 0;
+        unsigned b1t = 0xFFFFFFFFu, b2t = 0xFFFFFFFFu;
+        if (pause > 0) // wave-uniform, the same in all wavefronts
+        {
+            for (int step = 0; step < steps; ++step)
+            {
+                const int c = (step * TPK_WAVE + lane) * FPS_WAVES + wave;
+                if (c < cells)
+                {
+                    const int v = cell_max[c];
+                    const unsigned t = cell_tie[c];
+                    if (fps_above(v, t, b1v, b1t))
+                    {
+                        b1v = v;
+                        b1t = t;
+                        b1c = c;
+                    }
+                }
+            }
+            int v1, all_v;
+            const int l1 = winning_lane(b1v, b1t, v1);
+            const unsigned t1 = __builtin_amdgcn_readlane(b1t, l1);
+            const float4 mine = cell_best[__builtin_amdgcn_readlane(b1c, l1)];
+            if (lane == 0)
+            {
+                cand_val[par][wave] = v1;
+                cand_tie[par][wave] = t1;
+                lone[par][wave] = mine;
+            }
+            lds_barrier();
+            const int wl = winning_lane(lane < FPS_WAVES ? cand_val[par][lane] : INT_MIN,
+                                        lane < FPS_WAVES ? cand_tie[par][lane] : 0xFFFFFFFFu, all_v);
+            fetched = lone[par][wl];
+            if (all_v < 0) // no eligible point in the whole cloud: the reference's reduction yields index 0
+                fetched = make_float4(p0x, p0y, p0z, 0.f);
+            if (tid == 0)
+                out[j] = __float_as_int(fetched.w);
+            ns = 1;
+            j += 1;
+            --pause;
+            continue;
+        }
+        for (int step = 0; step < steps; ++step)
+        {
+            const int c = (step * TPK_WAVE + lane) * FPS_WAVES + wave;
+            if (c < cells)
+            {
+                const int v = cell_max[c], v2 = cell_max2[c];
+                const unsigned t = cell_tie[c], t2 = cell_tie2[c];
+                if (fps_above(v, t, b1v, b1t))
+                {
+                    b2v = b1v;
+                    b2t = b1t;
+                    b1v = v;
+                    b1t = t;
+                    b1c = c;
+                }
+                else if (fps_above(v, t, b2v, b2t))
+                {
+                    b2v = v;
+                    b2t = t;
+                }
+                if (fps_above(v2, t2, b2v, b2t))
+                {
+                    b2v = v2;
+                    b2t = t2;
+                }
+            }
+        }
+        {
+            int v1, v2, v3 = INT_MIN;
+            const int l1 = winning_lane(b1v, b1t, v1);
+            const unsigned t1 = __builtin_amdgcn_readlane(b1t, l1);
+            const int c1 = __builtin_amdgcn_readlane(b1c, l1);
+            const int left_v = lane == l1 ? b2v : b1v;
+            const unsigned left_t = lane == l1 ? b2t : b1t;
+            const int l2 = winning_lane(left_v, left_t, v2);
+            const unsigned t2 = __builtin_amdgcn_readlane(left_t, l2);
+            const int c2 = __builtin_amdgcn_readlane(b1c, l2);
+            const bool two = l2 != l1; // (else the second best is something of the first lane's: not published)
+            unsigned t3 = 0xFFFFFFFFu;
+            if (two)
+            {
+                const int rest_v = (lane == l1 || lane == l2) ? b2v : b1v;
+                const unsigned rest_t = (lane == l1 || lane == l2) ? b2t : b1t;
+                const int l3 = winning_lane(rest_v, rest_t, v3);
+                t3 = __builtin_amdgcn_readlane(rest_t, l3);
+            }
+            if (lane == 0)
+            {
+                cand_val[par][wave * 2 + 0] = v1;
+                cand_tie[par][wave * 2 + 0] = t1;
+                cand_cell[par][wave * 2 + 0] = c1;
+                cand_val[par][wave * 2 + 1] = two ? v2 : INT_MIN;
+                cand_tie[par][wave * 2 + 1] = two ? t2 : 0xFFFFFFFFu;
+                cand_cell[par][wave * 2 + 1] = two ? c2 : 0;
+                kept_val[par][wave] = two ? v3 : v2;
+                kept_tie[par][wave] = two ? t3 : t2;
+            }
+        }
+        lds_barrier();
+
+        // 4. the list is sorted out by all wavefronts together.  First every wavefront finds the places of its own
+        // published points among all of them (lane (c, o): is point o above my point c?).
+        {
+            const int c = lane / FPC_CANDS, o = lane % FPC_CANDS;
+            const int mine = wave * FPC_PUB + (c < FPC_PUB ? c : 0);
+            const int mv = cand_val[par][mine], ov = cand_val[par][o];
+            const unsigned mt = cand_tie[par][mine], ot = cand_tie[par][o];
+            // (points that are not published are all alike: the lower number first)
+            const bool higher = fps_above(ov, ot, mv, mt) || (ov == mv && ot == mt && o < mine);
+            const unsigned long long above = __ballot(c < FPC_PUB && higher);
+            if (o == 0 && c < FPC_PUB)
+                order[par][__builtin_popcountll((above >> (c * FPC_CANDS)) & ((1ull << FPC_CANDS) - 1ull))] = mine;
+        }
+        lds_barrier();
+        // Then wavefront k looks at the point of place k: the point of place 0 is the reference's choice; a later
+        // one may follow when it is above everything unpublished and none of the points before it changes its
+        // minimum (lane i: point i).
+        if (wave < FPC_T)
+        {
+            const int at = order[par][wave], before = order[par][lane < wave ? lane : 0];
+            const int val = cand_val[par][at];
+            const unsigned tie = cand_tie[par][at];
+            float4 rec = cell_best[cand_cell[par][at]];
+            const float4 earlier = cell_best[cand_cell[par][before]];
+            int kept_v;
+            const int hv = lane < FPS_WAVES ? kept_val[par][lane] : INT_MIN;
+            const unsigned ht = lane < FPS_WAVES ? kept_tie[par][lane] : 0xFFFFFFFFu;
+            const int kl = winning_lane(hv, ht, kept_v);
+            const unsigned kept_t = __builtin_amdgcn_readlane(ht, kl);
+            const bool spoiled = lane < wave && ordered_bits(tpk_dist2(rec.x, rec.y, rec.z, earlier.x, earlier.y, earlier.z)) < val;
+            // (its minimum must be above 0: the samples before it drop to 0 and keep their tie keys)
+            const bool may = wave == 0 || (__ballot(spoiled) == 0ull && fps_above(val, tie, kept_v, kept_t) && val > 0);
+            if (wave == 0 && val < 0) // no eligible point in the whole cloud: the reference's reduction yields index 0
+                rec = make_float4(p0x, p0y, p0z, 0.f);
+            if (lane == 0)
+            {
+                taken[par][wave] = rec;
+                follows[par][wave] = may ? 1 : 0;
+            }
+        }
+        lds_barrier();
+        int accept = static_cast<int>(__builtin_ctzll(~__ballot(lane < FPC_T && follows[par][lane < FPC_T ? lane : 0] != 0)));
+        accept = min(accept, npoint - j); // (>= 1: the point of place 0 always follows)
+        if (wave == 0 && lane < accept)
+            out[j + lane] = __float_as_int(taken[par][lane].w);
+        fetched = taken[par][lane < accept ? lane : 0];
+        ns = accept;
+        j += accept;
+        if (accept > 1)
+            penalty = 0;
+        else
+        {
+            pause = penalty;
+            penalty = penalty ? min(2 * penalty, 32) : 1;
+        }
+    }
+}
+
 // Clouds too large for registers: points and running minima stream from global memory.
 __global__ __launch_bounds__(FPS_THREADS) void fps_streaming_kernel(
     int n, int npoint, int log2_bs, int groups, const float* __restrict__ xyz,
@@ -1269,11 +1610,17 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
         int st = launch_curve_cells(cloud, none, nullptr, s);
         if (st != TPK_OK)
             return st;
+#ifdef FPS_ONE_PER_ROUND
         const size_t lds = static_cast<size_t>(l.cells) * 48 + FPS_LIVE_CAPACITY * FPS_WAVES * sizeof(unsigned short);
-        st = tpk_allow_lds(reinterpret_cast<const void*>(fps_cells_kernel), lds);
+        auto kernel = fps_cells_kernel;
+#else
+        const size_t lds = static_cast<size_t>(l.cells) * 56 + FPS_LIVE_CAPACITY * FPS_WAVES * sizeof(unsigned);
+        auto kernel = fps_cells_batched_kernel;
+#endif
+        st = tpk_allow_lds(reinterpret_cast<const void*>(kernel), lds);
         if (st != TPK_OK)
             return st;
-        hipLaunchKernelGGL(fps_cells_kernel, dim3(b), dim3(FPS_THREADS), lds, s, n, npoint, log2_bs, groups, l.cells,
+        hipLaunchKernelGGL(kernel, dim3(b), dim3(FPS_THREADS), lds, s, n, npoint, log2_bs, groups, l.cells,
                            xyz, cloud.sorted, cloud.boxes, reinterpret_cast<float*>(w + l.temp), idx_out);
     }
     else
