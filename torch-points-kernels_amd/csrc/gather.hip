@@ -147,17 +147,37 @@ __global__ __launch_bounds__(G_THREADS) void gather_fwd_lds_kernel(
     const int c0 = rb * rows_per_block;
     const int nrows = min(rows_per_block, c - c0);
 
-    const float* __restrict__ s = src + (static_cast<int64_t>(cloud) * c + c0) * m;
-    stage_copy(rows, s, static_cast<unsigned>(nrows) * static_cast<unsigned>(m));
-    __syncthreads();
-
     idx += static_cast<int64_t>(cloud) * n * K;
     if (WEIGHTED)
         weight += static_cast<int64_t>(cloud) * n * K;
     float* __restrict__ o = out + (static_cast<int64_t>(cloud) * c + c0) * n;
-
     const int64_t jbeg = static_cast<int64_t>(jpart) * jlen;
     const int64_t jend = tpk_min64(n, jbeg + jlen);
+    const float* __restrict__ s = src + (static_cast<int64_t>(cloud) * c + c0) * m;
+
+    if (WEIGHTED)
+    {
+        // Bound by the random LDS reads: a column's indices and weights are requested one column ahead, the
+        // first before the rows are staged, so that no lane waits for them between its reads.
+        int64_t j = jbeg + threadIdx.x;
+        Column<K, WEIGHTED, IdxT> next;
+        if (j < jend)
+            next.load(idx, weight, j);
+        stage_copy(rows, s, static_cast<unsigned>(nrows) * static_cast<unsigned>(m));
+        __syncthreads();
+        for (; j < jend; j += G_THREADS)
+        {
+            const Column<K, WEIGHTED, IdxT> col = next;
+            next.load(idx, weight, tpk_min64(j + G_THREADS, jend - 1));
+#pragma unroll
+            for (int r = 0; r < G_MAX_ROWS; ++r)
+                if (r < nrows)
+                    o[static_cast<int64_t>(r) * n + j] = col.combine(rows + r * m);
+        }
+        return;
+    }
+    stage_copy(rows, s, static_cast<unsigned>(nrows) * static_cast<unsigned>(m));
+    __syncthreads();
     for (int64_t j = jbeg + threadIdx.x; j < jend; j += G_THREADS)
     {
         Column<K, WEIGHTED, IdxT> col;
