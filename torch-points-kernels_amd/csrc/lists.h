@@ -280,18 +280,30 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
     // entry that takes the last one knows that it ends the list.
     int2* const queue = reinterpret_cast<int2*>(below_total + 2) + wave * L_QUEUE;
     int queued = 0, placed = 0; // (wave-uniform)
+    // An entry's weight is a trip to memory: the 64 entries taken from the queue wait for theirs while the next
+    // ones are queued, and go to their places when the queue has filled again (or at the end).
+    bool waiting = false; // per lane: an entry taken from the queue, not yet placed
+    int waiting_rank = 0, waiting_target = 0;
+    ListEntry<WEIGHTED> waiting_entry;
+    auto place_waiting = [&]() {
+        if (waiting)
+            place(waiting_rank, waiting_target, waiting_entry);
+        waiting = false;
+    };
     auto place_queued = [&](int count) {
+        place_waiting();
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         if (lane < count)
         {
             const int2 item = queue[(placed + lane) & (L_QUEUE - 1)];
             const int e = item.x, t = item.y - i0;
             const int left = atomicSub(&counters[t], 1); // places free before this entry took one
-            ListEntry<WEIGHTED> entry;
-            entry.j = ((e / K) * 4) | (left == 1 ? L_LAST : 0);
+            waiting_entry.j = ((e / K) * 4) | (left == 1 ? L_LAST : 0);
             if constexpr (WEIGHTED)
-                entry.w = weight[e];
-            place(ends[t] - left, item.y, entry);
+                waiting_entry.w = weight[e];
+            waiting_rank = ends[t] - left;
+            waiting_target = item.y;
+            waiting = true;
         }
         placed += count;
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -327,6 +339,7 @@ __global__ __launch_bounds__(G_THREADS) void build_lists_kernel(ListJob<WEIGHTED
             enqueue(e0 + u * G_THREADS, iv[u]);
     }
     place_queued(queued - placed);
+    place_waiting();
 }
 
 // Describes the job of building the lists of `clouds` clouds of `m` targets and `cloud_total`
