@@ -185,7 +185,8 @@ __global__ __launch_bounds__(G_THREADS) void gather_fwd_lds_kernel(
 #pragma unroll
         for (int r = 0; r < G_MAX_ROWS; ++r)
             if (r < nrows)
-                o[static_cast<int64_t>(r) * n + j] = col.combine(rows + r * m);
+                // (written once, read by nobody here: past the caches, -3 % on config 3b)
+                __builtin_nontemporal_store(col.combine(rows + r * m), &o[static_cast<int64_t>(r) * n + j]);
     }
 }
 
