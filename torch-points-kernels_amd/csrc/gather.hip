@@ -37,6 +37,7 @@ namespace {
 
 constexpr int G_MAX_ROWS = 8;
 constexpr int G_LDS_BUDGET = 131072; // bytes of LDS for the staged rows
+constexpr int G_PLAIN_BLOCKS = 1024; // workgroups the plain gather aims at (four per compute unit, two at a time)
 
 template <int K, bool WEIGHTED, typename IdxT>
 struct Column
@@ -575,13 +576,21 @@ int gather_fwd(int b, int c, int m, int64_t n, const float* src, const IdxT* idx
         return TPK_ERR_INVALID_ARG; // columns to fill but nothing to gather from
     if (!src || !idx || !out || (WEIGHTED && !weight))
         return TPK_ERR_INVALID_ARG;
-    const int r = rows_for(m, c);
+    int r = rows_for(m, c);
+    // The plain gather is bound by its stores and gains from two workgroups per compute unit that stage and store
+    // at different times, and from row blocks that are not split by columns (every split stages the rows again):
+    // fewer rows per workgroup while that gives more workgroups, down to two rows (with one row the indices, read
+    // once per row block, become the larger stream).  Config 3b: 8 rows x 2 column parts 62 us, 4 rows 59, 2 rows 55,
+    // 1 row 78.
+    if (!WEIGHTED)
+        while (r > 2 && static_cast<int64_t>(b) * tpk_ceil_div(c, r) < G_PLAIN_BLOCKS)
+            r = (r + 1) / 2;
     if (r > 0)
     {
         const int row_blocks = static_cast<int>(tpk_ceil_div(c, r));
         // Split the columns so that a few hundred workgroups exist, but keep each part at
         // least as long as a row (so staging a row block stays the smaller share of traffic).
-        int64_t jsplit = tpk_ceil_div(WEIGHTED ? 256 : 512, static_cast<int64_t>(row_blocks) * b);
+        int64_t jsplit = tpk_ceil_div(WEIGHTED ? 256 : G_PLAIN_BLOCKS, static_cast<int64_t>(row_blocks) * b);
         const int64_t max_split = n / (m > G_THREADS ? m : G_THREADS);
         if (jsplit > max_split)
             jsplit = max_split;
@@ -594,7 +603,7 @@ int gather_fwd(int b, int c, int m, int64_t n, const float* src, const IdxT* idx
         const size_t lds = static_cast<size_t>(r) * m * sizeof(float);
         // Measured on MI355X: the weighted 3-neighbour gather (LDS-read bound) is fastest with one
         // workgroup per compute unit and die-local cloud placement; the plain gather (store
-        // bound) with two rounds of workgroups and the default placement.
+        // bound) with two workgroups per compute unit at a time and the default placement.
         auto kernel = gather_fwd_lds_kernel<K, WEIGHTED, IdxT, WEIGHTED>;
         int st = allow_lds(kernel, lds);
         if (st != TPK_OK)
