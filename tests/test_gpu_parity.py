@@ -321,6 +321,8 @@ def test_ball_query_full_config4(tpk, oracle, dev):
         (tuple([50] * 200), 0.04, 0.3, 16),         # two queries per cloud: 32 clouds among 64 consecutive queries
         ((40000,), 0.3, 0.012, 32),                 # most balls hold the query point only
         ((90000, 20000), 0.05, 0.04, 32),           # 6 windows x 27 bins: more (window, bin) pairs than lanes
+        ((500000, 24288), 0.002, 0.01, 16),         # 64 windows of 8192 rows, 62 of them one cloud's
+        ((330000, 200000), 0.002, 0.01, 16),        # more rows than 64 windows of 8192: windows of 16384
     ],
 )
 def test_ball_query_partial_cell_search_parity(tpk, oracle, dev, sizes, qfrac, r, ns):

@@ -726,7 +726,7 @@ constexpr int NG_RUN = 16; // consecutive cells that share a second-level box in
 // ---------------------------------------------------------------------------------------
 // Ball query over bins, packed layout (several clouds back to back, sorted cloud id per point).
 //
-// The support array is cut into windows of CURVE_MAX_POINTS consecutive rows, each ordered on its
+// The support array is cut into windows of 8192 or 16384 (bqb_window_shift) consecutive rows, each ordered on its
 // own (curve_cells_kernel), which groups a window's points by the cell of a 16^3 grid over the
 // window's bounding box; the ordering kernel also leaves where each such bin ends.  One
 // wavefront serves one query: it reads which support rows belong to the query's cloud (found for
@@ -742,6 +742,16 @@ constexpr int NG_RUN = 16; // consecutive cells that share a second-level box in
 // serial scan itself, 64 rows per step with early exit: those are the dense
 // neighbourhoods, where the scan ends soon.
 // ---------------------------------------------------------------------------------------
+// Rows per window of the packed ball query, as a shift.  Windows of 8192 rows are ordered faster and by twice as
+// many workgroups (config 4: 15 windows of 16384 rows leave most of the chip idle while they are ordered: 61 ->
+// 57 us with 8192, 58 with 4096); a lane per window limits a cloud to 64 windows, so arrays above 64 x 8192 rows
+// keep windows of 16384.
+constexpr int BQB_SMALL_SHIFT = 13;
+inline int bqb_window_shift(int64_t size_x)
+{
+    return size_x <= (static_cast<int64_t>(TPK_WAVE) << BQB_SMALL_SHIFT) ? BQB_SMALL_SHIFT : 14;
+}
+static_assert((1 << 14) == CURVE_MAX_POINTS, "the larger window is what the ordering kernel holds at most");
 constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
 
 // Range of 16^3-grid cells along one axis that [v - r, v + r] can touch.  The interval is widened
@@ -759,7 +769,7 @@ __device__ __forceinline__ void bin_range(float v, float r, float lo, float scal
 // further down does with the points of a cell).
 template <bool SORTED>
 __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
-    int size_x, int size_y, float radius, float radius2, int nsample, const float* __restrict__ x,
+    int size_x, int size_y, int window_shift, float radius, float radius2, int nsample, const float* __restrict__ x,
     const float* __restrict__ y, const float4* __restrict__ sorted_x, const int* __restrict__ bin_ends,
     const float4* __restrict__ grids, const int2* __restrict__ cloud_rows, int64_t* __restrict__ idx,
     float* __restrict__ dist)
@@ -800,8 +810,8 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
         best = wave_merge_ascending(best < cand ? best : cand, lane);
         admit = read_lane_key(best, nsample - 1);
     };
-    const int wx0 = s0 / CURVE_MAX_POINTS;
-    const int windows = s1 > s0 ? (s1 - 1) / CURVE_MAX_POINTS - wx0 + 1 : 0;
+    const int wx0 = s0 >> window_shift;
+    const int windows = s1 > s0 ? ((s1 - 1) >> window_shift) - wx0 + 1 : 0;
     bool serial = windows > TPK_WAVE; // answer by the scan in index order instead
     if (!serial && windows > 0)
     {
@@ -850,7 +860,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 const int* __restrict__ ends = bin_ends + static_cast<int64_t>(wx) * CURVE_BINS;
                 start = bin ? ends[bin - 1] : 0;
                 size = ends[bin] - start;
-                start += wx * CURVE_MAX_POINTS;
+                start += wx << window_shift;
             }
             const int before = wave_exclusive_sum(size);
             const int total = __builtin_amdgcn_readlane(before + size, TPK_WAVE - 1);
@@ -1405,11 +1415,12 @@ struct BallLayout
 BallLayout ball_layout(int64_t size_x, int64_t size_y)
 {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
-    const size_t wx = static_cast<size_t>((size_x + CURVE_MAX_POINTS - 1) / CURVE_MAX_POINTS);
+    const size_t window = static_cast<size_t>(1) << bqb_window_shift(size_x);
+    const size_t wx = (static_cast<size_t>(size_x) + window - 1) / window;
     BallLayout l;
     size_t pos = 0;
     l.sorted_x = pos;
-    pos = up(pos + wx * CURVE_MAX_POINTS * sizeof(float4));
+    pos = up(pos + wx * window * sizeof(float4));
     l.bin_ends = pos;
     pos = up(pos + wx * CURVE_BINS * sizeof(int));
     l.grids = pos;
@@ -1445,7 +1456,8 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
     // (cloud ids are not used for the order: bins may mix the clouds of a window, rows tell them apart)
-    PointSet px{x, nullptr, size_x, size_x, CURVE_MAX_POINTS, reinterpret_cast<float4*>(w + l.sorted_x), nullptr,
+    const int window_shift = bqb_window_shift(size_x);
+    PointSet px{x, nullptr, size_x, size_x, 1 << window_shift, reinterpret_cast<float4*>(w + l.sorted_x), nullptr,
                 reinterpret_cast<int*>(w + l.bin_ends), reinterpret_cast<float4*>(w + l.grids)};
     PointSet none{nullptr, nullptr, 0, 1, CURVE_MAX_POINTS, nullptr, nullptr, nullptr, nullptr};
     const CloudRows rows{batch_x, batch_y, static_cast<int>(size_x), size_y, reinterpret_cast<int2*>(w + l.cloud_rows)};
@@ -1458,11 +1470,11 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
         return TPK_ERR_UNSUPPORTED;
     if (sorted)
         hipLaunchKernelGGL(ball_query_bins_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
-                           static_cast<int>(size_x), static_cast<int>(size_y), std::fabs(radius), radius2, nsample, x, y,
+                           static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
                            px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
     else
         hipLaunchKernelGGL(ball_query_bins_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
-                           static_cast<int>(size_x), static_cast<int>(size_y), std::fabs(radius), radius2, nsample, x, y,
+                           static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
                            px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
     return tpk_launch_status();
 }
