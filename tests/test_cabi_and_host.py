@@ -109,8 +109,10 @@ def test_library_exports_every_declared_symbol():
     lib.tpk_ball_query_partial_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
     assert lib.tpk_ball_query_partial_workspace_bytes(8191, 100, 16) == 0
     assert lib.tpk_ball_query_partial_workspace_bytes(40000, 100, 0) == 0
-    windows = 3  # 40000 support points in windows of 16384
-    assert lib.tpk_ball_query_partial_workspace_bytes(40000, 100, 16) == windows * (16384 * 16 + 4096 * 4) + 256 + 1024  # + the queries' cloud rows, 8 bytes each
+    windows = 5  # 40000 support points in windows of 8192 (arrays of at most 64 such windows)
+    assert lib.tpk_ball_query_partial_workspace_bytes(40000, 100, 16) == windows * (8192 * 16 + 4096 * 4) + 256 + 1024  # + the queries' cloud rows, 8 bytes each
+    windows = 37  # 600000 support points: windows of 16384
+    assert lib.tpk_ball_query_partial_workspace_bytes(600000, 100, 16) == windows * (16384 * 16 + 4096 * 4) + 1280 + 1024
 
 
 def test_argument_errors_are_reported_without_a_gpu():
