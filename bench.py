@@ -224,8 +224,11 @@ def _all_pairs_entry(call, pairs, steps, warmup, valu_kernel):
     executed = _executed(call)
     roof = _roof_flops(executed, pairs, 8, ev)
     table, commit = _profile_table(VALU_FILE, ("VALUBusy", "VALUUtilization"))
-    if valu_kernel in table:
-        roof["valu"] = {"valu_busy_pct": table[valu_kernel].get("VALUBusy"),
+    # the instance a launch picks depends on the sizes: take whichever of the named instances the summary holds
+    names = [k for k in ((valu_kernel,) if isinstance(valu_kernel, str) else valu_kernel) if k in table]
+    if names:
+        valu_kernel = names[0]
+        roof["valu"] = {"kernel": valu_kernel, "valu_busy_pct": table[valu_kernel].get("VALUBusy"),
                         "valu_lane_utilisation_pct": table[valu_kernel].get("VALUUtilization"),
                         "source": "profiles/" + os.path.basename(VALU_FILE), "measured_at_commit": commit}
     return {"what": "the same configuration through the C ABI's scan of all pairs (workspace == NULL; three_nn: "
@@ -438,7 +441,7 @@ def bench_others(dev, steps, warmup, with_cpu):
                               "of uneven density (here they return at once)")
     e["all_pairs_kernel"] = _all_pairs_entry(lambda lib, st: lib.tpk_three_nn_all_pairs_f32(
         unknown.shape[0], unknown.shape[1], known.shape[1], _p(unknown), _p(known), _p(nn_d), _p(nn_i), st),
-        pairs, max(3, steps // 4), 1, "three_nn_kernel<4>")
+        pairs, max(3, steps // 4), 1, ("three_nn_kernel<1>", "three_nn_kernel<2>", "three_nn_kernel<4>"))
     if ref is not None:
         sub = 4  # clouds
         secs = _cpu_time(lambda: ref.dense_knn(w["known"][:sub], w["unknown"][:sub], 3))
@@ -664,6 +667,130 @@ def bench_others(dev, steps, warmup, with_cpu):
     return out
 
 
+def headline_object(fps, steps, warmup, device):
+    """The full record of a run: the headline keys, the headline's roofline and cpu_baseline objects with their
+    prose, and (added by the caller) the per-operator entries under "ops"."""
+    full = {
+        "metric": "furthest_point_sample ms/batch",
+        "value": fps["wall_ms"],
+        "unit": "ms/batch",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": fps["wall_ms"],
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: furthest_point_sample B=16 clouds x N=16384 points (8 Gaussian clusters "
+                               "sigma=0.05 + 10% uniform), npoint=4096, start index 0, int32 out"},
+        "roofline": fps["roofline"],
+        "kernel_ms": fps["kernel_ms"],
+        "device": device,
+    }
+    if "cpu_baseline" in fps:
+        full["cpu_baseline"] = fps["cpu_baseline"]
+    return full
+
+
+DETAIL_FILE = os.path.join("gpurun_out", "bench_full.json")
+LINE_LIMIT = 4096  # bytes of the printed line; whoever runs this script may keep only the end of its output
+
+
+def _write_detail(full):
+    """Writes the full record (every operator with its workload text, notes and sources) next to the other
+    results of a GPU run; returns the path relative to the repository, or None when it cannot be written."""
+    try:
+        os.makedirs(os.path.join(ROOT, os.path.dirname(DETAIL_FILE)), exist_ok=True)
+        with open(os.path.join(ROOT, DETAIL_FILE), "w") as f:
+            json.dump(full, f, indent=1)
+        return DETAIL_FILE
+    except OSError:
+        return None
+
+
+def _sig(x, digits=4):
+    """Numbers to `digits` significant digits (a printed line, not an archive)."""
+    if isinstance(x, float):
+        return float("%.*g" % (digits, x))
+    return x
+
+
+def _compact_roofline(r):
+    keep = ("bound", "achieved", "peak", "unit", "frac", "traffic", "executed_pairs", "algorithmic_pairs",
+            "algorithmic_rate")
+    out = {k: _sig(r[k]) for k in keep if k in r}
+    if r.get("bound") == "mfma":
+        out["bound_detail"] = "fp32 VALU, unfused (no MFMA: inner dimension 3)"
+    valu = r.get("valu")
+    if valu:
+        out["valu"] = {"busy_pct": _sig(valu.get("valu_busy_pct")), "lanes_pct": _sig(valu.get("valu_lane_utilisation_pct"))}
+    return out
+
+
+def _compact_op(e):
+    """One operator as a row of the printed table: kernel ms (HIP events), roofline fraction of EXECUTED work
+    (or of algorithmic bytes), the algorithmic fraction for the pruned distance scans, measured HBM traffic
+    over algorithmic bytes, and the CPU figure in the operator's own unit."""
+    row = {"ms": _sig(e.get("kernel_ms"))}
+    if "value" in e:
+        row["v"] = _sig(e["value"], 3)
+        row["unit"] = e.get("metric")
+    r = e.get("roofline")
+    if r:
+        row["bound"] = "valu" if r.get("bound") == "mfma" else r.get("bound")
+        row["frac"] = _sig(r.get("frac"), 3)
+        if "algorithmic_rate" in r:
+            row["alg_frac"] = _sig(r["algorithmic_rate"] / r["peak"], 3)
+        if r.get("traffic") and e.get("algorithmic_bytes"):
+            row["traffic_x"] = _sig(r["traffic"] / e["algorithmic_bytes"], 3)
+    ap = e.get("all_pairs_kernel")
+    if ap:
+        row["all_pairs"] = {"ms": _sig(ap["kernel_ms"]), "frac": _sig(ap["roofline"]["frac"], 3)}
+    c = e.get("cpu_baseline")
+    if c:
+        row["cpu"] = _sig(c["value"], 3)
+        if c["unit"] != e.get("metric"):
+            row["cpu_unit"] = c["unit"]
+    return row
+
+
+# Operators of the BASELINE configurations first; the others leave the printed line first when it is too long.
+OPS_ORDER = ("ball_query_dense", "ball_query_partial_dense", "three_nn", "three_interpolate_fwd", "three_interpolate_bwd",
+             "grouping_fwd", "grouping_bwd", "chamfer_fwd", "chamfer_bwd", "ball_query_dense_sorted",
+             "ball_query_partial_dense_sorted", "knn_k16", "grow_proximity", "instance_iou", "gridding_fwd", "gridding_bwd",
+             "cubic_feature_sampling_fwd", "cubic_feature_sampling_bwd")
+
+
+def compact_line(full, detail_file=None, limit=LINE_LIMIT):
+    """The ONE line this script prints, at most `limit` bytes: the headline keys, the headline's roofline and
+    cpu_baseline without prose, and one short row per operator.  Everything else is in the detail file."""
+    line = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                 "higher_is_better", "scaling", "vs_baseline", "dtype", "data") if k in full}
+    line["value"] = _sig(full["value"], 6)
+    line["ms_per_step"] = _sig(full["ms_per_step"], 6)
+    line["value_is"] = "wall clock of the timed steps / steps; ops.*.v likewise (wall-based, in ops.*.unit); ops.*.ms = HIP-event time of the operator's kernels"
+    line["config"] = {"workload": "configs[1]: furthest_point_sample B=16 N=16384 npoint=4096"}
+    line["kernel_ms"] = _sig(full.get("kernel_ms"), 6)
+    line["roofline"] = _compact_roofline(full["roofline"])
+    c = full.get("cpu_baseline")
+    if c:
+        line["cpu_baseline"] = {"value": _sig(c["value"]), "unit": c["unit"], "cores": c["cores"], "kind": c["kind"],
+                                "sample": c["sample"][:96]}
+    if detail_file:
+        line["detail"] = detail_file
+    ops = full.get("ops") or {}
+    names = [n for n in OPS_ORDER if n in ops] + [n for n in ops if n not in OPS_ORDER]
+    line["ops"] = {n: _compact_op(ops[n]) for n in names}
+    text = json.dumps(line, separators=(",", ":"))
+    while len(text) > limit and names:
+        line["ops"].pop(names.pop())
+        line["ops_dropped"] = line.get("ops_dropped", 0) + 1
+        text = json.dumps(line, separators=(",", ":"))
+    return text
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -700,30 +827,11 @@ def main():
 
     with_cpu = not args.no_cpu
     fps = bench_fps(dev, args.steps, args.warmup, with_cpu)
-    line = {
-        "metric": "furthest_point_sample ms/batch",
-        "value": fps["wall_ms"],
-        "unit": "ms/batch",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": fps["wall_ms"],
-        "higher_is_better": False,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": "configs[1]: furthest_point_sample B=16 clouds x N=16384 points (8 Gaussian clusters "
-                               "sigma=0.05 + 10% uniform), npoint=4096, start index 0, int32 out"},
-        "roofline": fps["roofline"],
-        "kernel_ms": fps["kernel_ms"],
-        "device": torch.cuda.get_device_name(0),
-    }
-    if "cpu_baseline" in fps:
-        line["cpu_baseline"] = fps["cpu_baseline"]
+    full = headline_object(fps, args.steps, args.warmup, torch.cuda.get_device_name(0))
     if args.ops == "all":
-        line["ops"] = bench_others(dev, max(5, args.steps), args.warmup, with_cpu)
-    print(json.dumps(line))
+        full["ops"] = bench_others(dev, max(5, args.steps), args.warmup, with_cpu)
+    detail = _write_detail(full)
+    print(compact_line(full, detail))
 
 
 if __name__ == "__main__":

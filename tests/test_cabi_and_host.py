@@ -235,3 +235,45 @@ def test_product_package_does_not_reference_the_oracle():
             if f.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_bench_line_is_short_and_parses():
+    """bench.py prints ONE line; a harness that keeps only the end of the output must still find all of it.
+    Built here from canned numbers (no GPU): 18 operators with long workload texts and notes."""
+    import json
+
+    import bench
+
+    prose = "x" * 900
+    roof_f = {"bound": "mfma", "achieved": 0.578912345, "peak": 157.3, "unit": "TFLOP/s", "frac": 0.0036801234,
+              "traffic": 3779123.0, "executed_pairs": 86222336, "algorithmic_pairs": 1073479680,
+              "algorithmic_rate": 7.2081234, "algorithmic_speedup": 12.45, "note": prose,
+              "valu": {"valu_busy_pct": 4.3, "valu_lane_utilisation_pct": 75.8, "source": prose, "measured_at_commit": "abc"}}
+    roof_b = {"bound": "hbm", "achieved": 2394.123456, "peak": 8000.0, "unit": "GB/s", "frac": 0.299265432,
+              "traffic": 242912345.0, "traffic_source": prose, "traffic_measured_at_commit": "abc", "note": prose}
+    cpu = {"value": 5894.123456, "unit": "ms/batch", "cores": 16, "kind": "reference", "sample": prose}
+    fps = {"wall_ms": 1.4968812345, "kernel_ms": 1.489371234, "roofline": roof_f, "cpu_baseline": cpu}
+    full = bench.headline_object(fps, 20, 3, "AMD Instinct MI355X")
+    full["ops"] = {}
+    for i, name in enumerate(bench.OPS_ORDER):
+        e = {"workload": prose, "metric": "queries/s", "value": 1.23456789e9, "kernel_ms": 0.0123456789, "wall_ms": 0.02,
+             "roofline": dict(roof_f if i % 2 else roof_b), "algorithmic_bytes": 174063616, "pairs": 1 << 30,
+             "cpu_baseline": dict(cpu, unit="queries/s")}
+        if i % 3 == 0:
+            e["all_pairs_kernel"] = {"what": prose, "kernel_ms": 1.116123, "wall_ms": 1.2, "roofline": dict(roof_f)}
+        full["ops"][name] = e
+    text = bench.compact_line(full, bench.DETAIL_FILE)
+    assert "\n" not in text and len(text) < 4096, len(text)
+    line = json.loads(text)
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in line, key
+    assert line["value"] == line["ms_per_step"] == 1.49688
+    assert set(line["roofline"]) >= {"bound", "achieved", "peak", "unit", "frac", "traffic"}
+    assert line["roofline"]["bound"] in ("hbm", "mfma") and "note" not in line["roofline"]
+    assert set(line["cpu_baseline"]) == {"value", "unit", "cores", "kind", "sample"} and line["cpu_baseline"]["cores"] == 16
+    assert list(line["ops"]) == list(bench.OPS_ORDER) and "ops_dropped" not in line
+    assert line["ops"]["three_interpolate_bwd"]["ms"] == 0.01235
+    # a line that would be too long sheds the operators outside the BASELINE configurations first
+    short = json.loads(bench.compact_line(full, bench.DETAIL_FILE, limit=2600))
+    assert short["ops_dropped"] > 0 and "ball_query_dense" in short["ops"] and "roofline" in short
