@@ -336,3 +336,78 @@ def test_gpu_only_operators_refuse_cpu_tensors(pkg):
         pkg.chamfer_dist.chamfer_dist(torch.rand(1, 4, 3), torch.rand(1, 4, 3))
     with pytest.raises(NotImplementedError):
         pkg.gridding(torch.rand(1, 4, 3) * 2 - 1, 8)
+
+
+def test_edge_list_mode(pkg, ref_cpu):
+    """mode = 1 (cpu/src/neighbors.cpp:107-135, :257-291): edges (support index, query row) with distances (E, 1)."""
+    from torch_points_kernels import points_cpu
+
+    g = torch.Generator().manual_seed(5)
+    support, query = torch.rand(300, 3, generator=g), torch.rand(40, 3, generator=g)
+    query[7] = 5.0  # a query without neighbours
+    idx, dist = points_cpu.ball_query(support, query, 0.15, 6, 0, True)
+    edges, d2 = points_cpu.ball_query(support, query, 0.15, 6, 1, True)
+    assert edges.shape[1] == 2 and d2.shape == (edges.shape[0], 1) and edges.dtype == torch.int64 and d2.dtype == torch.float32
+    want = []
+    for i in range(40):
+        used = int((dist[i] != -1).sum())
+        if used == 0:
+            want.append((0, i, -1.0))  # the reference's stand-in for "no neighbour" is kept as an edge
+        want += [(int(idx[i, j]), i, float(dist[i, j])) for j in range(used)]
+    assert [(int(a), int(b), float(c)) for (a, b), c in zip(edges.tolist(), d2[:, 0].tolist())] == want
+    assert (7 in edges[:, 1].tolist()) and d2[edges[:, 1] == 7, 0].tolist() == [-1.0]
+    x, y = torch.rand(900, 3, generator=g), torch.rand(120, 3, generator=g)
+    y[3] = -4.0
+    bx = torch.sort(torch.randint(0, 3, (900,), generator=g))[0]
+    by = torch.sort(torch.randint(0, 3, (120,), generator=g))[0]
+    idx, dist = points_cpu.batch_ball_query(x, y, bx, by, 0.12, 5, 0, True)
+    edges, d2 = points_cpu.batch_ball_query(x, y, bx, by, 0.12, 5, 1, True)
+    keep = dist != -1
+    rows = torch.arange(120).unsqueeze(1).expand_as(idx)
+    assert torch.equal(edges[:, 0], idx[keep]) and torch.equal(edges[:, 1], rows[keep]) and torch.equal(d2[:, 0], dist[keep])
+    assert 3 not in edges[:, 1].tolist()  # packed layout: a row without neighbours contributes nothing
+    if ref_cpu is not None:
+        for got, want in zip(points_cpu.ball_query(support, query, 0.15, 6, 1, True), ref_cpu.ball_query(support, query, 0.15, 6, 1, True)):
+            assert torch.equal(got, want)
+        for got, want in zip(points_cpu.ball_query(support, query, 0.15, -1, 1, True), ref_cpu.ball_query(support, query, 0.15, -1, 1, True)):
+            assert torch.equal(got, want)
+        for got, want in zip((edges, d2), ref_cpu.batch_ball_query(x, y, bx, by, 0.12, 5, 1, True)):
+            assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_rows_that_are_not_finite(pkg, dtype):
+    """A NaN or infinite coordinate in the support cloud: never a neighbour inside a radius, last among the nearest;
+    every other answer is what the cloud without those rows gives."""
+    g = torch.Generator().manual_seed(21)
+    clean = torch.rand(1, 700, 3, generator=g, dtype=dtype)
+    bad_rows = [0, 5, 333, 699, 700, 701]
+    support = torch.empty(1, 706, 3, dtype=dtype)
+    keep = [i for i in range(706) if i not in bad_rows]
+    support[0, keep] = clean[0, :700]
+    support[0, 0] = torch.tensor([float("nan"), 0.5, 0.5], dtype=dtype)
+    support[0, 5] = torch.tensor([0.5, float("inf"), 0.5], dtype=dtype)
+    support[0, 333] = torch.tensor([float("-inf"), float("nan"), 0.1], dtype=dtype)
+    support[0, 699] = float("nan")
+    support[0, 700] = float("inf")
+    support[0, 701] = torch.tensor([0.2, 0.2, float("-inf")], dtype=dtype)
+    query = torch.rand(1, 90, 3, generator=g, dtype=dtype)
+    remap = torch.tensor(keep)
+    idx, d2 = pkg.knn(support, query, 9)
+    cidx, cd2 = pkg.knn(clean, query, 9)
+    assert torch.equal(idx, remap[cidx]) and torch.equal(d2, cd2)
+    ridx, rd = pkg.ball_query(0.2, 12, support, query, mode="dense", sort=True)
+    cridx, crd = pkg.ball_query(0.2, 12, clean, query, mode="dense", sort=True)
+    hit = crd != -1
+    assert torch.equal(rd, crd) and torch.equal(ridx[hit], remap[cridx][hit])
+    dist, i3 = pkg.three_nn(query, support)
+    cdist, ci3 = pkg.three_nn(query, clean)
+    assert torch.equal(i3.long(), remap[ci3.long()]) and torch.equal(dist, cdist)
+    # more neighbours asked for than finite rows exist: the others follow, in index order
+    few = support[:, :8].clone()
+    idx, d2 = pkg.knn(few, query[:, :4], 8)
+    assert idx[0, :, 6:].tolist() == [[0, 5]] * 4 and not torch.isfinite(d2[0, :, 6:]).any()
+    # a query that is not finite has no neighbour inside any radius
+    q = torch.tensor([[[float("nan"), 0.5, 0.5], [float("inf"), 0.5, 0.5]]], dtype=dtype)
+    ridx, rd = pkg.ball_query(0.5, 4, clean, q, mode="dense", sort=True)
+    assert (rd == -1).all() and (ridx == 0).all()

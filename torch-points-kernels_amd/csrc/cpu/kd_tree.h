@@ -13,6 +13,7 @@
 #pragma once
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <limits>
 #include <vector>
@@ -26,13 +27,20 @@ inline T squared_distance(const T* a, const T* b)
     return (dx * dx + dy * dy) + dz * dz;
 }
 
-// A neighbour candidate; ordered by distance, equal distances by index.
+// A neighbour candidate; ordered by distance, equal distances by index.  A distance that is not a number
+// (a point or query with NaN, or inf - inf) counts as infinite, so that the order stays total: such
+// candidates come last, by index.
 template <typename T>
 struct Neighbour
 {
     T d2;
     int64_t index;
-    bool operator<(const Neighbour& o) const { return d2 < o.d2 || (d2 == o.d2 && index < o.index); }
+    static T rank(T v) { return std::isnan(v) ? std::numeric_limits<T>::infinity() : v; }
+    bool operator<(const Neighbour& o) const
+    {
+        const T a = rank(d2), b = rank(o.d2);
+        return a < b || (a == b && index < o.index);
+    }
 };
 
 template <typename T>
@@ -41,16 +49,23 @@ class KdTree
   public:
     static constexpr int LEAF = 12; // points per leaf
 
-    // points: n rows of (x, y, z); the tree keeps its own reordered copy.
-    KdTree(const T* points, int64_t n) : n_(n)
+    // points: n rows of (x, y, z); the tree keeps its own reordered copy.  Rows with a coordinate that is not
+    // finite stay out of the tree (they cannot be ordered along an axis): they follow the tree's points, in
+    // index order, no radius search ever reports them, and `nearest` offers them after the tree's points.
+    KdTree(const T* points, int64_t n) : n_(n), finite_(0)
     {
         order_.resize(static_cast<size_t>(n));
         for (int64_t i = 0; i < n; ++i)
-            order_[static_cast<size_t>(i)] = i;
-        if (n > 0)
+            if (std::isfinite(points[3 * i]) && std::isfinite(points[3 * i + 1]) && std::isfinite(points[3 * i + 2]))
+                order_[static_cast<size_t>(finite_++)] = i;
+        int64_t at = finite_;
+        for (int64_t i = 0; i < n; ++i)
+            if (!(std::isfinite(points[3 * i]) && std::isfinite(points[3 * i + 1]) && std::isfinite(points[3 * i + 2])))
+                order_[static_cast<size_t>(at++)] = i;
+        if (finite_ > 0)
         {
-            nodes_.reserve(static_cast<size_t>(2 * (n / LEAF + 1)));
-            build(points, 0, n);
+            nodes_.reserve(static_cast<size_t>(2 * (finite_ / LEAF + 1)));
+            build(points, 0, finite_);
         }
         xyz_.resize(static_cast<size_t>(3 * n));
         for (int64_t i = 0; i < n; ++i)
@@ -64,7 +79,7 @@ class KdTree
     template <typename Visit>
     void within(const T* q, T r2, Visit&& visit) const
     {
-        if (n_ == 0)
+        if (finite_ == 0)
             return;
         int stack[64];
         int top = 0;
@@ -103,9 +118,21 @@ class KdTree
             int node;
             T bound; // squared distance to the plane that separates the query from this subtree
         };
+        auto offer = [&](const Neighbour<T>& c) {
+            if (count == k && !(c < best[k - 1]))
+                return;
+            int64_t at = count < k ? count++ : k - 1;
+            while (at > 0 && c < best[at - 1])
+            {
+                best[at] = best[at - 1];
+                --at;
+            }
+            best[at] = c;
+        };
         Pending stack[64];
         int top = 0;
-        stack[top++] = Pending{0, T(0)};
+        if (finite_ > 0)
+            stack[top++] = Pending{0, T(0)};
         while (top > 0)
         {
             const Pending p = stack[--top];
@@ -116,18 +143,7 @@ class KdTree
             if (node.dim < 0)
             {
                 for (int64_t i = node.lo; i < node.hi; ++i)
-                {
-                    const Neighbour<T> c{squared_distance(q, &xyz_[static_cast<size_t>(3 * i)]), order_[static_cast<size_t>(i)]};
-                    if (count == k && !(c < best[k - 1]))
-                        continue;
-                    int64_t at = count < k ? count++ : k - 1;
-                    while (at > 0 && c < best[at - 1])
-                    {
-                        best[at] = best[at - 1];
-                        --at;
-                    }
-                    best[at] = c;
-                }
+                    offer(Neighbour<T>{squared_distance(q, &xyz_[static_cast<size_t>(3 * i)]), order_[static_cast<size_t>(i)]});
                 continue;
             }
             const T diff = q[node.dim] - node.split;
@@ -136,6 +152,8 @@ class KdTree
             stack[top++] = Pending{far, diff * diff};
             stack[top++] = Pending{near, T(0)};
         }
+        for (int64_t i = finite_; i < n_; ++i) // the rows outside the tree
+            offer(Neighbour<T>{squared_distance(q, &xyz_[static_cast<size_t>(3 * i)]), order_[static_cast<size_t>(i)]});
         return count;
     }
 
@@ -191,6 +209,7 @@ class KdTree
     }
 
     int64_t n_;
+    int64_t finite_; // the tree holds the first finite_ positions
     std::vector<int64_t> order_; // position in the tree's arrays -> index in the caller's cloud
     std::vector<T> xyz_;         // the points in tree order
     std::vector<Node> nodes_;

@@ -53,6 +53,11 @@ struct ListEntry<false>
 };
 constexpr int L_LAST = static_cast<int>(0x80000000u);
 constexpr int L_NOTHING = 0x7ffffffc - 3 * 0x40000; // (rows further down, at multiples of the row size, stay out of range too)
+// The walker multiplies the offset by the number of rows it stages side by side (1, 2 or 4), in 32 bits: every
+// product has to stay beyond the LDS.
+static_assert(static_cast<uint32_t>(L_NOTHING) * 1u >= TPK_LDS_BYTES && static_cast<uint32_t>(L_NOTHING) * 2u >= TPK_LDS_BYTES &&
+                  static_cast<uint32_t>(L_NOTHING) * 4u >= TPK_LDS_BYTES,
+              "an entry that refers to nothing must read beyond the LDS whatever the number of staged rows");
 
 constexpr int L_SPANS = G_THREADS / TPK_WAVE; // spans of targets per cloud: one per wavefront of the walker
 constexpr int L_MAX_SPAN = 15360;             // targets of a span: their bookkeeping (2 ints each) fits in LDS

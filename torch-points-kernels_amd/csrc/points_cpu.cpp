@@ -154,7 +154,41 @@ at::Tensor rows_to_tensor(const std::vector<float>& v, int64_t rows, int64_t wid
 
 void check_mode(int mode)
 {
-    TORCH_CHECK(mode == 0, "only mode = 0 (a matrix of neighbours) is built; the Python layer never asks for edge lists");
+    TORCH_CHECK(mode == 0 || mode == 1, "mode must be 0 (a matrix of neighbours) or 1 (a list of edges)");
+}
+
+// mode = 1 of the reference (cpu/src/neighbors.cpp:107-135, :257-291; cpu/src/ball_query.cpp:45-51, :120-126): the
+// neighbour matrix as a list of edges (support index, query row) with their squared distances (E, 1), query rows in
+// order, a row's neighbours in the order of the matrix.  Unused slots of the matrix hold distance -1.  In the
+// one-cloud search a query without neighbours keeps the reference's stand-in (0, -1) as an edge (`keep_empty`); in the
+// packed layout such a row contributes nothing.
+std::pair<at::Tensor, at::Tensor> matrix_to_edges(const at::Tensor& idx, const at::Tensor& dist, bool keep_empty)
+{
+    const int64_t rows = idx.size(0), width = idx.size(1);
+    const int64_t* pi = idx.data_ptr<int64_t>();
+    const float* pd = dist.data_ptr<float>();
+    std::vector<int64_t> edges;
+    std::vector<float> d2;
+    for (int64_t i = 0; i < rows; ++i)
+    {
+        int64_t used = 0;
+        while (used < width && pd[i * width + used] != -1.0f)
+            ++used;
+        if (used == 0 && keep_empty)
+        {
+            edges.push_back(0);
+            edges.push_back(i);
+            d2.push_back(-1.0f);
+        }
+        for (int64_t j = 0; j < used; ++j)
+        {
+            edges.push_back(pi[i * width + j]);
+            edges.push_back(i);
+            d2.push_back(pd[i * width + j]);
+        }
+    }
+    const int64_t count = static_cast<int64_t>(d2.size());
+    return {rows_to_tensor(edges, count, 2), rows_to_tensor(d2, count, 1)};
 }
 
 // support (N, 3), query (M, 3) of one cloud -> (idx (M, width) int64, dist2 (M, width) float32)
@@ -172,7 +206,10 @@ std::pair<at::Tensor, at::Tensor> ball_query(at::Tensor support, at::Tensor quer
         width = radius_search<scalar_t>(support.data_ptr<scalar_t>(), support.size(0), query.data_ptr<scalar_t>(), query.size(0),
                                         radius, q.integral, max_num, sorted, 0, true, 1, idx, dist);
     });
-    return {rows_to_tensor(idx, query.size(0), width), rows_to_tensor(dist, query.size(0), width)};
+    const at::Tensor out_idx = rows_to_tensor(idx, query.size(0), width), out_dist = rows_to_tensor(dist, query.size(0), width);
+    if (mode == 1)
+        return matrix_to_edges(out_idx, out_dist, true);
+    return {out_idx, out_dist};
 }
 
 // Argument order of the reference (cpu/src/ball_query.cpp:127-146 with the swap at :137): the first tensor holds the
@@ -230,8 +267,8 @@ std::pair<at::Tensor, at::Tensor> batch_ball_query(at::Tensor support, at::Tenso
     query_batch = query_batch.contiguous();
     const int64_t nq = query.size(0), ns = support.size(0);
     if (nq == 0)
-        return {torch::empty({0, std::max(max_num, 0)}, torch::dtype(torch::kLong)),
-                torch::empty({0, std::max(max_num, 0)}, torch::dtype(torch::kFloat))};
+        return {torch::empty({0, mode == 1 ? 2 : std::max(max_num, 0)}, torch::dtype(torch::kLong)),
+                torch::empty({0, mode == 1 ? 1 : std::max(max_num, 0)}, torch::dtype(torch::kFloat))};
     const int64_t clouds = query_batch.data_ptr<int64_t>()[nq - 1] + 1;
     TORCH_CHECK(ns > 0 && clouds == support_batch.data_ptr<int64_t>()[ns - 1] + 1,
                 "Both batches need to have the same number of samples.");
@@ -264,6 +301,8 @@ std::pair<at::Tensor, at::Tensor> batch_ball_query(at::Tensor support, at::Tenso
             std::copy_n(dist[k].data() + (q - qs[k]) * widths[k], widths[k], out_dist.data_ptr<float>() + q * width);
         }
     }
+    if (mode == 1)
+        return matrix_to_edges(out_idx, out_dist, false);
     return {out_idx, out_dist};
 }
 
