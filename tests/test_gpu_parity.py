@@ -3,8 +3,9 @@
 
 Bar: integer outputs (neighbour / sample / argmin indices, hit counts) bit-exact; ball-query,
 three_nn and chamfer distances bit-exact too (same unfused fp32 arithmetic); interpolated
-features bit-exact forward; gradients (atomic accumulation, unordered) within
-rtol 1e-5 / atol 1e-6 of the oracle's in-order sums.
+features bit-exact forward; gradients within rtol 1e-5 / atol 1e-6 of the oracle's in-order sums, plus - for
+the scatter sums, whose terms the kernels add in another order - two units in the last place of the sum of the
+terms' magnitudes (needed by a handful of elements in 10^7: _assert_scatter_sum_close counts them).
 """
 import sys
 
@@ -30,20 +31,36 @@ def _np(t):
     return t.detach().cpu().numpy()
 
 
-def _assert_scatter_sum_close(got, want, abs_sum):
-    """Scatter-add results: the kernels add in no fixed order (as the reference's atomics do),
-    the oracle in index order.  Both are fp32 sums of the same terms, so they agree to
-    rtol/atol plus a reordering allowance proportional to the sum of the terms' magnitudes
-    (which matters only where the terms cancel)."""
+REORDER_ULPS = 2.0  # allowance for a different order of summation, in units of 2^-23 * sum of |terms|
+
+
+def _assert_scatter_sum_close(got, want, abs_sum, where=""):
+    """Scatter-add results: the kernels add a target's terms in the order of its list (the reference's
+    atomics: in no fixed order), the oracle in index order.  Both are fp32 sums of the same terms, so they
+    agree to rtol/atol plus a reordering allowance proportional to the sum of the terms' magnitudes, which
+    matters only where the terms cancel.  Returns (elements outside the strict bound, worst error in units
+    of 2^-23 * sum of |terms| among those) and appends them to gpurun_out/gradient_tolerance.jsonl."""
+    import json
+    import os
+
     err = np.abs(got - want)
     strict = ATOL + RTOL * np.abs(want)
     outside = err > strict
-    # how much of the result needs the reordering allowance at all (printed with -s / on failure)
-    print("[tolerance] %d of %d elements outside rtol %g / atol %g before the reordering allowance; worst error %g "
-          "(%.2f x the strict bound there)" % (outside.sum(), outside.size, RTOL, ATOL, err.max(),
-                                               (err / strict).max()), file=sys.stderr, flush=True)
-    bad = err > strict + 1e-6 * abs_sum
+    ulp = np.float32(2.0 ** -23) * abs_sum
+    worst_ulps = float((err[outside] / np.maximum(ulp[outside], 1e-30)).max()) if outside.any() else 0.0
+    record = {"case": where or os.environ.get("PYTEST_CURRENT_TEST", ""), "elements": int(outside.size),
+              "outside_strict": int(outside.sum()), "worst_error": float(err.max()),
+              "worst_over_strict": float((err / strict).max()), "worst_outside_in_ulps_of_abs_sum": worst_ulps}
+    print("[tolerance] %s" % json.dumps(record), file=sys.stderr, flush=True)
+    try:
+        os.makedirs("gpurun_out", exist_ok=True)
+        with open(os.path.join("gpurun_out", "gradient_tolerance.jsonl"), "a") as f:
+            f.write(json.dumps(record) + "\n")
+    except OSError:
+        pass
+    bad = err > strict + REORDER_ULPS * ulp
     assert not bad.any(), "%d of %d elements differ, worst %g" % (bad.sum(), bad.size, err.max())
+    return int(outside.sum()), worst_ulps
 
 
 def _in_threads(fn, tasks, workers=16):
@@ -788,7 +805,9 @@ def test_interpolate_full_config3a(tpk, oracle, dev):
     out.backward(w["grad_out"].to(dev))
     want = oracle.three_interpolate_grad(w["grad_out"].numpy(), wi, _np(weight), known.shape[1])
     abs_sum = oracle.three_interpolate_grad(w["grad_out"].abs().numpy(), wi, _np(weight), known.shape[1])
-    _assert_scatter_sum_close(_np(feats.grad), want, abs_sum)
+    outside, _ = _assert_scatter_sum_close(_np(feats.grad), want, abs_sum)
+    # measured: 0 of 8 388 608 elements outside rtol 1e-5 / atol 1e-6 (the order of a list varies from run to run)
+    assert outside <= 8
 
 
 # ------------------------------------------------------------------ grouping
@@ -838,7 +857,10 @@ def test_grouping_full_config3b(tpk, oracle, dev):
     out.backward(w["grad_out"].to(dev))
     want = oracle.grouping_operation_grad(w["grad_out"].numpy(), w["idx"].numpy(), f.shape[2])
     abs_sum = oracle.grouping_operation_grad(w["grad_out"].abs().numpy(), w["idx"].numpy(), f.shape[2])
-    _assert_scatter_sum_close(_np(f.grad), want, abs_sum)
+    outside, _ = _assert_scatter_sum_close(_np(f.grad), want, abs_sum)
+    # measured: 1 of 8 388 608 elements outside rtol 1e-5 / atol 1e-6, by less than one unit in the last place of
+    # the sum of the terms' magnitudes (a sum of 8 terms that cancel)
+    assert outside <= 8
 
 
 # ------------------------------------------------------------------ knn (general k)
