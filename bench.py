@@ -39,6 +39,8 @@ TRAFFIC_KERNELS = {
     "fps": ["fps_pruned_kernel<16, 1024, 4, true>"],
     "three_interpolate_fwd": ["gather_fwd_lds_kernel<3, true, int, true>"],
     "three_interpolate_bwd": ["build_lists_kernel<3, true, int>", "gather_bwd_lists_kernel<3, true, 2>"],
+    "three_interpolate_bwd_lists": ["gather_bwd_lists_kernel<3, true, 2>"],
+    "grouping_bwd_lists": ["gather_bwd_lists_kernel<1, false, 1>"],
     "grouping_fwd": ["gather_fwd_lds_kernel<1, false, long, false>"],
     "grouping_bwd": ["build_lists_kernel<1, false, long>", "gather_bwd_lists_kernel<1, false, 1>"],
     "chamfer_bwd": ["chamfer_bwd_chains_kernel<float>"],
@@ -254,6 +256,17 @@ def _executed(call):
     assert st == 0, "counting call failed with status %d" % st
     assert lib.tpk_work_read_reset(ctypes.byref(n)) == 0
     return int(n.value)
+
+
+def _autograd_split(forward_recording, backward_from_lists, nbytes, steps, warmup, key):
+    """The two halves of a gather's training step as autograd runs them: the forward pass that also inverts the index
+    and the backward pass that walks the lists."""
+    wall_f, ev_f = _time_gpu(forward_recording, steps, warmup)
+    lists = forward_recording()[1]
+    wall_b, ev_b = _time_gpu(lambda: backward_from_lists(lists), steps, warmup)
+    return {"what": "forward pass with autograd recording (gather, then the lists for the backward pass), then the backward "
+                    "pass over those lists", "forward_kernel_ms": ev_f, "forward_wall_ms": wall_f, "backward_kernel_ms": ev_b,
+            "backward_wall_ms": wall_b, "backward_roofline": _roof_bytes(nbytes, ev_b, key)}
 
 
 def _p(t):
@@ -589,9 +602,15 @@ def bench_others(dev, steps, warmup, with_cpu):
                              "sample": "%d of 16 clouds, reference cpu/src/interpolate.cpp scalar loops" % sub}
     out["three_interpolate_fwd"] = e
     wall, ev = _time_gpu(lambda: nat.three_interpolate_grad(gout, idx, weight, m), steps, warmup)
-    e = {"workload": "configs[2]a: three_interpolate backward grad (16,128,16384) -> (16,128,4096)", "metric": "GB/s",
-         "value": nbytes / (wall * 1e-3) / 1e9, "kernel_ms": ev, "wall_ms": wall,
+    e = {"workload": "configs[2]a: three_interpolate backward grad (16,128,16384) -> (16,128,4096); the call of the "
+                     "reference's interface, which gets (grad_out, idx, weight) and inverts the index itself",
+         "metric": "GB/s", "value": nbytes / (wall * 1e-3) / 1e9, "kernel_ms": ev, "wall_ms": wall,
          "roofline": _roof_bytes(nbytes, ev, "three_interpolate_bwd"), "algorithmic_bytes": nbytes}
+    # the same gradient as autograd computes it: the forward pass, knowing that a backward pass follows, also inverts
+    # the index, and the backward pass walks the lists
+    e["as_autograd_runs_it"] = _autograd_split(
+        lambda: nat.three_interpolate_recording(feats, idx, weight),
+        lambda lists: nat.three_interpolate_grad_lists(gout, lists, m), nbytes, steps, warmup, "three_interpolate_bwd_lists")
     if ref is not None:
         secs = _cpu_time(lambda: ref.knn_interpolate_grad(w["grad_out"][:sub], idx64, wc, m))
         e["cpu_baseline"] = {"value": (nbytes * sub / 16) / secs / 1e9, "unit": "GB/s", "cores": 1, "kind": "reference",
@@ -620,9 +639,13 @@ def bench_others(dev, steps, warmup, with_cpu):
     out["grouping_fwd"] = e
     n = feats.shape[2]
     wall, ev = _time_gpu(lambda: nat.grouping_operation_grad(gout, gidx, n), steps, warmup)
-    out["grouping_bwd"] = {"workload": "configs[2]b: grouping_operation backward", "metric": "GB/s",
+    out["grouping_bwd"] = {"workload": "configs[2]b: grouping_operation backward (the stand-alone call, which inverts the index "
+                                       "itself)", "metric": "GB/s",
                            "value": nbytes / (wall * 1e-3) / 1e9, "kernel_ms": ev, "wall_ms": wall,
                            "roofline": _roof_bytes(nbytes, ev, "grouping_bwd"), "algorithmic_bytes": nbytes}
+    out["grouping_bwd"]["as_autograd_runs_it"] = _autograd_split(
+        lambda: nat.grouping_operation_recording(feats, gidx),
+        lambda lists: nat.grouping_operation_grad_lists(gout, lists, n), nbytes, steps, warmup, "grouping_bwd_lists")
     del feats, gidx, gout
 
     # configs[4]: chamfer fwd/bwd
@@ -745,6 +768,10 @@ def _compact_op(e):
             row["alg_frac"] = _sig(r["algorithmic_rate"] / r["peak"], 3)
         if r.get("traffic") and e.get("algorithmic_bytes"):
             row["traffic_x"] = _sig(r["traffic"] / e["algorithmic_bytes"], 3)
+    ag = e.get("as_autograd_runs_it")
+    if ag:
+        row["autograd"] = {"fwd_ms": _sig(ag["forward_kernel_ms"]), "bwd_ms": _sig(ag["backward_kernel_ms"]),
+                           "bwd_frac": _sig(ag["backward_roofline"]["frac"], 3)}
     ap = e.get("all_pairs_kernel")
     if ap:
         row["all_pairs"] = {"ms": _sig(ap["kernel_ms"]), "frac": _sig(ap["roofline"]["frac"], 3)}

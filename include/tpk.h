@@ -64,10 +64,21 @@ int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* workspace,
  *   idx (b, m, nsample) int64         dist (b, m, nsample) float32 (squared)
  * First `nsample` support points in index order with d2 < radius*radius; unused idx slots
  * repeat the first hit (0 when there is none), unused dist slots are -1.
+ * Clouds of 1024 .. 8192 points are searched through buckets of cells that every workgroup
+ * builds in LDS.  Larger clouds need a `workspace` for anything better than a scan of all
+ * pairs (tpk_ball_query_dense_workspace_bytes() bytes - 0 for sizes not served that way -,
+ * 256-byte aligned, contents arbitrary before and after): the points are ordered in windows
+ * along a space filling curve and a query only looks into the bins its ball touches, as in the
+ * packed layout below.  tpk_ball_query_dense_f32 is the call without a workspace.  Same results
+ * every way.
  * ------------------------------------------------------------------------------------- */
 int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int nsample,
                              const float* new_xyz, const float* xyz, int64_t* idx, float* dist,
                              void* stream);
+size_t tpk_ball_query_dense_workspace_bytes(int b, int n, int m, int nsample);
+int tpk_ball_query_dense_ws_f32(int b, int n, int m, float radius, int nsample,
+                                const float* new_xyz, const float* xyz, int64_t* idx, float* dist,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Ball query, packed variable-length layout.
@@ -204,6 +215,20 @@ size_t tpk_three_interpolate_grad_workspace_bytes(int b, int n, int m);
 int tpk_three_interpolate_grad_f32(int b, int c, int n, int m, const float* grad_out,
                                    const int32_t* idx, const float* weight, float* grad_points,
                                    void* workspace, size_t workspace_bytes, void* stream);
+/* The two halves of tpk_three_interpolate_grad_f32 on their own, for callers that know at the
+ * time of the FORWARD pass that a backward pass will follow (autograd is recording): the lists
+ * depend on (idx, weight) only, so they can be built then, the backward pass is the walk alone, and
+ * several backward passes share one inversion.  `lists`: tpk_three_interpolate_grad_workspace_bytes()
+ * bytes, 256-byte aligned, kept by the caller from one call to the other (read-only in the second, so
+ * one set of lists serves any number of backward passes).  TPK_ERR_UNSUPPORTED: the lists do not serve
+ * the shape (the size function returns 0); use tpk_three_interpolate_grad_f32.  The reference has no
+ * counterpart: its backward is three_interpolate_grad_kernel_wrapper with atomics
+ * (cuda/src/interpolate_gpu.cu:122-164). */
+int tpk_three_interpolate_lists_f32(int b, int n, int m, const int32_t* idx, const float* weight,
+                                    void* lists, size_t lists_bytes, void* stream);
+int tpk_three_interpolate_grad_lists_f32(int b, int c, int n, int m, const float* grad_out,
+                                         void* lists, size_t lists_bytes, float* grad_points,
+                                         void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Grouping (gather of feature columns), forward and backward.
@@ -221,6 +246,12 @@ size_t tpk_group_grad_workspace_bytes(int b, int n, int npoint, int nsample);
 int tpk_group_grad_f32(int b, int c, int n, int npoint, int nsample, const float* grad_out,
                        const int64_t* idx, float* grad_features, void* workspace,
                        size_t workspace_bytes, void* stream);
+/* The two halves of tpk_group_grad_f32 on their own, as for the interpolation above (`lists`:
+ * tpk_group_grad_workspace_bytes() bytes). */
+int tpk_group_lists(int b, int n, int npoint, int nsample, const int64_t* idx, void* lists,
+                    size_t lists_bytes, void* stream);
+int tpk_group_grad_lists_f32(int b, int c, int n, int npoint, int nsample, const float* grad_out,
+                             void* lists, size_t lists_bytes, float* grad_features, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Chamfer distance, forward (both directions) and backward.

@@ -22,8 +22,9 @@ def _declared_symbols():
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
     for want in (
-        "tpk_fps_f32", "tpk_fps_workspace_bytes", "tpk_ball_query_dense_f32", "tpk_ball_query_partial_workspace_bytes", "tpk_ball_query_partial_f32",
+        "tpk_fps_f32", "tpk_fps_workspace_bytes", "tpk_ball_query_dense_f32", "tpk_ball_query_dense_workspace_bytes", "tpk_ball_query_dense_ws_f32", "tpk_ball_query_partial_workspace_bytes", "tpk_ball_query_partial_f32",
         "tpk_three_nn_workspace_bytes", "tpk_three_nn_f32", "tpk_knn_workspace_bytes", "tpk_knn_f32", "tpk_three_interpolate_f32", "tpk_three_interpolate_grad_f32", "tpk_group_f32",
+        "tpk_three_interpolate_lists_f32", "tpk_three_interpolate_grad_lists_f32", "tpk_group_lists", "tpk_group_grad_lists_f32",
         "tpk_group_grad_f32", "tpk_chamfer_fwd_workspace_bytes", "tpk_chamfer_fwd_f32", "tpk_chamfer_fwd_f64", "tpk_chamfer_bwd_f32",
         "tpk_chamfer_bwd_f64", "tpk_grow_proximity_workspace_bytes", "tpk_grow_proximity", "tpk_instance_iou", "tpk_gridding_f32", "tpk_gridding_f64", "tpk_gridding_grad_f32",
         "tpk_gridding_grad_f64", "tpk_cubic_feature_sampling_f32", "tpk_cubic_feature_sampling_f64",

@@ -241,6 +241,40 @@ def test_ball_query_dense_over_cells(tpk, oracle, dev, kind, B, N, M, r, ns):
     np.testing.assert_array_equal(_np(dist), want_dist)
 
 
+@pytest.mark.parametrize("kind", ["uniform", "clusters", "flat", "non_finite", "offset_1e4"])
+@pytest.mark.parametrize("B,N,M,r,ns", [(2, 8193, 2500, 0.04, 16), (1, 20000, 2100, 0.03, 32), (3, 20000, 700, 0.25, 8),
+                                        (1, 100000, 450, 0.015, 64), (1, 100000, 420, 0.2, 20), (2, 12289, 1700, 0.05, 100),
+                                        (2, 9000, 50, 0.05, 16)])
+def test_ball_query_dense_large_clouds(tpk, oracle, dev, kind, B, N, M, r, ns):
+    # clouds above 8192 points do not fit in LDS: the dense layout takes the bin walk of the packed layout under its
+    # own rules (strict <, indices inside the cloud, the first hit repeated behind the last); sparse balls (a few
+    # points), dense ones (thousands: the walk hands over to the scan in index order) and windows that hold the end
+    # of one cloud and the beginning of the next; the last shape has too few pairs to pay for the ordering and keeps
+    # the scan of all pairs
+    g = torch.Generator().manual_seed(3 * N + M)
+    xyz = torch.rand(B, N, 3, generator=g)
+    new_xyz = xyz[:, torch.randperm(N, generator=g)[:M]].clone() + 0.003 * torch.randn(B, M, 3, generator=g)
+    if kind == "clusters":
+        centres = torch.rand(B, 7, 3, generator=g)
+        xyz = torch.stack([centres[b, torch.randint(0, 7, (N,), generator=g)] for b in range(B)]) + 0.02 * torch.randn(B, N, 3, generator=g)
+        new_xyz = xyz[:, :M].clone() + 0.002
+        new_xyz[:, ::5] += 3.0  # queries far from every point
+    elif kind == "flat":
+        xyz[..., 1] = -0.75
+        new_xyz[..., 1] = -0.75 + 0.3 * r
+    elif kind == "non_finite":
+        xyz[:, 11, 0] = float("nan")
+        xyz[:, N // 2, 2] = float("inf")
+        new_xyz[:, 2, 1] = float("nan")
+        new_xyz[:, 3, 0] = -float("inf")
+    elif kind.startswith("offset"):
+        xyz, new_xyz = xyz + float(kind[7:]), new_xyz + float(kind[7:])
+    idx, dist = tpk.ball_query(r, ns, xyz.to(dev), new_xyz.contiguous().to(dev), mode="dense")
+    want_idx, want_dist = oracle.ball_query_dense(r, ns, xyz.numpy(), new_xyz.contiguous().numpy())
+    np.testing.assert_array_equal(_np(idx), want_idx)
+    np.testing.assert_array_equal(_np(dist), want_dist)
+
+
 def _packed_case(seed, sizes, qfrac, jitter):
     g = torch.Generator().manual_seed(seed)
     xs, ys, bx, by = [], [], [], []
@@ -808,6 +842,58 @@ def test_interpolate_full_config3a(tpk, oracle, dev):
     outside, _ = _assert_scatter_sum_close(_np(feats.grad), want, abs_sum)
     # measured: 0 of 8 388 608 elements outside rtol 1e-5 / atol 1e-6 (the order of a list varies from run to run)
     assert outside <= 8
+
+
+def test_backward_over_lists_built_in_the_forward_pass(tpk, oracle, dev):
+    """With autograd recording, the forward pass also builds the per-target lists and the
+    backward pass only walks them: same gradient as the stand-alone call (which builds them itself), for
+    both gathers; one set of lists serves several backward passes; without a gradient nothing is built."""
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    feats, idx, w, gout = _interp_case(3, 21, 700, 5000, 99)
+    f, i, wt, go = feats.to(dev), idx.to(dev), w.to(dev), gout.to(dev)
+    out, lists = native.three_interpolate_recording(f, i, wt)
+    assert lists.numel() > 0 and lists.dtype == torch.uint8
+    np.testing.assert_array_equal(_np(out), oracle.three_interpolate(feats.numpy(), idx.numpy(), w.numpy()))
+    want = oracle.three_interpolate_grad(gout.numpy(), idx.numpy(), w.numpy(), 700)
+    abs_sum = oracle.three_interpolate_grad(gout.abs().numpy(), idx.numpy(), w.numpy(), 700)
+    first = native.three_interpolate_grad_lists(go, lists, 700)
+    _assert_scatter_sum_close(_np(first), want, abs_sum)
+    assert torch.equal(native.three_interpolate_grad_lists(go, lists, 700), first)  # (the walk leaves the lists as they are)
+    _assert_scatter_sum_close(_np(native.three_interpolate_grad(go, i, wt, 700)), want, abs_sum)
+    fr = f.clone().requires_grad_(True)
+    y = tpk.three_interpolate(fr, i, wt)
+    y.backward(go, retain_graph=True)
+    once = fr.grad.clone()
+    y.backward(go)
+    _assert_scatter_sum_close(_np(once), want, abs_sum)
+    _assert_scatter_sum_close(_np(fr.grad), 2 * want, 2 * abs_sum)
+    # on a stream of the caller's own
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fs = f.clone().requires_grad_(True)
+        tpk.three_interpolate(fs, i, wt).backward(go)
+    torch.cuda.current_stream().wait_stream(side)
+    _assert_scatter_sum_close(_np(fs.grad), want, abs_sum)
+    # grouping
+    g = torch.Generator().manual_seed(5)
+    feats = torch.randn(2, 9, 3000, generator=g)
+    gidx = torch.randint(0, 3000, (2, 300, 16), generator=g)
+    gg = torch.randn(2, 9, 300, 16, generator=g)
+    out, lists = native.grouping_operation_recording(feats.to(dev), gidx.to(dev))
+    np.testing.assert_array_equal(_np(out), oracle.grouping_operation(feats.numpy(), gidx.numpy()))
+    want = oracle.grouping_operation_grad(gg.numpy(), gidx.numpy(), 3000)
+    abs_sum = oracle.grouping_operation_grad(gg.abs().numpy(), gidx.numpy(), 3000)
+    _assert_scatter_sum_close(_np(native.grouping_operation_grad_lists(gg.to(dev), lists, 3000)), want, abs_sum)
+    _assert_scatter_sum_close(_np(native.grouping_operation_grad(gg.to(dev), gidx.to(dev), 3000)), want, abs_sum)
+    # shapes the lists do not serve (too many targets for LDS): empty lists, and autograd takes the other backward pass
+    feats, idx, w, gout = _interp_case(1, 3, 60000, 900, 7)
+    out, lists = native.three_interpolate_recording(feats.to(dev), idx.to(dev), w.to(dev))
+    assert lists.numel() == 0
+    fb = feats.to(dev).requires_grad_(True)
+    tpk.three_interpolate(fb, idx.to(dev), w.to(dev)).backward(gout.to(dev))
+    _assert_scatter_sum_close(_np(fb.grad), oracle.three_interpolate_grad(gout.numpy(), idx.numpy(), w.numpy(), 60000),
+                              oracle.three_interpolate_grad(gout.abs().numpy(), idx.numpy(), w.numpy(), 60000))
 
 
 # ------------------------------------------------------------------ grouping

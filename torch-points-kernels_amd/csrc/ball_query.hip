@@ -686,9 +686,14 @@ int tpk_cells_ball_query_dense(int b, int n, int m, float radius, float radius2,
     return tpk_launch_status();
 }
 
-extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int nsample,
-                                        const float* new_xyz, const float* xyz, int64_t* idx,
-                                        float* dist, void* stream)
+extern "C" size_t tpk_ball_query_dense_workspace_bytes(int b, int n, int m, int nsample)
+{
+    return tpk_grid_ball_query_dense_workspace_bytes(b, n, m, nsample);
+}
+
+extern "C" int tpk_ball_query_dense_ws_f32(int b, int n, int m, float radius, int nsample,
+                                           const float* new_xyz, const float* xyz, int64_t* idx,
+                                           float* dist, void* workspace, size_t workspace_bytes, void* stream)
 {
     if (b < 0 || n < 0 || m < 0 || nsample < 0)
         return TPK_ERR_INVALID_ARG;
@@ -706,7 +711,16 @@ extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int n
         return TPK_ERR_UNSUPPORTED;
     const float radius2 = radius * radius; // fp32 product, as the reference kernel forms it
     {
+        // clouds of 1024 .. 8192 points: buckets of cells in LDS
         const int st = tpk_cells_ball_query_dense(b, n, m, radius, radius2, nsample, false, new_xyz, xyz, idx, dist, tpk_stream(stream));
+        if (st != TPK_ERR_UNSUPPORTED)
+            return st;
+    }
+    if (workspace)
+    {
+        // larger clouds: ordered in windows, a walk over the bins the ball touches
+        const int st = tpk_grid_ball_query_dense(b, n, m, radius, radius2, nsample, new_xyz, xyz, idx, dist, workspace,
+                                                 workspace_bytes, tpk_stream(stream));
         if (st != TPK_ERR_UNSUPPORTED)
             return st;
     }
@@ -717,6 +731,13 @@ extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int n
         hipLaunchKernelGGL(ball_query_dense_kernel<BQ_Q>, dim3(static_cast<unsigned>(blocks)), dim3(BQ_THREADS), 0,
                            tpk_stream(stream), n, m, static_cast<int>(bpc), radius2, nsample, new_xyz, xyz, idx, dist);
     return tpk_launch_status();
+}
+
+extern "C" int tpk_ball_query_dense_f32(int b, int n, int m, float radius, int nsample,
+                                        const float* new_xyz, const float* xyz, int64_t* idx,
+                                        float* dist, void* stream)
+{
+    return tpk_ball_query_dense_ws_f32(b, n, m, radius, nsample, new_xyz, xyz, idx, dist, nullptr, 0, stream);
 }
 
 extern "C" size_t tpk_ball_query_partial_workspace_bytes(int64_t size_x, int64_t size_y, int nsample)

@@ -691,6 +691,53 @@ int launch_bwd_lists(int b, int c, int m, int64_t n, const BwdShape& sh, const f
     return tpk_launch_status();
 }
 
+// The shape of the list path for (b, n, m), or rows == 0 where the lists do not serve it.
+template <int K>
+BwdShape list_shape(int b, int m, int64_t n)
+{
+    BwdShape sh = bwd_shape(n > 0 ? n : 1, m);
+    if (n <= 0 || m <= 0 || n * K > 0x7fffffffLL || static_cast<int64_t>(b) * sh.parts > 0x7fffffffLL)
+        sh.rows = 0;
+    return sh;
+}
+
+// Inverts the index of every cloud into `lists` (lists_workspace_bytes() bytes).  TPK_ERR_UNSUPPORTED: the
+// list path does not serve this shape.
+template <int K, bool WEIGHTED, typename IdxT>
+int gather_lists(int b, int m, int64_t n, const IdxT* idx, const float* weight, void* lists_memory, size_t lists_bytes,
+                 hipStream_t s)
+{
+    const BwdShape sh = list_shape<K>(b, m, n);
+    const size_t need = lists_workspace_bytes<K, WEIGHTED>(b, m, n);
+    if (sh.rows == 0 || need == 0)
+        return TPK_ERR_UNSUPPORTED;
+    if (!lists_memory || lists_bytes < need || (reinterpret_cast<uintptr_t>(lists_memory) & 15u))
+        return TPK_ERR_WORKSPACE;
+    const int64_t part_total = static_cast<int64_t>(sh.part_len) * K;
+    const Lists<WEIGHTED> lists = lists_at<WEIGHTED>(lists_memory, static_cast<int64_t>(b) * sh.parts, m, part_total);
+    return launch_build_lists<K, WEIGHTED, IdxT>(b, m, n * K, part_total, idx, weight, lists, s);
+}
+
+// The backward pass over lists that gather_lists() built for the same (b, n, m).
+template <int K, bool WEIGHTED>
+int gather_bwd_from_lists(int b, int c, int m, int64_t n, const float* grad_out, void* lists_memory, size_t lists_bytes,
+                          float* grad_src, hipStream_t s)
+{
+    const BwdShape sh = list_shape<K>(b, m, n);
+    const size_t need = lists_workspace_bytes<K, WEIGHTED>(b, m, n);
+    if (sh.rows == 0 || need == 0)
+        return TPK_ERR_UNSUPPORTED;
+    if (!lists_memory || lists_bytes < need || (reinterpret_cast<uintptr_t>(lists_memory) & 15u))
+        return TPK_ERR_WORKSPACE;
+    const Lists<WEIGHTED> lists =
+        lists_at<WEIGHTED>(lists_memory, static_cast<int64_t>(b) * sh.parts, m, static_cast<int64_t>(sh.part_len) * K);
+    if (sh.rows == 4)
+        return launch_bwd_lists<K, WEIGHTED, 4>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+    if (sh.rows == 2)
+        return launch_bwd_lists<K, WEIGHTED, 2>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+    return launch_bwd_lists<K, WEIGHTED, 1>(b, c, m, n, sh, grad_out, lists, grad_src, s);
+}
+
 template <int K, bool WEIGHTED, typename IdxT>
 int gather_bwd(int b, int c, int m, int64_t n, const float* grad_out, const IdxT* idx,
                const float* weight, float* grad_src, void* workspace, size_t workspace_bytes,
@@ -703,23 +750,12 @@ int gather_bwd(int b, int c, int m, int64_t n, const float* grad_out, const IdxT
     if (!grad_src || (n > 0 && (!grad_out || !idx || (WEIGHTED && !weight))))
         return TPK_ERR_INVALID_ARG;
     // The list path needs entry positions that fit an int, and the workspace.
-    const BwdShape sh = bwd_shape(n > 0 ? n : 1, m);
-    const bool fits = n > 0 && sh.rows > 0 && n * K <= 0x7fffffffLL &&
-                      static_cast<int64_t>(b) * sh.parts <= 0x7fffffffLL;
     const size_t need = lists_workspace_bytes<K, WEIGHTED>(b, m, n);
-    if (fits && workspace && need > 0 && workspace_bytes >= need)
+    if (n > 0 && workspace && need > 0 && workspace_bytes >= need && list_shape<K>(b, m, n).rows > 0)
     {
-        const int64_t part_total = static_cast<int64_t>(sh.part_len) * K;
-        const Lists<WEIGHTED> lists = lists_at<WEIGHTED>(workspace, static_cast<int64_t>(b) * sh.parts, m, part_total);
-        int st = launch_build_lists<K, WEIGHTED, IdxT>(b, m, n * K, part_total, idx, weight, lists, s);
+        int st = gather_lists<K, WEIGHTED, IdxT>(b, m, n, idx, weight, workspace, workspace_bytes, s);
         if (st == TPK_OK)
-        {
-            if (sh.rows == 4)
-                return launch_bwd_lists<K, WEIGHTED, 4>(b, c, m, n, sh, grad_out, lists, grad_src, s);
-            if (sh.rows == 2)
-                return launch_bwd_lists<K, WEIGHTED, 2>(b, c, m, n, sh, grad_out, lists, grad_src, s);
-            return launch_bwd_lists<K, WEIGHTED, 1>(b, c, m, n, sh, grad_out, lists, grad_src, s);
-        }
+            return gather_bwd_from_lists<K, WEIGHTED>(b, c, m, n, grad_out, workspace, workspace_bytes, grad_src, s);
         if (st != TPK_ERR_UNSUPPORTED)
             return st;
     }
@@ -785,4 +821,50 @@ extern "C" int tpk_group_grad_f32(int b, int c, int n, int npoint, int nsample,
     return gather_bwd<1, false, int64_t>(b, c, n, static_cast<int64_t>(npoint) * nsample, grad_out,
                                          idx, nullptr, grad_features, workspace, workspace_bytes,
                                          tpk_stream(stream));
+}
+
+extern "C" int tpk_three_interpolate_lists_f32(int b, int n, int m, const int32_t* idx, const float* weight, void* lists,
+                                               size_t lists_bytes, void* stream)
+{
+    if (b < 0 || n < 0 || m < 0)
+        return TPK_ERR_INVALID_ARG;
+    if (b > 0 && n > 0 && m > 0 && (!idx || !weight))
+        return TPK_ERR_INVALID_ARG;
+    return gather_lists<3, true, int32_t>(b, m, n, idx, weight, lists, lists_bytes, tpk_stream(stream));
+}
+
+extern "C" int tpk_three_interpolate_grad_lists_f32(int b, int c, int n, int m, const float* grad_out, void* lists,
+                                                    size_t lists_bytes, float* grad_points, void* stream)
+{
+    if (b < 0 || c < 0 || n < 0 || m < 0)
+        return TPK_ERR_INVALID_ARG;
+    if (b == 0 || c == 0 || m == 0)
+        return TPK_OK;
+    if (!grad_out || !grad_points)
+        return TPK_ERR_INVALID_ARG;
+    return gather_bwd_from_lists<3, true>(b, c, m, n, grad_out, lists, lists_bytes, grad_points, tpk_stream(stream));
+}
+
+extern "C" int tpk_group_lists(int b, int n, int npoint, int nsample, const int64_t* idx, void* lists, size_t lists_bytes,
+                               void* stream)
+{
+    if (b < 0 || n < 0 || npoint < 0 || nsample < 0)
+        return TPK_ERR_INVALID_ARG;
+    const int64_t columns = static_cast<int64_t>(npoint) * nsample;
+    if (b > 0 && n > 0 && columns > 0 && !idx)
+        return TPK_ERR_INVALID_ARG;
+    return gather_lists<1, false, int64_t>(b, n, columns, idx, nullptr, lists, lists_bytes, tpk_stream(stream));
+}
+
+extern "C" int tpk_group_grad_lists_f32(int b, int c, int n, int npoint, int nsample, const float* grad_out, void* lists,
+                                        size_t lists_bytes, float* grad_features, void* stream)
+{
+    if (b < 0 || c < 0 || n < 0 || npoint < 0 || nsample < 0)
+        return TPK_ERR_INVALID_ARG;
+    if (b == 0 || c == 0 || n == 0)
+        return TPK_OK;
+    if (!grad_out || !grad_features)
+        return TPK_ERR_INVALID_ARG;
+    return gather_bwd_from_lists<1, false>(b, c, n, static_cast<int64_t>(npoint) * nsample, grad_out, lists, lists_bytes,
+                                           grad_features, tpk_stream(stream));
 }

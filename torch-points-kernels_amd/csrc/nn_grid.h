@@ -47,3 +47,11 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
                                 const float* x, const float* y, const int64_t* batch_x,
                                 const int64_t* batch_y, int64_t* idx, float* dist, void* workspace,
                                 size_t workspace_bytes, hipStream_t stream);
+
+// Ball query, dense layout (b clouds of n points, m queries each; cuda/src/ball_query_gpu.cu:9-52), for clouds
+// above 8192 points: the bin walk of the packed layout under the dense layout's rules (hit: squared distance
+// < radius2; indices inside the cloud; the slots behind the last hit repeat the first, 0 without any; distance -1).
+size_t tpk_grid_ball_query_dense_workspace_bytes(int b, int n, int m, int nsample);
+int tpk_grid_ball_query_dense(int b, int n, int m, float radius, float radius2, int nsample, const float* new_xyz,
+                              const float* xyz, int64_t* idx, float* dist, void* workspace, size_t workspace_bytes,
+                              hipStream_t stream);

@@ -753,6 +753,8 @@ inline int bqb_window_shift(int64_t size_x)
 }
 static_assert((1 << 14) == CURVE_MAX_POINTS, "the larger window is what the ordering kernel holds at most");
 constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
+constexpr int BQB_DENSE_MIN_POINTS = 8192; // dense layout: clouds above this take the bin walk (smaller ones fit in LDS whole)
+constexpr int64_t BQB_DENSE_MIN_PAIRS = 40000000; // ... when the call has at least this many (query, point) pairs
 
 // Range of 16^3-grid cells along one axis that [v - r, v + r] can touch.  The interval is widened
 // by a few ulps of its ends so that a point the fp32 radius test accepts is never left out.
@@ -767,13 +769,18 @@ __device__ __forceinline__ void bin_range(float v, float r, float lo, float scal
 // first nsample in row order with squared distance <= radius2: the wavefront keeps its 64 best (distance, row)
 // keys sorted across the lanes and merges the hits of a step into them (as the wavefront-per-query kernel
 // further down does with the points of a cell).
-template <bool SORTED>
+// DENSE (unsorted only): the dense layout's rules instead (cuda/src/ball_query_gpu.cu:9-52) - clouds of dense_n
+// consecutive rows with dense_m consecutive queries each (no cloud_rows), a hit has squared distance < radius2
+// (strict), indices count from the cloud's first row, and the slots behind the last hit repeat the first hit
+// (0 without any) with distance -1.
+template <bool SORTED, bool DENSE>
 __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     int size_x, int size_y, int window_shift, float radius, float radius2, int nsample, const float* __restrict__ x,
     const float* __restrict__ y, const float4* __restrict__ sorted_x, const int* __restrict__ bin_ends,
     const float4* __restrict__ grids, const int2* __restrict__ cloud_rows, int64_t* __restrict__ idx,
-    float* __restrict__ dist)
+    float* __restrict__ dist, int dense_n, int dense_m)
 {
+    static_assert(!(SORTED && DENSE), "the sorted query of the dense layout has a kernel of its own");
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
     __shared__ int hit_rows[WAVES][BQB_HITS];
     __shared__ float hit_dists[WAVES][BQB_HITS];
@@ -790,8 +797,18 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
 
     const float ux = y[q * 3 + 0], uy = y[q * 3 + 1], uz = y[q * 3 + 2];
     const float qx = to_vector_register(ux), qy = to_vector_register(uy), qz = to_vector_register(uz);
-    const int2 cloud = cloud_rows[q]; // the support rows of the query's cloud
-    const int s0 = cloud.x, s1 = cloud.y;
+    int s0, s1; // the support rows of the query's cloud
+    if constexpr (DENSE)
+    {
+        s0 = static_cast<int>(q / dense_m) * dense_n;
+        s1 = s0 + dense_n;
+    }
+    else
+    {
+        const int2 cloud = cloud_rows[q];
+        s0 = cloud.x;
+        s1 = cloud.y;
+    }
     const int64_t out = q * nsample;
     TPK_WORK_DECL
 
@@ -885,7 +902,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                     offer(has && d < radius2 && row >= s0 && row < s1, d, row);
                     continue;
                 }
-                const bool hit = has && d <= radius2 && row >= s0 && row < s1;
+                const bool hit = has && (DENSE ? d < radius2 : d <= radius2) && row >= s0 && row < s1;
                 const unsigned long long mask = __ballot(hit);
                 if (mask == 0)
                     continue;
@@ -952,12 +969,19 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
             rank += rows[j] < my_row ? 1 : 0;
         if (lane < cnt && rank < nsample)
         {
-            idx[out + rank] = my_row;
+            idx[out + rank] = DENSE ? my_row - s0 : my_row;
             dist[out + rank] = my_dist;
+        }
+        int64_t filler = -1;
+        if constexpr (DENSE)
+        {
+            // the first hit of the scan in index order = the lowest row among the hits
+            const unsigned long long lowest = __ballot(lane < cnt && rank == 0);
+            filler = lowest ? __shfl(my_row, __builtin_ctzll(lowest)) - s0 : 0;
         }
         for (int s = cnt + lane; s < nsample; s += TPK_WAVE)
         {
-            idx[out + s] = -1;
+            idx[out + s] = filler;
             dist[out + s] = -1.0f;
         }
         TPK_WORK_FLUSH
@@ -967,6 +991,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     // Serial semantics directly: lanes hold 64 consecutive support rows; ballot + prefix count
     // give the hits their slots in index order; stop after nsample hits.
     cnt = 0;
+    int first_hit = -1; // (dense layout: the row that fills the slots behind the last hit)
     constexpr int BATCH = 4; // loads of four steps in flight
     for (int base = s0; base < s1 && cnt < nsample; base += BATCH * TPK_WAVE)
     {
@@ -985,20 +1010,22 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
             const int pos = base + u * TPK_WAVE + lane;
             const float d = tpk_dist2(qx, qy, qz, px[u], py[u], pz[u]);
             TPK_WORK_ADD(1);
-            const bool hit = pos < s1 && d <= radius2;
+            const bool hit = pos < s1 && (DENSE ? d < radius2 : d <= radius2);
             const unsigned long long mask = __ballot(hit);
             const int slot = cnt + static_cast<int>(tpk_prefix_count(mask));
             if (hit && slot < nsample)
             {
-                idx[out + slot] = pos;
+                idx[out + slot] = DENSE ? pos - s0 : pos;
                 dist[out + slot] = d;
             }
+            if (DENSE && first_hit < 0 && mask != 0)
+                first_hit = base + u * TPK_WAVE + __builtin_ctzll(mask) - s0;
             cnt += __builtin_popcountll(mask);
         }
     }
     for (int s = cnt + lane; s < nsample; s += TPK_WAVE)
     {
-        idx[out + s] = -1;
+        idx[out + s] = DENSE ? max(first_hit, 0) : -1;
         dist[out + s] = -1.0f;
     }
     TPK_WORK_FLUSH
@@ -1469,12 +1496,63 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
     if (sorted)
-        hipLaunchKernelGGL(ball_query_bins_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+        hipLaunchKernelGGL((ball_query_bins_kernel<true, false>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
                            static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
-                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
+                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist, 0, 0);
     else
-        hipLaunchKernelGGL(ball_query_bins_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+        hipLaunchKernelGGL((ball_query_bins_kernel<false, false>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
                            static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
-                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist);
+                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist, 0, 0);
+    return tpk_launch_status();
+}
+
+namespace {
+
+// The dense layout takes the bin walk for clouds too large for the buckets of cells in LDS (ball_query.hip):
+// the b clouds of n points are one array of b * n rows, cut into windows like the packed layout's.
+bool ball_bins_dense_supported(int b, int n, int m, int nsample)
+{
+    // Ordering the points costs 17 - 30 us before the first query is answered, in which time the scan of all pairs
+    // tests BQB_DENSE_MIN_PAIRS pairs: calls with fewer pairs keep the scan.  (What the host cannot know is how many
+    // points a ball holds.  Where it holds hundreds, the scan in index order ends after a fraction of the cloud and
+    // the walk over the bins has nothing to skip: measured 66 against 34 us for 4 x 20000 points, 5000 queries
+    // each, 670 points per ball, and 222 against 162 us for 100000 points with 420 per ball - against 32 and 130 us,
+    // 39 and 817 us where a ball holds a few points.)
+    return n > BQB_DENSE_MIN_POINTS && b > 0 && m > 0 && nsample > 0 && static_cast<int64_t>(b) * n < (1LL << 30) &&
+           static_cast<int64_t>(b) * m <= 0x7fffffffLL && static_cast<int64_t>(b) * n * m >= BQB_DENSE_MIN_PAIRS;
+}
+
+} // namespace
+
+size_t tpk_grid_ball_query_dense_workspace_bytes(int b, int n, int m, int nsample)
+{
+    return ball_bins_dense_supported(b, n, m, nsample) ? ball_layout(static_cast<int64_t>(b) * n, 0).total : 0;
+}
+
+int tpk_grid_ball_query_dense(int b, int n, int m, float radius, float radius2, int nsample, const float* new_xyz,
+                              const float* xyz, int64_t* idx, float* dist, void* workspace, size_t workspace_bytes,
+                              hipStream_t s)
+{
+    if (!ball_bins_dense_supported(b, n, m, nsample))
+        return TPK_ERR_UNSUPPORTED;
+    const int64_t size_x = static_cast<int64_t>(b) * n, size_y = static_cast<int64_t>(b) * m;
+    const BallLayout l = ball_layout(size_x, 0);
+    if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return TPK_ERR_WORKSPACE;
+    char* w = static_cast<char*>(workspace);
+    const int window_shift = bqb_window_shift(size_x);
+    PointSet px{xyz, nullptr, size_x, size_x, 1 << window_shift, reinterpret_cast<float4*>(w + l.sorted_x), nullptr,
+                reinterpret_cast<int*>(w + l.bin_ends), reinterpret_cast<float4*>(w + l.grids)};
+    PointSet none{nullptr, nullptr, 0, 1, CURVE_MAX_POINTS, nullptr, nullptr, nullptr, nullptr};
+    int st = launch_curve_cells(px, none, nullptr, s);
+    if (st != TPK_OK)
+        return st;
+    constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
+    const int64_t blocks = tpk_ceil_div(size_y, WAVES);
+    if (blocks > 0x7fffffffLL)
+        return TPK_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((ball_query_bins_kernel<false, true>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+                       static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, xyz,
+                       new_xyz, px.sorted, px.bin_ends, px.grid, static_cast<const int2*>(nullptr), idx, dist, n, m);
     return tpk_launch_status();
 }

@@ -257,6 +257,57 @@ at::Tensor three_interpolate_grad(at::Tensor grad_out, at::Tensor idx, at::Tenso
     return output;
 }
 
+// three_interpolate for a caller that will ask for the gradient (autograd is recording): with the forward
+// pass the index is inverted into the per-target lists that the backward pass walks (include/tpk.h,
+// tpk_three_interpolate_lists_f32), so that the backward pass is the walk alone and several backward passes
+// share one inversion.  Returns (output, lists); `lists` is empty where the list path does not serve the shape
+// (then three_interpolate_grad is the backward pass).  No counterpart in the reference, whose backward scatters
+// with atomics.  (Inverting on a second stream beside the gather was measured: the two event waits between the
+// streams cost more than the 18 us they hide - 198 us per call against 52 us one after the other.)
+std::pair<at::Tensor, at::Tensor> three_interpolate_recording(at::Tensor points, at::Tensor idx, at::Tensor weight)
+{
+    check_contiguous(idx, "idx");
+    check_contiguous(weight, "weight");
+    check_gpu(points, "points");
+    check_gpu(idx, "idx");
+    check_gpu(weight, "weight");
+    check_dtype(idx, at::kInt, "idx");
+    check_f32(weight, "weight");
+    TORCH_CHECK(points.dim() == 3 && idx.dim() == 3 && idx.size(2) == 3 && weight.sizes() == idx.sizes(),
+                "points (B, c, m), idx and weight (B, n, 3) expected");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(points.device());
+    const int b = as_int(idx.size(0), "batch size"), n = as_int(idx.size(1), "n"), m = as_int(points.size(2), "m");
+    const size_t bytes = tpk_three_interpolate_grad_workspace_bytes(b, n, m);
+    if (bytes == 0)
+        return {three_interpolate(points, idx, weight), torch::empty({0}, at::device(points.device()).dtype(at::kByte))};
+    at::Tensor lists = torch::empty({static_cast<int64_t>(bytes)}, at::device(points.device()).dtype(at::kByte));
+    at::Tensor output = three_interpolate(points, idx, weight);
+    check_status(tpk_three_interpolate_lists_f32(b, n, m, idx.data_ptr<int32_t>(), weight.data_ptr<float>(), lists.data_ptr(),
+                                                 bytes, current_stream(points)),
+                 "three_interpolate (lists for the backward pass)");
+    return {output, lists};
+}
+
+// The backward pass over the lists three_interpolate_recording() returned.
+at::Tensor three_interpolate_grad_lists(at::Tensor grad_out, at::Tensor lists, const int m)
+{
+    check_contiguous(grad_out, "grad_out");
+    check_f32(grad_out, "grad_out");
+    check_gpu(grad_out, "grad_out");
+    check_gpu(lists, "lists");
+    check_same_device(grad_out, lists, "grad_out and lists");
+    TORCH_CHECK(grad_out.dim() == 3, "grad_out must have shape (B, c, n)");
+    TORCH_CHECK(lists.scalar_type() == at::kByte && lists.is_contiguous() && m >= 0, "lists as three_interpolate_recording returned them");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_out.device());
+    at::Tensor output = torch::empty({grad_out.size(0), grad_out.size(1), m}, at::device(grad_out.device()).dtype(at::kFloat));
+    check_status(tpk_three_interpolate_grad_lists_f32(as_int(grad_out.size(0), "batch size"), as_int(grad_out.size(1), "channels"),
+                                                      as_int(grad_out.size(2), "n"), m, grad_out.data_ptr<float>(),
+                                                      lists.data_ptr(), static_cast<size_t>(lists.numel()),
+                                                      output.data_ptr<float>(), current_stream(grad_out)),
+                 "three_interpolate_grad (from lists)");
+    return output;
+}
+
 // cuda/src/ball_query.cpp:15-36.  Query centres first, as in the reference.
 // sorted: the nsample nearest neighbours within the radius, nearest first (what the reference
 // computes for CPU tensors with sort=True, cpu/src/ball_query.cpp:127-146).
@@ -295,12 +346,18 @@ std::pair<at::Tensor, at::Tensor> ball_query_dense(at::Tensor new_xyz, at::Tenso
                      "ball_query_dense (sorted)");
         return std::make_pair(idx, dist);
     }
-    check_status(tpk_ball_query_dense_f32(
-                     as_int(xyz.size(0), "batch size"), as_int(xyz.size(1), "support points"),
-                     as_int(new_xyz.size(1), "query points"), radius, nsample,
-                     new_xyz.data_ptr<float>(), xyz.data_ptr<float>(), idx.data_ptr<int64_t>(),
-                     dist.data_ptr<float>(), current_stream(new_xyz)),
-                 "ball_query_dense");
+    {
+        const int b = as_int(xyz.size(0), "batch size"), n = as_int(xyz.size(1), "support points");
+        const int m = as_int(new_xyz.size(1), "query points");
+        const size_t ws_bytes = tpk_ball_query_dense_workspace_bytes(b, n, m, nsample);
+        at::Tensor ws;
+        if (ws_bytes)
+            ws = torch::empty({static_cast<int64_t>(ws_bytes)}, new_xyz.options().dtype(torch::kUInt8));
+        check_status(tpk_ball_query_dense_ws_f32(b, n, m, radius, nsample, new_xyz.data_ptr<float>(), xyz.data_ptr<float>(),
+                                                 idx.data_ptr<int64_t>(), dist.data_ptr<float>(),
+                                                 ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, current_stream(new_xyz)),
+                     "ball_query_dense");
+    }
     return std::make_pair(idx, dist);
 }
 
@@ -601,6 +658,46 @@ at::Tensor grouping_operation_grad(at::Tensor grad_out, at::Tensor idx, const in
     return out;
 }
 
+// grouping_operation for a caller that will ask for the gradient: as three_interpolate_recording.
+std::pair<at::Tensor, at::Tensor> grouping_operation_recording(at::Tensor features, at::Tensor idx)
+{
+    check_contiguous(idx, "idx");
+    check_gpu(features, "features");
+    check_gpu(idx, "idx");
+    check_dtype(idx, at::kLong, "idx");
+    TORCH_CHECK(features.dim() == 3 && idx.dim() == 3, "features (B, C, N) and idx (B, npoint, nsample) expected");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(features.device());
+    const int b = as_int(idx.size(0), "batch size"), n = as_int(features.size(2), "N");
+    const int npoint = as_int(idx.size(1), "npoint"), nsample = as_int(idx.size(2), "nsample");
+    const size_t bytes = tpk_group_grad_workspace_bytes(b, n, npoint, nsample);
+    if (bytes == 0)
+        return {grouping_operation(features, idx), torch::empty({0}, at::device(features.device()).dtype(at::kByte))};
+    at::Tensor lists = torch::empty({static_cast<int64_t>(bytes)}, at::device(features.device()).dtype(at::kByte));
+    at::Tensor output = grouping_operation(features, idx);
+    check_status(tpk_group_lists(b, n, npoint, nsample, idx.data_ptr<int64_t>(), lists.data_ptr(), bytes, current_stream(features)),
+                 "grouping_operation (lists for the backward pass)");
+    return {output, lists};
+}
+
+at::Tensor grouping_operation_grad_lists(at::Tensor grad_out, at::Tensor lists, const int n)
+{
+    check_contiguous(grad_out, "grad_out");
+    check_f32(grad_out, "grad_out");
+    check_gpu(grad_out, "grad_out");
+    check_gpu(lists, "lists");
+    check_same_device(grad_out, lists, "grad_out and lists");
+    TORCH_CHECK(grad_out.dim() == 4, "grad_out must have shape (B, C, npoint, nsample)");
+    TORCH_CHECK(lists.scalar_type() == at::kByte && lists.is_contiguous() && n >= 0, "lists as grouping_operation_recording returned them");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_out.device());
+    at::Tensor out = torch::empty({grad_out.size(0), grad_out.size(1), n}, at::device(grad_out.device()).dtype(at::kFloat));
+    check_status(tpk_group_grad_lists_f32(as_int(grad_out.size(0), "batch size"), as_int(grad_out.size(1), "channels"), n,
+                                          as_int(grad_out.size(2), "npoint"), as_int(grad_out.size(3), "nsample"),
+                                          grad_out.data_ptr<float>(), lists.data_ptr(), static_cast<size_t>(lists.numel()),
+                                          out.data_ptr<float>(), current_stream(grad_out)),
+                 "grouping_operation_grad (from lists)");
+    return out;
+}
+
 // cuda/src/chamfer_dist.cpp:3-6 -> cuda/src/chamfer_dist_gpu.cu:157-184
 std::vector<torch::Tensor> chamfer_dist(torch::Tensor xyz1, torch::Tensor xyz2)
 {
@@ -724,6 +821,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("cubic_feature_sampling_grad", &cubic_feature_sampling_grad);
     m.def("three_interpolate", &three_interpolate);
     m.def("three_interpolate_grad", &three_interpolate_grad);
+    m.def("three_interpolate_recording", &three_interpolate_recording);
+    m.def("three_interpolate_grad_lists", &three_interpolate_grad_lists);
     m.def("ball_query_dense", &ball_query_dense, pybind11::arg("new_xyz"), pybind11::arg("xyz"), pybind11::arg("radius"),
           pybind11::arg("nsample"), pybind11::arg("sorted") = false);
     m.def("ball_query_partial_dense", &ball_query_partial_dense, pybind11::arg("x"), pybind11::arg("y"),
@@ -731,6 +830,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           pybind11::arg("sorted") = false);
     m.def("grouping_operation", &grouping_operation);
     m.def("grouping_operation_grad", &grouping_operation_grad);
+    m.def("grouping_operation_recording", &grouping_operation_recording);
+    m.def("grouping_operation_grad_lists", &grouping_operation_grad_lists);
     m.def("chamfer_dist", &chamfer_dist);
     m.def("chamfer_dist_grad", &chamfer_dist_grad);
     m.def("tpk_version", &tpk_version);

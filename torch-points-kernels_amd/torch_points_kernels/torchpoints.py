@@ -49,14 +49,23 @@ class ThreeInterpolate(Function):
     def forward(ctx, features, idx, weight):
         B, c, m = features.size()
         ctx.three_interpolate_for_backward = (idx, weight, m)
+        ctx.three_interpolate_lists = None
         if features.is_cuda:
+            if ctx.needs_input_grad[0]:
+                # a backward pass will follow: what it needs of (idx, weight) - the index inverted into lists per
+                # target - is built now, and the backward pass only walks it (and any further backward pass shares it)
+                out, lists = native().three_interpolate_recording(features.contiguous(), idx.contiguous(), weight.contiguous())
+                ctx.three_interpolate_lists = lists if lists.numel() else None
+                return out
             return native().three_interpolate(features, idx, weight)
         return host().knn_interpolate(features, idx, weight)
 
     @staticmethod
     def backward(ctx, grad_out):
         idx, weight, m = ctx.three_interpolate_for_backward
-        if grad_out.is_cuda:
+        if grad_out.is_cuda and ctx.three_interpolate_lists is not None:
+            grad_features = native().three_interpolate_grad_lists(grad_out.contiguous(), ctx.three_interpolate_lists, m)
+        elif grad_out.is_cuda:
             grad_features = native().three_interpolate_grad(grad_out.contiguous(), idx, weight, m)
         else:
             grad_features = host().knn_interpolate_grad(grad_out.contiguous(), idx, weight, m)
@@ -77,11 +86,19 @@ class GroupingOperation(Function):
     @staticmethod
     def forward(ctx, features, idx):
         ctx.grouping_for_backward = (idx, features.size(2))
+        ctx.grouping_lists = None
+        if ctx.needs_input_grad[0]:
+            # (as in ThreeInterpolate: the lists the backward pass walks are built with the forward pass)
+            out, lists = native().grouping_operation_recording(features.contiguous(), idx.contiguous())
+            ctx.grouping_lists = lists if lists.numel() else None
+            return out
         return native().grouping_operation(features.contiguous(), idx.contiguous())
 
     @staticmethod
     def backward(ctx, grad_out):
         idx, n = ctx.grouping_for_backward
+        if ctx.grouping_lists is not None:
+            return native().grouping_operation_grad_lists(grad_out.contiguous(), ctx.grouping_lists, n), None
         return native().grouping_operation_grad(grad_out.contiguous(), idx.contiguous(), n), None
 
 
