@@ -617,6 +617,23 @@ def test_fps_several_samples_per_round(tpk, oracle, dev, B, N, npoint, kind):
     np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(xyz.contiguous().numpy(), npoint))
 
 
+@pytest.mark.parametrize("N", [16384, 40000])
+def test_fps_lattice_half_random_half(tpk, oracle, dev, N):
+    # Half of the cloud lies on a lattice (rounds with equal maxima: one sample each, by the reference's tie rule, and
+    # the next rounds go there at once), half is random (rounds of several samples): sampling half of all points
+    # alternates between the two kinds of rounds thousands of times, in the register kernel and in the one with cells
+    # in memory.
+    g = torch.Generator().manual_seed(N)
+    side = int(round((N // 2) ** (1.0 / 3.0))) + 1
+    axis = torch.arange(side, dtype=torch.float32) * 0.125
+    lattice = torch.stack(torch.meshgrid(axis, axis, axis, indexing="ij"), -1).reshape(-1, 3)[: N // 2] + 0.25
+    scattered = torch.rand(N - N // 2, 3, generator=g) * (side * 0.125) + 0.25
+    scattered[:, 0] += side * 0.125 + 0.3  # beside the lattice, so that both halves keep being sampled
+    cloud = torch.cat([lattice, scattered])[torch.randperm(N, generator=g)].unsqueeze(0).contiguous()
+    out = tpk.furthest_point_sample(cloud.to(dev), N // 2)
+    np.testing.assert_array_equal(_np(out), oracle.furthest_point_sample(cloud.numpy(), N // 2))
+
+
 def test_fps_full_config2(tpk, oracle, dev):
     w = W.cfg2_fps()
     xyz = w["xyz"].to(dev)

@@ -559,9 +559,7 @@ extern "C" int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbo
                 for (int sweep = 0; sweep < CL_SWEEPS; ++sweep)
                     launch(sweep);
                 int last = 0;
-                hipError_t e = hipMemcpyAsync(&last, changed + CL_SWEEPS - 1, sizeof(int), hipMemcpyDeviceToHost, s);
-                if (e == hipSuccess)
-                    e = hipStreamSynchronize(s);
+                const hipError_t e = static_cast<hipError_t>(tpk_read_back(&last, changed + CL_SWEEPS - 1, sizeof(int), s));
                 cluster_clear_kernel<<<1, CL_THREADS, 0, s>>>(changed);
                 if (e != hipSuccess || last == 0)
                     return e;
@@ -589,9 +587,7 @@ extern "C" int tpk_grow_proximity(int64_t n, int nsample, const int64_t* neighbo
         return (int)e;
     cluster_describe_kernel<<<blocks1, CL_THREADS, 0, s>>>(ni, packed, scanned, number, seeds, starts);
     u64 totals = 0;
-    e = hipMemcpyAsync(&totals, scanned + n, sizeof(u64), hipMemcpyDeviceToHost, s);
-    if (e == hipSuccess)
-        e = hipStreamSynchronize(s);
+    e = static_cast<hipError_t>(tpk_read_back(&totals, scanned + n, sizeof(u64), s));
     if (e != hipSuccess)
         return (int)e;
     const int clusters = (int)(totals >> 32);

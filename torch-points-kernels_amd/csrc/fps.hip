@@ -10,7 +10,7 @@
 //   up to 16384 points   fps_pruned_kernel: up to 32 points per lane in registers, cloud
 //                        ordered along a space filling curve so that most updates can be
 //                        skipped exactly (described at the kernel);
-//   up to 163840 points  fps_cells_kernel: the cloud ordered along the curve into cells of 64
+//   up to 163840 points  fps_cells_batched_kernel: the cloud ordered along the curve into cells of 64
 //                        points that stay in memory (the caller's workspace); boxes, largest
 //                        distance and best point of every cell in LDS; a round touches only
 //                        the cells the new sample can change (described at the kernel);
@@ -277,20 +277,17 @@ __global__ __launch_bounds__(THREADS) void fps_resident_kernel(
 // The fp32 box distance is compared with a relative margin of 2e-6, several times the rounding
 // error of either side, so a skipped update is provably a no-op.
 //
-// Selection.  Each lane keeps the maximum of every group and of all its points; a wavefront
-// whose groups were all skipped keeps these from the round before.  The workgroup maximum is
-// one LDS atomic max per 16-lane row (after a DPP reduction) and a barrier.  Only a wavefront
-// that holds the maximum then looks for the slot: group per lane by compare/select, the
-// winning lane's group and member through wave-uniform (GPR-indexed) register reads.  It
-// publishes the point's coordinates and sorted position in LDS and counts itself as winner;
-// after the second barrier every wavefront reads the new sample from there.  The wavefronts
-// that wait for the winner reset the words of the next round and store the previous round's
-// index, which keeps both off the critical path.
+// Selection.  Each lane keeps the largest and second largest running minimum of every group; a
+// wavefront publishes its two best points of different lanes (value, coordinates, sorted
+// position: found per lane by compare/select, then through wave-uniform, GPR-indexed register
+// reads) and the largest minimum it keeps to itself, and a round takes as many of the published
+// points as follow each other as samples (described where the loop begins): several samples per
+// round, each round's box tests one instruction sequence whatever their number.
 //
-// Equal maxima.  When the winners' count is not exactly one (several points hold the maximum,
-// or no point is eligible) the round is resolved by the reference's tie key over all points
-// holding the maximum, through a copy of the running minima in LDS (slots are not in index
-// order here, so the key is computed from the original index kept in the sort keys).
+// Equal maxima.  When several points hold the maximum, or no point is eligible, the round takes one
+// sample by the reference's tie key over all points holding the maximum, through a copy of the
+// running minima in LDS (slots are not in index order here, so the key is computed from the
+// original index kept in the sort keys).
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ unsigned tie_key(int k, int log2_bs, int ref_groups)
 {
@@ -341,7 +338,7 @@ __device__ __forceinline__ int sorted_position(int g, int wave, int e, int lane)
     return ((g * WAVES + wave) * GS + e) * TPK_WAVE + lane;
 }
 
-template <int PPT, int THREADS, int GS, bool BATCHED>
+template <int PPT, int THREADS, int GS>
 __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     int n, int npoint, int log2_bs, int ref_groups, int key_capacity,
     const float* __restrict__ xyz, int32_t* __restrict__ out)
@@ -359,7 +356,6 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     int* const bins = t_copy + PPT * THREADS; // CURVE_BINS words
     __shared__ int wave_totals[WAVES];
     __shared__ RoundWords words[2];
-    __shared__ float4 record[2];      // x, y, z of the round's winner and its sorted position
     __shared__ int cloud_box[6];      // ordered ints: min x,y,z then max x,y,z
     __shared__ int group_box[WAVES * NG * 6]; // the same per (wavefront, group) cell
 
@@ -419,9 +415,9 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     }
     __syncthreads();
     // lane g of every 16-lane row tests this wavefront's group g; lanes beyond NG hold an empty box
-    // (BATCHED: row g tests group g, its lane k against sample k of the round)
-    static_assert(!BATCHED || NG <= 4, "one row of lanes per group");
-    const int my_group = BATCHED ? lane >> 4 : lane & 15;
+    // (row g of the lanes tests group g, its lane k against sample k of the round)
+    static_assert(NG <= 4, "one row of lanes per group");
+    const int my_group = lane >> 4;
     float blo[3], bhi[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a)
@@ -441,20 +437,16 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
     }
 
     const float p0x = xyz[0], p0y = xyz[1], p0z = xyz[2];
-    float vx = p0x, vy = p0y, vz = p0z;         // the last sample (the same in every lane)
     int bound = ordered_bits(__builtin_inff()); // no running minimum exceeds this
     const bool row_head = (lane & 15) == 0;
     int best = g[0]; // this lane's largest running minimum and that of its row of 16 lanes
 #pragma unroll
     for (int gi = 1; gi < NG; ++gi)
         best = max(best, g[gi]);
-    int row_val = row_all_max_i32(best);
-    int pending = -1; // sorted position of the previous round's sample while its index is unstored
     if (tid == 0)
         out[0] = 0;
     TPK_WORK_DECL
 
-    if constexpr (BATCHED)
     {
         // Several samples per round.  After a round's updates let c0 > c1 > c2 ... be the points in the order of
         // their running minima.  c0 is the next sample.  If c1's minimum is not changed by c0 (c0 is no closer
@@ -718,175 +710,6 @@ __global__ __launch_bounds__(THREADS) void fps_pruned_kernel(
         TPK_WORK_FLUSH
         return;
     }
-    for (int j = 1; j < npoint; ++j)
-    {
-        const int par = j & 1;
-
-        // 1. which groups can change?  squared distance from the sample to the group's box
-        unsigned live; // bit g set: group g must be updated
-        {
-            const float dx = fmaxf(fmaxf(blo[0] - vx, vx - bhi[0]), 0.f);
-            const float dy = fmaxf(fmaxf(blo[1] - vy, vy - bhi[1]), 0.f);
-            const float dz = fmaxf(fmaxf(blo[2] - vz, vz - bhi[2]), 0.f);
-            const float lb = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz)) * 0.999998f;
-            // an empty box gives lb = +inf (never live); NaN compares false -> live
-            const bool skip = lb >= __int_as_float(bound);
-            live = static_cast<unsigned>(__ballot(!skip)) & ((1u << NG) - 1u);
-        }
-
-        // 2. distance update of the live groups; a wavefront without any keeps its maxima
-        if (live != 0)
-        {
-#pragma unroll
-            for (int gi = 0; gi < NG; ++gi)
-            {
-                if ((live >> gi) & 1u) // uniform over the wavefront
-                {
-                    TPK_WORK_ADD(GS);
-#pragma unroll
-                    for (int e = 0; e < GS; ++e)
-                    {
-                        const int i = gi * GS + e;
-                        const float d = tpk_dist2(x[i], y[i], z[i], vx, vy, vz);
-                        t[i] = min(t[i], ordered_bits(d));
-                        g[gi] = e == 0 ? t[i] : max(g[gi], t[i]);
-                    }
-                }
-            }
-            best = g[0];
-#pragma unroll
-            for (int gi = 1; gi < NG; ++gi)
-                best = max(best, g[gi]);
-            row_val = row_all_max_i32(best); // DPP reduction over each 16-lane row
-        }
-
-        // 3. workgroup maximum: one LDS atomic per row
-        if (row_head)
-            lds_atomic_max_i32(&words[par].max_val, row_val);
-        lds_barrier();
-        const int gv_lanes = words[par].max_val;
-        const int gv = __builtin_amdgcn_readfirstlane(gv_lanes);
-
-        // 4. only a wavefront holding the maximum looks for the slot and publishes the point
-        const unsigned long long top = __ballot(best == gv);
-        if (top == 0)
-        {
-            // Nothing to publish: the wait for the winner is used to prepare the words of the
-            // next round and to store the previous round's index.  Two wavefronts are in charge
-            // of the store; with a single winner at least one of them comes through here.
-            if (lane == 0)
-            {
-                words[par ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
-                if (pending >= 0 && (wave == (j & (WAVES - 1)) || wave == ((j + 1) & (WAVES - 1))))
-                    out[j - 1] = static_cast<int>(sort_keys[pending] & 0x3FFFu);
-            }
-        }
-        else
-        {
-            int my_grp = 0, my_hits = 0;
-#pragma unroll
-            for (int gi = NG - 1; gi >= 0; --gi)
-            {
-                const bool m = g[gi] == best;
-                my_grp = m ? gi : my_grp;
-                my_hits += m ? 1 : 0;
-            }
-            const int wl = __builtin_ctzll(top);
-            const int grp = __builtin_amdgcn_readlane(my_grp, wl);
-            // members of that group (uniform index into the registers), first match per lane
-            int hits = 0, my_e = 0;
-#pragma unroll
-            for (int e = GS - 1; e >= 0; --e)
-            {
-                const bool m = t[grp * GS + e] == gv;
-                my_e = m ? e : my_e;
-                hits += m ? 1 : 0;
-            }
-            const int ce = __builtin_amdgcn_readlane(my_e, wl);
-            // one group and one member of it hold the maximum in lane wl, and no other lane does
-            const bool single = __builtin_popcountll(top) == 1 &&
-                                __builtin_amdgcn_readlane(my_hits + hits, wl) == 2;
-            const int slot = grp * GS + ce;
-            const float cx = x[slot], cy = y[slot], cz = z[slot];
-            if (lane == wl)
-            {
-                const int pos = sorted_position<WAVES, GS>(grp, wave, ce, lane);
-                record[par] = make_float4(cx, cy, cz, __int_as_float(pos));
-                lds_atomic_add_u32(&words[par].winners, single ? 1 : 2);
-            }
-        }
-        lds_barrier();
-        float4 rec = record[par];
-        const int winners = __builtin_amdgcn_readfirstlane(words[par].winners);
-
-        // The index of a single winner is stored during the next round (see above).
-        const int previous = pending;
-        pending = __builtin_amdgcn_readfirstlane(__float_as_int(rec.w));
-        if (winners != 1)
-        {
-            // Rare: several points hold the maximum (or none is eligible).  Every wavefront
-            // may have been busy publishing, so what the waiting ones do is done here.
-            pending = -1; // this round's index is stored below
-            if (tid == 0)
-            {
-                words[par ^ 1] = RoundWords{INT_MIN, 0, 0xFFFFFFFFu, 0};
-                if (previous >= 0)
-                    out[j - 1] = static_cast<int>(sort_keys[previous] & 0x3FFFu);
-            }
-            if (gv < 0)
-            {
-                // No eligible point in the whole cloud: the reference's reduction yields index 0.
-                rec = make_float4(p0x, p0y, p0z, 0.f);
-                if (tid == 0)
-                    out[j] = 0;
-                lds_barrier();
-            }
-            else
-            {
-                // The smallest tie key decides.  The running minima go through LDS so that
-                // this path can loop over the slots without indexing registers dynamically.
-#pragma unroll
-                for (int i = 0; i < PPT; ++i)
-                    t_copy[i * THREADS + tid] = t[i];
-                unsigned my_tk = 0xFFFFFFFFu;
-                int my_q = 0;
-#pragma clang loop unroll(disable)
-                for (int i = 0; i < PPT; ++i)
-                {
-                    const int q = sorted_position<WAVES, GS>(i / GS, wave, i % GS, lane);
-                    if (t_copy[i * THREADS + tid] == gv && q < n)
-                    {
-                        const unsigned tk =
-                            tie_key(static_cast<int>(sort_keys[q] & 0x3FFFu), log2_bs, ref_groups);
-                        if (tk < my_tk)
-                        {
-                            my_tk = tk;
-                            my_q = q;
-                        }
-                    }
-                }
-                if (my_tk != 0xFFFFFFFFu)
-                    atomicMin(&words[par].min_tie, my_tk);
-                lds_barrier();
-                if (my_tk == words[par].min_tie) // tie keys are distinct: exactly one lane
-                {
-                    const int k = static_cast<int>(sort_keys[my_q] & 0x3FFFu);
-                    record[par] = make_float4(xyz[k * 3 + 0], xyz[k * 3 + 1], xyz[k * 3 + 2],
-                                              __int_as_float(my_q));
-                    out[j] = k;
-                }
-                lds_barrier();
-                rec = record[par];
-            }
-        }
-        vx = rec.x;
-        vy = rec.y;
-        vz = rec.z;
-        bound = gv_lanes;
-    }
-    if (tid == 0 && pending >= 0)
-        out[npoint - 1] = static_cast<int>(sort_keys[pending] & 0x3FFFu);
-    TPK_WORK_FLUSH
 }
 
 constexpr int FPS_CELL_WINDOW = CURVE_MAX_POINTS;            // points ordered together
@@ -894,7 +717,6 @@ constexpr int FPS_WINDOW_CELLS = FPS_CELL_WINDOW / NG_CELL;  // 256
 constexpr int FPS_MAX_CELLS = 2560;                          // cells whose state fits in LDS
 constexpr int FPS_CELL_POINTS = FPS_MAX_CELLS * NG_CELL;     // 163840
 constexpr int FPS_LIVE_CAPACITY = (FPS_MAX_CELLS + FPS_THREADS - 1) / FPS_THREADS * TPK_WAVE; // live cells per wavefront
-constexpr int FPS_CELL_BATCH = 4;                            // cells whose points a wavefront requests together
 
 // Clouds too large for registers.  The cloud has been cut into windows of 16384 consecutive
 // points, each ordered along the curve into 256 cells of 64 (curve_cells_kernel): records
@@ -908,164 +730,8 @@ constexpr int FPS_CELL_BATCH = 4;                            // cells whose poin
 // to wavefront c mod 16 (neighbours on the curve go to different wavefronts): the wavefront
 // tests the boxes of its cells (one per lane and step), then updates the live ones - 64 points
 // per cell, a few cells' loads in flight together - and renews their LDS entries.  After a
-// Every wavefront then finds the best of its cells, the 16 results are exchanged through LDS
-// and reduced as in the other kernels.  One barrier per round.
-// dynamic LDS: 48 bytes per cell + FPS_LIVE_CAPACITY * 16 * 2.
-__global__ __launch_bounds__(FPS_THREADS) void fps_cells_kernel(
-    int n, int npoint, int log2_bs, int groups, int cells, const float* __restrict__ xyz,
-    const float4* __restrict__ sorted, const float4* __restrict__ boxes, float* __restrict__ temp,
-    int32_t* __restrict__ out)
-{
-    extern __shared__ float4 cell_best[];                                  // [cells] x, y, z, index
-    float* const box = reinterpret_cast<float*>(cell_best + cells);        // [6][cells] lo.xyz, hi.xyz
-    int* const cell_max = reinterpret_cast<int*>(box + 6 * cells);         // [cells] bits of the largest minimum
-    unsigned* const cell_tie = reinterpret_cast<unsigned*>(cell_max + cells); // [cells]
-    unsigned short* const live_all = reinterpret_cast<unsigned short*>(cell_tie + cells);
-    __shared__ WaveRecord records[2][FPS_WAVES];
-
-    xyz += static_cast<int64_t>(blockIdx.x) * n * 3;
-    sorted += static_cast<int64_t>(blockIdx.x) * cells * NG_CELL;
-    boxes += static_cast<int64_t>(blockIdx.x) * cells * NG_BOX;
-    temp += static_cast<int64_t>(blockIdx.x) * cells * NG_CELL;
-    out += static_cast<int64_t>(blockIdx.x) * npoint;
-    const int tid = threadIdx.x;
-    const int lane = tid & (TPK_WAVE - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
-    unsigned short* const live = live_all + wave * FPS_LIVE_CAPACITY;
-    const int steps = (cells + FPS_THREADS - 1) / FPS_THREADS; // cells per lane
-    const unsigned bs_mask = (1u << log2_bs) - 1u;
-    auto tie_key = [&](unsigned k) __attribute__((always_inline)) {
-        const unsigned rev = log2_bs ? (__brev(k & bs_mask) >> (32 - log2_bs)) : 0u;
-        return rev * static_cast<unsigned>(groups) + (k >> log2_bs);
-    };
-
-    // Set-up: minima, boxes and largest minima (best points are found by the first update).
-    for (int c = wave; c < cells; c += FPS_WAVES)
-    {
-        const float4 r = sorted[c * NG_CELL + lane];
-        const bool takes_part = __float_as_int(r.w) != 0x7FFFFFFF && eligible(r.x, r.y, r.z);
-        temp[c * NG_CELL + lane] = takes_part ? 1e10f : -1.0f;
-        const bool any = __ballot(takes_part) != 0;
-        if (lane < 6)
-        {
-            const float4 b = boxes[c * NG_BOX + lane / 3];
-            const int a = lane % 3;
-            box[lane * cells + c] = a == 0 ? b.x : a == 1 ? b.y : b.z;
-        }
-        if (lane == 6)
-        {
-            cell_max[c] = ordered_bits(any ? 1e10f : -1.0f);
-            cell_tie[c] = 0xFFFFFFFFu;
-        }
-    }
-    const float p0x = xyz[0], p0y = xyz[1], p0z = xyz[2];
-    float sx = p0x, sy = p0y, sz = p0z;
-    if (tid == 0)
-        out[0] = 0;
-    __syncthreads();
-
-    for (int j = 1; j < npoint; ++j)
-    {
-        // 1. the live cells among this wavefront's
-        int count = 0;
-        for (int step = 0; step < steps; ++step)
-        {
-            const int c = (step * TPK_WAVE + lane) * FPS_WAVES + wave;
-            bool is_live = false;
-            if (c < cells)
-            {
-                const float dx = fmaxf(fmaxf(box[0 * cells + c] - sx, sx - box[3 * cells + c]), 0.f);
-                const float dy = fmaxf(fmaxf(box[1 * cells + c] - sy, sy - box[4 * cells + c]), 0.f);
-                const float dz = fmaxf(fmaxf(box[2 * cells + c] - sz, sz - box[5 * cells + c]), 0.f);
-                const float lb = __builtin_fmaf(dx, dx, __builtin_fmaf(dy, dy, dz * dz));
-                is_live = lb * 0.999998f < __int_as_float(cell_max[c]);
-            }
-            const unsigned long long mask = __ballot(is_live);
-            if (is_live)
-                live[count + tpk_prefix_count(mask)] = static_cast<unsigned short>(c);
-            count += __builtin_popcountll(mask);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-
-        // 2. their points: new minima, and the cell's best point
-        for (int i0 = 0; i0 < count; i0 += FPS_CELL_BATCH)
-        {
-            int c[FPS_CELL_BATCH];
-            float4 r[FPS_CELL_BATCH];
-            float m[FPS_CELL_BATCH];
-#pragma unroll
-            for (int u = 0; u < FPS_CELL_BATCH; ++u)
-            {
-                c[u] = __builtin_amdgcn_readfirstlane(static_cast<int>(live[min(i0 + u, count - 1)]));
-                r[u] = sorted[c[u] * NG_CELL + lane];
-                m[u] = temp[c[u] * NG_CELL + lane];
-            }
-#pragma unroll
-            for (int u = 0; u < FPS_CELL_BATCH; ++u)
-            {
-                if (i0 + u >= count) // wave-uniform
-                    break;
-                const float d = tpk_dist2(r[u].x, r[u].y, r[u].z, sx, sy, sz);
-                const int old_bits = ordered_bits(m[u]);
-                const int new_bits = min(ordered_bits(d), old_bits); // -1 stays -1
-                if (new_bits != old_bits)
-                    temp[c[u] * NG_CELL + lane] = __int_as_float(new_bits);
-                const unsigned k = static_cast<unsigned>(__float_as_int(r[u].w));
-                const unsigned tk = tie_key(k);
-                int cell_val;
-                const int wl = winning_lane(new_bits, tk, cell_val);
-                if (lane == wl)
-                {
-                    cell_max[c[u]] = cell_val;
-                    cell_tie[c[u]] = tk;
-                    cell_best[c[u]] = make_float4(r[u].x, r[u].y, r[u].z, __int_as_float(static_cast<int>(k)));
-                }
-            }
-        }
-
-        // 3. the best of this wavefront's cells (steps 1 - 3 touch no other wavefront's cells, so
-        // the records below are the only exchange: one barrier per round, records double buffered)
-        int best = INT_MIN, best_cell = 0;
-        unsigned best_tk = 0xFFFFFFFFu;
-        for (int step = 0; step < steps; ++step)
-        {
-            const int c = (step * TPK_WAVE + lane) * FPS_WAVES + wave;
-            if (c < cells)
-            {
-                const int v = cell_max[c];
-                const unsigned t = cell_tie[c];
-                const bool better = v > best || (v == best && t < best_tk);
-                best = better ? v : best;
-                best_tk = better ? t : best_tk;
-                best_cell = better ? c : best_cell;
-            }
-        }
-        int wave_val;
-        const int wl = winning_lane(best, best_tk, wave_val);
-        const int wave_cell = __builtin_amdgcn_readlane(best_cell, wl);
-        const float4 b = cell_best[wave_cell];
-        if (lane == 0)
-        {
-            WaveRecord rec;
-            rec.val = wave_val;
-            rec.tk = __builtin_amdgcn_readlane(best_tk, wl);
-            rec.k = __float_as_int(b.w);
-            rec.x = b.x;
-            rec.y = b.y;
-            rec.z = b.z;
-            records[j & 1][wave] = rec;
-        }
-        lds_barrier();
-        int k, gv_unused;
-        reduce_records<FPS_WAVES>(records[j & 1], lane, p0x, p0y, p0z, k, sx, sy, sz, gv_unused);
-        if (tid == 0)
-            out[j] = k;
-    }
-}
-
-
-// The same with several samples per round, as in fps_pruned_kernel: after a round's updates the points with the
+// Every wavefront then finds the best of its cells and the results are exchanged through LDS.
+// Several samples are taken per round, as in fps_pruned_kernel: after a round's updates the points with the
 // largest running minima follow each other as samples as long as none of them changes the next one's minimum.
 // Here the order is by (minimum, then the reference's tie key), which is strict - equal minima need no separate
 // path - and a candidate's coordinates are at hand in LDS (the best point of its cell).  LDS also keeps every
@@ -1501,19 +1167,13 @@ void launch_resident(int b, int n, int npoint, int log2_bs, int groups, const fl
 }
 
 
-#ifdef FPS_ONE_PER_ROUND
-constexpr bool FPS_BATCHED = false;
-#else
-constexpr bool FPS_BATCHED = true;
-#endif
-
-template <int PPT, int THREADS, int GS, bool BATCHED>
+template <int PPT, int THREADS, int GS>
 int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float* xyz,
                   int32_t* out, hipStream_t s)
 {
     const int key_capacity = n > CURVE_BINS ? (n + 63) & ~63 : CURVE_BINS; // (the ordering borrows CURVE_BINS words)
     const size_t lds = (static_cast<size_t>(key_capacity) + static_cast<size_t>(PPT) * THREADS + CURVE_BINS) * sizeof(unsigned);
-    auto kernel = fps_pruned_kernel<PPT, THREADS, GS, BATCHED>;
+    auto kernel = fps_pruned_kernel<PPT, THREADS, GS>;
     const int allowed = tpk_allow_lds(reinterpret_cast<const void*>(kernel), lds);
     if (allowed != TPK_OK)
         return allowed;
@@ -1587,18 +1247,16 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
     // groups for the winner to search) except between 4097 and 8192 points.
     if (n <= 512)
         launch_resident<1, FPS_THREADS>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
-    // (FPS_BATCHED: several samples per round; a build with -DFPS_ONE_PER_ROUND keeps the loop that takes one, for
-    // comparison)
     else if (n <= 512 * 2)
-        return launch_pruned<2, 512, 1, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<2, 512, 1>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 4)
-        return launch_pruned<2, 1024, 2, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<2, 1024, 2>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 8)
-        return launch_pruned<4, 1024, 4, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<4, 1024, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= 512 * 16)
-        return launch_pruned<16, 512, 4, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<16, 512, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_REGISTER_POINTS)
-        return launch_pruned<16, 1024, 4, FPS_BATCHED>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
+        return launch_pruned<16, 1024, 4>(b, n, npoint, log2_bs, groups, xyz, idx_out, s);
     else if (n <= FPS_CELL_POINTS && workspace && workspace_bytes >= cell_layout(b, n).total)
     {
         // Cells of 64 points in memory, their summaries in LDS.
@@ -1610,13 +1268,8 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
         int st = launch_curve_cells(cloud, none, nullptr, s);
         if (st != TPK_OK)
             return st;
-#ifdef FPS_ONE_PER_ROUND
-        const size_t lds = static_cast<size_t>(l.cells) * 48 + FPS_LIVE_CAPACITY * FPS_WAVES * sizeof(unsigned short);
-        auto kernel = fps_cells_kernel;
-#else
         const size_t lds = static_cast<size_t>(l.cells) * 56 + FPS_LIVE_CAPACITY * FPS_WAVES * sizeof(unsigned);
         auto kernel = fps_cells_batched_kernel;
-#endif
         st = tpk_allow_lds(reinterpret_cast<const void*>(kernel), lds);
         if (st != TPK_OK)
             return st;

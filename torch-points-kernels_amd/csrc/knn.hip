@@ -468,11 +468,10 @@ extern "C" int tpk_ball_query_sorted_partial_f32(int64_t size_x, int64_t size_y,
     int64_t* ranges_dev = static_cast<int64_t*>(workspace);
     hipLaunchKernelGGL(cloud_ranges_kernel, dim3(5), dim3(KNN_THREADS), 0, s, size_x, size_y, batch_x, batch_y, ranges_dev);
     int64_t ranges[2 * (NP_MAX_CLOUDS + 1)];
-    hipError_t e = hipMemcpyAsync(ranges, ranges_dev, sizeof(ranges), hipMemcpyDeviceToHost, s);
-    if (e == hipSuccess)
-        e = hipStreamSynchronize(s);
-    if (e != hipSuccess)
-        return static_cast<int>(e);
+    static_assert(sizeof(ranges) <= TPK_READ_BACK_BYTES, "the cloud ranges fit the pinned buffer");
+    const int read = tpk_read_back(ranges, ranges_dev, sizeof(ranges), s);
+    if (read != TPK_OK)
+        return read;
     const int64_t* rx = ranges;
     const int64_t* ry = ranges + NP_MAX_CLOUDS + 1;
     void* grid_ws = static_cast<char*>(workspace) + NP_RANGES_BYTES;

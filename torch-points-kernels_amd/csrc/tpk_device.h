@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -68,6 +69,34 @@ static inline int tpk_allow_lds(const void* kernel, size_t bytes)
     if (e != hipSuccess)
         return static_cast<int>(e);
     have = ask;
+    return TPK_OK;
+}
+
+// Copies `bytes` (at most TPK_READ_BACK_BYTES) from device memory at `src` to `dst` behind the work on `stream` and
+// waits for them: for the entry points whose next step depends on what the device computed.  The copy lands in a
+// small pinned buffer that every host thread allocates once and keeps (a copy into pageable memory is staged by the
+// runtime, which blocks the host for longer than the data takes).
+constexpr size_t TPK_READ_BACK_BYTES = 32768;
+static inline int tpk_read_back(void* dst, const void* src, size_t bytes, hipStream_t stream)
+{
+    static thread_local void* pinned = nullptr;
+    if (bytes > TPK_READ_BACK_BYTES)
+        return TPK_ERR_INVALID_ARG;
+    if (!pinned)
+    {
+        const hipError_t made = hipHostMalloc(&pinned, TPK_READ_BACK_BYTES, hipHostMallocDefault);
+        if (made != hipSuccess)
+        {
+            pinned = nullptr;
+            return static_cast<int>(made);
+        }
+    }
+    hipError_t e = hipMemcpyAsync(pinned, src, bytes, hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(stream);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    memcpy(dst, pinned, bytes);
     return TPK_OK;
 }
 
