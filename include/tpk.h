@@ -5,8 +5,11 @@
  * Every entry point takes plain device pointers and sizes, launches on the HIP stream
  * passed as `stream` (a hipStream_t cast to void*; NULL = the null stream), never
  * allocates, never synchronises the host (exceptions, documented below: tpk_grow_proximity and
- * tpk_ball_query_sorted_partial_f32 with a workspace and nsample > 64) and keeps no state between calls.  The caller
- * owns all memory.  All arrays are dense row-major ("contiguous").  Outputs need not be
+ * tpk_ball_query_sorted_partial_f32 with a workspace and nsample > 64) and keeps no state between calls
+ * (exception: tpk_three_nn_static_f32, whose scratch memory is an array inside the library that all calls on a GPU
+ * share).  The first call of a kernel on a device makes a few runtime calls on the host (the kernel's LDS limit;
+ * for tpk_three_nn_static_f32 also the address of its array): a caller that captures HIP graphs makes one call
+ * of the same shape outside the capture first.  The caller owns all memory.  All arrays are dense row-major ("contiguous").  Outputs need not be
  * initialised: every element of every output array is written by the call.
  *
  * Return value: TPK_OK (0); a negative TPK_ERR_* for a rejected argument (nothing was
@@ -168,8 +171,11 @@ int tpk_three_nn_all_pairs_f32(int b, int n, int m, const float* unknown, const 
  * the library runs on holds one until the process ends).  The call allocates and frees nothing.
  * Shapes whose workspace (tpk_three_nn_workspace_bytes()) exceeds the array are rejected with
  * TPK_ERR_TOO_LARGE before anything is launched; shapes that need no workspace run the all
- * pairs scan.  All calls on one GPU share that GPU's array: calls that overlap there (different
- * streams or host threads) race; calls on one stream are safe.
+ * pairs scan.  All calls on one GPU share that GPU's array, its contents (the per-cloud words
+ * included) are whatever the last call left: calls that overlap there (different streams or host
+ * threads) race; calls on one stream are safe.  The first call on a device looks up the array's
+ * address and sets the kernels' LDS limits (host runtime calls, no allocation): make one call per
+ * device before capturing a graph that contains this entry point.
  * ------------------------------------------------------------------------------------- */
 #define TPK_THREE_NN_STATIC_SCRATCH_BYTES (8u << 20)
 size_t tpk_three_nn_static_scratch_bytes(void);

@@ -1685,3 +1685,76 @@ def test_extension_rejects_bad_tensors(tpk, dev):
     with pytest.raises(RuntimeError):
         tpk.three_interpolate(torch.rand(2, 4, 16, device=dev), torch.zeros(2, 8, 3, dtype=torch.int64, device=dev),
                               torch.rand(2, 8, 3, device=dev))  # idx must be int32, as three_nn returns it
+
+
+def test_lists_layout_and_fillers(dev):
+    """The inverted index that the backward gathers walk, read back from the device: every index entry appears once in
+    the list of its target, a target nobody refers to owns one empty entry, the last entry of every list is marked, and
+    the places that fill a span's last row refer to nothing - as offset 0x7ff3fffc, which the walker relies on to lie
+    beyond the LDS (reads there return zero)."""
+    import ctypes
+    import os
+
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "torch-points-kernels_amd",
+                                   "torch_points_kernels", "libtpk_hip.so"))
+    lib.tpk_three_interpolate_grad_workspace_bytes.restype = ctypes.c_size_t
+    NOTHING, LAST, SPANS, WAVE, GAP = 0x7FF3FFFC, 0x80000000, 16, 64, 128
+    for b, n, m in ((2, 3000, 500), (1, 20001, 130), (3, 700, 40)):
+        g = torch.Generator().manual_seed(n + m)
+        idx = torch.randint(0, m, (b, n, 3), generator=g, dtype=torch.int32)
+        idx[idx == 7] = 8  # target 7 keeps an empty list
+        weight = torch.rand(b, n, 3, generator=g)
+        nbytes = lib.tpk_three_interpolate_grad_workspace_bytes(b, n, m)
+        assert nbytes > 0
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        di, dw = idx.to(dev), weight.to(dev)
+        st = lib.tpk_three_interpolate_lists_f32(b, n, m, ctypes.c_void_p(di.data_ptr()), ctypes.c_void_p(dw.data_ptr()),
+                                                 ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(nbytes), None)
+        assert st == 0
+        torch.cuda.synchronize()
+        raw = ws.cpu().numpy()
+        # the shape the library chose: rows of grad_out staged together, columns per part (gather.hip, bwd_shape)
+        span = -(-m // SPANS)
+        n4 = (n + 3) & ~3
+        for r in (4, 2, 1):
+            room = min(40960 // r - span * SPANS, 32768 // r) & ~3
+            if room >= n4 or (r == 1 and room >= 4096):
+                part_len = min(n4, room)
+                break
+        parts = -(-n // part_len)
+        cloud_parts = b * parts
+        align = lambda v: (v + 255) & ~255
+        capacity = ((part_len * 3 + m + 63) & ~63) + GAP * SPANS + 64
+        regions = raw[: cloud_parts * SPANS * 16].view(np.int32).reshape(cloud_parts, SPANS, 4)
+        off = align(cloud_parts * SPANS * 16) + align(cloud_parts * SPANS * WAVE * 4)
+        entries = raw[off : off + cloud_parts * capacity * 8].view(np.uint32).reshape(cloud_parts, capacity, 2)
+        weights = raw[off : off + cloud_parts * capacity * 8].view(np.float32).reshape(cloud_parts, capacity, 2)[..., 1]
+        for cp in range(cloud_parts):
+            cloud, part = divmod(cp, parts)
+            col0 = part * part_len
+            cols = min(part_len, n - col0)
+            want = {}
+            for j in range(cols):
+                for k in range(3):
+                    want.setdefault(int(idx[cloud, col0 + j, k]), []).append((j, float(weight[cloud, col0 + j, k])))
+            for s in range(SPANS):
+                base, length, steps, _ = (int(v) for v in regions[cp, s])
+                t0, t1 = min(s * span, m), min((s + 1) * span, m)
+                assert steps == -(-length // WAVE)
+                ranks = np.arange(steps * WAVE)
+                at = base + (ranks % max(steps, 1)) * WAVE + ranks // max(steps, 1)  # rank q -> lane q / c, step q % c
+                js, ws_ = entries[cp, at, 0], weights[cp, at]
+                # behind the last entry of the span: entries that refer to nothing
+                assert (js[length:] == NOTHING).all() and (ws_[length:] == 0).all()
+                target, got = t0, {}
+                for q in range(length):
+                    j = int(js[q])
+                    if (j & 0x7FFFFFFF) != NOTHING:
+                        got.setdefault(target, []).append(((j & 0x7FFFFFFF) >> 2, float(ws_[q])))
+                    else:
+                        assert j == (NOTHING | LAST) and target not in want  # the one entry of an empty list
+                    if j & LAST:
+                        target += 1
+                assert target == t1
+                for t in range(t0, t1):
+                    assert sorted(got.get(t, [])) == sorted(want.get(t, [])), (cp, s, t)
