@@ -36,7 +36,7 @@ VALU_FILE = os.path.join(PROFILES, "distance_scans_valu_utilisation.txt")
 
 # Kernels whose HBM traffic adds up to one launch of an operator (names as rocprofv3 prints them).
 TRAFFIC_KERNELS = {
-    "fps": ["fps_pruned_kernel<16, 1024, 4, true>"],
+    "fps": ["fps_pruned_kernel<16, 1024, 4>"],
     "three_interpolate_fwd": ["gather_fwd_lds_kernel<3, true, int, true>"],
     "three_interpolate_bwd": ["build_lists_kernel<3, true, int>", "gather_bwd_lists_kernel<3, true, 2>"],
     "three_interpolate_bwd_lists": ["gather_bwd_lists_kernel<3, true, 2>"],
@@ -47,9 +47,9 @@ TRAFFIC_KERNELS = {
 }
 # Kernels whose VALU counters describe a distance scan.
 VALU_KERNELS = {
-    "fps": "fps_pruned_kernel<16, 1024, 4, true>",
+    "fps": "fps_pruned_kernel<16, 1024, 4>",
     "ball_query_dense": "ball_query_dense_cells_kernel<false>",
-    "ball_query_partial_dense": "ball_query_bins_kernel<false>",
+    "ball_query_partial_dense": "ball_query_bins_kernel<false, false>",
     "three_nn": "three_nn_cells_kernel",
     "chamfer_fwd": "chamfer_grid_kernel",
 }
