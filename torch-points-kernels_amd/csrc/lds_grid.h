@@ -3,15 +3,18 @@
 //
 // Build: bounding box of the finite coordinates, up to LG_AXIS cells per axis and LG_CELLS in all sized for
 // about LG_PER_CELL points per cell (a flat cloud gets a flat grid), a count per cell (LDS atomics that also
-// hand every point its place inside its cell), a prefix sum, the points written cell by cell as four arrays
-// (x, y, z, index).  Search: cells are numbered x first, so the (up to) three cells of a row (y, z) are one run
-// of consecutive places; a lane walks the runs around its query point by point - its own cell first, a row is
+// hand every point its place inside its cell), a prefix sum, the points written cell by cell as records
+// (x, y, z, index) of 16 bytes.  Search: cells are numbered x first, so the (up to) three cells of a row (y, z)
+// are one run of consecutive places; a lane walks the runs around its query point by point - its own cell first, a row is
 // passed over when its distance in (y, z) already exceeds the bound the lane's best entries set - and the answer
 // is final when that bound is smaller than the distance to every face of the examined block that has cells
 // behind it; otherwise the faces that are too near are pushed out by one layer of cells each and only the new
-// layers are examined.  Lanes of a wavefront walk different cells: LDS serves their scattered 4-byte reads at
-// a third of the rate of consecutive ones, which is what the search is bound by together with the issue of the
-// distance arithmetic.
+// layers are examined.  The lanes of a wavefront examine their runs together - a run takes the wavefront as many
+// steps as the longest of its 64 runs has points, about twice the average - and what bounds the search is the issue
+// of its instructions (four wavefronts share a SIMD): 17 for a candidate, 45 to set up a run.  The build is
+// bound the same way - every instruction of it costs the workgroup 16 clocks - hence the grid's shape comes
+// from the first wavefront alone, and a point is one 16-byte record: one LDS write when it is placed, one read
+// per candidate (four arrays x, y, z, index: 2.5 us more per call on 16 clouds of 4096 points, 16384 queries each).
 #pragma once
 
 #include "tpk_device.h"
@@ -48,6 +51,31 @@ __device__ __forceinline__ float lg_wave_min(float v)
     return fminf(fminf(tpk_read_lane(v, 0), tpk_read_lane(v, 16)), fminf(tpk_read_lane(v, 32), tpk_read_lane(v, 48)));
 }
 
+// Minimum / maximum of two numbers that are not NaN, in one instruction (fminf / fmaxf first turn a signalling
+// NaN that cannot occur here into a quiet one, an instruction per operand).
+__device__ __forceinline__ float lg_min(float a, float b)
+{
+    float r;
+    asm("v_min_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float lg_max(float a, float b)
+{
+    float r;
+    asm("v_max_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+// A float as an integer that orders the same way, and back.
+__device__ __forceinline__ int lg_ordered(float f)
+{
+    const int b = __float_as_int(f);
+    return b >= 0 ? b : b ^ 0x7FFFFFFF;
+}
+__device__ __forceinline__ float lg_unordered(int b)
+{
+    return __int_as_float(b >= 0 ? b : b ^ 0x7FFFFFFF);
+}
+
 // Cell along one axis, clamped to the grid (NaN goes to cell 0).
 __device__ __forceinline__ int lg_cell(float t, int cells)
 {
@@ -63,8 +91,7 @@ __device__ __forceinline__ unsigned long long lg_key(float d, int i)
 
 struct LdsGrid
 {
-    float *sx, *sy, *sz; // [m] each: the points cell by cell
-    int* si;             // [m] their indices
+    float4* points;      // [m] the points cell by cell: x, y, z, index
     int* starts;         // [LG_STARTS] first place of every cell, then the number of points
     float lo[3], inv[3], width[3];
     int cells[3];
@@ -77,18 +104,17 @@ struct LdsGrid
 __device__ __forceinline__ void lds_grid_build(LdsGrid& g, unsigned char* lds, const float* __restrict__ known, int m,
                                                int index_base)
 {
-    float* const sx = g.sx = reinterpret_cast<float*>(lds);
-    float* const sy = g.sy = sx + m;
-    float* const sz = g.sz = sy + m;
-    int* const si = g.si = reinterpret_cast<int*>(sz + m);
-    int* const starts = g.starts = si + m;
-    __shared__ float box_parts[6][LG_WAVES]; // per wavefront: min x, y, z then -max x, y, z
-    __shared__ float box[6];
+    float4* const points = g.points = reinterpret_cast<float4*>(lds);
+    int* const starts = g.starts = reinterpret_cast<int*>(points + m);
+    __shared__ int box[6];      // ordered ints: min x, y, z then max x, y, z of the finite coordinates
+    __shared__ float shape[12]; // lo, inv, width, cells of the grid, from the first wavefront
     __shared__ int wave_totals[LG_WAVES];
     __shared__ int crowding; // sum over the cells of count^2
     const int tid = threadIdx.x;
     const int lane = tid & (TPK_WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / TPK_WAVE);
+    if (tid < 6)
+        box[tid] = tid < 3 ? 0x7FFFFFFF : INT_MIN;
     __syncthreads();
 
     // ---- the cloud's points and bounding box (finite coordinates only) ----
@@ -106,88 +132,92 @@ __device__ __forceinline__ void lds_grid_build(LdsGrid& g, unsigned char* lds, c
     if (tid == 0)
         crowding = 0;
     {
+        // (rows past the end repeat the last point: no effect on the box)
         const float inf = __builtin_inff();
-        float ends[6] = {inf, inf, inf, inf, inf, inf}; // (minima of -max: one kind of reduction)
+        float lows[3] = {inf, inf, inf}, highs[3] = {-inf, -inf, -inf};
 #pragma unroll
         for (int u = 0; u < LG_PER_THREAD; ++u)
         {
-            // (rows past the end repeat the last point: no effect on the box)
             const float v[3] = {px[u], py[u], pz[u]};
 #pragma unroll
             for (int a = 0; a < 3; ++a)
-                if (fabsf(v[a]) < inf)
-                {
-                    ends[a] = fminf(ends[a], v[a]);
-                    ends[3 + a] = fminf(ends[3 + a], -v[a]);
-                }
+            {
+                const bool finite = fabsf(v[a]) < inf;
+                lows[a] = lg_min(lows[a], finite ? v[a] : inf);
+                highs[a] = lg_max(highs[a], finite ? v[a] : -inf);
+            }
         }
 #pragma unroll
-        for (int a = 0; a < 6; ++a)
+        for (int a = 0; a < 3; ++a)
         {
-            const float e = lg_wave_min(ends[a]);
+            const int low = ~wave_max_i32(~lg_ordered(lows[a])), high = wave_max_i32(lg_ordered(highs[a]));
             if (lane == 0)
-                box_parts[a][wave] = e;
-        }
-    }
-    __syncthreads();
-    if (wave == 0)
-    {
-#pragma unroll
-        for (int a = 0; a < 6; ++a)
-        {
-            const float e = lg_row_min(box_parts[a][lane & (LG_WAVES - 1)]);
-            if (lane == 0)
-                box[a] = e;
+            {
+                atomicMin(&box[a], low);
+                atomicMax(&box[3 + a], high);
+            }
         }
     }
     __syncthreads();
 
     // ---- the grid: about LG_PER_CELL points per cell, cells as cubic as LG_AXIS per axis and LG_CELLS in
-    // all allow (a flat cloud gets a flat grid of up to 64 x 64 cells) ----
-    float lo[3], inv[3], width[3];
-    int cells[3];
+    // all allow (a flat cloud gets a flat grid of up to 64 x 64 cells).  The first wavefront works it out, its
+    // lanes trying 64 sizes at a time. ----
+    if (wave == 0)
     {
-        float extent[3], longest = 0.0f;
+        float low[3], extent[3], longest = 0.0f;
 #pragma unroll
         for (int a = 0; a < 3; ++a)
         {
-            lo[a] = box[a];
-            extent[a] = -box[3 + a] - lo[a]; // (NaN or -inf for a cloud without finite coordinates)
+            low[a] = lg_unordered(box[a]);
+            extent[a] = lg_unordered(box[3 + a]) - low[a]; // (NaN or -inf for a cloud without finite coordinates)
             extent[a] = extent[a] > 0.0f ? extent[a] : 0.0f;
             longest = fmaxf(longest, extent[a]);
         }
+        float share[3]; // of the longest axis
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+            share[a] = longest > 0.0f ? extent[a] / longest : 0.0f;
         // cells per axis for `along` cells along the longest axis, and their product
         auto fit = [&](float along, int (&count)[3]) __attribute__((always_inline)) {
             int all = 1;
 #pragma unroll
             for (int a = 0; a < 3; ++a)
             {
-                const float f = longest > 0.0f ? fminf(extent[a] / longest * along + 0.5f, static_cast<float>(LG_AXIS)) : 1.0f;
+                const float f = longest > 0.0f ? fminf(share[a] * along + 0.5f, static_cast<float>(LG_AXIS)) : 1.0f;
                 count[a] = f >= 1.0f ? static_cast<int>(f) : 1;
                 all *= count[a];
             }
             return all;
         };
-        // (the product grows with `along`: the largest value that stays within the cells wanted, by bisection)
+        // (the product grows with `along`: the largest of the sizes tried that stays within the cells wanted, in
+        // steps of 2 up to 2 * LG_AXIS, then in steps of 1 / 32 inside the step found)
         const int wanted = static_cast<int>(fminf(static_cast<float>(LG_CELLS), fmaxf(static_cast<float>(m) / LG_PER_CELL, 1.0f)));
-        float few = 0.0f, many = 2.0f * LG_AXIS;
-        for (int step = 0; step < 12; ++step)
+        int count[3];
+        const int coarse = __builtin_popcountll(__ballot(fit(2.0f * static_cast<float>(lane + 1), count) <= wanted));
+        const int fine = __builtin_popcountll(__ballot(fit(2.0f * static_cast<float>(coarse) + static_cast<float>(lane + 1) * (1.0f / 32.0f), count) <= wanted));
+        fit(2.0f * static_cast<float>(coarse) + static_cast<float>(fine) * (1.0f / 32.0f), count);
+        if (lane < 3)
         {
-            const float mid = 0.5f * (few + many);
-            int count[3];
-            if (fit(mid, count) > wanted)
-                many = mid;
-            else
-                few = mid;
+            const float e = lane == 0 ? extent[0] : lane == 1 ? extent[1] : extent[2];
+            const float l = lane == 0 ? low[0] : lane == 1 ? low[1] : low[2];
+            const int k = lane == 0 ? count[0] : lane == 1 ? count[1] : count[2];
+            shape[lane] = e > 0.0f ? l : 0.0f;
+            shape[3 + lane] = e > 0.0f ? static_cast<float>(k) / e : 0.0f;
+            shape[6 + lane] = e / static_cast<float>(k);
+            shape[9 + lane] = __int_as_float(k);
         }
-        fit(few, cells);
+    }
+    __syncthreads();
+    float lo[3], inv[3], width[3];
+    int cells[3];
 #pragma unroll
-        for (int a = 0; a < 3; ++a)
-        {
-            inv[a] = extent[a] > 0.0f ? static_cast<float>(cells[a]) / extent[a] : 0.0f;
-            width[a] = extent[a] / static_cast<float>(cells[a]);
-            lo[a] = extent[a] > 0.0f ? lo[a] : 0.0f;
-        }
+    for (int a = 0; a < 3; ++a)
+    {
+        lo[a] = shape[a];
+        inv[a] = shape[3 + a];
+        width[a] = shape[6 + a];
+        cells[a] = __float_as_int(shape[9 + a]);
     }
 
     // ---- count per cell; the count before a point's own increment is its place inside the cell ----
@@ -231,10 +261,7 @@ __device__ __forceinline__ void lds_grid_build(LdsGrid& g, unsigned char* lds, c
         if (tid + u * LG_THREADS < m)
         {
             const int at = starts[placed[u] >> 16] + (placed[u] & 0xFFFF);
-            sx[at] = px[u];
-            sy[at] = py[u];
-            sz[at] = pz[u];
-            si[at] = index_base + tid + u * LG_THREADS;
+            points[at] = make_float4(px[u], py[u], pz[u], __int_as_float(index_base + tid + u * LG_THREADS));
         }
     __syncthreads();
     g.crowd = static_cast<float>(crowding) / static_cast<float>(m);
@@ -253,10 +280,7 @@ __device__ __forceinline__ void lds_grid_build(LdsGrid& g, unsigned char* lds, c
 template <typename Best>
 __device__ __forceinline__ void lds_grid_search(const LdsGrid& g, float qx, float qy, float qz, Best& best TPK_WORK_PARAM)
 {
-    const float* const sx = g.sx;
-    const float* const sy = g.sy;
-    const float* const sz = g.sz;
-    const int* const si = g.si;
+    const float4* const points = g.points;
     const int* const starts = g.starts;
     const float(&lo)[3] = g.lo;
     const float(&inv)[3] = g.inv;
@@ -279,7 +303,7 @@ __device__ __forceinline__ void lds_grid_search(const LdsGrid& g, float qx, floa
         return k == c[a] ? 0.0f : fmaxf(gap - slack[a], 0.0f) * width[a];
     };
     // The runs of a box of cells, one per (y, z), point by point.  A run no point of which can beat the
-    // bound so far is passed over.  (The index is read only when the distance does not rule it out.)
+    // bound so far is passed over.
     auto examine = [&](int x0, int x1, int y0, int y1, int z0, int z1) __attribute__((always_inline)) {
         const int run = x1 - x0 + 1;
         int y = y0, z = z0, pos = 0, end = 0;
@@ -304,9 +328,10 @@ __device__ __forceinline__ void lds_grid_search(const LdsGrid& g, float qx, floa
                 continue;
             }
             TPK_WORK_ADD(1);
-            const float d = tpk_dist2(qx, qy, qz, sx[pos], sy[pos], sz[pos]);
+            const float4 p = points[pos];
+            const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
             if (d <= best.bound())
-                best.offer(lg_key(d, si[pos]));
+                best.offer(lg_key(d, __float_as_int(p.w)));
             ++pos;
         }
     };
@@ -383,9 +408,10 @@ __device__ __forceinline__ void lds_grid_scan_all(const LdsGrid& g, int m, float
     for (int k = 0; k < m; ++k)
     {
         TPK_WORK_ADD(1);
-        const float d = tpk_dist2(qx, qy, qz, g.sx[k], g.sy[k], g.sz[k]);
+        const float4 p = g.points[k];
+        const float d = tpk_dist2(qx, qy, qz, p.x, p.y, p.z);
         if (d <= best.bound())
-            best.offer(lg_key(d, g.si[k]));
+            best.offer(lg_key(d, __float_as_int(p.w)));
     }
 }
 
