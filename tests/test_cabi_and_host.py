@@ -59,7 +59,12 @@ def test_library_exports_every_declared_symbol():
     lib.tpk_fps_workspace_bytes.restype = ctypes.c_size_t
     assert lib.tpk_fps_workspace_bytes(4, 16384) == 0
     # 16385..163840 points: records (16 B), boxes (160 B per cell of 64) and minima (4 B) of whole windows of 16384
-    assert lib.tpk_fps_workspace_bytes(4, 50000) == 4 * 4 * 256 * (64 * 16 + 160 + 64 * 4)
+    # and, for the coarse order in front: a record (16 B) and a place (4 B) per point, and per chunk of 16384 points
+    # of the batch two clouds' spans (16 B), boxes (48 B) and counts (2 x 4096 x 4 B), every array a multiple of 256 B
+    up = lambda v: (v + 255) // 256 * 256
+    chunks = (4 * 50000 + 16383) // 16384
+    coarse = up(4 * 50000 * 16) + up(4 * 50000 * 4) + up(chunks * 16) + up(chunks * 48) + up(chunks * 2 * 4096 * 4)
+    assert lib.tpk_fps_workspace_bytes(4, 50000) == 4 * 4 * 256 * (64 * 16 + 160 + 64 * 4) + coarse
     assert lib.tpk_fps_workspace_bytes(2, 200000) == 2 * 200000 * 4  # larger: the minima only
     # searches over curve-ordered cells: 16 bytes per point padded to cells of 64, 160 bytes per cell;
     # 0 = the shape is served by the all-pairs scan, no workspace wanted

@@ -32,6 +32,9 @@ struct PointSet
     int* wide_first;      // optional (with boxes) [windows][cells]: the window's cells, those with much wider boxes than
                           // the window's average first - the cells whose queries take a search longest
     const int* only;      // optional [clouds]: a cloud whose word is 0 is left out (dense layout)
+    const float4* records; // optional [total]: the points as (x, y, z, index) records to be read instead of xyz -
+                           // an array that has been brought into a coarse order (coarse_order.h), whose records
+                           // carry the numbers the points had before
 };
 
 __host__ __device__ inline int set_cells(const PointSet& s)
@@ -152,6 +155,7 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     const int n = static_cast<int>(tpk_min64(set.stride, set.cloud_points - in_cloud));
     const int cells = set_cells(set);
     const float* __restrict__ xyz = set.xyz + start * 3;
+    const float4* __restrict__ records = set.records ? set.records + start : nullptr;
     const int64_t* __restrict__ group = set.group ? set.group + start : nullptr;
     float4* __restrict__ sorted = set.sorted + window * cells * NG_CELL;
     float4* __restrict__ boxes = set.boxes ? set.boxes + window * cells * NG_BOX : nullptr;
@@ -169,9 +173,19 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
     for (int u = 0; u < PER; ++u)
     {
         const int k = min(tid + u * NG_SORT_THREADS, n - 1);
+        if (records)
+        {
+            const float4 r = records[k];
+            p[u][0] = r.x;
+            p[u][1] = r.y;
+            p[u][2] = r.z;
+        }
+        else
+        {
 #pragma unroll
-        for (int a = 0; a < 3; ++a)
-            p[u][a] = xyz[k * 3 + a];
+            for (int a = 0; a < 3; ++a)
+                p[u][a] = xyz[k * 3 + a];
+        }
     }
     // (with cloud ids: how far a point's id lies above the window's first, cut at 7)
     int id_offset[PER];
@@ -274,11 +288,22 @@ __global__ __launch_bounds__(NG_SORT_THREADS) void curve_cells_kernel(PointSet s
 #pragma unroll
         for (int u = 0; u < PER; ++u)
             place[u] = tid + u * NG_SORT_THREADS < n ? atomicAdd(&bins[bin[u]], 1) : -1;
+        // (records: the number a point had before the coarse order - read once more, the line is still near)
+        int number[PER];
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            number[u] = static_cast<int>(in_cloud) + tid + u * NG_SORT_THREADS;
+        if (records)
+        {
+#pragma unroll
+            for (int u = 0; u < PER; ++u)
+                if (place[u] >= 0)
+                    number[u] = __float_as_int(records[tid + u * NG_SORT_THREADS].w);
+        }
 #pragma unroll
         for (int u = 0; u < PER; ++u)
             if (place[u] >= 0)
-                sorted[place[u]] = make_float4(p[u][0], p[u][1], p[u][2],
-                                               __int_as_float(static_cast<int>(in_cloud) + tid + u * NG_SORT_THREADS));
+                sorted[place[u]] = make_float4(p[u][0], p[u][1], p[u][2], __int_as_float(number[u]));
     }
     const int padded = cells * NG_CELL;
     {

@@ -28,7 +28,7 @@
 // k among its own equal maxima, and the halving tree then prefers the thread whose number
 // has the smaller bit-reversal.  Both rules together are "smallest tie key", with
 //   key(k) = bitrev(k mod BS) * ceil(n / BS) + floor(k / BS).
-#include "curve_cells.h"
+#include "coarse_order.h"
 
 #include <cmath>
 
@@ -1186,7 +1186,7 @@ int launch_pruned(int b, int n, int npoint, int log2_bs, int groups, const float
 struct CellLayout
 {
     int cells; // per cloud
-    size_t sorted, boxes, temp, total;
+    size_t sorted, boxes, temp, coarse, total;
 };
 CellLayout cell_layout(int b, int n)
 {
@@ -1197,7 +1197,9 @@ CellLayout cell_layout(int b, int n)
     l.sorted = 0;
     l.boxes = up(all * NG_CELL * sizeof(float4));
     l.temp = up(l.boxes + all * NG_BOX * sizeof(float4));
-    l.total = up(l.temp + all * NG_CELL * sizeof(float));
+    l.coarse = up(l.temp + all * NG_CELL * sizeof(float));
+    // (clouds of many windows are brought into a coarse order first: coarse_order.h)
+    l.total = n >= CO_MIN_ROWS ? up(l.coarse + coarse_layout(static_cast<int64_t>(b) * n).total) : l.coarse;
     return l;
 }
 
@@ -1265,7 +1267,16 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
         PointSet cloud{xyz, nullptr, static_cast<int64_t>(b) * n, n, FPS_CELL_WINDOW,
                        reinterpret_cast<float4*>(w + l.sorted), reinterpret_cast<float4*>(w + l.boxes), nullptr, nullptr};
         PointSet none{nullptr, nullptr, 0, 1, FPS_CELL_WINDOW, nullptr, nullptr, nullptr, nullptr};
-        int st = launch_curve_cells(cloud, none, nullptr, s);
+        int st = TPK_OK;
+        if (n >= CO_MIN_ROWS)
+        {
+            // windows that are neighbourhoods instead of samples of the whole cloud: cells half as wide
+            st = launch_coarse_order(xyz, nullptr, static_cast<int64_t>(b) * n, n, true, CO_MIN_ROWS, w + l.coarse, s);
+            if (st != TPK_OK)
+                return st;
+            cloud.records = reinterpret_cast<const float4*>(w + l.coarse);
+        }
+        st = launch_curve_cells(cloud, none, nullptr, s);
         if (st != TPK_OK)
             return st;
         const size_t lds = static_cast<size_t>(l.cells) * 56 + FPS_LIVE_CAPACITY * FPS_WAVES * sizeof(unsigned);
