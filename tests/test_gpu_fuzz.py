@@ -59,8 +59,8 @@ def _packed(rng, kind, sizes_from, max_queries):
 
 
 def _fps(rng, kind, tpk, nat, oracle, dev):
-    B = int(rng.integers(1, 3))
-    n = int(rng.choice([300, 513, 700, 1024, 1500, 3000, 5000, 9000, 16384, 16390, 21000, 40000]))
+    B = int(rng.integers(1, 4))
+    n = int(rng.choice([300, 513, 700, 1024, 1500, 3000, 5000, 9000, 16384, 16390, 21000, 33000, 40000, 70000]))
     npoint = int(rng.integers(1, min(n, 600 if n <= 16384 else 120)))
     x = _cloud(rng, B, n, kind) + (0.0 if kind != 3 else 0.3)
     _eq(tpk.furthest_point_sample(x.to(dev), npoint), oracle.furthest_point_sample(x.numpy(), npoint), "fps %s" % ((B, n, npoint, kind),))
@@ -177,7 +177,7 @@ def _ball_packed(rng, kind, tpk, nat, oracle, dev):
 
 def _ball_dense(rng, kind, tpk, nat, oracle, dev):
     B = int(rng.integers(1, 4))
-    n = int(rng.choice([1, 40, 512, 777, 3000, 4096, 17000]))
+    n = int(rng.choice([1, 40, 512, 777, 3000, 4096, 17000, 20000, 70000]))
     m = int(rng.choice([1, 100, 512, 1024, 3000]))
     r = float(rng.choice([0.01, 0.05, 0.1, 0.3, 1.0]))
     ns = int(rng.choice([1, 5, 16, 32, 64, 100]))
