@@ -1352,6 +1352,45 @@ def test_chamfer_parity(tpk, oracle, dev, B, n, m, dtype):
     np.testing.assert_allclose(_np(gb), wb, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_chamfer_backward_skewed_indices(tpk, dev, dtype):
+    # The backward pass keeps, per range of points, the other cloud's points that chose one of them in LDS, with
+    # room for the share of the other cloud a range expects and a third more.  Here every point of the second cloud
+    # names one of the first 900 points of the first (some of them hundreds of times), so one range meets all 16384
+    # and takes the chains of point numbers instead; the first cloud's indices are uniform (entries in LDS); the
+    # second pair has them the other way round.  Checked against sums formed in float64, to the stated tolerance
+    # plus the reordering allowance.
+    B, n, m = 2, 16384, 16384
+    g = torch.Generator().manual_seed(9)
+    a, b = torch.rand(B, n, 3, generator=g, dtype=dtype), torch.rand(B, m, 3, generator=g, dtype=dtype)
+    i1 = torch.randint(0, m, (B, n), generator=g, dtype=torch.int32)
+    i2 = (torch.rand(B, m, generator=g) ** 3 * 900).to(torch.int32)
+    i1[1], i2[1] = (torch.rand(n, generator=g) ** 3 * 900).to(torch.int32), torch.randint(0, n, (m,), generator=g, dtype=torch.int32)
+    g1, g2 = torch.randn(B, n, generator=g, dtype=dtype), torch.randn(B, m, generator=g, dtype=dtype)
+    native = __import__("torch_points_kernels._native", fromlist=["native"]).native()
+    ga, gb = native.chamfer_dist_grad(a.to(dev), b.to(dev), i1.to(dev), i2.to(dev), g1.to(dev), g2.to(dev))
+    an, bn, g1n, g2n = (t.numpy().astype(np.float64) for t in (a, b, g1, g2))
+    wa, wb, ma, mb = (np.zeros((B, k, 3)) for k in (n, m, n, m))
+    for c in range(B):
+        j1, j2 = i1[c].numpy().astype(np.int64), i2[c].numpy().astype(np.int64)
+        t1 = 2 * g1n[c][:, None] * (an[c] - bn[c][j1])  # d dist1[i] / d xyz1[i]; its negative goes to xyz2[j1[i]]
+        t2 = 2 * g2n[c][:, None] * (bn[c] - an[c][j2])
+        wa[c] += t1
+        wb[c] += t2
+        np.add.at(wb[c], j1, -t1)
+        np.add.at(wa[c], j2, -t2)
+        ma[c] += np.abs(t1)
+        mb[c] += np.abs(t2)
+        np.add.at(mb[c], j1, np.abs(t1))
+        np.add.at(ma[c], j2, np.abs(t2))
+    if dtype == torch.float64:
+        np.testing.assert_allclose(_np(ga), wa, rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(_np(gb), wb, rtol=1e-12, atol=1e-12)
+    else:
+        _assert_scatter_sum_close(_np(ga), wa.astype(np.float32), ma.astype(np.float32), "chamfer backward, skewed indices, xyz1")
+        _assert_scatter_sum_close(_np(gb), wb.astype(np.float32), mb.astype(np.float32), "chamfer backward, skewed indices, xyz2")
+
+
 def test_chamfer_ties_take_lowest_index(tpk, oracle, dev):
     a = torch.zeros(1, 300, 3)
     b = torch.full((1, 3000, 3), 5.0)

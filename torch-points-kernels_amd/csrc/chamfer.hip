@@ -261,23 +261,41 @@ __global__ __launch_bounds__(256) void chamfer_bwd_scatter_kernel(
 // Backward without float atomics and without workspace.  A workgroup owns a range of points
 // ("targets") of one cloud of one pair.  It first threads the points of the OTHER cloud that
 // chose one of its targets as nearest neighbour into per-target chains held in LDS: one LDS
-// integer exchange per point (head[target] <- point, next[point] <- old head).  Then one lane per
+// integer exchange per point (head[target] <- entry, next[entry] <- old head).  Then one lane per
 // target adds the target's own term and walks its chain (most chains hold zero to two points).
 // Every output is written once, nothing is zero-filled.  The order of a chain is the order in
 // which the exchanges happened to be served, so - as with the reference's atomics - the sum of
 // a point with several terms may differ in the last bits from run to run.
-// dynamic LDS: (points of the larger cloud + targets per workgroup) ints.
+//
+// What a chain holds: the workgroup reads the other cloud's indices in order anyway, so for a point that chose one
+// of its targets it reads the point's coordinates and gradient in the same pass - consecutive addresses - and
+// keeps them in LDS as the chain's entry (x, y, z, 2 g; next).  The walk then reads LDS only, and the one
+// scattered read per target that remains is the target's own nearest point.  (Entries that name the other
+// cloud's points, their coordinates and gradients fetched during the walk, were the first version: four scattered
+// 4- and 12-byte reads per target, and a compute unit serves a scattered read at about 1.7 clocks per lane
+// whatever its width - 8800 of 10500 clocks per 1024 targets.)  A range's share of the other cloud is about
+// range / points of it; room is kept for `capacity` entries, and a workgroup that meets more (a range that
+// much of the other cloud chose) builds chains of point numbers instead, as before.
+// dynamic LDS: lds_ints ints.
 constexpr int CHB_THREADS = 1024;
-constexpr int CHB_LDS_INTS = 38912; // 152 KiB: chains of the other cloud's points + heads of a range
+constexpr int CHB_LDS_INTS = 38912; // 152 KiB
+
+// LDS words of one entry: four values and the link.
+template <typename T>
+constexpr int chb_entry_ints()
+{
+    return 4 * static_cast<int>(sizeof(T) / sizeof(int)) + 1;
+}
 
 template <typename T>
 __global__ __launch_bounds__(CHB_THREADS) void chamfer_bwd_chains_kernel(
-    int n, int m, int clouds, int splits, int range1, int range2, const T* __restrict__ xyz1,
+    int n, int m, int clouds, int splits, int range1, int range2, int lds_ints, const T* __restrict__ xyz1,
     const T* __restrict__ xyz2, const int32_t* __restrict__ idx1, const int32_t* __restrict__ idx2,
     const T* __restrict__ grad_dist1, const T* __restrict__ grad_dist2, T* __restrict__ grad_xyz1,
     T* __restrict__ grad_xyz2)
 {
-    extern __shared__ int chain_lds[];
+    extern __shared__ __align__(16) int chain_lds[];
+    __shared__ int entries; // entries asked for (may exceed the room)
     // logical workgroup = ((cloud * 2 + direction) * splits + split); those of a pair run on one
     // die, whose L2 then serves the random reads into the pair's points
     const int lin = static_cast<int>(xcd_local_block(blockIdx.x, gridDim.x));
@@ -292,8 +310,6 @@ __global__ __launch_bounds__(CHB_THREADS) void chamfer_bwd_chains_kernel(
     const int t1 = min(t0 + range, npts);
     if (t0 >= t1)
         return; // (the whole workgroup: no barrier has been passed yet)
-    int* const next = chain_lds;
-    int* const head = chain_lds + nother;
     const int tid = threadIdx.x;
     const T* __restrict__ own = (second ? xyz2 : xyz1) + static_cast<int64_t>(cloud) * npts * 3;
     const T* __restrict__ other = (second ? xyz1 : xyz2) + static_cast<int64_t>(cloud) * nother * 3;
@@ -303,8 +319,15 @@ __global__ __launch_bounds__(CHB_THREADS) void chamfer_bwd_chains_kernel(
     const T* __restrict__ other_g = (second ? grad_dist1 : grad_dist2) + static_cast<int64_t>(cloud) * nother;
     T* __restrict__ out = (second ? grad_xyz2 : grad_xyz1) + static_cast<int64_t>(cloud) * npts * 3;
 
+    // entries in LDS: values [capacity][4], links [capacity], heads [range]
+    const int capacity = min(nother, (lds_ints - range) / chb_entry_ints<T>());
+    T* const values = reinterpret_cast<T*>(chain_lds);
+    int* const links = chain_lds + capacity * (chb_entry_ints<T>() - 1);
+    int* head = links + capacity;
     for (int t = tid; t < t1 - t0; t += CHB_THREADS)
         head[t] = -1;
+    if (tid == 0)
+        entries = 0;
     __syncthreads();
     constexpr int BATCH = 8; // index loads in flight per thread
     for (int j0 = tid; j0 < nother; j0 += BATCH * CHB_THREADS)
@@ -316,94 +339,162 @@ __global__ __launch_bounds__(CHB_THREADS) void chamfer_bwd_chains_kernel(
             const int j = j0 + u * CHB_THREADS;
             k[u] = j < nother ? other_idx[j] : -1;
         }
+        // (read by every lane, wanted or not: a wavefront's 64 consecutive points cost a few lines, where reads
+        // under the test cost as much as scattered ones - a lane at a time)
+        T ox[BATCH], oy[BATCH], oz[BATCH], og[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+        {
+            const int j = min(j0 + u * CHB_THREADS, nother - 1);
+            ox[u] = other[j * 3 + 0];
+            oy[u] = other[j * 3 + 1];
+            oz[u] = other[j * 3 + 2];
+            og[u] = other_g[j] * 2;
+        }
 #pragma unroll
         for (int u = 0; u < BATCH; ++u)
             if (k[u] >= t0 && k[u] < t1)
             {
-                const int j = j0 + u * CHB_THREADS;
-                next[j] = atomicExch(&head[k[u] - t0], j);
+                // (one request per entry: a request for all of a lane's entries of the batch at once - lanes
+                // asking for different numbers - was slower, 20 against 15.5 us)
+                const int e = atomicAdd(&entries, 1);
+                if (e < capacity)
+                {
+                    links[e] = atomicExch(&head[k[u] - t0], e);
+                    values[e * 4 + 0] = ox[u];
+                    values[e * 4 + 1] = oy[u];
+                    values[e * 4 + 2] = oz[u];
+                    values[e * 4 + 3] = og[u];
+                }
             }
     }
     __syncthreads();
-    // Several targets per lane at a time, so that their dependent reads (own index -> that point;
-    // chain head -> point -> next) travel together.
-    constexpr int TPT = 1;
-    for (int kb = t0 + tid; kb < t1; kb += TPT * CHB_THREADS)
+    const bool in_lds = entries <= capacity;
+    int* const next = chain_lds; // (chains of point numbers: links [nother], heads [range])
+    if (!in_lds)
     {
-        T px[TPT], py[TPT], pz[TPT], g[TPT], ax[TPT], ay[TPT], az[TPT];
-        int j2[TPT], j[TPT];
-#pragma unroll
-        for (int u = 0; u < TPT; ++u)
+        __syncthreads(); // (every wavefront has read the count)
+        head = chain_lds + nother;
+        for (int t = tid; t < t1 - t0; t += CHB_THREADS)
+            head[t] = -1;
+        __syncthreads();
+        for (int j0 = tid; j0 < nother; j0 += BATCH * CHB_THREADS)
         {
-            const int k = min(kb + u * CHB_THREADS, t1 - 1);
-            px[u] = own[k * 3 + 0];
-            py[u] = own[k * 3 + 1];
-            pz[u] = own[k * 3 + 2];
-            j2[u] = own_idx[k];
-            g[u] = own_g[k] * 2;
-            j[u] = kb + u * CHB_THREADS < t1 ? head[k - t0] : -1;
-        }
+            int k[BATCH];
 #pragma unroll
-        for (int u = 0; u < TPT; ++u)
-        {
-            ax[u] = g[u] * (px[u] - other[j2[u] * 3 + 0]);
-            ay[u] = g[u] * (py[u] - other[j2[u] * 3 + 1]);
-            az[u] = g[u] * (pz[u] - other[j2[u] * 3 + 2]);
-        }
-        // The chains are followed in LDS first, CHAIN links at a time, and the points they name are
-        // requested together: the reads from memory do not wait for one another.
-        constexpr int CHAIN = 2;
-        while (true)
-        {
-            bool any = false;
-#pragma unroll
-            for (int u = 0; u < TPT; ++u)
-                any = any || j[u] >= 0;
-            if (!any)
-                break;
-            int link[TPT][CHAIN];
-#pragma unroll
-            for (int u = 0; u < TPT; ++u)
-#pragma unroll
-                for (int l = 0; l < CHAIN; ++l)
-                {
-                    link[u][l] = j[u];
-                    j[u] = j[u] >= 0 ? next[j[u]] : -1;
-                }
-            T gj[TPT][CHAIN], ox[TPT][CHAIN], oy[TPT][CHAIN], oz[TPT][CHAIN];
-#pragma unroll
-            for (int u = 0; u < TPT; ++u)
-#pragma unroll
-                for (int l = 0; l < CHAIN; ++l)
-                {
-                    const int jj = link[u][l] >= 0 ? link[u][l] : 0;
-                    gj[u][l] = other_g[jj] * 2;
-                    ox[u][l] = other[jj * 3 + 0];
-                    oy[u][l] = other[jj * 3 + 1];
-                    oz[u][l] = other[jj * 3 + 2];
-                }
-#pragma unroll
-            for (int u = 0; u < TPT; ++u)
-#pragma unroll
-                for (int l = 0; l < CHAIN; ++l)
-                    if (link[u][l] >= 0)
-                    {
-                        ax[u] = ax[u] + -(gj[u][l] * (ox[u][l] - px[u]));
-                        ay[u] = ay[u] + -(gj[u][l] * (oy[u][l] - py[u]));
-                        az[u] = az[u] + -(gj[u][l] * (oz[u][l] - pz[u]));
-                    }
-        }
-#pragma unroll
-        for (int u = 0; u < TPT; ++u)
-        {
-            const int k = kb + u * CHB_THREADS;
-            if (k < t1)
+            for (int u = 0; u < BATCH; ++u)
             {
-                out[k * 3 + 0] = ax[u];
-                out[k * 3 + 1] = ay[u];
-                out[k * 3 + 2] = az[u];
+                const int j = j0 + u * CHB_THREADS;
+                k[u] = j < nother ? other_idx[j] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+                if (k[u] >= t0 && k[u] < t1)
+                {
+                    const int j = j0 + u * CHB_THREADS;
+                    next[j] = atomicExch(&head[k[u] - t0], j);
+                }
+        }
+        __syncthreads();
+    }
+    if (in_lds)
+    {
+        // Several targets per lane at a time, so that their dependent reads (own index -> that point) travel together.
+        constexpr int TPT = 4;
+        for (int kb = t0 + tid; kb < t1; kb += TPT * CHB_THREADS)
+        {
+            T px[TPT], py[TPT], pz[TPT], g[TPT];
+            int j2[TPT], j[TPT];
+#pragma unroll
+            for (int u = 0; u < TPT; ++u)
+            {
+                const int k = min(kb + u * CHB_THREADS, t1 - 1);
+                px[u] = own[k * 3 + 0];
+                py[u] = own[k * 3 + 1];
+                pz[u] = own[k * 3 + 2];
+                j2[u] = own_idx[k];
+                g[u] = own_g[k] * 2;
+                j[u] = kb + u * CHB_THREADS < t1 ? head[k - t0] : -1;
+            }
+            T qx[TPT], qy[TPT], qz[TPT];
+#pragma unroll
+            for (int u = 0; u < TPT; ++u)
+            {
+                qx[u] = other[j2[u] * 3 + 0];
+                qy[u] = other[j2[u] * 3 + 1];
+                qz[u] = other[j2[u] * 3 + 2];
+            }
+#pragma unroll
+            for (int u = 0; u < TPT; ++u)
+            {
+                T ax = g[u] * (px[u] - qx[u]);
+                T ay = g[u] * (py[u] - qy[u]);
+                T az = g[u] * (pz[u] - qz[u]);
+                int e = j[u];
+                while (e >= 0)
+                {
+                    const T vx = values[e * 4 + 0], vy = values[e * 4 + 1], vz = values[e * 4 + 2], vg = values[e * 4 + 3];
+                    e = links[e];
+                    ax = ax + -(vg * (vx - px[u]));
+                    ay = ay + -(vg * (vy - py[u]));
+                    az = az + -(vg * (vz - pz[u]));
+                }
+                const int k = kb + u * CHB_THREADS;
+                if (k < t1)
+                {
+                    out[k * 3 + 0] = ax;
+                    out[k * 3 + 1] = ay;
+                    out[k * 3 + 2] = az;
+                }
             }
         }
+        return;
+    }
+    for (int k = t0 + tid; k < t1; k += CHB_THREADS)
+    {
+        const T px = own[k * 3 + 0], py = own[k * 3 + 1], pz = own[k * 3 + 2];
+        const int j2 = own_idx[k];
+        const T g = own_g[k] * 2;
+        int j = head[k - t0];
+        T ax = g * (px - other[j2 * 3 + 0]);
+        T ay = g * (py - other[j2 * 3 + 1]);
+        T az = g * (pz - other[j2 * 3 + 2]);
+        {
+            // The chains are followed in LDS first, CHAIN links at a time, and the points they name are
+            // requested together: the reads from memory do not wait for one another.
+            constexpr int CHAIN = 2;
+            while (j >= 0)
+            {
+                int link[CHAIN];
+#pragma unroll
+                for (int l = 0; l < CHAIN; ++l)
+                {
+                    link[l] = j;
+                    j = j >= 0 ? next[j] : -1;
+                }
+                T gj[CHAIN], ox[CHAIN], oy[CHAIN], oz[CHAIN];
+#pragma unroll
+                for (int l = 0; l < CHAIN; ++l)
+                {
+                    const int jj = link[l] >= 0 ? link[l] : 0;
+                    gj[l] = other_g[jj] * 2;
+                    ox[l] = other[jj * 3 + 0];
+                    oy[l] = other[jj * 3 + 1];
+                    oz[l] = other[jj * 3 + 2];
+                }
+#pragma unroll
+                for (int l = 0; l < CHAIN; ++l)
+                    if (link[l] >= 0)
+                    {
+                        ax = ax + -(gj[l] * (ox[l] - px));
+                        ay = ay + -(gj[l] * (oy[l] - py));
+                        az = az + -(gj[l] * (oz[l] - pz));
+                    }
+            }
+        }
+        out[k * 3 + 0] = ax;
+        out[k * 3 + 1] = ay;
+        out[k * 3 + 2] = az;
     }
 }
 
@@ -492,18 +583,28 @@ int chamfer_bwd(int b, int n, int m, const T* xyz1, const T* xyz2, const int32_t
         splits = splits < 1 ? 1 : splits;
         while (larger + tpk_ceil_div(larger, splits) > CHB_LDS_INTS && splits < most)
             ++splits;
+        // (room for the entries a range expects - its share of the other cloud - and a third more)
+        auto with_entries = [&](int parts) {
+            const int64_t range = tpk_ceil_div(larger, parts);
+            return range + chb_entry_ints<T>() * (range + range / 3 + 64);
+        };
+        while (with_entries(splits) > CHB_LDS_INTS && splits < most)
+            ++splits;
         const int range1 = static_cast<int>(tpk_ceil_div(n, splits)), range2 = static_cast<int>(tpk_ceil_div(m, splits));
+        const int range = range1 > range2 ? range1 : range2;
         const int64_t groups = 2 * static_cast<int64_t>(b) * splits;
-        if (larger + (range1 > range2 ? range1 : range2) <= CHB_LDS_INTS && groups <= 0x7fffffffLL &&
-            static_cast<int64_t>(larger) * 3 <= 0x7fffffffLL)
+        if (larger + range <= CHB_LDS_INTS && groups <= 0x7fffffffLL && static_cast<int64_t>(larger) * 3 <= 0x7fffffffLL)
         {
-            const size_t lds = (static_cast<size_t>(larger) + (range1 > range2 ? range1 : range2)) * sizeof(int);
+            // every point of the other cloud as an entry where that fits; else all of the LDS
+            const int64_t all = range + static_cast<int64_t>(chb_entry_ints<T>()) * larger;
+            const int lds_ints = static_cast<int>(all <= CHB_LDS_INTS ? (all > larger + range ? all : larger + range) : CHB_LDS_INTS);
+            const size_t lds = static_cast<size_t>(lds_ints) * sizeof(int);
             const int allowed = allow_lds(chamfer_bwd_chains_kernel<T>, lds);
             if (allowed != TPK_OK)
                 return allowed;
             hipLaunchKernelGGL(chamfer_bwd_chains_kernel<T>, dim3(static_cast<unsigned>(groups)), dim3(CHB_THREADS), lds, s,
-                               n, m, b, splits, range1, range2, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2, grad_xyz1,
-                               grad_xyz2);
+                               n, m, b, splits, range1, range2, lds_ints, xyz1, xyz2, idx1, idx2, grad_dist1, grad_dist2,
+                               grad_xyz1, grad_xyz2);
             return tpk_launch_status();
         }
     }
