@@ -753,7 +753,7 @@ inline int bqb_window_shift(int64_t size_x)
 }
 static_assert((1 << 14) == CURVE_MAX_POINTS, "the larger window is what the ordering kernel holds at most");
 constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
-constexpr int BQB_BLOCKS = 64;     // bins, or blocks of bins, of one window that a ball's cube is cut into at most
+constexpr int BQB_BLOCKS = 64;     // bins, or blocks of bins, of one compact window that a ball's cube is cut into at most
 constexpr int BQB_DENSE_MIN_POINTS = 8192; // dense layout: clouds above this take the bin walk (smaller ones fit in LDS whole)
 constexpr int64_t BQB_DENSE_MIN_PAIRS = 40000000; // ... when the call has at least this many (query, point) pairs
 
@@ -783,7 +783,10 @@ __device__ __forceinline__ bool cube_misses(float v, float r, float lo, float sc
 // consecutive rows with dense_m consecutive queries each (no cloud_rows), a hit has squared distance < radius2
 // (strict), indices count from the cloud's first row, and the slots behind the last hit repeat the first hit
 // (0 without any) with distance -1.
-template <bool SORTED, bool DENSE>
+// COMPACT: the windows are neighbourhoods (the rows were brought into the coarse order first): a window whose box the
+// ball misses is passed over, and where a ball touches more than BQB_BLOCKS bins of a window it is cut into blocks of
+// bins instead of handing the query to the scan.
+template <bool SORTED, bool DENSE, bool COMPACT>
 __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     int size_x, int size_y, int window_shift, float radius, float radius2, int nsample, const float* __restrict__ x,
     const float* __restrict__ y, const float4* __restrict__ sorted_x, const int* __restrict__ bin_ends,
@@ -853,24 +856,26 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
             bin_range(uz, radius, origin.z, scale.z, fz, lz);
             // The cube's bins, or - where it touches more than BQB_BLOCKS of them - the aligned blocks of 2^3, 4^3 or
             // 8^3 bins it touches, or the whole window: such a block is one run of consecutive bins on the curve.
-            while ((lx - fx + 1) * (ly - fy + 1) * (lz - fz + 1) > BQB_BLOCKS)
-            {
-                ++level;
-                fx >>= 1, lx >>= 1, fy >>= 1, ly >>= 1, fz >>= 1, lz >>= 1;
-            }
+            if constexpr (COMPACT)
+                while ((lx - fx + 1) * (ly - fy + 1) * (lz - fz + 1) > BQB_BLOCKS)
+                {
+                    ++level;
+                    fx >>= 1, lx >>= 1, fy >>= 1, ly >>= 1, fz >>= 1, lz >>= 1;
+                }
             const int nx = lx - fx + 1, ny = ly - fy + 1;
             nbins = nx * ny * (lz - fz + 1);
             // (a window of a cloud in coarse order is a neighbourhood: most balls lie outside its box)
-            if (cube_misses(ux, radius, origin.x, scale.x) || cube_misses(uy, radius, origin.y, scale.y) ||
-                cube_misses(uz, radius, origin.z, scale.z))
-                nbins = 0;
+            if constexpr (COMPACT)
+                if (cube_misses(ux, radius, origin.x, scale.x) || cube_misses(uy, radius, origin.y, scale.y) ||
+                    cube_misses(uz, radius, origin.z, scale.z))
+                    nbins = 0;
             block = fx | (fy << 4) | (fz << 8) | ((nx - 1) << 12) | ((ny - 1) << 16) | (lane << 26);
         }
         const int pairs_before = wave_exclusive_sum(nbins);
         const int pairs = __builtin_amdgcn_readlane(pairs_before + nbins, TPK_WAVE - 1);
-        // (a ball that touches more than 512 blocks in all covers so much of its cloud that the scan in index
-        // order ends early)
-        serial = pairs > 8 * TPK_WAVE;
+        // (a ball that touches more than 512 bins or blocks in all - windows that span their cloud: more than 64
+        // bins of one window - covers so much of its cloud that the scan in index order ends early)
+        serial = pairs > 8 * TPK_WAVE || (!COMPACT && __ballot(nbins > TPK_WAVE) != 0);
         // 64 (window, bin) pairs at a time; nearly always there are no more than that
         auto walk_pairs = [&](int pair0) __attribute__((always_inline)) {
             // one descriptor per pair, written by the window's lane: a window's block holds a few bins, so a loop
@@ -885,7 +890,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
             // switched off hands out nothing)
             const int d = marks[lane];
             const int window = (d >> 26) & 63;
-            const int l = __shfl(level, window);
+            const int l = COMPACT ? __shfl(level, window) : 0;
             if (pair0 + lane < pairs)
             {
                 const int i = (d >> 20) & 63;
@@ -1546,14 +1551,11 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
     const int64_t blocks = tpk_ceil_div(size_y, WAVES);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    if (sorted)
-        hipLaunchKernelGGL((ball_query_bins_kernel<true, false>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
-                           static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
-                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist, 0, 0);
-    else
-        hipLaunchKernelGGL((ball_query_bins_kernel<false, false>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
-                           static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
-                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist, 0, 0);
+    auto kernel = sorted ? (coarse ? ball_query_bins_kernel<true, false, true> : ball_query_bins_kernel<true, false, false>)
+                         : (coarse ? ball_query_bins_kernel<false, false, true> : ball_query_bins_kernel<false, false, false>);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, static_cast<int>(size_x),
+                       static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y, px.sorted, px.bin_ends,
+                       px.grid, rows.rows, idx, dist, 0, 0);
     return tpk_launch_status();
 }
 
@@ -1611,7 +1613,8 @@ int tpk_grid_ball_query_dense(int b, int n, int m, float radius, float radius2, 
     const int64_t blocks = tpk_ceil_div(size_y, WAVES);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((ball_query_bins_kernel<false, true>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+    auto kernel = coarse ? ball_query_bins_kernel<false, true, true> : ball_query_bins_kernel<false, true, false>;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
                        static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, xyz,
                        new_xyz, px.sorted, px.bin_ends, px.grid, static_cast<const int2*>(nullptr), idx, dist, n, m);
     return tpk_launch_status();
