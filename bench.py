@@ -49,7 +49,7 @@ TRAFFIC_KERNELS = {
 VALU_KERNELS = {
     "fps": "fps_pruned_kernel<16, 1024, 4>",
     "ball_query_dense": "ball_query_dense_cells_kernel<false>",
-    "ball_query_partial_dense": "ball_query_bins_kernel<false, false, false>",
+    "ball_query_partial_dense": "ball_query_bins_kernel<false, false>",
     "three_nn": "three_nn_cells_kernel",
     "chamfer_fwd": "chamfer_grid_kernel",
 }

@@ -385,54 +385,6 @@ def test_ball_query_partial_cell_search_parity(tpk, oracle, dev, sizes, qfrac, r
     np.testing.assert_array_equal(_np(dist), wd)
 
 
-@pytest.mark.parametrize("r,ns", [(0.008, 16), (0.03, 24), (0.06, 8)])
-def test_ball_query_partial_coarse_order(tpk, oracle, dev, r, ns):
-    # A packed array of 262144 rows or more with 131072 queries or more: the clouds of 65536 points or more are
-    # brought into a coarse order first, so that a window of 16384 rows is a neighbourhood; small clouds between
-    # them keep their places.  Radii: a few bins of a window per ball; more bins than the walk takes one by one
-    # (blocks of 8 or 64 bins); more than 64 points per ball in the large clouds (the scan in index order).
-    # The answer of a query does not depend on the other queries: every third query, asked alone, takes the walk
-    # without the coarse order (which the tests above pin against the oracle); every 97th is compared with the
-    # oracle directly.
-    sizes = (70000, 300, 16000, 180000) + (50,) * 20 + (66000, 9)
-    x, y, bx, by = _packed_case(5, sizes, 0.5, 0.0007)
-    y, by = torch.cat([y, y + 0.004]), torch.cat([by, by])
-    order = torch.sort(by, stable=True).indices
-    y, by = y[order].contiguous(), by[order].contiguous()
-    assert x.shape[0] >= 262144 and y.shape[0] >= 131072
-    xd, bxd = x.to(dev), bx.to(dev)
-    idx, dist = tpk.ball_query(r, ns, xd, y.to(dev), mode="partial_dense", batch_x=bxd, batch_y=by.to(dev))
-    part = slice(1, None, 3)
-    idx3, dist3 = tpk.ball_query(r, ns, xd, y[part].contiguous().to(dev), mode="partial_dense", batch_x=bxd,
-                                 batch_y=by[part].contiguous().to(dev))
-    assert y[part].shape[0] < 131072
-    np.testing.assert_array_equal(_np(idx)[part], _np(idx3))
-    np.testing.assert_array_equal(_np(dist)[part], _np(dist3))
-    few = slice(5, None, 97)
-    wi, wd = oracle.ball_query_partial_dense(r, ns, x.numpy(), y[few].contiguous().numpy(), bx.numpy(), by[few].contiguous().numpy())
-    np.testing.assert_array_equal(_np(idx)[few], wi)
-    np.testing.assert_array_equal(_np(dist)[few], wd)
-
-
-@pytest.mark.parametrize("B,N,M,r,ns", [(1, 300000, 140000, 0.012, 16), (2, 270000, 70000, 0.035, 12)])
-def test_ball_query_dense_coarse_order(tpk, oracle, dev, B, N, M, r, ns):
-    # the same for the dense layout: clouds of 262144 points or more with 131072 queries or more in all
-    g = torch.Generator().manual_seed(N + M)
-    xyz = torch.rand(B, N, 3, generator=g)
-    xyz[:, : N // 3] = xyz[:, : N // 3] * 0.2 + 0.4  # a third of every cloud in a fifth of its extent
-    new_xyz = (xyz[:, torch.randperm(N, generator=g)[:M]] + 0.002 * torch.randn(B, M, 3, generator=g)).contiguous()
-    idx, dist = tpk.ball_query(r, ns, xyz.to(dev), new_xyz.to(dev), mode="dense")
-    half = new_xyz[:, ::3].contiguous()
-    assert B * half.shape[1] < 131072
-    idx3, dist3 = tpk.ball_query(r, ns, xyz.to(dev), half.to(dev), mode="dense")
-    np.testing.assert_array_equal(_np(idx)[:, ::3], _np(idx3))
-    np.testing.assert_array_equal(_np(dist)[:, ::3], _np(dist3))
-    few = new_xyz[:, 7::211].contiguous()
-    wi, wd = oracle.ball_query_dense(r, ns, xyz.numpy(), few.numpy())
-    np.testing.assert_array_equal(_np(idx)[:, 7::211], wi)
-    np.testing.assert_array_equal(_np(dist)[:, 7::211], wd)
-
-
 def test_ball_query_partial_cell_search_edges(tpk, oracle, dev):
     g = torch.Generator().manual_seed(21)
     # points exactly on the sphere count (<=); duplicated support points; a query cloud without support

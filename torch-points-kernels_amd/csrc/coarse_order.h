@@ -1,21 +1,19 @@
-// A coarse spatial order for clouds of many windows.
+// A coarse spatial order for clouds of more than one window.
 //
 // The ordering kernel (curve_cells.h) orders windows of at most CURVE_MAX_POINTS consecutive points.  A cloud of
-// many windows, taken as it comes, gives windows that each span the whole cloud: a search looks into all of them.
-// Here the rows of every large cloud - from a number of rows the caller names, more than one chunk - are first brought into the order of the 4096
-// cells of a 16^3 grid over the cloud's bounding box, along the same curve as inside a window, so that consecutive
-// windows of the result are compact neighbourhoods; the ordering kernel then reads the result instead of the
-// caller's array.  The result is an array of records (x, y, z, number the row had): rows of smaller clouds keep
-// their places, a large cloud's rows are permuted among its own places, so the rows of a cloud remain the same
-// range of the array.
+// several windows, taken as it comes, gives windows that each span the whole cloud, and cells of 64 points as wide
+// as if the cloud had 16384 points.  Here the rows of every cloud of a batch - clouds of the same size, more than
+// one chunk each - are first brought into the order of the 4096 cells of a 16^3 grid over the cloud's bounding
+// box, along the same curve as inside a window, so that consecutive windows of the result are compact
+// neighbourhoods; the ordering kernel then reads the result instead of the caller's array.  The result is an array
+// of records (x, y, z, number the row had inside its cloud); a cloud's rows are permuted among its own places.
 //
-// A counting sort over chunks of CO_CHUNK rows, four launches: (1) every chunk finds the (at most two) large
-// clouds it holds rows of - the cloud of its first row and the cloud of its last row; a cloud that lies inside
-// a chunk is not large - and the bounding box of its rows of either; (2) every chunk forms the boxes of its clouds
-// from the chunks' boxes, counts its rows per cell and gives every row its rank among the chunk's rows of the
-// same cell; (3) one workgroup per large cloud turns the counts of the cloud's chunks into first places, cell after
-// cell and inside a cell chunk after chunk; (4) every row goes to its place.  Clouds are either given by a sorted
-// id per row (packed layout: the ends of the two clouds are found by binary search) or all of the same size.
+// A counting sort over chunks of CO_CHUNK rows of the batch, four launches: (1) every chunk finds the bounding box
+// of its rows of either of the (at most two) clouds it holds rows of - the cloud of its first row and the cloud of
+// its last row; (2) every chunk forms the boxes of its clouds from the chunks' boxes, counts its rows per cell and
+// gives every row its rank among the chunk's rows of the same cell; (3) one workgroup per cloud turns the counts of
+// the cloud's chunks into first places, cell after cell and inside a cell chunk after chunk; (4) every row goes to
+// its place.
 #pragma once
 
 #include "curve_cells.h"
@@ -27,21 +25,17 @@ constexpr int CO_CHUNK = CURVE_MAX_POINTS;
 constexpr int CO_PER = CO_CHUNK / CO_THREADS;
 constexpr int CO_SHIFT = 14;
 static_assert((1 << CO_SHIFT) == CO_CHUNK, "a place is (cell << CO_SHIFT) | rank");
-constexpr int CO_MIN_ROWS = CO_CHUNK + 1; // the fewest rows a caller may call large: a cloud inside a chunk never is
-constexpr unsigned CO_STAYS = 0xFFFFFFFFu;                           // place of a row that keeps its place
+constexpr int CO_MIN_ROWS = CO_CHUNK + 1; // rows of a cloud at least: a chunk then holds rows of two clouds at most
 
 struct CoarseOrder
 {
     const float* xyz;     // [rows][3]
-    const int64_t* batch; // sorted cloud id per row, or nullptr: clouds of cloud_rows consecutive rows
-    int rows;
-    int cloud_rows;       // (without ids)
-    int number_in_cloud;  // records carry the row's number inside its cloud instead of in the array (without ids)
-    int large;            // a cloud is large from this many rows on (>= CO_MIN_ROWS)
+    int rows;             // of the batch: clouds of cloud_rows consecutive rows
+    int cloud_rows;
     float4* records;      // out [rows]
-    unsigned* places;     // [rows] (cell << CO_SHIFT) | rank among the chunk's rows of the cell, or CO_STAYS
-    int4* spans;          // [chunks] rows [x, y) of the large cloud the chunk's first row lies in, [z, w) of another
-                          // large cloud that begins inside the chunk; (0, 0): none
+    unsigned* places;     // [rows] (cell << CO_SHIFT) | rank among the chunk's rows of the cell
+    int4* spans;          // [chunks] rows [x, y) of the cloud the chunk's first row lies in, [z, w) of the cloud that
+                          // begins inside the chunk; (0, 0): none
     int* boxes;           // [chunks][2][6] ordered ints: box of the chunk's rows of either cloud
     int* counts;          // [chunks][2][CURVE_BINS] rows per cell, then first places inside the cloud
 };
@@ -95,7 +89,7 @@ __global__ __launch_bounds__(CO_THREADS) void coarse_spans_kernel(CoarseOrder jo
     const int n = min(CO_CHUNK, job.rows - first);
     const float* __restrict__ xyz = job.xyz + static_cast<int64_t>(first) * 3;
 
-    // the rows of this thread: tid, tid + 1024, ... (requested before the clouds are known)
+    // the rows of this thread: tid, tid + 1024, ... (all requested before the first is used)
     float p[CO_PER][3];
 #pragma unroll
     for (int u = 0; u < CO_PER; ++u)
@@ -109,29 +103,14 @@ __global__ __launch_bounds__(CO_THREADS) void coarse_spans_kernel(CoarseOrder jo
         box[tid] = tid % 6 < 3 ? 0x7FFFFFFF : INT_MIN;
     if (tid < TPK_WAVE)
     {
-        int a0, a1, b0 = 0, b1 = 0;
         const int last = first + n - 1;
-        if (job.batch)
+        const int a0 = first / job.cloud_rows * job.cloud_rows, a1 = a0 + job.cloud_rows;
+        int b0 = 0, b1 = 0;
+        if (last >= a1)
         {
-            const int64_t id_a = job.batch[first], id_b = job.batch[last];
-            wave_equal_range(job.batch, job.rows, id_a, lane, a0, a1);
-            if (id_b != id_a) // (uniform over the wavefront)
-                wave_equal_range(job.batch, job.rows, id_b, lane, b0, b1);
+            b0 = a1;
+            b1 = b0 + job.cloud_rows;
         }
-        else
-        {
-            a0 = first / job.cloud_rows * job.cloud_rows;
-            a1 = a0 + job.cloud_rows;
-            if (last >= a1)
-            {
-                b0 = a1;
-                b1 = b0 + job.cloud_rows;
-            }
-        }
-        if (a1 - a0 < job.large)
-            a0 = a1 = 0;
-        if (b1 - b0 < job.large)
-            b0 = b1 = 0;
         if (tid == 0)
         {
             span = make_int4(a0, a1, b0, b1);
@@ -140,8 +119,6 @@ __global__ __launch_bounds__(CO_THREADS) void coarse_spans_kernel(CoarseOrder jo
     }
     __syncthreads();
     const int4 s = span;
-    if (s.y == 0 && s.w == 0)
-        return; // no row of a large cloud here
 #pragma unroll
     for (int slot = 0; slot < 2; ++slot)
     {
@@ -190,12 +167,6 @@ __global__ __launch_bounds__(CO_THREADS) void coarse_count_kernel(CoarseOrder jo
     const int first = chunk * CO_CHUNK;
     const int n = min(CO_CHUNK, job.rows - first);
     const int4 s = job.spans[chunk];
-    if (s.y == 0 && s.w == 0)
-    {
-        for (int k = tid; k < n; k += CO_THREADS)
-            job.places[first + k] = CO_STAYS;
-        return;
-    }
     const float* __restrict__ xyz = job.xyz + static_cast<int64_t>(first) * 3;
     float p[CO_PER][3];
 #pragma unroll
@@ -236,12 +207,10 @@ __global__ __launch_bounds__(CO_THREADS) void coarse_count_kernel(CoarseOrder jo
     for (int u = 0; u < CO_PER; ++u)
     {
         const int row = first + tid + u * CO_THREADS;
-        place[u] = CO_STAYS;
+        place[u] = 0;
         if (tid + u * CO_THREADS >= n)
             continue;
-        const bool in_a = row >= s.x && row < s.y, in_b = row >= s.z && row < s.w;
-        if (!in_a && !in_b)
-            continue;
+        const bool in_a = row < s.y; // (else in the second cloud)
         const CurveGrid& grid = in_a ? grid_a : grid_b;
         unsigned cell[3];
 #pragma unroll
@@ -260,7 +229,7 @@ __global__ __launch_bounds__(CO_THREADS) void coarse_count_kernel(CoarseOrder jo
             job.counts[static_cast<int64_t>(chunk) * 2 * CURVE_BINS + i] = (&counts[0][0])[i];
 }
 
-// (3) first places: workgroup 2 * chunk + slot serves the large cloud that begins in that chunk as that slot.
+// (3) first places: workgroup 2 * chunk + slot serves the cloud that begins in that chunk as that slot.
 __global__ __launch_bounds__(CO_THREADS) void coarse_scan_kernel(CoarseOrder job)
 {
     __shared__ int wave_totals[CO_THREADS / TPK_WAVE];
@@ -323,30 +292,22 @@ __global__ __launch_bounds__(CO_THREADS) void coarse_place_kernel(CoarseOrder jo
         const int row = first + k;
         const unsigned place = job.places[row];
         const float x = xyz[k * 3 + 0], y = xyz[k * 3 + 1], z = xyz[k * 3 + 2];
-        int to = row, number = row;
-        if (place != CO_STAYS)
-        {
-            const bool in_a = row >= s.x && row < s.y;
-            const int begin = in_a ? s.x : s.z;
-            to = begin + counts[(in_a ? 0 : CURVE_BINS) + (place >> CO_SHIFT)] + static_cast<int>(place & (CO_CHUNK - 1));
-        }
-        if (job.number_in_cloud)
-            number = row % job.cloud_rows;
-        job.records[to] = make_float4(x, y, z, __int_as_float(number));
+        const bool in_a = row < s.y;
+        const int begin = in_a ? s.x : s.z;
+        const int to = begin + counts[(in_a ? 0 : CURVE_BINS) + (place >> CO_SHIFT)] + static_cast<int>(place & (CO_CHUNK - 1));
+        job.records[to] = make_float4(x, y, z, __int_as_float(row - begin));
     }
 }
 
 // Enqueues the four kernels.  `scratch`: coarse_layout(rows).total bytes, 256-byte aligned; the records lie at its
 // start.
-inline int launch_coarse_order(const float* xyz, const int64_t* batch, int64_t rows, int64_t cloud_rows,
-                               bool number_in_cloud, int large, void* scratch, hipStream_t s)
+inline int launch_coarse_order(const float* xyz, int64_t rows, int64_t cloud_rows, void* scratch, hipStream_t s)
 {
-    if (rows <= 0 || rows >= (1LL << 30) || large < CO_MIN_ROWS || (!batch && (cloud_rows < large || cloud_rows > rows)))
+    if (rows <= 0 || rows >= (1LL << 30) || cloud_rows < CO_MIN_ROWS || cloud_rows > rows)
         return TPK_ERR_UNSUPPORTED;
     const CoarseLayout l = coarse_layout(rows);
     char* const w = static_cast<char*>(scratch);
-    CoarseOrder job{xyz, batch, static_cast<int>(rows), static_cast<int>(batch ? 0 : cloud_rows), number_in_cloud ? 1 : 0, large,
-                    reinterpret_cast<float4*>(w + l.records), reinterpret_cast<unsigned*>(w + l.places),
+    CoarseOrder job{xyz, static_cast<int>(rows), static_cast<int>(cloud_rows), reinterpret_cast<float4*>(w + l.records), reinterpret_cast<unsigned*>(w + l.places),
                     reinterpret_cast<int4*>(w + l.spans), reinterpret_cast<int*>(w + l.boxes),
                     reinterpret_cast<int*>(w + l.counts)};
     const unsigned chunks = static_cast<unsigned>(co_chunks(rows));

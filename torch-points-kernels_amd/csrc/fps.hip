@@ -1271,7 +1271,7 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
         if (n >= CO_MIN_ROWS)
         {
             // windows that are neighbourhoods instead of samples of the whole cloud: cells half as wide
-            st = launch_coarse_order(xyz, nullptr, static_cast<int64_t>(b) * n, n, true, CO_MIN_ROWS, w + l.coarse, s);
+            st = launch_coarse_order(xyz, static_cast<int64_t>(b) * n, n, w + l.coarse, s);
             if (st != TPK_OK)
                 return st;
             cloud.records = reinterpret_cast<const float4*>(w + l.coarse);

@@ -21,7 +21,7 @@
 // 160 bytes per cell (its box and those of its four runs of 16 points).  The curve ordering works
 // in LDS on at most 16384 points: a larger cloud (up to 163840 points) is ordered in windows of
 // 16384 consecutive points, which the search sees as more - and wider - cells of the same cloud.
-#include "coarse_order.h"
+#include "curve_cells.h"
 
 #include <algorithm>
 #include <cmath>
@@ -753,7 +753,6 @@ inline int bqb_window_shift(int64_t size_x)
 }
 static_assert((1 << 14) == CURVE_MAX_POINTS, "the larger window is what the ordering kernel holds at most");
 constexpr int BQB_HITS = TPK_WAVE; // hits a wavefront collects before it falls back to the scan
-constexpr int BQB_BLOCKS = 64;     // bins, or blocks of bins, of one compact window that a ball's cube is cut into at most
 constexpr int BQB_DENSE_MIN_POINTS = 8192; // dense layout: clouds above this take the bin walk (smaller ones fit in LDS whole)
 constexpr int64_t BQB_DENSE_MIN_PAIRS = 40000000; // ... when the call has at least this many (query, point) pairs
 
@@ -766,15 +765,6 @@ __device__ __forceinline__ void bin_range(float v, float r, float lo, float scal
     last = static_cast<int>(curve_grid_cell((v + r) + slack, lo, scale) >> 2);
 }
 
-// [v - r, v + r], widened the same way, lies wholly below or above the grid's extent along the axis: no point of
-// the window can lie within r of v.  (Grid coordinates run from 0 to 63.999; a window whose points share the
-// coordinate has scale 0 and is never ruled out.)
-__device__ __forceinline__ bool cube_misses(float v, float r, float lo, float scale)
-{
-    const float slack = (fabsf(v) + r) * 1e-6f + 1e-30f;
-    return (((v + r) + slack) - lo) * scale < 0.0f || (((v - r) - slack) - lo) * scale >= 64.0f;
-}
-
 // SORTED: the nsample (<= 64) NEAREST points with squared distance < radius2, nearest first, instead of the
 // first nsample in row order with squared distance <= radius2: the wavefront keeps its 64 best (distance, row)
 // keys sorted across the lanes and merges the hits of a step into them (as the wavefront-per-query kernel
@@ -783,10 +773,7 @@ __device__ __forceinline__ bool cube_misses(float v, float r, float lo, float sc
 // consecutive rows with dense_m consecutive queries each (no cloud_rows), a hit has squared distance < radius2
 // (strict), indices count from the cloud's first row, and the slots behind the last hit repeat the first hit
 // (0 without any) with distance -1.
-// COMPACT: the windows are neighbourhoods (the rows were brought into the coarse order first): a window whose box the
-// ball misses is passed over, and where a ball touches more than BQB_BLOCKS bins of a window it is cut into blocks of
-// bins instead of handing the query to the scan.
-template <bool SORTED, bool DENSE, bool COMPACT>
+template <bool SORTED, bool DENSE>
 __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     int size_x, int size_y, int window_shift, float radius, float radius2, int nsample, const float* __restrict__ x,
     const float* __restrict__ y, const float4* __restrict__ sorted_x, const int* __restrict__ bin_ends,
@@ -846,7 +833,7 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
     if (!serial && windows > 0)
     {
         // lane w: the block of bins that the ball's cube touches in window wx0 + w
-        int nbins = 0, block = 0, level = 0;
+        int nbins = 0, block = 0;
         if (lane < windows)
         {
             const float4 origin = grids[(wx0 + lane) * 2 + 0], scale = grids[(wx0 + lane) * 2 + 1];
@@ -854,28 +841,15 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
             bin_range(ux, radius, origin.x, scale.x, fx, lx);
             bin_range(uy, radius, origin.y, scale.y, fy, ly);
             bin_range(uz, radius, origin.z, scale.z, fz, lz);
-            // The cube's bins, or - where it touches more than BQB_BLOCKS of them - the aligned blocks of 2^3, 4^3 or
-            // 8^3 bins it touches, or the whole window: such a block is one run of consecutive bins on the curve.
-            if constexpr (COMPACT)
-                while ((lx - fx + 1) * (ly - fy + 1) * (lz - fz + 1) > BQB_BLOCKS)
-                {
-                    ++level;
-                    fx >>= 1, lx >>= 1, fy >>= 1, ly >>= 1, fz >>= 1, lz >>= 1;
-                }
             const int nx = lx - fx + 1, ny = ly - fy + 1;
             nbins = nx * ny * (lz - fz + 1);
-            // (a window of a cloud in coarse order is a neighbourhood: most balls lie outside its box)
-            if constexpr (COMPACT)
-                if (cube_misses(ux, radius, origin.x, scale.x) || cube_misses(uy, radius, origin.y, scale.y) ||
-                    cube_misses(uz, radius, origin.z, scale.z))
-                    nbins = 0;
             block = fx | (fy << 4) | (fz << 8) | ((nx - 1) << 12) | ((ny - 1) << 16) | (lane << 26);
         }
         const int pairs_before = wave_exclusive_sum(nbins);
         const int pairs = __builtin_amdgcn_readlane(pairs_before + nbins, TPK_WAVE - 1);
-        // (a ball that touches more than 512 bins or blocks in all - windows that span their cloud: more than 64
-        // bins of one window - covers so much of its cloud that the scan in index order ends early)
-        serial = pairs > 8 * TPK_WAVE || (!COMPACT && __ballot(nbins > TPK_WAVE) != 0);
+        // (a ball that touches more than 64 bins of one window, or 512 in all, covers so much of
+        // its cloud that the scan in index order ends early)
+        serial = __ballot(nbins > TPK_WAVE) != 0 || pairs > 8 * TPK_WAVE;
         // 64 (window, bin) pairs at a time; nearly always there are no more than that
         auto walk_pairs = [&](int pair0) __attribute__((always_inline)) {
             // one descriptor per pair, written by the window's lane: a window's block holds a few bins, so a loop
@@ -886,14 +860,10 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 marks[pairs_before + i - pair0] = block | (i << 20);
             // lane p: where the points of pair pair0 + p start in the ordered array, and how many
             int start = 0, size = 0;
-            // (the level of a pair's window sits in the window's lane; fetched by all lanes: a lane that is
-            // switched off hands out nothing)
-            const int d = marks[lane];
-            const int window = (d >> 26) & 63;
-            const int l = COMPACT ? __shfl(level, window) : 0;
             if (pair0 + lane < pairs)
             {
-                const int i = (d >> 20) & 63;
+                const int d = marks[lane];
+                const int i = (d >> 20) & 63, window = (d >> 26) & 63;
                 const int fx = d & 15, fy = (d >> 4) & 15, fz = (d >> 8) & 15;
                 const int nx = ((d >> 12) & 15) + 1, ny = ((d >> 16) & 15) + 1;
                 const int wx = wx0 + window;
@@ -903,12 +873,10 @@ __global__ __launch_bounds__(NG_SCAN_THREADS) void ball_query_bins_kernel(
                 const int in_plane = i - iz * nx * ny;
                 const int iy = static_cast<int>((static_cast<float>(in_plane) + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(nx)));
                 const int ix = in_plane - iy * nx;
-                // (a block of level l: the 8^l bins from the position of its first cell, cut to a multiple of 8^l)
-                const unsigned span = 1u << (3 * l);
-                const unsigned bin = curve_bin_table.bin[((fx + ix) << l) | (((fy + iy) << l) << 4) | (((fz + iz) << l) << 8)] & ~(span - 1u);
+                const unsigned bin = curve_bin_table.bin[(fx + ix) | ((fy + iy) << 4) | ((fz + iz) << 8)];
                 const int* __restrict__ ends = bin_ends + static_cast<int64_t>(wx) * CURVE_BINS;
                 start = bin ? ends[bin - 1] : 0;
-                size = ends[bin + span - 1u] - start;
+                size = ends[bin] - start;
                 start += wx << window_shift;
             }
             const int before = wave_exclusive_sum(size);
@@ -1468,21 +1436,10 @@ namespace {
 
 struct BallLayout
 {
-    size_t sorted_x, bin_ends, grids, cloud_rows, coarse, total;
+    size_t sorted_x, bin_ends, grids, cloud_rows, total;
 };
 
-// When the support points are brought into the coarse order first (coarse_order.h): a query then looks into a
-// few windows instead of all windows of its cloud, 1.0 against 1.7 ns per query on a cloud of 300000 points, and
-// the four launches in front cost 45 - 60 us - they pay from about 65000 queries on (measured, 300000 points,
-// radius 0.02: 300000 queries 547 -> 355 us, 30000 queries 84 -> 114 us).  What the host knows of a packed array
-// is its length, not that of its clouds: `rows` is the array's length there, the cloud's in the dense layout.
-constexpr int BQB_COARSE_CLOUD = 4 * CO_CHUNK; // a cloud takes part from this many rows on
-inline bool ball_coarse_pays(int64_t rows, int64_t queries)
-{
-    return rows >= 262144 && queries >= 131072;
-}
-
-BallLayout ball_layout(int64_t size_x, int64_t size_y, bool coarse)
+BallLayout ball_layout(int64_t size_x, int64_t size_y)
 {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
     const size_t window = static_cast<size_t>(1) << bqb_window_shift(size_x);
@@ -1497,9 +1454,6 @@ BallLayout ball_layout(int64_t size_x, int64_t size_y, bool coarse)
     pos = up(pos + wx * 2 * sizeof(float4));
     l.cloud_rows = pos;
     pos = up(pos + static_cast<size_t>(size_y) * sizeof(int2));
-    l.coarse = pos;
-    if (coarse)
-        pos = up(pos + coarse_layout(size_x).total);
     l.total = pos;
     return l;
 }
@@ -1514,7 +1468,7 @@ bool ball_bins_supported(int64_t size_x, int64_t size_y, int nsample)
 
 size_t tpk_grid_ball_query_workspace_bytes(int64_t size_x, int64_t size_y, int nsample)
 {
-    return ball_bins_supported(size_x, size_y, nsample) ? ball_layout(size_x, size_y, ball_coarse_pays(size_x, size_y)).total : 0;
+    return ball_bins_supported(size_x, size_y, nsample) ? ball_layout(size_x, size_y).total : 0;
 }
 
 int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, float radius2, int nsample, bool sorted,
@@ -1524,8 +1478,7 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
 {
     if (!ball_bins_supported(size_x, size_y, nsample) || (sorted && nsample > TPK_WAVE))
         return TPK_ERR_UNSUPPORTED;
-    const bool coarse = ball_coarse_pays(size_x, size_y);
-    const BallLayout l = ball_layout(size_x, size_y, coarse);
+    const BallLayout l = ball_layout(size_x, size_y);
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
@@ -1535,27 +1488,21 @@ int tpk_grid_ball_query_partial(int64_t size_x, int64_t size_y, float radius, fl
                 reinterpret_cast<int*>(w + l.bin_ends), reinterpret_cast<float4*>(w + l.grids)};
     PointSet none{nullptr, nullptr, 0, 1, CURVE_MAX_POINTS, nullptr, nullptr, nullptr, nullptr};
     const CloudRows rows{batch_x, batch_y, static_cast<int>(size_x), size_y, reinterpret_cast<int2*>(w + l.cloud_rows)};
-    int st = TPK_OK;
-    if (coarse)
-    {
-        // large clouds first into a coarse order of their own, so that their windows are compact
-        st = launch_coarse_order(x, batch_x, size_x, 0, false, BQB_COARSE_CLOUD, w + l.coarse, s);
-        if (st != TPK_OK)
-            return st;
-        px.records = reinterpret_cast<const float4*>(w + l.coarse);
-    }
-    st = launch_curve_cells(px, none, nullptr, s, rows);
+    int st = launch_curve_cells(px, none, nullptr, s, rows);
     if (st != TPK_OK)
         return st;
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
     const int64_t blocks = tpk_ceil_div(size_y, WAVES);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    auto kernel = sorted ? (coarse ? ball_query_bins_kernel<true, false, true> : ball_query_bins_kernel<true, false, false>)
-                         : (coarse ? ball_query_bins_kernel<false, false, true> : ball_query_bins_kernel<false, false, false>);
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s, static_cast<int>(size_x),
-                       static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y, px.sorted, px.bin_ends,
-                       px.grid, rows.rows, idx, dist, 0, 0);
+    if (sorted)
+        hipLaunchKernelGGL((ball_query_bins_kernel<true, false>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+                           static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
+                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist, 0, 0);
+    else
+        hipLaunchKernelGGL((ball_query_bins_kernel<false, false>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+                           static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, x, y,
+                           px.sorted, px.bin_ends, px.grid, rows.rows, idx, dist, 0, 0);
     return tpk_launch_status();
 }
 
@@ -1579,7 +1526,7 @@ bool ball_bins_dense_supported(int b, int n, int m, int nsample)
 
 size_t tpk_grid_ball_query_dense_workspace_bytes(int b, int n, int m, int nsample)
 {
-    return ball_bins_dense_supported(b, n, m, nsample) ? ball_layout(static_cast<int64_t>(b) * n, 0, ball_coarse_pays(n, static_cast<int64_t>(b) * m)).total : 0;
+    return ball_bins_dense_supported(b, n, m, nsample) ? ball_layout(static_cast<int64_t>(b) * n, 0).total : 0;
 }
 
 int tpk_grid_ball_query_dense(int b, int n, int m, float radius, float radius2, int nsample, const float* new_xyz,
@@ -1589,8 +1536,7 @@ int tpk_grid_ball_query_dense(int b, int n, int m, float radius, float radius2, 
     if (!ball_bins_dense_supported(b, n, m, nsample))
         return TPK_ERR_UNSUPPORTED;
     const int64_t size_x = static_cast<int64_t>(b) * n, size_y = static_cast<int64_t>(b) * m;
-    const bool coarse = ball_coarse_pays(n, size_y);
-    const BallLayout l = ball_layout(size_x, 0, coarse);
+    const BallLayout l = ball_layout(size_x, 0);
     if (!workspace || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return TPK_ERR_WORKSPACE;
     char* w = static_cast<char*>(workspace);
@@ -1598,23 +1544,14 @@ int tpk_grid_ball_query_dense(int b, int n, int m, float radius, float radius2, 
     PointSet px{xyz, nullptr, size_x, size_x, 1 << window_shift, reinterpret_cast<float4*>(w + l.sorted_x), nullptr,
                 reinterpret_cast<int*>(w + l.bin_ends), reinterpret_cast<float4*>(w + l.grids)};
     PointSet none{nullptr, nullptr, 0, 1, CURVE_MAX_POINTS, nullptr, nullptr, nullptr, nullptr};
-    int st = TPK_OK;
-    if (coarse)
-    {
-        st = launch_coarse_order(xyz, nullptr, size_x, n, false, BQB_COARSE_CLOUD, w + l.coarse, s);
-        if (st != TPK_OK)
-            return st;
-        px.records = reinterpret_cast<const float4*>(w + l.coarse);
-    }
-    st = launch_curve_cells(px, none, nullptr, s);
+    int st = launch_curve_cells(px, none, nullptr, s);
     if (st != TPK_OK)
         return st;
     constexpr int WAVES = NG_SCAN_THREADS / TPK_WAVE;
     const int64_t blocks = tpk_ceil_div(size_y, WAVES);
     if (blocks > 0x7fffffffLL)
         return TPK_ERR_UNSUPPORTED;
-    auto kernel = coarse ? ball_query_bins_kernel<false, true, true> : ball_query_bins_kernel<false, true, false>;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
+    hipLaunchKernelGGL((ball_query_bins_kernel<false, true>), dim3(static_cast<unsigned>(blocks)), dim3(NG_SCAN_THREADS), 0, s,
                        static_cast<int>(size_x), static_cast<int>(size_y), window_shift, std::fabs(radius), radius2, nsample, xyz,
                        new_xyz, px.sorted, px.bin_ends, px.grid, static_cast<const int2*>(nullptr), idx, dist, n, m);
     return tpk_launch_status();
