@@ -1188,6 +1188,11 @@ struct CellLayout
     int cells; // per cloud
     size_t sorted, boxes, temp, coarse, total;
 };
+// Clouds of more than one window are brought into a coarse order first (coarse_order.h), in batches it can index.
+bool fps_coarse_first(int b, int n)
+{
+    return n >= CO_MIN_ROWS && static_cast<int64_t>(b) * n < (1LL << 30);
+}
 CellLayout cell_layout(int b, int n)
 {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
@@ -1198,8 +1203,7 @@ CellLayout cell_layout(int b, int n)
     l.boxes = up(all * NG_CELL * sizeof(float4));
     l.temp = up(l.boxes + all * NG_BOX * sizeof(float4));
     l.coarse = up(l.temp + all * NG_CELL * sizeof(float));
-    // (clouds of many windows are brought into a coarse order first: coarse_order.h)
-    l.total = n >= CO_MIN_ROWS ? up(l.coarse + coarse_layout(static_cast<int64_t>(b) * n).total) : l.coarse;
+    l.total = fps_coarse_first(b, n) ? up(l.coarse + coarse_layout(static_cast<int64_t>(b) * n).total) : l.coarse;
     return l;
 }
 
@@ -1268,7 +1272,7 @@ extern "C" int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* wor
                        reinterpret_cast<float4*>(w + l.sorted), reinterpret_cast<float4*>(w + l.boxes), nullptr, nullptr};
         PointSet none{nullptr, nullptr, 0, 1, FPS_CELL_WINDOW, nullptr, nullptr, nullptr, nullptr};
         int st = TPK_OK;
-        if (n >= CO_MIN_ROWS)
+        if (fps_coarse_first(b, n))
         {
             // windows that are neighbourhoods instead of samples of the whole cloud: cells half as wide
             st = launch_coarse_order(xyz, static_cast<int64_t>(b) * n, n, w + l.coarse, s);
