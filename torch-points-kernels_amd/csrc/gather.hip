@@ -195,6 +195,10 @@ constexpr int GB_LDS_FLOATS = TPK_LDS_BYTES / 4; // floats of LDS a workgroup of
 constexpr int GB_STAGE_FLOATS = 32768; // at most this many of them hold the staged piece of grad_out (128 KiB)
 constexpr int GB_FETCH = GB_STAGE_FLOATS / 4 / G_THREADS; // 16-byte loads per lane that bring in a piece: 8
 constexpr int GB_AHEAD = 8;            // rows of list entries a wavefront has requested ahead of the one it adds
+constexpr int GB_HOLD = 36;            // rows of list entries a lane keeps in registers where a piece's entries are held
+// The walk that holds a piece's entries in registers: one row per pass, 4-byte entries.
+template <int K, bool WEIGHTED, int R>
+constexpr bool GB_HOLD_FOR = K == 1 && !WEIGHTED && R == 1;
 
 typedef int int2_vec __attribute__((ext_vector_type(2)));
 
@@ -273,7 +277,8 @@ __device__ __forceinline__ void carried_in(const float (&open)[R], bool starts, 
 // grad_out streams from memory while the lists are walked: every lane requests its 16-byte loads of
 // the NEXT piece into registers during the walk (a wavefront's loads complete in order, so the entry
 // requests behind them wait for them: every wavefront does this at another point of its walk) and
-// writes them to LDS between the two barriers that end the piece.
+// writes them to LDS between the two barriers that end the piece.  (Lists without weights over whole rows, one
+// row per pass: the entries of a piece fit in registers and are requested a piece ahead - see GB_HOLD_FOR.)
 // dynamic LDS: R * part_len floats (the piece) + R * L_SPANS * span floats (the sums).
 template <int K, bool WEIGHTED, int R>
 __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
@@ -362,6 +367,121 @@ __global__ __launch_bounds__(G_THREADS, 1) void gather_bwd_lists_kernel(
         }
     };
 
+    if constexpr (GB_HOLD_FOR<K, WEIGHTED, R>)
+    {
+        // Entries held in registers (this instance: 4-byte entries, whole rows as pieces).  A wavefront's loads
+        // complete in order, so an entry requested behind the 16-byte loads of the next piece waits for that
+        // piece - for most of the time a piece takes.  Here a piece's entries are all requested before the next
+        // piece is, right after the walk of the piece before, and kept in registers: the walk itself then asks
+        // memory for nothing, and the next piece is requested at its very beginning, by all wavefronts at once.
+        // (Spans of more than GB_HOLD rows of entries fetch the rest one row at a time.)
+        if (vector_loads)
+        {
+            struct Span
+            {
+                __amdgpu_buffer_rsrc_t ebuf;
+                uint32_t first;
+                int steps, first_slot;
+            };
+            auto describe = [&](int piece) __attribute__((always_inline)) {
+                const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
+                const int64_t cloud_part = static_cast<int64_t>(unit / row_groups) * parts + part;
+                const int4 region = lists.regions[cloud_part * L_SPANS + wave];
+                Span sp;
+                sp.steps = __builtin_amdgcn_readfirstlane(region.z);
+                sp.first_slot = (lists.first_target[(cloud_part * L_SPANS + wave) * TPK_WAVE + lane] - t0) * (R * 4);
+                sp.ebuf = memory_buffer(lists.entries + cloud_part * lists.capacity, static_cast<uint32_t>(lists.capacity) * ENTRY_BYTES);
+                sp.first = (static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(region.x)) + static_cast<uint32_t>(lane)) * ENTRY_BYTES;
+                return sp;
+            };
+            auto entry = [&](const Span& sp, int i) __attribute__((always_inline)) {
+                const uint32_t row = static_cast<uint32_t>(min(i, sp.steps - 1)) * (TPK_WAVE * ENTRY_BYTES); // wave-uniform
+                return __builtin_amdgcn_raw_buffer_load_b32(sp.ebuf, sp.first, row, 0);
+            };
+            int held[GB_HOLD];
+            auto request_all = [&](const Span& sp) __attribute__((always_inline)) {
+                if (sp.steps > 0)
+                {
+#pragma unroll
+                    for (int u = 0; u < GB_HOLD; ++u)
+                        held[u] = entry(sp, u);
+                }
+            };
+            fetch(0);
+            Span cur = describe(0);
+            request_all(cur);
+            stage_fetched();
+            for (int piece = 0; piece < pieces; ++piece)
+            {
+                const int unit = unit0 + piece / parts, part = piece - (piece / parts) * parts;
+                const int cloud = unit / row_groups, c0 = (unit - cloud * row_groups) * R;
+                const int nrows = min(R, c - c0);
+                // (what the next piece's entries are found by, requested before the next piece itself)
+                Span next = cur;
+                if (piece + 1 < pieces)
+                    next = describe(piece + 1);
+                lds_barrier(); // the piece is in LDS
+                const char* const staged = reinterpret_cast<const char*>(rows);
+                char* const put_at = reinterpret_cast<char*>(sums);
+                float acc = 0.f;
+                int slot = cur.first_slot;
+                auto take = [&](int j) __attribute__((always_inline)) {
+                    acc += *reinterpret_cast<const float*>(staged + (static_cast<unsigned>(j) & 0x7fffffffu));
+                    const bool ends = j < 0; // the entry ends a list
+                    if (ends)
+                        *reinterpret_cast<float*>(put_at + slot) = acc;
+                    acc = ends ? 0.f : acc;
+                    slot += ends ? 4 : 0;
+                };
+                // The next piece is requested while this one is walked, a load every few steps: a compute unit takes
+                // requests at 64 bytes a clock, 2000 clocks for a piece, and a wavefront that issues its eight loads
+                // in one go stands still that long.
+                int next_source_rows;
+                unsigned next_len;
+                const float* __restrict__ next_source = piece + 1 < pieces ? piece_source(piece + 1, next_source_rows, next_len) : nullptr;
+                constexpr int EVERY = GB_HOLD / GB_FETCH; // steps between two loads
+#pragma unroll
+                for (int u = 0; u < GB_HOLD; ++u)
+                {
+                    if (u % EVERY == 0 && u / EVERY < GB_FETCH)
+                    {
+                        const unsigned col = (static_cast<unsigned>(u / EVERY) * G_THREADS + tid) * 4u;
+                        fetched[u / EVERY] = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (next_source && col < next_len)
+                            fetched[u / EVERY] = *reinterpret_cast<const float4*>(next_source + col);
+                    }
+                    if (u < cur.steps) // (wave-uniform)
+                        take(held[u]);
+                }
+                for (int i = GB_HOLD; i < cur.steps; ++i)
+                    take(entry(cur, i));
+                // the first list every lane ended, with what the lanes before carried into it
+                float open[1] = {acc}, carry[1];
+                const bool ended_one = slot != cur.first_slot;
+                carried_in<1>(open, ended_one, lane, carry);
+                if (ended_one)
+                    *reinterpret_cast<float*>(put_at + cur.first_slot) += carry[0];
+                float* __restrict__ d = grad_src + (static_cast<int64_t>(cloud) * c + c0) * m + t0;
+                for (int t = lane; t < width; t += TPK_WAVE)
+                {
+                    if (0 < nrows)
+                    {
+                        const float v = sums[t];
+                        float* const at = d + t;
+                        *at = part == 0 ? v : *at + v;
+                    }
+                }
+                // (the next piece's entries, behind the stores: requested before them, or one by one during the walk, the
+                // call was 2.5 us slower)
+                if (piece + 1 < pieces)
+                    request_all(next);
+                cur = next;
+                lds_barrier(); // everybody is done with the piece
+                stage_fetched();
+            }
+            return;
+        }
+    }
     if (vector_loads)
     {
         fetch(0);
