@@ -7,6 +7,7 @@ features bit-exact forward; gradients within rtol 1e-5 / atol 1e-6 of the oracle
 the scatter sums, whose terms the kernels add in another order - two units in the last place of the sum of the
 terms' magnitudes (needed by a handful of elements in 10^7: _assert_scatter_sum_close counts them).
 """
+import os
 import sys
 
 import numpy as np
@@ -32,6 +33,7 @@ def _np(t):
 
 
 REORDER_ULPS = 2.0  # allowance for a different order of summation, in units of 2^-23 * sum of |terms|
+TOLERANCE_LOG = os.path.join("gpurun_out", "gradient_tolerance.jsonl")  # one line per comparison
 
 
 def _assert_scatter_sum_close(got, want, abs_sum, where=""):
@@ -39,7 +41,7 @@ def _assert_scatter_sum_close(got, want, abs_sum, where=""):
     atomics: in no fixed order), the oracle in index order.  Both are fp32 sums of the same terms, so they
     agree to rtol/atol plus a reordering allowance proportional to the sum of the terms' magnitudes, which
     matters only where the terms cancel.  Returns (elements outside the strict bound, worst error in units
-    of 2^-23 * sum of |terms| among those) and appends them to gpurun_out/gradient_tolerance.jsonl."""
+    of 2^-23 * sum of |terms| among those) and appends them to the file TOLERANCE_LOG names."""
     import json
     import os
 
@@ -53,8 +55,8 @@ def _assert_scatter_sum_close(got, want, abs_sum, where=""):
               "worst_over_strict": float((err / strict).max()), "worst_outside_in_ulps_of_abs_sum": worst_ulps}
     print("[tolerance] %s" % json.dumps(record), file=sys.stderr, flush=True)
     try:
-        os.makedirs("gpurun_out", exist_ok=True)
-        with open(os.path.join("gpurun_out", "gradient_tolerance.jsonl"), "a") as f:
+        os.makedirs(os.path.dirname(TOLERANCE_LOG), exist_ok=True)
+        with open(TOLERANCE_LOG, "a") as f:
             f.write(json.dumps(record) + "\n")
     except OSError:
         pass
