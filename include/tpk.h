@@ -52,8 +52,8 @@ const char* tpk_status_string(int status);
  * `workspace` replaces the reference's `temp` tensor: it is needed only when n exceeds
  * what one workgroup keeps in registers (16384 points); tpk_fps_workspace_bytes() says how
  * many bytes (0 = none needed, NULL may be passed).  Up to 163840 points it also holds the
- * cloud in curve order (about 22 bytes per point); with 4 bytes per point or more, but less
- * than that, the call still works, several times slower.
+ * cloud in curve order and what orders it (45 - 52 bytes per point); with 4 bytes per point
+ * or more, but less than that, the call still works, several times slower.
  * ------------------------------------------------------------------------------------- */
 size_t tpk_fps_workspace_bytes(int b, int n);
 int tpk_fps_f32(int b, int n, int npoint, const float* xyz, void* workspace,
